@@ -1,0 +1,180 @@
+/*
+ * sparsetir_amd -- C ABI of the MI355X (gfx950) implementation of the kernels that
+ * SparseTIR generates for SpMM / SDDMM / BSR / RGMS, and of its format-decomposition pass.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and -1 on failure; stir_last_error() then gives
+ *     the reason (same convention as TVMAPISetLastError / TVMGetLastError,
+ *     include/tvm/runtime/c_runtime_api.h:181-190 of the reference).
+ *   - All index arrays are int32, all buffers are flat and contiguous, exactly the layout
+ *     the reference's lowered functions take (src/tir/transforms/lower_sparse_buffer.cc:46-58).
+ *   - "d_" parameters are device pointers on the current HIP device; others are host pointers.
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream).  Launches are
+ *     asynchronous, like the reference's ROCMWrappedFunc (src/runtime/rocm/rocm_module.cc:146-189).
+ *   - Kernels write into caller-owned outputs; outputs that are accumulated with atomics
+ *     (hyb, RGMS) must be zero-filled by the caller, as in the reference
+ *     (examples/spmm/bench_spmm.py:206, examples/rgms/rgcn/bench_rgcn_tensorcore.py:843).
+ */
+#ifndef SPARSETIR_AMD_H_
+#define SPARSETIR_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Message of the last failure on the calling thread. */
+const char* stir_last_error(void);
+
+/* Library version string. */
+const char* stir_version(void);
+
+/* ------------------------------------------------------------------ format pass (host) */
+
+/*
+ * ColumnPartHyb, src/sparse/format.cc:46-168 (Python: python/tvm/sparse/format.py:89-116).
+ * Two calls: _sizes fills nrows[num_col_parts*num_buckets] (ELL rows per (part, bucket),
+ * part-major); _fill writes, for k = part*num_buckets + bucket, row_indices[k] (nrows[k]),
+ * col_indices[k] and mask[k] (nrows[k]*buckets[bucket]) -- all host int32, fully written.
+ */
+int stir_column_part_hyb_sizes(int32_t num_rows, int32_t num_cols, const int32_t* indptr,
+                               const int32_t* indices, int32_t num_col_parts,
+                               const int32_t* buckets, int32_t num_buckets, int64_t* nrows);
+int stir_column_part_hyb_fill(int32_t num_rows, int32_t num_cols, const int32_t* indptr,
+                              const int32_t* indices, int32_t num_col_parts,
+                              const int32_t* buckets, int32_t num_buckets,
+                              int32_t* const* row_indices, int32_t* const* col_indices,
+                              int32_t* const* mask);
+
+/*
+ * CSFToELL3D, src/sparse/format.cc:180-343 (Python: python/tvm/sparse/format.py:142-170).
+ * _sizes fills groups[num_buckets]; _fill writes per bucket b: indptr[b] (num_rels+1),
+ * row_indices[b] (groups*rows_bkt[b]), col_indices[b] / mask[b] (groups*rows_bkt[b]*cols_bkt[b]).
+ */
+int stir_csf_to_ell3d_sizes(int32_t num_rels, const int32_t* indptr0, const int32_t* indices0,
+                            const int32_t* indptr1, const int32_t* indices1,
+                            const int32_t* rows_bkt, const int32_t* cols_bkt,
+                            int32_t num_buckets, int64_t* groups);
+int stir_csf_to_ell3d_fill(int32_t num_rels, const int32_t* indptr0, const int32_t* indices0,
+                           const int32_t* indptr1, const int32_t* indices1,
+                           const int32_t* rows_bkt, const int32_t* cols_bkt,
+                           int32_t num_buckets, int32_t* const* indptr,
+                           int32_t* const* row_indices, int32_t* const* col_indices,
+                           int32_t* const* mask);
+
+/*
+ * ConDense, src/sparse/format.cc:353-429 (Python: python/tvm/sparse/format.py:119-139).
+ * _sizes fills group_indptr[ceil(n/t)+1] and *num_groups; _fill writes tile_indices
+ * (num_groups*g) and mask (num_groups*t*g).
+ */
+int stir_condense_sizes(int32_t n, const int32_t* indptr, const int32_t* indices, int32_t t,
+                        int32_t g, int32_t* group_indptr, int64_t* num_groups);
+int stir_condense_fill(int32_t n, const int32_t* indptr, const int32_t* indices, int32_t t,
+                       int32_t g, int32_t* tile_indices, int32_t* mask);
+
+/* ---------------------------------------------------------------- format pass (device) */
+
+/*
+ * ColumnPartHyb on the GPU, bit-exact with the host routine above for CSR input whose
+ * column indices ascend within each row (the reference runs this on the CPU only,
+ * src/sparse/format.cc:58-59; unsorted rows are reported as an error here).
+ * d_workspace must hold stir_column_part_hyb_device_workspace_bytes(...) bytes and must
+ * stay untouched between the _sizes and the _fill call.  _sizes synchronises the stream
+ * to return nrows on the host; _fill writes device arrays through host tables of
+ * device pointers (k = part*num_buckets + bucket).
+ */
+size_t stir_column_part_hyb_device_workspace_bytes(int32_t num_rows, int32_t num_col_parts,
+                                                   int32_t num_buckets);
+int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols,
+                                      const int32_t* d_indptr, const int32_t* d_indices,
+                                      int32_t num_col_parts, const int32_t* buckets,
+                                      int32_t num_buckets, void* d_workspace, int64_t* nrows,
+                                      void* stream);
+int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols,
+                                     const int32_t* d_indptr, const int32_t* d_indices,
+                                     int32_t num_col_parts, const int32_t* buckets,
+                                     int32_t num_buckets, void* d_workspace,
+                                     int32_t* const* d_row_indices,
+                                     int32_t* const* d_col_indices, int32_t* const* d_mask,
+                                     void* stream);
+
+/* ------------------------------------------------------------------------------ kernels */
+
+/*
+ * CSR row-split SpMM fp32, C[i,:] = sum_p A[p] * B[indices[p],:].
+ * Argument list of the reference's built operator: [A, B, C, indptr, indices]
+ * (examples/spmm/bench_spmm_naive.py:121-129; lowered form
+ * tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:22-70).  Rows without
+ * nonzeros are written as zeros (the GPU schedule's init block, bench_spmm_naive.py:113).
+ */
+int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
+                      const float* d_B, float* d_C, const int32_t* d_indptr,
+                      const int32_t* d_indices, void* stream);
+
+/*
+ * hyb SpMM fp32: all ELL buckets of all column partitions in one launch.
+ * The reference specialises and builds one fused kernel per (graph, bucket list)
+ * (examples/spmm/bench_spmm.py:116-199); the plan is that built object.  Bucket k =
+ * part*num_buckets + bucket has width bucket_widths[bucket], nrows[k] ELL rows and the
+ * device arrays d_A[k] (nrows*width f32), d_rows[k] (nrows), d_cols[k] (nrows*width), the
+ * (A_k, rows_k, cols_k) triples of the reference's argument list (bench_spmm.py:208-222).
+ * A bucket is accumulated with atomics when num_col_parts > 1 or it is the last bucket of
+ * its partition, and stored otherwise (bench_spmm.py:170).  The plan keeps the pointers,
+ * not copies: the arrays must outlive it.
+ */
+typedef struct stir_hyb_plan stir_hyb_plan;
+int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,
+                         int32_t num_buckets, const int32_t* bucket_widths,
+                         const int64_t* nrows, const float* const* d_A,
+                         const int32_t* const* d_rows, const int32_t* const* d_cols);
+int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B, float* d_C,
+                      void* stream);
+int stir_hyb_plan_destroy(stir_hyb_plan* plan);
+
+/*
+ * SDDMM fp32.  _preproc is the reference's binary-search block: mid[e] = index of the row
+ * that owns nonzero e (tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:531-551);
+ * stir_sddmm_f32 computes C[e] = <A[mid[e],:], B[indices[e],:]> with the reference's
+ * argument list [A, B, C, indptr, indices, mid] (examples/sddmm/bench_sddmm.py:170).
+ */
+int stir_sddmm_preproc(int32_t m, int64_t nnz, const int32_t* d_indptr, int32_t* d_mid,
+                       void* stream);
+int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
+                   const float* d_B, float* d_C, const int32_t* d_indptr,
+                   const int32_t* d_indices, const int32_t* d_mid, void* stream);
+
+/*
+ * BSR SpMM on MFMA, 16-bit inputs, fp32 accumulation; argument list [A, X, Y, indptr,
+ * indices] of examples/blocksparse/bsr_spmm.py:427-432.  A: nnzb*blk*blk, X: nb*blk*feat,
+ * Y: mb*blk*feat.  dtype: STIR_F16 or STIR_BF16 for A and X; out_dtype: the same 16-bit
+ * type or STIR_F32.  blk must be 16 or 32 and feat a multiple of 32.
+ */
+enum { STIR_F16 = 0, STIR_BF16 = 1, STIR_F32 = 2 };
+int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk,
+                  int32_t feat, int64_t nnzb, const void* d_A, const void* d_X, void* d_Y,
+                  const int32_t* d_indptr, const int32_t* d_indices, void* stream);
+
+/*
+ * RGMS (relational gather-matmul-scatter), fp16 inputs, fp32 accumulation and output,
+ * on the ELL3D buckets produced by CSFToELL3D.  Mirrors the built operator of
+ * examples/rgms/rgcn/bench_rgcn_tensorcore.py:838-851: W is [R, feat_in, feat_out], X is
+ * [n, feat_in], Y (zero-filled by the caller) is [m, feat_out] fp32; per bucket b the
+ * arrays d_A[b] (groups*rb*cb fp16 edge weights, the 0/1 mask in the reference), d_rows[b]
+ * (groups*rb), d_cols[b] (groups*rb*cb) and d_mids[b] (groups: relation of each group).
+ */
+typedef struct stir_rgms_plan stir_rgms_plan;
+int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int32_t* rows_bkt,
+                          const int32_t* cols_bkt, const int64_t* groups,
+                          const void* const* d_A, const int32_t* const* d_rows,
+                          const int32_t* const* d_cols, const int32_t* const* d_mids);
+int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
+                  int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
+                  float* d_Y, void* stream);
+int stir_rgms_plan_destroy(stir_rgms_plan* plan);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSETIR_AMD_H_ */

@@ -1,0 +1,48 @@
+// Shared host-side helpers for the C ABI: last-error string and HIP status checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+namespace stir {
+
+// Thread-local message returned by stir_last_error(); the same convention as
+// TVMAPISetLastError / TVMGetLastError (include/tvm/runtime/c_runtime_api.h:181-190
+// in the reference): an entry point returns -1 after recording why.
+void set_error(const char* fmt, ...);
+const char* get_error();
+
+inline int fail(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+inline int fail(const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  set_error("%s", buf);
+  return -1;
+}
+
+}  // namespace stir
+
+#define STIR_HIP(expr)                                                                     \
+  do {                                                                                     \
+    hipError_t _e = (expr);                                                                \
+    if (_e != hipSuccess)                                                                  \
+      return stir::fail("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__,   \
+                        __LINE__);                                                         \
+  } while (0)
+
+#define STIR_REQUIRE(cond, ...)                   \
+  do {                                            \
+    if (!(cond)) return stir::fail(__VA_ARGS__);  \
+  } while (0)
+
+#define STIR_LAUNCH_CHECK() STIR_HIP(hipGetLastError())
+
+namespace stir {
+constexpr int kWave = 64;
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+}  // namespace stir

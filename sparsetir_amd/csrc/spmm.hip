@@ -1,0 +1,461 @@
+// CSR row-split SpMM and hyb (bucketed ELL) SpMM for gfx950, fp32.
+//
+// Both kernels are gathers of dense feature rows: per nonzero one row of B (feat*4 bytes)
+// is read, scaled and summed.  The feature row is spread over a "lane group" of G lanes,
+// each lane owning float4 chunks, so one wavefront (64 lanes) serves 64/G nonzeros per
+// step with fully coalesced 16-byte loads.  Column indices and values are fetched once per
+// wavefront with one coalesced load (lane l holds slot l of the 64-slot tile) and handed to
+// the lane groups through cross-lane reads, so no lane issues a redundant index load.
+#include "common.h"
+#include "../../include/sparsetir_amd.h"
+
+namespace {
+
+using stir::kWave;
+
+struct alignas(16) HybBucket {
+  const float* A;
+  const int32_t* rows;
+  const int32_t* cols;
+  int64_t nrows;
+  int64_t tile_begin;  // first wave tile of this bucket in the fused launch
+  int32_t width;
+  int32_t log2w;   // log2(width) when the bucket runs in slot-tile mode, else -1
+  int32_t atomic;  // accumulate with atomics instead of storing
+  int32_t pad;
+};
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+
+__device__ __forceinline__ void fma4(float4& acc, float a, const float4& x) {
+  acc.x = fmaf(a, x.x, acc.x);
+  acc.y = fmaf(a, x.y, acc.y);
+  acc.z = fmaf(a, x.z, acc.z);
+  acc.w = fmaf(a, x.w, acc.w);
+}
+
+__device__ __forceinline__ void atomic_add4(float* p, const float4& v) {
+  __hip_atomic_fetch_add(p + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_fetch_add(p + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_fetch_add(p + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_fetch_add(p + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Sum `acc` over the lane groups whose group index differs in the bits [G, limit).
+template <int G, int REP>
+__device__ __forceinline__ void reduce_groups(float4 (&acc)[REP], int limit) {
+#pragma unroll
+  for (int off = G; off < kWave; off <<= 1) {
+    if (off < limit) {
+#pragma unroll
+      for (int r = 0; r < REP; ++r) {
+        acc[r].x += __shfl_xor(acc[r].x, off, kWave);
+        acc[r].y += __shfl_xor(acc[r].y, off, kWave);
+        acc[r].z += __shfl_xor(acc[r].z, off, kWave);
+        acc[r].w += __shfl_xor(acc[r].w, off, kWave);
+      }
+    }
+  }
+}
+
+template <int G, int REP>
+__device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int gl,
+                                          const float4 (&acc)[REP], bool atomic) {
+  float* base = C + row * feat + gl * 4;
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    if (atomic)
+      atomic_add4(base + r * G * 4, acc[r]);
+    else
+      *reinterpret_cast<float4*>(base + r * G * 4) = acc[r];
+  }
+}
+
+// ----------------------------------------------------------------------------- CSR SpMM
+// One wavefront per row; the 64/G lane groups take the row's nonzeros round-robin and
+// their partial sums are combined with cross-lane adds at the end.
+template <int G, int REP>
+__global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, const float* __restrict__ A,
+                                                       const float* __restrict__ B,
+                                                       float* __restrict__ C,
+                                                       const int32_t* __restrict__ indptr,
+                                                       const int32_t* __restrict__ indices) {
+  constexpr int NG = kWave / G;
+  constexpr int UNROLL = 4;
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const int g = lane / G, gl = lane % G;
+  const int start = indptr[row], end = indptr[row + 1];
+  float4 acc[REP];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  for (int base = start; base < end; base += kWave) {
+    const int p = base + lane;
+    const int my_col = p < end ? indices[p] : 0;
+    const float my_val = p < end ? A[p] : 0.f;
+    const int cnt = min(kWave, end - base);
+    for (int j0 = 0; j0 < cnt; j0 += NG * UNROLL) {
+      float4 x[UNROLL][REP];
+      float v[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int j = j0 + u * NG + g;  // < 64 because NG*UNROLL divides 64
+        const int col = __shfl(my_col, j, kWave);
+        v[u] = __shfl(my_val, j, kWave);
+        const float* bp = B + (int64_t)col * feat + gl * 4;
+#pragma unroll
+        for (int r = 0; r < REP; ++r)
+          x[u][r] = (j < cnt) ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+        for (int r = 0; r < REP; ++r) fma4(acc[r], v[u], x[u][r]);
+    }
+  }
+  reduce_groups<G, REP>(acc, kWave);
+  if (g == 0) write_row<G, REP>(C, row, feat, gl, acc, false);
+}
+
+// Any feature width: one wavefront per row, lane l owns features l, l+64, ...
+__global__ __launch_bounds__(256) void csr_spmm_generic_kernel(int m, int feat, const float* __restrict__ A,
+                                                               const float* __restrict__ B,
+                                                               float* __restrict__ C,
+                                                               const int32_t* __restrict__ indptr,
+                                                               const int32_t* __restrict__ indices) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const int start = indptr[row], end = indptr[row + 1];
+  for (int f = lane; f < feat; f += kWave) {
+    float acc = 0.f;
+    for (int p = start; p < end; ++p) acc = fmaf(A[p], B[(int64_t)indices[p] * feat + f], acc);
+    C[(int64_t)row * feat + f] = acc;
+  }
+}
+
+// ----------------------------------------------------------------------------- hyb SpMM
+// Slot-tile mode (power-of-two width <= 64): a wavefront owns 64 consecutive ELL slots,
+// i.e. 64/width whole ELL rows.  Lane group g owns slots [g*G, g*G+G) of the tile.
+template <int G, int REP, int LOG2W>
+__device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, int feat,
+                                              const float* __restrict__ B, float* __restrict__ C,
+                                              int lane) {
+  constexpr int W = 1 << LOG2W;
+  constexpr int CH = G < 8 ? G : 8;  // gathers in flight per lane
+  const int g = lane / G, gl = lane % G;
+  const int64_t slot0 = t * kWave;
+  const int64_t nslots = bk.nrows << LOG2W;
+  const int64_t s = slot0 + lane;
+  const int my_col = s < nslots ? bk.cols[s] : 0;
+  const float my_val = s < nslots ? bk.A[s] : 0.f;
+  constexpr int ROWS = kWave >> LOG2W;  // ELL rows per tile
+  const int64_t row0 = slot0 >> LOG2W;
+  int my_row = -1;
+  if (lane < ROWS && row0 + lane < bk.nrows) my_row = bk.rows[row0 + lane];
+  const bool atomic = bk.atomic != 0;
+
+  float4 acc[REP];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  // The chunk loop stays rolled so that only CH gathers (not all G) are live at once.
+#pragma unroll 1
+  for (int c = 0; c < G; c += CH) {
+    float4 x[CH][REP];
+    float v[CH];
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+      const int sl = g * G + c + u;
+      const int col = __shfl(my_col, sl, kWave);
+      v[u] = __shfl(my_val, sl, kWave);
+      const float* bp = B + (int64_t)col * feat + gl * 4;
+#pragma unroll
+      for (int r = 0; r < REP; ++r) x[u][r] = ld4(bp + r * G * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < CH; ++u) {
+#pragma unroll
+      for (int r = 0; r < REP; ++r) fma4(acc[r], v[u], x[u][r]);
+      if constexpr (W <= G) {
+        // end of an ELL row inside this lane group; for W <= CH this folds to a constant
+        if (((c + u + 1) & (W - 1)) == 0) {
+          const int out_row = __shfl(my_row, (g * G + c + u) >> LOG2W, kWave);
+          if (out_row >= 0) write_row<G, REP>(C, out_row, feat, gl, acc, atomic);
+#pragma unroll
+          for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+    }
+  }
+  if constexpr (W > G) {
+    // an ELL row spans W/G lane groups: combine them, the first group of the row writes
+    reduce_groups<G, REP>(acc, W);
+    const int out_row = __shfl(my_row, (g * G) >> LOG2W, kWave);
+    if (((g * G) & (W - 1)) == 0 && out_row >= 0)
+      write_row<G, REP>(C, out_row, feat, gl, acc, atomic);
+  }
+}
+
+// Row mode (any width): a wavefront owns one ELL row and walks it 64 slots at a time.
+template <int G, int REP>
+__device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int feat,
+                                             const float* __restrict__ B, float* __restrict__ C,
+                                             int lane) {
+  constexpr int CH = G < 8 ? G : 8;
+  const int g = lane / G, gl = lane % G;
+  const int w = bk.width;
+  const int32_t* cols = bk.cols + t * w;
+  const float* vals = bk.A + t * w;
+  float4 acc[REP];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int c0 = 0; c0 < w; c0 += kWave) {
+    const int s = c0 + lane;
+    const int my_col = s < w ? cols[s] : 0;
+    const float my_val = s < w ? vals[s] : 0.f;
+#pragma unroll 1
+    for (int c = 0; c < G; c += CH) {
+      float4 x[CH][REP];
+      float v[CH];
+#pragma unroll
+      for (int u = 0; u < CH; ++u) {
+        const int sl = g * G + c + u;
+        const int col = __shfl(my_col, sl, kWave);
+        v[u] = __shfl(my_val, sl, kWave);
+        const float* bp = B + (int64_t)col * feat + gl * 4;
+        const bool live = c0 + sl < w;
+#pragma unroll
+        for (int r = 0; r < REP; ++r)
+          x[u][r] = live ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < CH; ++u)
+#pragma unroll
+        for (int r = 0; r < REP; ++r) fma4(acc[r], v[u], x[u][r]);
+    }
+  }
+  reduce_groups<G, REP>(acc, kWave);
+  if (g == 0) write_row<G, REP>(C, bk.rows[t], feat, gl, acc, bk.atomic != 0);
+}
+
+__device__ __forceinline__ int find_bucket(const HybBucket* __restrict__ table, int nb,
+                                           int64_t tile) {
+  int lo = 0, hi = nb - 1;  // largest k with tile_begin[k] <= tile
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[mid].tile_begin <= tile)
+      lo = mid;
+    else
+      hi = mid - 1;
+  }
+  return lo;
+}
+
+template <int G, int REP>
+__global__ __launch_bounds__(256) void hyb_spmm_kernel(const HybBucket* __restrict__ table, int nb,
+                                                       int64_t total_tiles, int feat,
+                                                       const float* __restrict__ B,
+                                                       float* __restrict__ C) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t tile = (int64_t)blockIdx.x * 4 + wave;
+  if (tile >= total_tiles) return;
+  const int k = find_bucket(table, nb, tile);
+  const HybBucket bk = table[k];
+  const int64_t t = tile - bk.tile_begin;
+  switch (bk.log2w) {
+    case 0: hyb_slot_tile<G, REP, 0>(bk, t, feat, B, C, lane); break;
+    case 1: hyb_slot_tile<G, REP, 1>(bk, t, feat, B, C, lane); break;
+    case 2: hyb_slot_tile<G, REP, 2>(bk, t, feat, B, C, lane); break;
+    case 3: hyb_slot_tile<G, REP, 3>(bk, t, feat, B, C, lane); break;
+    case 4: hyb_slot_tile<G, REP, 4>(bk, t, feat, B, C, lane); break;
+    case 5: hyb_slot_tile<G, REP, 5>(bk, t, feat, B, C, lane); break;
+    case 6: hyb_slot_tile<G, REP, 6>(bk, t, feat, B, C, lane); break;
+    default: hyb_row_tile<G, REP>(bk, t, feat, B, C, lane); break;
+  }
+}
+
+// Any feature width: one wavefront per ELL row, lane l owns features l, l+64, ...
+__global__ __launch_bounds__(256) void hyb_spmm_generic_kernel(const HybBucket* __restrict__ table,
+                                                               int nb, int64_t total_rows, int feat,
+                                                               const float* __restrict__ B,
+                                                               float* __restrict__ C) {
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= total_rows) return;
+  const int k = find_bucket(table, nb, tile);
+  const HybBucket bk = table[k];
+  const int64_t t = tile - bk.tile_begin;
+  const int w = bk.width;
+  const int64_t out_row = bk.rows[t];
+  for (int f = lane; f < feat; f += kWave) {
+    float acc = 0.f;
+    for (int s = 0; s < w; ++s)
+      acc = fmaf(bk.A[t * w + s], B[(int64_t)bk.cols[t * w + s] * feat + f], acc);
+    float* dst = C + out_row * feat + f;
+    if (bk.atomic)
+      __hip_atomic_fetch_add(dst, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+      *dst = acc;
+  }
+}
+
+int log2_exact(int64_t x) {
+  int l = 0;
+  while ((int64_t(1) << l) < x) ++l;
+  return l;
+}
+
+}  // namespace
+
+struct stir_hyb_plan {
+  int32_t m, n, num_col_parts, num_buckets;
+  int device;
+  int nk;                         // buckets with at least one ELL row
+  HybBucket* d_table_tiles;       // tile_begin counted in wave tiles (vectorised kernel)
+  HybBucket* d_table_rows;        // tile_begin counted in ELL rows (generic kernel)
+  int64_t total_tiles, total_rows;
+};
+
+extern "C" {
+
+int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
+                      const float* d_B, float* d_C, const int32_t* d_indptr,
+                      const int32_t* d_indices, void* stream) {
+  STIR_REQUIRE(m >= 0 && n >= 0 && feat > 0 && nnz >= 0, "csr_spmm: bad sizes m=%d n=%d feat=%d", m, n, feat);
+  if (m == 0) return 0;
+  STIR_REQUIRE(d_B && d_C && d_indptr && (nnz == 0 || (d_A && d_indices)), "csr_spmm: null pointer argument");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)stir::ceil_div(m, 4)), block(256);
+#define STIR_CSR(G, REP) \
+  hipLaunchKernelGGL((csr_spmm_kernel<G, REP>), grid, block, 0, st, m, feat, d_A, d_B, d_C, d_indptr, d_indices)
+  switch (feat) {
+    case 32: STIR_CSR(8, 1); break;
+    case 64: STIR_CSR(16, 1); break;
+    case 128: STIR_CSR(32, 1); break;
+    case 256: STIR_CSR(64, 1); break;
+    case 512: STIR_CSR(64, 2); break;
+    default:
+      hipLaunchKernelGGL(csr_spmm_generic_kernel, grid, block, 0, st, m, feat, d_A, d_B, d_C, d_indptr, d_indices);
+  }
+#undef STIR_CSR
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,
+                         int32_t num_buckets, const int32_t* bucket_widths, const int64_t* nrows,
+                         const float* const* d_A, const int32_t* const* d_rows,
+                         const int32_t* const* d_cols) {
+  STIR_REQUIRE(plan, "hyb_plan_create: plan is null");
+  STIR_REQUIRE(m >= 0 && n >= 0 && num_col_parts > 0 && num_buckets > 0, "hyb_plan_create: bad sizes");
+  for (int b = 0; b < num_buckets; ++b)
+    STIR_REQUIRE(bucket_widths[b] > 0, "hyb_plan_create: bucket width %d is not positive", bucket_widths[b]);
+  const int total = num_col_parts * num_buckets;
+  HybBucket* host = new HybBucket[total > 0 ? 2 * total : 1];
+  HybBucket* host_rows = host + total;
+  int nk = 0;
+  int64_t tiles = 0, rows = 0;
+  for (int k = 0; k < total; ++k) {
+    if (nrows[k] < 0) {
+      delete[] host;
+      return stir::fail("hyb_plan_create: nrows[%d] is negative", k);
+    }
+    if (nrows[k] == 0) continue;
+    if (!d_A[k] || !d_rows[k] || !d_cols[k]) {
+      delete[] host;
+      return stir::fail("hyb_plan_create: bucket %d has rows but a null array", k);
+    }
+    const int b = k % num_buckets;
+    const int w = bucket_widths[b];
+    HybBucket e;
+    e.A = d_A[k];
+    e.rows = d_rows[k];
+    e.cols = d_cols[k];
+    e.nrows = nrows[k];
+    e.width = w;
+    e.atomic = (num_col_parts > 1 || b == num_buckets - 1) ? 1 : 0;
+    e.pad = 0;
+    const bool slot_mode = stir::is_pow2(w) && w <= kWave;
+    e.log2w = slot_mode ? log2_exact(w) : -1;
+    e.tile_begin = tiles;
+    host[nk] = e;
+    tiles += slot_mode ? stir::ceil_div(nrows[k] * w, kWave) : nrows[k];
+    e.tile_begin = rows;
+    host_rows[nk] = e;
+    rows += nrows[k];
+    ++nk;
+  }
+  stir_hyb_plan* p = new stir_hyb_plan();
+  p->m = m;
+  p->n = n;
+  p->num_col_parts = num_col_parts;
+  p->num_buckets = num_buckets;
+  p->nk = nk;
+  p->total_tiles = tiles;
+  p->total_rows = rows;
+  p->d_table_tiles = nullptr;
+  p->d_table_rows = nullptr;
+  hipError_t e = hipGetDevice(&p->device);
+  if (e == hipSuccess && nk > 0) {
+    e = hipMalloc(reinterpret_cast<void**>(&p->d_table_tiles), sizeof(HybBucket) * 2 * nk);
+    if (e == hipSuccess) {
+      p->d_table_rows = p->d_table_tiles + nk;
+      e = hipMemcpy(p->d_table_tiles, host, sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
+      if (e == hipSuccess)
+        e = hipMemcpy(p->d_table_rows, host_rows, sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
+    }
+  }
+  delete[] host;
+  if (e != hipSuccess) {
+    if (p->d_table_tiles) (void)hipFree(p->d_table_tiles);
+    delete p;
+    return stir::fail("hyb_plan_create: %s", hipGetErrorString(e));
+  }
+  *plan = p;
+  return 0;
+}
+
+int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B, float* d_C,
+                      void* stream) {
+  STIR_REQUIRE(plan, "hyb_spmm: plan is null");
+  STIR_REQUIRE(feat > 0, "hyb_spmm: feat=%d", feat);
+  if (plan->nk == 0) return 0;
+  STIR_REQUIRE(d_B && d_C, "hyb_spmm: null pointer argument");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  dim3 block(256);
+  const int64_t nblocks = stir::ceil_div(plan->total_tiles, 4);
+  STIR_REQUIRE(nblocks < (int64_t(1) << 31), "hyb_spmm: %lld tiles exceed one launch", (long long)plan->total_tiles);
+  dim3 grid((unsigned)nblocks);
+#define STIR_HYB(G, REP)                                                                        \
+  hipLaunchKernelGGL((hyb_spmm_kernel<G, REP>), grid, block, 0, st, plan->d_table_tiles, plan->nk, \
+                     plan->total_tiles, feat, d_B, d_C)
+  switch (feat) {
+    case 32: STIR_HYB(8, 1); break;
+    case 64: STIR_HYB(16, 1); break;
+    case 128: STIR_HYB(32, 1); break;
+    case 256: STIR_HYB(64, 1); break;
+    case 512: STIR_HYB(64, 2); break;
+    default: {
+      const int64_t rb = stir::ceil_div(plan->total_rows, 4);
+      STIR_REQUIRE(rb < (int64_t(1) << 31), "hyb_spmm: %lld rows exceed one launch", (long long)plan->total_rows);
+      hipLaunchKernelGGL(hyb_spmm_generic_kernel, dim3((unsigned)rb), block, 0, st, plan->d_table_rows,
+                         plan->nk, plan->total_rows, feat, d_B, d_C);
+    }
+  }
+#undef STIR_HYB
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+int stir_hyb_plan_destroy(stir_hyb_plan* plan) {
+  if (!plan) return 0;
+  if (plan->d_table_tiles) (void)hipFree(plan->d_table_tiles);
+  delete plan;
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,171 @@
+"""Format-decomposition routines with the reference's Python surface.
+
+Mirrors ``python/tvm/sparse/format.py`` of the reference: ``column_part_hyb`` (:89-116),
+``condense`` (:119-139) and ``csf_to_ell3d`` (:142-170) keep their names, argument order and
+return nesting.  Where the reference takes ``tvm.nd`` CPU arrays and returns nested
+``Array<NDArray>``, these take numpy arrays / CPU torch tensors and return nested lists of
+numpy ``int32`` arrays.  ``column_part_hyb`` additionally accepts CUDA torch tensors, in which
+case the decomposition runs on the GPU and returns CUDA tensors.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+
+
+def _host_i32(a, name):
+    """int32 contiguous numpy view of a numpy array / CPU torch tensor (reference:
+    'Only support int32 index data type', src/sparse/format.cc:56-59)."""
+    if hasattr(a, "detach") and hasattr(a, "numpy"):
+        if a.device.type != "cpu":
+            raise _lib.SparseTIRError(f"Only support {name} conversion on CPU.")
+        a = a.detach().numpy()
+    a = np.asarray(a)
+    if a.dtype != np.int32:
+        raise _lib.SparseTIRError(
+            f"Only support int32 index data type, got {a.dtype.itemsize * 8} bits for {name}.")
+    return np.ascontiguousarray(a)
+
+
+def _vp(a):
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _is_cuda_tensor(a):
+    return hasattr(a, "is_cuda") and a.is_cuda
+
+
+def column_part_hyb(num_rows, num_cols, indptr_nd, indices_nd, num_col_parts, buckets):
+    """Partition a CSR matrix by columns and collect rows into ELL buckets by their number of
+    nonzeros per partition.
+
+    Returns ``(row_indices, col_indices, mask)``; each is a list over column partitions of
+    lists over buckets of int32 arrays shaped ``(nrows,)``, ``(nrows, b)``, ``(nrows, b)``.
+    """
+    if _is_cuda_tensor(indptr_nd) or _is_cuda_tensor(indices_nd):
+        return _column_part_hyb_device(num_rows, num_cols, indptr_nd, indices_nd,
+                                       num_col_parts, buckets)
+    L = _lib.lib()
+    indptr = _host_i32(indptr_nd, "indptr")
+    indices = _host_i32(indices_nd, "indices")
+    if indptr.shape[0] != num_rows + 1:
+        raise _lib.SparseTIRError("ColumnPartHyb: indptr must have num_rows + 1 entries")
+    widths = np.ascontiguousarray(np.asarray(list(buckets), dtype=np.int32))
+    nb = len(widths)
+    nk = num_col_parts * nb
+    nrows = np.zeros(max(nk, 1), np.int64)
+    _lib.check(L.stir_column_part_hyb_sizes(num_rows, num_cols, _vp(indptr), _vp(indices),
+                                            num_col_parts, _vp(widths), nb, _vp(nrows)))
+    rows = [np.empty(int(nrows[k]), np.int32) for k in range(nk)]
+    cols = [np.empty((int(nrows[k]), int(widths[k % nb])), np.int32) for k in range(nk)]
+    mask = [np.empty((int(nrows[k]), int(widths[k % nb])), np.int32) for k in range(nk)]
+    _lib.check(L.stir_column_part_hyb_fill(
+        num_rows, num_cols, _vp(indptr), _vp(indices), num_col_parts, _vp(widths), nb,
+        _lib.ptr_table([a.ctypes.data for a in rows]),
+        _lib.ptr_table([a.ctypes.data for a in cols]),
+        _lib.ptr_table([a.ctypes.data for a in mask])))
+    nest = lambda xs: [[xs[p * nb + b] for b in range(nb)] for p in range(num_col_parts)]
+    return nest(rows), nest(cols), nest(mask)
+
+
+def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, buckets):
+    import torch
+
+    L = _lib.lib()
+    for t, name in ((indptr, "indptr"), (indices, "indices")):
+        if not _is_cuda_tensor(t):
+            raise _lib.SparseTIRError("ColumnPartHyb(device): indptr and indices must both be CUDA tensors")
+        if t.dtype != torch.int32:
+            raise _lib.SparseTIRError(
+                f"Only support int32 index data type, got {t.element_size() * 8} bits for {name}.")
+    indptr, indices = indptr.contiguous(), indices.contiguous()
+    if indptr.shape[0] != num_rows + 1:
+        raise _lib.SparseTIRError("ColumnPartHyb: indptr must have num_rows + 1 entries")
+    dev = indptr.device
+    widths = np.ascontiguousarray(np.asarray(list(buckets), dtype=np.int32))
+    nb = len(widths)
+    nk = num_col_parts * nb
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        ws_bytes = L.stir_column_part_hyb_device_workspace_bytes(num_rows, num_col_parts, nb)
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+        nrows = np.zeros(max(nk, 1), np.int64)
+        _lib.check(L.stir_column_part_hyb_device_sizes(
+            num_rows, num_cols, ctypes.c_void_p(indptr.data_ptr()),
+            ctypes.c_void_p(indices.data_ptr()), num_col_parts, _vp(widths), nb,
+            ctypes.c_void_p(ws.data_ptr()), _vp(nrows), stream))
+        rows = [torch.empty(int(nrows[k]), dtype=torch.int32, device=dev) for k in range(nk)]
+        cols = [torch.empty((int(nrows[k]), int(widths[k % nb])), dtype=torch.int32, device=dev)
+                for k in range(nk)]
+        mask = [torch.empty((int(nrows[k]), int(widths[k % nb])), dtype=torch.int32, device=dev)
+                for k in range(nk)]
+        _lib.check(L.stir_column_part_hyb_device_fill(
+            num_rows, num_cols, ctypes.c_void_p(indptr.data_ptr()),
+            ctypes.c_void_p(indices.data_ptr()), num_col_parts, _vp(widths), nb,
+            ctypes.c_void_p(ws.data_ptr()),
+            _lib.ptr_table([a.data_ptr() for a in rows]),
+            _lib.ptr_table([a.data_ptr() for a in cols]),
+            _lib.ptr_table([a.data_ptr() for a in mask]), stream))
+        # the workspace is read by the fill kernels: keep it alive until they are done
+        torch.cuda.current_stream().synchronize()
+    nest = lambda xs: [[xs[p * nb + b] for b in range(nb)] for p in range(num_col_parts)]
+    return nest(rows), nest(cols), nest(mask)
+
+
+def condense(indptr_nd, indices_nd, t, g):
+    """Condense a CSR matrix to (t x 1) tiles and group g tiles together.
+
+    Returns ``(group_indptr, tile_indices, mask)`` shaped ``(ceil(n/t)+1,)``, ``(G, g)``,
+    ``(G, t, g)``.
+    """
+    L = _lib.lib()
+    indptr = _host_i32(indptr_nd, "indptr")
+    indices = _host_i32(indices_nd, "indices")
+    n = indptr.shape[0] - 1
+    if t <= 0 or g <= 0:
+        raise _lib.SparseTIRError(f"ConDense: t={t} g={g} must be positive")
+    tiles = (n + t - 1) // t
+    gptr = np.empty(tiles + 1, np.int32)
+    ng = np.zeros(1, np.int64)
+    _lib.check(L.stir_condense_sizes(n, _vp(indptr), _vp(indices), t, g, _vp(gptr), _vp(ng)))
+    G = int(ng[0])
+    tile_indices = np.empty((G, g), np.int32)
+    mask = np.empty((G, t, g), np.int32)
+    _lib.check(L.stir_condense_fill(n, _vp(indptr), _vp(indices), t, g, _vp(tile_indices),
+                                    _vp(mask)))
+    return gptr, tile_indices, mask
+
+
+def csf_to_ell3d(csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1, nnz_rows_bkt,
+                 nnz_cols_bkt):
+    """Convert CSF (relation -> row -> column) to the bucketed ELL3D format.
+
+    Returns ``(indptr, row_indices, col_indices, mask)``, each a list over buckets, shaped
+    ``(R+1,)``, ``(G, rb)``, ``(G, rb, cb)``, ``(G, rb, cb)``.
+    """
+    L = _lib.lib()
+    p0 = _host_i32(csf_indptr_0, "csf_indptr_0")
+    i0 = _host_i32(csf_indices_0, "csf_indices_0")
+    p1 = _host_i32(csf_indptr_1, "csf_indptr_1")
+    i1 = _host_i32(csf_indices_1, "csf_indices_1")
+    rb = np.ascontiguousarray(np.asarray(list(nnz_rows_bkt), dtype=np.int32))
+    cb = np.ascontiguousarray(np.asarray(list(nnz_cols_bkt), dtype=np.int32))
+    if len(rb) != len(cb):
+        raise _lib.SparseTIRError("Input nnz_rows and nnz_cols should have same length.")
+    nb = len(cb)
+    num_rels = p0.shape[0] - 1
+    groups = np.zeros(max(nb, 1), np.int64)
+    _lib.check(L.stir_csf_to_ell3d_sizes(num_rels, _vp(p0), _vp(i0), _vp(p1), _vp(i1), _vp(rb),
+                                         _vp(cb), nb, _vp(groups)))
+    out_ptr = [np.empty(num_rels + 1, np.int32) for _ in range(nb)]
+    rows = [np.empty((int(groups[b]), int(rb[b])), np.int32) for b in range(nb)]
+    cols = [np.empty((int(groups[b]), int(rb[b]), int(cb[b])), np.int32) for b in range(nb)]
+    mask = [np.empty((int(groups[b]), int(rb[b]), int(cb[b])), np.int32) for b in range(nb)]
+    _lib.check(L.stir_csf_to_ell3d_fill(
+        num_rels, _vp(p0), _vp(i0), _vp(p1), _vp(i1), _vp(rb), _vp(cb), nb,
+        _lib.ptr_table([a.ctypes.data for a in out_ptr]),
+        _lib.ptr_table([a.ctypes.data for a in rows]),
+        _lib.ptr_table([a.ctypes.data for a in cols]),
+        _lib.ptr_table([a.ctypes.data for a in mask])))
+    return out_ptr, rows, cols, mask

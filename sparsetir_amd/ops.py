@@ -1,0 +1,296 @@
+"""The built operators: what ``tvm.build(mod, target=...)`` hands the reference's scripts.
+
+Each ``build_*`` function returns a callable that takes the same flat device arrays, in the
+same order, as the operator the reference builds for that kernel, and launches the
+hand-written gfx950 kernel through the C ABI on torch's current stream:
+
+  build_csrmm         f(A, B, C, indptr, indices)             examples/spmm/bench_spmm_naive.py:121-129
+  build_hyb_csrmm     f(B, C, A_0, rows_0, cols_0, ...)       examples/spmm/bench_spmm.py:208-225
+  build_sddmm_preproc f(A, B, C, indptr, indices, mid)        examples/sddmm/bench_sddmm.py:106-115
+  build_sddmm         f(A, B, C, indptr, indices, mid)        examples/sddmm/bench_sddmm.py:170-171
+  build_bsrmm         f(A, X, Y, indptr, indices)             examples/blocksparse/bsr_spmm.py:427-433
+  build_rgms          f(W, X, Y, (A_k, rows_k, cols_k)..., mids_k...)
+                                                               examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
+
+Arrays are torch CUDA tensors (device memory and streams only).  Arguments are checked the
+way the reference's generated host stub checks DLTensors (src/tir/transforms/arg_binder.cc:152+):
+one dimension, exact dtype, exact length, contiguous, all on one device.  Operators also offer
+``time_evaluator(number)``, the reference's protocol of one discarded call followed by the
+mean of ``number`` back-to-back launches between device events
+(src/runtime/profiling.cc:742-797).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None and t.numel() > 0 else 0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class _Operator:
+    name = "main"
+    entry_name = "main"
+
+    def _check(self, args, spec):
+        """spec: list of (label, dtype, length)."""
+        if len(args) != len(spec):
+            raise _lib.SparseTIRError(f"{self.name}: num_args should be {len(spec)}")
+        dev = None
+        for i, (t, (label, dtype, length)) in enumerate(zip(args, spec)):
+            if not isinstance(t, torch.Tensor):
+                raise _lib.SparseTIRError(f"{self.name}: Expect arg[{i}] to be pointer")
+            if not t.is_cuda:
+                raise _lib.SparseTIRError(f"{self.name}: arg[{i}] ({label}) must be a device array")
+            if t.dim() != 1:
+                raise _lib.SparseTIRError(f"{self.name}: {label}.ndim is expected to equal 1")
+            if t.dtype != dtype:
+                raise _lib.SparseTIRError(
+                    f"{self.name}: {label}.dtype is expected to be {dtype}, got {t.dtype}")
+            if t.shape[0] != length:
+                raise _lib.SparseTIRError(
+                    f"{self.name}: {label}.shape[0] is expected to be {length}, got {t.shape[0]}")
+            if not t.is_contiguous():
+                raise _lib.SparseTIRError(f"{self.name}: {label} is expected to be compact")
+            if dev is None:
+                dev = t.device
+            elif t.device != dev:
+                raise _lib.SparseTIRError(f"{self.name}: all arrays must be on one device")
+        return dev
+
+    def time_evaluator(self, number=100):
+        """Returns g(*args) -> mean seconds per call over ``number`` launches after one
+        discarded call, timed with device events on the current stream."""
+        def run(*args):
+            self(*args)
+            start = torch.cuda.Event(enable_timing=True)
+            stop = torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(number):
+                self(*args)
+            stop.record()
+            stop.synchronize()
+            return start.elapsed_time(stop) / 1e3 / number
+        return run
+
+
+class CsrMM(_Operator):
+    name = "csrmm"
+
+    def __init__(self, m, n, feat, nnz):
+        self.m, self.n, self.feat, self.nnz = int(m), int(n), int(feat), int(nnz)
+        self.L = _lib.lib()
+
+    def __call__(self, a, b, c, indptr, indices):
+        f32, i32 = torch.float32, torch.int32
+        dev = self._check([a, b, c, indptr, indices],
+                          [("A", f32, self.nnz), ("B", f32, self.n * self.feat),
+                           ("C", f32, self.m * self.feat), ("indptr", i32, self.m + 1),
+                           ("indices", i32, self.nnz)])
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_csr_spmm_f32(self.m, self.n, self.feat, self.nnz, _ptr(a),
+                                                _ptr(b), _ptr(c), _ptr(indptr), _ptr(indices),
+                                                _stream()))
+
+
+class HybCsrMM(_Operator):
+    """All ELL buckets of all column partitions in one launch.  ``nrows`` lists the ELL rows
+    of every bucket, partition-major, the quantity the reference specialises the kernel with
+    (examples/spmm/bench_spmm.py:146-152)."""
+    name = "hyb_csrmm"
+
+    def __init__(self, m, n, feat, num_col_parts, buckets, nrows):
+        self.m, self.n, self.feat = int(m), int(n), int(feat)
+        self.parts, self.buckets = int(num_col_parts), [int(b) for b in buckets]
+        self.nrows = [int(r) for r in nrows]
+        if len(self.nrows) != self.parts * len(self.buckets):
+            raise _lib.SparseTIRError("hyb_csrmm: nrows must have num_col_parts*len(buckets) entries")
+        self.L = _lib.lib()
+        self._plan = None
+        self._key = None
+        self._keep = None
+
+    def _spec(self):
+        f32, i32 = torch.float32, torch.int32
+        spec = [("B", f32, self.n * self.feat), ("C", f32, self.m * self.feat)]
+        nb = len(self.buckets)
+        for k, r in enumerate(self.nrows):
+            w = self.buckets[k % nb]
+            tag = f"{k // nb}_{k % nb}"
+            spec += [(f"A_{tag}", f32, r * w), (f"rows_{tag}", i32, r), (f"cols_{tag}", i32, r * w)]
+        return spec
+
+    def _drop_plan(self):
+        if self._plan is not None:
+            self.L.stir_hyb_plan_destroy(self._plan)
+            self._plan = None
+
+    def __del__(self):
+        try:
+            self._drop_plan()
+        except Exception:
+            pass
+
+    def __call__(self, b, c, *triples):
+        dev = self._check([b, c, *triples], self._spec())
+        key = (dev,) + tuple(t.data_ptr() for t in triples)
+        with torch.cuda.device(dev):
+            if key != self._key:
+                self._drop_plan()
+                nk = len(self.nrows)
+                widths = (ctypes.c_int32 * len(self.buckets))(*self.buckets)
+                nrows = (ctypes.c_int64 * max(nk, 1))(*self.nrows)
+                plan = ctypes.c_void_p()
+                A = _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in triples[0::3]])
+                R = _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in triples[1::3]])
+                Cc = _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in triples[2::3]])
+                _lib.check(self.L.stir_hyb_plan_create(ctypes.byref(plan), self.m, self.n, self.parts,
+                                                       len(self.buckets), widths, nrows, A, R, Cc))
+                self._plan, self._key = plan, key
+                self._keep = triples  # the plan stores pointers into these arrays
+            _lib.check(self.L.stir_hyb_spmm_f32(self._plan, self.feat, _ptr(b), _ptr(c), _stream()))
+
+
+class SddmmPreproc(_Operator):
+    name = "sddmm_preproc"
+
+    def __init__(self, m, n, feat, nnz):
+        self.m, self.n, self.feat, self.nnz = int(m), int(n), int(feat), int(nnz)
+        self.L = _lib.lib()
+
+    def _spec(self):
+        f32, i32 = torch.float32, torch.int32
+        return [("A", f32, self.m * self.feat), ("B", f32, self.n * self.feat),
+                ("C", f32, self.nnz), ("indptr", i32, self.m + 1), ("indices", i32, self.nnz),
+                ("mid", i32, self.nnz)]
+
+    def __call__(self, a, b, c, indptr, indices, mid):
+        dev = self._check([a, b, c, indptr, indices, mid], self._spec())
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_sddmm_preproc(self.m, self.nnz, _ptr(indptr), _ptr(mid), _stream()))
+
+
+class Sddmm(SddmmPreproc):
+    name = "sddmm"
+
+    def __call__(self, a, b, c, indptr, indices, mid):
+        dev = self._check([a, b, c, indptr, indices, mid], self._spec())
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_sddmm_f32(self.m, self.n, self.feat, self.nnz, _ptr(a), _ptr(b),
+                                             _ptr(c), _ptr(indptr), _ptr(indices), _ptr(mid),
+                                             _stream()))
+
+
+_DT = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+
+
+class BsrMM(_Operator):
+    name = "bsrmm"
+
+    def __init__(self, mb, nb, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):
+        self.mb, self.nb, self.nnzb, self.blk, self.feat = map(int, (mb, nb, nnzb, blk, feat))
+        self.dtype = dtype
+        self.out_dtype = dtype if out_dtype is None else out_dtype
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise _lib.SparseTIRError("bsrmm: inputs must be float16 or bfloat16")
+        self.L = _lib.lib()
+
+    def __call__(self, a, x, y, indptr, indices):
+        i32 = torch.int32
+        dev = self._check([a, x, y, indptr, indices],
+                          [("A", self.dtype, self.nnzb * self.blk * self.blk),
+                           ("X", self.dtype, self.nb * self.blk * self.feat),
+                           ("Y", self.out_dtype, self.mb * self.blk * self.feat),
+                           ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb)])
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_bsr_spmm(_DT[self.dtype], _DT[self.out_dtype], self.mb, self.nb,
+                                            self.blk, self.feat, self.nnzb, _ptr(a), _ptr(x), _ptr(y),
+                                            _ptr(indptr), _ptr(indices), _stream()))
+
+
+class Rgms(_Operator):
+    """RGMS on ELL3D buckets.  ``groups`` lists the group count of every bucket, ``rows_bkt`` /
+    ``cols_bkt`` the ELL rows per group and slots per ELL row."""
+    name = "rgms"
+
+    def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
+        self.m, self.n, self.R = int(m), int(n), int(num_rels)
+        self.fin, self.fout = int(feat_in), int(feat_out)
+        self.rb, self.cb = [int(v) for v in rows_bkt], [int(v) for v in cols_bkt]
+        self.groups = [int(v) for v in groups]
+        self.L = _lib.lib()
+        self._plan = None
+        self._key = None
+        self._keep = None
+
+    def _spec(self):
+        f16, f32, i32 = torch.float16, torch.float32, torch.int32
+        spec = [("W", f16, self.R * self.fin * self.fout), ("X", f16, self.n * self.fin),
+                ("Y", f32, self.m * self.fout)]
+        for k, g in enumerate(self.groups):
+            spec += [(f"A_{k}", f16, g * self.rb[k] * self.cb[k]), (f"rows_{k}", i32, g * self.rb[k]),
+                     (f"cols_{k}", i32, g * self.rb[k] * self.cb[k])]
+        for k, g in enumerate(self.groups):
+            spec.append((f"mids_{k}", i32, g))
+        return spec
+
+    def _drop_plan(self):
+        if self._plan is not None:
+            self.L.stir_rgms_plan_destroy(self._plan)
+            self._plan = None
+
+    def __del__(self):
+        try:
+            self._drop_plan()
+        except Exception:
+            pass
+
+    def __call__(self, w, x, y, *rest):
+        dev = self._check([w, x, y, *rest], self._spec())
+        nb = len(self.groups)
+        triples, mids = rest[:3 * nb], rest[3 * nb:]
+        key = (dev,) + tuple(t.data_ptr() for t in rest)
+        with torch.cuda.device(dev):
+            if key != self._key:
+                self._drop_plan()
+                plan = ctypes.c_void_p()
+                rb = (ctypes.c_int32 * nb)(*self.rb)
+                cb = (ctypes.c_int32 * nb)(*self.cb)
+                groups = (ctypes.c_int64 * nb)(*self.groups)
+                tab = lambda ts: _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in ts])
+                _lib.check(self.L.stir_rgms_plan_create(ctypes.byref(plan), nb, rb, cb, groups,
+                                                        tab(triples[0::3]), tab(triples[1::3]),
+                                                        tab(triples[2::3]), tab(mids)))
+                self._plan, self._key, self._keep = plan, key, rest
+            _lib.check(self.L.stir_rgms_f16(self._plan, self.m, self.n, self.R, self.fin, self.fout,
+                                            _ptr(w), _ptr(x), _ptr(y), _stream()))
+
+
+def build_csrmm(m, n, feat, nnz):
+    return CsrMM(m, n, feat, nnz)
+
+
+def build_hyb_csrmm(m, n, feat, num_col_parts, buckets, nrows):
+    return HybCsrMM(m, n, feat, num_col_parts, buckets, nrows)
+
+
+def build_sddmm_preproc(m, n, feat, nnz):
+    return SddmmPreproc(m, n, feat, nnz)
+
+
+def build_sddmm(m, n, feat, nnz):
+    return Sddmm(m, n, feat, nnz)
+
+
+def build_bsrmm(mb, nb, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):
+    return BsrMM(mb, nb, nnzb, blk, feat, dtype, out_dtype)
+
+
+def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
+    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups)

@@ -1,0 +1,47 @@
+"""The C-ABI library loads and exports exactly the entry points include/sparsetir_amd.h
+declares (no compute calls: this runs without a GPU)."""
+import ctypes
+import os
+import re
+
+import sparsetir_amd._lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sparsetir_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(stir_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_what_the_binding_lists():
+    assert declared_symbols() == sorted(L.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(L.LIB_PATH), "build with `python -m sparsetir_amd.build`"
+    lib = ctypes.CDLL(L.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_version_and_error_string():
+    lib = L.lib()
+    assert b"gfx950" in lib.stir_version()
+    rc = lib.stir_condense_sizes(1, None, None, 0, 0, None, None)
+    assert rc == -1
+    assert b"ConDense" in lib.stir_last_error()
+
+
+def test_no_product_file_touches_the_oracle():
+    """The shipped package must not import, link or run anything under oracle/."""
+    pkg = os.path.join(ROOT, "sparsetir_amd")
+    for base, _, files in os.walk(pkg):
+        if os.path.basename(base) == "build":
+            continue
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".h")):
+                text = open(os.path.join(base, f), errors="ignore").read()
+                assert "import oracle" not in text and "from oracle" not in text, f
+                assert "sparsetir_oracle" not in text, f
