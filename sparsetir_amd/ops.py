@@ -87,12 +87,12 @@ class CsrMM(_Operator):
         self.m, self.n, self.feat, self.nnz = int(m), int(n), int(feat), int(nnz)
         self.L = _lib.lib()
 
-    def __call__(self, a, b, c, indptr, indices):
+    def __call__(self, *args):
         f32, i32 = torch.float32, torch.int32
-        dev = self._check([a, b, c, indptr, indices],
-                          [("A", f32, self.nnz), ("B", f32, self.n * self.feat),
-                           ("C", f32, self.m * self.feat), ("indptr", i32, self.m + 1),
-                           ("indices", i32, self.nnz)])
+        dev = self._check(args, [("A", f32, self.nnz), ("B", f32, self.n * self.feat),
+                                 ("C", f32, self.m * self.feat), ("indptr", i32, self.m + 1),
+                                 ("indices", i32, self.nnz)])
+        a, b, c, indptr, indices = args
         with torch.cuda.device(dev):
             _lib.check(self.L.stir_csr_spmm_f32(self.m, self.n, self.feat, self.nnz, _ptr(a),
                                                 _ptr(b), _ptr(c), _ptr(indptr), _ptr(indices),
@@ -137,8 +137,9 @@ class HybCsrMM(_Operator):
         except Exception:
             pass
 
-    def __call__(self, b, c, *triples):
-        dev = self._check([b, c, *triples], self._spec())
+    def __call__(self, *args):
+        dev = self._check(args, self._spec())
+        b, c, triples = args[0], args[1], args[2:]
         key = (dev,) + tuple(t.data_ptr() for t in triples)
         with torch.cuda.device(dev):
             if key != self._key:
@@ -170,8 +171,9 @@ class SddmmPreproc(_Operator):
                 ("C", f32, self.nnz), ("indptr", i32, self.m + 1), ("indices", i32, self.nnz),
                 ("mid", i32, self.nnz)]
 
-    def __call__(self, a, b, c, indptr, indices, mid):
-        dev = self._check([a, b, c, indptr, indices, mid], self._spec())
+    def __call__(self, *args):
+        dev = self._check(args, self._spec())
+        a, b, c, indptr, indices, mid = args
         with torch.cuda.device(dev):
             _lib.check(self.L.stir_sddmm_preproc(self.m, self.nnz, _ptr(indptr), _ptr(mid), _stream()))
 
@@ -179,8 +181,9 @@ class SddmmPreproc(_Operator):
 class Sddmm(SddmmPreproc):
     name = "sddmm"
 
-    def __call__(self, a, b, c, indptr, indices, mid):
-        dev = self._check([a, b, c, indptr, indices, mid], self._spec())
+    def __call__(self, *args):
+        dev = self._check(args, self._spec())
+        a, b, c, indptr, indices, mid = args
         with torch.cuda.device(dev):
             _lib.check(self.L.stir_sddmm_f32(self.m, self.n, self.feat, self.nnz, _ptr(a), _ptr(b),
                                              _ptr(c), _ptr(indptr), _ptr(indices), _ptr(mid),
@@ -201,13 +204,13 @@ class BsrMM(_Operator):
             raise _lib.SparseTIRError("bsrmm: inputs must be float16 or bfloat16")
         self.L = _lib.lib()
 
-    def __call__(self, a, x, y, indptr, indices):
+    def __call__(self, *args):
         i32 = torch.int32
-        dev = self._check([a, x, y, indptr, indices],
-                          [("A", self.dtype, self.nnzb * self.blk * self.blk),
-                           ("X", self.dtype, self.nb * self.blk * self.feat),
-                           ("Y", self.out_dtype, self.mb * self.blk * self.feat),
-                           ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb)])
+        dev = self._check(args, [("A", self.dtype, self.nnzb * self.blk * self.blk),
+                                 ("X", self.dtype, self.nb * self.blk * self.feat),
+                                 ("Y", self.out_dtype, self.mb * self.blk * self.feat),
+                                 ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb)])
+        a, x, y, indptr, indices = args
         with torch.cuda.device(dev):
             _lib.check(self.L.stir_bsr_spmm(_DT[self.dtype], _DT[self.out_dtype], self.mb, self.nb,
                                             self.blk, self.feat, self.nnzb, _ptr(a), _ptr(x), _ptr(y),
@@ -251,8 +254,9 @@ class Rgms(_Operator):
         except Exception:
             pass
 
-    def __call__(self, w, x, y, *rest):
-        dev = self._check([w, x, y, *rest], self._spec())
+    def __call__(self, *args):
+        dev = self._check(args, self._spec())
+        w, x, y, rest = args[0], args[1], args[2], args[3:]
         nb = len(self.groups)
         triples, mids = rest[:3 * nb], rest[3 * nb:]
         key = (dev,) + tuple(t.data_ptr() for t in rest)

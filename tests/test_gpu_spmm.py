@@ -1,0 +1,217 @@
+"""GPU parity of CSR row-split SpMM and hyb SpMM (through the C ABI) against the CPU oracle.
+
+Tolerance: fp32, |got - want| <= 1e-5 * (|A| @ |X|) elementwise, i.e. relative 1e-5 measured
+against the magnitude of the terms that are summed (an rtol-only check against the result is
+meaningless where the terms cancel); the float64 closed form is the reference value.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparsetir_amd as st
+from sparsetir_amd import datasets, ops
+from sparsetir_amd._lib import SparseTIRError
+from helpers import random_csr, spmm_f64
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+def _check(got, indptr, indices, vals, x, what):
+    want = spmm_f64(indptr, indices, vals, x)
+    scale = spmm_f64(indptr, indices, np.abs(vals), np.abs(x))
+    err = np.abs(got.astype(np.float64) - want)
+    bad = err > RTOL * scale + 1e-30
+    assert not bad.any(), f"{what}: {bad.sum()} elements off, worst {err.max():.3e}"
+
+
+def _run_csr(dev, indptr, indices, vals, x, feat, fill=None):
+    m, n = len(indptr) - 1, x.shape[0]
+    f = ops.build_csrmm(m, n, feat, len(indices))
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    c = torch.full((m * feat,), float("nan") if fill is None else fill, dtype=torch.float32, device=dev)
+    f(t(vals), t(x.ravel()), c, t(indptr), t(indices))
+    torch.cuda.synchronize()
+    return c.cpu().numpy().reshape(m, feat)
+
+
+def test_csr_spmm_config1(dev):
+    g = datasets.config1()
+    got = _run_csr(dev, g["indptr"], g["indices"], g["values"], g["x"], g["feat"])
+    _check(got, g["indptr"], g["indices"], g["values"], g["x"], "config1")
+    # and against the C restatement of the reference's serial loop nest
+    ref = oracle.csrmm(g["values"], g["x"], g["indptr"], g["indices"], g["feat"])
+    scale = spmm_f64(g["indptr"], g["indices"], g["values"], np.abs(g["x"]))
+    assert np.all(np.abs(got - ref) <= 2 * RTOL * scale)
+
+
+@pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 48, 20, 1])
+def test_csr_spmm_feature_widths(dev, feat):
+    m, n = 1003, 777
+    indptr, indices = random_csr(m, n, 30000, feat, skew=1.2)
+    rng = np.random.default_rng(feat)
+    vals = rng.random(len(indices), dtype=np.float32)
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    got = _run_csr(dev, indptr, indices, vals, x, feat)
+    assert np.all(got[np.diff(indptr) == 0] == 0.0)  # rows without nonzeros are zeroed
+    _check(got, indptr, indices, vals, x, f"feat={feat}")
+
+
+def test_csr_spmm_edge_shapes(dev):
+    for m, n, nnz in [(1, 1, 1), (5, 3, 0), (0, 4, 0), (130, 2, 200)]:
+        indptr, indices = random_csr(m, n, nnz, 3)
+        rng = np.random.default_rng(0)
+        vals = rng.random(len(indices), dtype=np.float32)
+        x = rng.standard_normal((n, 64), dtype=np.float32)
+        got = _run_csr(dev, indptr, indices, vals, x, 64)
+        if m:
+            _check(got, indptr, indices, vals, x, f"shape {(m, n, nnz)}")
+
+
+def test_csr_spmm_long_row(dev):
+    # one row holding every column (the power-law tail)
+    m, n, feat = 9, 5000, 128
+    indptr = np.asarray([0, 3, n + 3] + [n + 3] * (m - 2), np.int32)
+    indices = np.concatenate([[1, 5, 9], np.arange(n)]).astype(np.int32)
+    rng = np.random.default_rng(5)
+    vals = rng.random(len(indices), dtype=np.float32)
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    got = _run_csr(dev, indptr, indices, vals, x, feat)
+    _check(got, indptr, indices, vals, x, "long row")
+
+
+def test_csr_spmm_argument_checks(dev):
+    f = ops.build_csrmm(4, 4, 32, 3)
+    z = lambda k, dt=torch.float32: torch.zeros(k, dtype=dt, device=dev)
+    good = [z(3), z(128), z(128), z(5, torch.int32), z(3, torch.int32)]
+    f(*good)
+    with pytest.raises(SparseTIRError, match="num_args"):
+        f(*good[:4])
+    with pytest.raises(SparseTIRError, match="dtype"):
+        f(good[0], good[1], good[2], z(5, torch.int64), good[4])
+    with pytest.raises(SparseTIRError, match="shape"):
+        f(good[0], z(127), good[2], good[3], good[4])
+    with pytest.raises(SparseTIRError, match="ndim"):
+        f(good[0], z(128).reshape(4, 32), good[2], good[3], good[4])
+    with pytest.raises(SparseTIRError, match="device"):
+        f(good[0].cpu(), good[1], good[2], good[3], good[4])
+
+
+# ------------------------------------------------------------------------------- hyb
+
+def _hyb_setup(dev, indptr, indices, m, n, parts, buckets, weighted, seed, device_format=False):
+    if device_format:
+        ti = lambda a: torch.from_numpy(a).to(dev)
+        rows, cols, mask = st.column_part_hyb(m, n, ti(indptr), ti(indices), parts, buckets)
+        tonp = lambda a: a.cpu().numpy()
+        rows = [[tonp(a) for a in p] for p in rows]
+        cols = [[tonp(a) for a in p] for p in cols]
+        mask = [[tonp(a) for a in p] for p in mask]
+    else:
+        rows, cols, mask = st.column_part_hyb(m, n, indptr, indices, parts, buckets)
+    rng = np.random.default_rng(seed)
+    triples_np = []
+    for p in range(parts):
+        for b in range(len(buckets)):
+            a = mask[p][b].astype(np.float32)
+            if weighted:
+                a = a * rng.random(a.shape, dtype=np.float32)
+            triples_np.append((a, rows[p][b], cols[p][b]))
+    return triples_np
+
+
+def _run_hyb(dev, m, n, feat, parts, buckets, triples_np, x):
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    f = ops.build_hyb_csrmm(m, n, feat, parts, buckets, [len(r) for _, r, _ in triples_np])
+    args = []
+    for a, r, c in triples_np:
+        args += [t(a.ravel()), t(r), t(c.ravel())]
+    cdev = torch.zeros(m * feat, dtype=torch.float32, device=dev)
+    f(t(x.ravel()), cdev, *args)
+    torch.cuda.synchronize()
+    return cdev.cpu().numpy().reshape(m, feat), (f, args)
+
+
+def _hyb_as_coo(triples_np):
+    """(row, col, value) of every slot with a nonzero weight, as a CSR for the float64 form."""
+    rr, cc, vv = [], [], []
+    for a, r, c in triples_np:
+        if len(r) == 0:
+            continue
+        sel = a != 0
+        rr.append(np.repeat(r[:, None], c.shape[1], 1)[sel])
+        cc.append(c[sel])
+        vv.append(a[sel])
+    return np.concatenate(rr), np.concatenate(cc), np.concatenate(vv)
+
+
+@pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 96, 7])
+@pytest.mark.parametrize("parts,buckets", [(1, [1, 2, 4, 8, 16, 32]), (2, [1, 2, 4, 8, 16, 32, 64, 128, 256, 512]),
+                                           (4, [2, 3, 7]), (3, [1])])
+def test_hyb_spmm_matches_oracle(dev, feat, parts, buckets):
+    m = n = 3001
+    indptr, indices = random_csr(m, n, 60000, 17, skew=1.3)
+    triples = _hyb_setup(dev, indptr, indices, m, n, parts, buckets, weighted=True, seed=feat)
+    x = np.random.default_rng(feat).standard_normal((n, feat), dtype=np.float32)
+    got, _ = _run_hyb(dev, m, n, feat, parts, buckets, triples, x)
+    want = oracle.hyb_spmm(m, feat, x, triples, parts)
+    import scipy.sparse as sp
+    r, c, v = _hyb_as_coo(triples)
+    scale = sp.csr_matrix((np.abs(v).astype(np.float64), (r, c)), shape=(m, n)) @ np.abs(x).astype(np.float64)
+    exact = sp.csr_matrix((v.astype(np.float64), (r, c)), shape=(m, n)) @ x.astype(np.float64)
+    assert np.all(np.abs(got - exact) <= RTOL * scale + 1e-30)
+    assert np.all(np.abs(got - want) <= 2 * RTOL * scale + 1e-30)
+
+
+def test_hyb_spmm_store_semantics_of_non_atomic_buckets(dev):
+    """With one column partition every bucket but the last stores (overwrites) its rows and
+    the last one accumulates (examples/spmm/bench_spmm.py:170-177): calling the operator
+    twice on the same C doubles only the rows of the last bucket."""
+    m = n = 500
+    feat, buckets = 64, [1, 2, 4]
+    indptr, indices = random_csr(m, n, 4000, 3, skew=1.0)
+    triples = _hyb_setup(dev, indptr, indices, m, n, 1, buckets, weighted=False, seed=0)
+    x = np.random.default_rng(0).standard_normal((n, feat), dtype=np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    f = ops.build_hyb_csrmm(m, n, feat, 1, buckets, [len(r) for _, r, _ in triples])
+    args = []
+    for a, r, c in triples:
+        args += [t(a.ravel()), t(r), t(c.ravel())]
+    cdev = torch.zeros(m * feat, dtype=torch.float32, device=dev)
+    f(t(x.ravel()), cdev, *args)
+    once = cdev.cpu().numpy().reshape(m, feat).copy()
+    f(t(x.ravel()), cdev, *args)
+    twice = cdev.cpu().numpy().reshape(m, feat)
+    last_rows = np.unique(triples[-1][1])
+    other = np.setdiff1d(np.arange(m), last_rows)
+    assert np.array_equal(twice[other], once[other])
+    assert np.allclose(twice[last_rows], 2 * once[last_rows], rtol=1e-6)
+
+
+@pytest.mark.parametrize("feat", [32, 128])
+def test_hyb_spmm_config2_against_csr_kernel_and_oracle(dev, feat):
+    g = datasets.config2()
+    m, n, parts, buckets = g["m"], g["n"], g["num_col_parts"], g["buckets"]
+    triples = _hyb_setup(dev, g["indptr"], g["indices"], m, n, parts, buckets, weighted=False, seed=0,
+                         device_format=True)
+    x = datasets.features(n, feat, seed=7)
+    got, _ = _run_hyb(dev, m, n, feat, parts, buckets, triples, x)
+    ones = np.ones(len(g["indices"]), np.float32)
+    _check(got, g["indptr"], g["indices"], ones, x, "config2 hyb")
+    csr = _run_csr(dev, g["indptr"], g["indices"], ones, x, feat)
+    scale = spmm_f64(g["indptr"], g["indices"], ones, np.abs(x))
+    assert np.all(np.abs(got - csr) <= 2 * RTOL * scale + 1e-30)
+    want = oracle.hyb_spmm(m, feat, x, triples, parts)
+    assert np.all(np.abs(got - want) <= 2 * RTOL * scale + 1e-30)
+
+
+def test_hyb_spmm_empty_and_degenerate(dev):
+    # no nonzeros at all: every bucket empty, C stays zero
+    m = n = 10
+    indptr = np.zeros(m + 1, np.int32)
+    indices = np.zeros(0, np.int32)
+    triples = _hyb_setup(dev, indptr, indices, m, n, 2, [1, 2], weighted=False, seed=0)
+    x = np.ones((n, 32), np.float32)
+    got, _ = _run_hyb(dev, m, n, 32, 2, [1, 2], triples, x)
+    assert np.all(got == 0)
