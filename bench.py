@@ -29,7 +29,10 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; scaled by a
 # plain copy of known size), keyed by workload signature.  None when not measured.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # profiles/hyb_spmm_config3_uniform.md: FETCH_SIZE 15,740,045 KiB x 2.0 + WRITE_SIZE 1,478,996 KiB x 1.0
+    "uniform/p1/b1-2-4-8-16-32-64-128-256-512/f128/s1.0": 33.75e9,
+}
 
 
 def parse():
@@ -44,7 +47,8 @@ def parse():
     ap.add_argument("--buckets", type=str, default=None, help="comma separated ELL widths")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip CSR / SDDMM side measurements")
-    ap.add_argument("--cpu-rows", type=int, default=300000, help="rows in the cpu_baseline sample")
+    ap.add_argument("--cpu-rows", type=int, default=10**9,
+                    help="rows in the cpu_baseline sample (default: every row, about 6 s on one core)")
     return ap.parse_args()
 
 
@@ -162,6 +166,23 @@ def main():
         log(f"[bench] cpu baseline: {cpu['value']:.2f} GFLOP/s on 1 core ({cpu_s:.2f}s); oracle check {oracle_ok}")
         del xh, ref, got
 
+    # Probes: a plain copy of known size (n*feat*4 bytes read and written; also the kernel the
+    # FETCH_SIZE / WRITE_SIZE counters are scaled by under rocprofv3 --pmc) and nnz gathers of
+    # feat*4-byte rows at pseudo-random indices (what the access pattern allows at best).
+    import ctypes
+    from sparsetir_amd import _lib
+    L = _lib.lib()
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    st0 = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    nbytes = (n * feat * 4) // 16 * 16
+    _, copy_s, _ = time_steps(lambda: _lib.check(L.stir_probe_copy(vp(x), vp(c_csr), nbytes, st0)), 3, 1, torch)
+    probes = {"copy_GBps": 2.0 * nbytes / copy_s / 1e9}
+    if feat in (32, 64, 128, 256):
+        _, gat_s, _ = time_steps(lambda: _lib.check(L.stir_probe_gather(vp(x), n, feat, nnz, vp(c_csr), st0)),
+                                 3, 1, torch)
+        probes["random_row_gather_GBps"] = nnz * feat * 4.0 / gat_s / 1e9
+    log(f"[bench] probes: {probes}")
+
     # ---- timed region
     wall, dev_mean, dev_min = time_steps(lambda: hyb(x, c, *triples), args.steps, args.warmup, torch)
     flops = 2.0 * nnz * feat
@@ -189,7 +210,8 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(sig),
                      "kernel": "hyb_spmm_kernel<32,1>" if feat == 128 else "hyb_spmm_kernel",
                      "kernel_ms_mean": dev_mean * 1e3, "kernel_ms_min": dev_min * 1e3,
-                     "algorithmic_bytes": alg_bytes,
+                     "algorithmic_bytes": alg_bytes, "probes": probes,
+                     "traffic_GBps": (MEASURED_TRAFFIC.get(sig) or 0) / dev_mean / 1e9 or None,
                      "uncached_gather_bytes": 4.0 * slots * feat + 8.0 * slots + 4.0 * m * feat},
         "cpu_baseline": cpu,
         "check": check,

@@ -1,0 +1,152 @@
+/*
+ * sparsetir_amd -- the operators with TVM's PackedFunc calling convention over DLPack tensors.
+ *
+ * Every operator below has the signature of TVMPackedCFunc
+ * (include/tvm/runtime/c_runtime_api.h:296-306 of the reference):
+ *
+ *   int f(TVMValue* args, int* type_codes, int num_args, TVMRetValueHandle ret, void* resource);
+ *
+ * returning 0 on success and -1 after recording a message (stir_last_error(), forwarded to
+ * TVMAPISetLastError when a hook is installed).  Array arguments are DLTensor* passed with type
+ * code kTVMDLTensorHandle, kTVMNDArrayHandle or kTVMOpaqueHandle, integer arguments are
+ * v_int64 with kTVMArgInt, exactly what the reference's generated host stubs accept
+ * (src/tir/transforms/make_packed_api.cc:243-248).  Arrays are checked like BindDLTensor does
+ * (src/tir/transforms/arg_binder.cc:152+): one dimension, dtype code/bits/lanes, compact strides,
+ * byte_offset applied, all on one device (kDLROCM, or kDLCUDA as PyTorch-ROCm exports it).
+ * Sizes are taken from the tensor shapes; what the shapes cannot give is passed as trailing
+ * integers (the reference bakes those into the built module when it specialises the kernel).
+ *
+ * The types below repeat the public DLPack / TVM C definitions so that this header stands alone;
+ * include <dlpack/dlpack.h> and <tvm/runtime/c_runtime_api.h> first to use the originals.
+ */
+#ifndef SPARSETIR_AMD_PACKED_H_
+#define SPARSETIR_AMD_PACKED_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef DLPACK_DLPACK_H_
+#define DLPACK_DLPACK_H_
+typedef enum {
+  kDLCPU = 1,
+  kDLCUDA = 2,
+  kDLCUDAHost = 3,
+  kDLROCM = 10,
+  kDLROCMHost = 11
+} DLDeviceType;
+typedef struct {
+  DLDeviceType device_type;
+  int32_t device_id;
+} DLDevice;
+typedef enum { kDLInt = 0U, kDLUInt = 1U, kDLFloat = 2U, kDLOpaqueHandle = 3U, kDLBfloat = 4U } DLDataTypeCode;
+typedef struct {
+  uint8_t code;
+  uint8_t bits;
+  uint16_t lanes;
+} DLDataType;
+typedef struct {
+  void* data;
+  DLDevice device;
+  int32_t ndim;
+  DLDataType dtype;
+  int64_t* shape;
+  int64_t* strides;
+  uint64_t byte_offset;
+} DLTensor;
+#endif /* DLPACK_DLPACK_H_ */
+
+#ifndef TVM_RUNTIME_C_RUNTIME_API_H_
+typedef union {
+  int64_t v_int64;
+  double v_float64;
+  void* v_handle;
+  const char* v_str;
+  DLDataType v_type;
+  DLDevice v_device;
+} TVMValue;
+typedef void* TVMRetValueHandle;
+typedef void* TVMFunctionHandle;
+typedef int (*TVMPackedCFunc)(TVMValue* args, int* type_codes, int num_args, TVMRetValueHandle ret,
+                              void* resource_handle);
+typedef void (*TVMPackedCFuncFinalizer)(void* resource_handle);
+enum {
+  kTVMArgInt = 0,
+  kTVMArgFloat = 2,
+  kTVMOpaqueHandle = 3,
+  kTVMNullptr = 4,
+  kTVMDLTensorHandle = 7,
+  kTVMNDArrayHandle = 13
+};
+#endif
+
+/*
+ * Operators (global names as registered by stir_register_all):
+ *
+ * "sparsetir.csrmm"          (A, B, C, indptr, indices)
+ *      examples/spmm/bench_spmm_naive.py:121-129
+ * "sparsetir.hyb_csrmm"      (B, C, A_0, rows_0, cols_0, ..., feat, num_col_parts)
+ *      examples/spmm/bench_spmm.py:208-225; bucket k of partition p is triple p*nb + k
+ * "sparsetir.sddmm_preproc"  (A, B, C, indptr, indices, mid)
+ * "sparsetir.sddmm"          (A, B, C, indptr, indices, mid)
+ *      examples/sddmm/bench_sddmm.py:106-115, 170-171
+ * "sparsetir.bsrmm"          (A, X, Y, indptr, indices, blk, feat)    A, X f16 or bf16
+ *      examples/blocksparse/bsr_spmm.py:427-433
+ * "sparsetir.rgms"           (W, X, Y, A_0, rows_0, cols_0, ..., mids_0, ..., feat_in, feat_out)
+ *      examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
+ *
+ * Format pass (host tensors, kDLCPU; the reference returns nested Array<NDArray>, which needs
+ * libtvm objects, so here a sizing call is followed by a fill call into caller-made tensors):
+ *
+ * "tir.sparse.ColumnPartHyb.sizes" (num_rows, num_cols, indptr, indices, num_col_parts, buckets, nrows_out)
+ * "tir.sparse.ColumnPartHyb.fill"  (num_rows, num_cols, indptr, indices, num_col_parts, buckets,
+ *                                   rows_0, cols_0, mask_0, rows_1, ...)      src/sparse/format.cc:46-168
+ *      buckets: int32 tensor; nrows_out: int64 tensor of num_col_parts*len(buckets).
+ *      With kDLROCM/kDLCUDA indptr and indices the decomposition runs on the GPU.
+ * "tir.sparse.CSFToELL3D.sizes"    (indptr0, indices0, indptr1, indices1, rows_bkt, cols_bkt, groups_out)
+ * "tir.sparse.CSFToELL3D.fill"     (indptr0, indices0, indptr1, indices1, rows_bkt, cols_bkt,
+ *                                   indptr_0, rows_0, cols_0, mask_0, indptr_1, ...) src/sparse/format.cc:180-343
+ * "tir.sparse.ConDense.sizes"      (indptr, indices, t, g, group_indptr_out, num_groups_out)
+ * "tir.sparse.ConDense.fill"       (indptr, indices, t, g, tile_indices_out, mask_out)  src/sparse/format.cc:353-429
+ */
+int stir_packed_csrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_hyb_csrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_sddmm_preproc(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_sddmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_bsrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_rgms(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_column_part_hyb_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_column_part_hyb_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_csf_to_ell3d_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_csf_to_ell3d_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_condense_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_condense_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
+
+/* Number of packed operators, and the i-th one's global name / function. */
+int stir_packed_count(void);
+const char* stir_packed_name(int i);
+TVMPackedCFunc stir_packed_func(int i);
+
+/*
+ * Registers every operator in a TVM runtime: pass the runtime's TVMFuncCreateFromCFunc
+ * (c_runtime_api.h:336) and TVMFuncRegisterGlobal (c_runtime_api.h:348).  override != 0
+ * replaces existing globals of the same name.  Returns 0, or the first failing status.
+ */
+int stir_register_all(int (*create_from_cfunc)(TVMPackedCFunc, void*, TVMPackedCFuncFinalizer,
+                                               TVMFunctionHandle*),
+                      int (*register_global)(const char*, TVMFunctionHandle, int), int override);
+
+/* Forward error messages to the host runtime (e.g. TVMAPISetLastError); NULL removes the hook. */
+void stir_set_error_hook(void (*hook)(const char* msg));
+
+/* Stream (hipStream_t) that packed operator calls made by this thread launch on; NULL = default.
+ * The reference keeps the same thread-local state behind TVMSetStream (c_runtime_api.h:482). */
+void stir_set_stream(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSETIR_AMD_PACKED_H_ */

@@ -1,0 +1,586 @@
+// TVM PackedFunc adapters: unpack TVMValue/DLTensor arguments, validate them the way the
+// reference's generated host stubs do, and call the plain C ABI.
+#include <cmath>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "common.h"
+#include "../../include/sparsetir_amd.h"
+#include "../../include/sparsetir_amd_packed.h"
+
+namespace {
+
+thread_local void* g_stream = nullptr;
+void (*g_error_hook)(const char*) = nullptr;
+
+int packed_fail(const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  stir::set_error("%s", buf);
+  if (g_error_hook) g_error_hook(buf);
+  return -1;
+}
+
+// Forward a failure of the plain C ABI (message already recorded) to the hook.
+int forward(int rc) {
+  if (rc != 0 && g_error_hook) g_error_hook(stir_last_error());
+  return rc;
+}
+
+enum Where { kHost, kDevice };
+
+struct Arr {
+  void* data = nullptr;
+  int64_t len = 0;
+  int device_type = 0, device_id = 0;
+};
+
+struct Args {
+  const char* fn;
+  TVMValue* v;
+  int* tc;
+  int n;
+  bool ok = true;
+  int dev_type = -1, dev_id = -1;
+
+  // Array argument i: one dimension, given dtype, compact, on the expected side.
+  Arr arr(int i, const char* name, uint8_t code, uint8_t bits, Where where) {
+    Arr a;
+    if (!ok) return a;
+    const int t = tc[i];
+    if (t != kTVMDLTensorHandle && t != kTVMNDArrayHandle && t != kTVMOpaqueHandle && t != kTVMNullptr) {
+      ok = false;
+      packed_fail("%s: Expect arg[%d] to be pointer", fn, i);
+      return a;
+    }
+    const DLTensor* d = t == kTVMNullptr ? nullptr : static_cast<const DLTensor*>(v[i].v_handle);
+    if (!d) {
+      ok = false;
+      packed_fail("%s: %s is expected to be a tensor, got null", fn, name);
+      return a;
+    }
+    if (d->ndim != 1) {
+      ok = false;
+      packed_fail("%s: %s.ndim is expected to equal 1", fn, name);
+      return a;
+    }
+    if (d->dtype.code != code || d->dtype.bits != bits || d->dtype.lanes != 1) {
+      ok = false;
+      packed_fail("%s: %s.dtype is expected to be code %d bits %d lanes 1, got code %d bits %d lanes %d", fn,
+                  name, code, bits, d->dtype.code, d->dtype.bits, d->dtype.lanes);
+      return a;
+    }
+    if (d->strides && d->shape[0] > 1 && d->strides[0] != 1) {
+      ok = false;
+      packed_fail("%s: %s.strides: expected to be compact array", fn, name);
+      return a;
+    }
+    const bool on_dev = d->device.device_type == kDLROCM || d->device.device_type == kDLCUDA;
+    const bool on_host = d->device.device_type == kDLCPU || d->device.device_type == kDLROCMHost ||
+                         d->device.device_type == kDLCUDAHost;
+    if ((where == kDevice && !on_dev) || (where == kHost && !on_host)) {
+      ok = false;
+      packed_fail("%s: %s is expected to be on the %s", fn, name, where == kDevice ? "GPU (kDLROCM)" : "CPU");
+      return a;
+    }
+    if (where == kDevice) {
+      if (dev_type < 0) {
+        dev_type = d->device.device_type;
+        dev_id = d->device.device_id;
+      } else if (dev_type != (int)d->device.device_type || dev_id != d->device.device_id) {
+        ok = false;
+        packed_fail("%s: Argument %s.device_id has an unsatisfied constraint: all arrays on one device", fn,
+                    name);
+        return a;
+      }
+    }
+    a.data = d->data ? static_cast<char*>(d->data) + d->byte_offset : nullptr;
+    a.len = d->shape[0];
+    a.device_type = d->device.device_type;
+    a.device_id = d->device.device_id;
+    return a;
+  }
+
+  // Device or host, whichever the tensor is on (format pass accepts both).
+  bool on_device(int i) const {
+    const int t = tc[i];
+    if (t != kTVMDLTensorHandle && t != kTVMNDArrayHandle && t != kTVMOpaqueHandle) return false;
+    const DLTensor* d = static_cast<const DLTensor*>(v[i].v_handle);
+    return d && (d->device.device_type == kDLROCM || d->device.device_type == kDLCUDA);
+  }
+
+  int64_t integer(int i, const char* name) {
+    if (!ok) return 0;
+    if (tc[i] != kTVMArgInt) {
+      ok = false;
+      packed_fail("%s: Expect arg[%d] (%s) to be int", fn, i, name);
+      return 0;
+    }
+    return v[i].v_int64;
+  }
+
+  bool count(int want) {
+    if (n != want) {
+      ok = false;
+      packed_fail("%s: num_args should be %d", fn, want);
+    }
+    return ok;
+  }
+
+  bool len(const Arr& a, const char* name, int64_t want) {
+    if (ok && a.len != want) {
+      ok = false;
+      packed_fail("%s: Argument %s.shape[0] has an unsatisfied constraint: %lld == %lld", fn, name,
+                  (long long)a.len, (long long)want);
+    }
+    return ok;
+  }
+};
+
+// Makes the arrays' device current for the call and restores the previous one.
+struct DeviceGuard {
+  int prev = -1;
+  bool switched = false;
+  int enter(int dev_id) {
+    if (dev_id < 0) return 0;
+    STIR_HIP(hipGetDevice(&prev));
+    if (prev != dev_id) {
+      STIR_HIP(hipSetDevice(dev_id));
+      switched = true;
+    }
+    return 0;
+  }
+  ~DeviceGuard() {
+    if (switched) (void)hipSetDevice(prev);
+  }
+};
+
+bool fits_i32(int64_t x) { return x >= 0 && x <= INT32_MAX; }
+
+// ---- cached plans for the plan-based kernels: rebuilt when any pointer or size changes
+struct HybKey {
+  std::vector<uintptr_t> ptrs;
+  std::vector<int64_t> nums;
+  bool operator==(const HybKey& o) const { return ptrs == o.ptrs && nums == o.nums; }
+};
+std::mutex g_plan_mutex;
+HybKey g_hyb_key;
+stir_hyb_plan* g_hyb_plan = nullptr;
+HybKey g_rgms_key;
+stir_rgms_plan* g_rgms_plan = nullptr;
+
+}  // namespace
+
+extern "C" {
+
+void stir_set_error_hook(void (*hook)(const char*)) { g_error_hook = hook; }
+void stir_set_stream(void* stream) { g_stream = stream; }
+
+int stir_packed_csrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.csrmm", v, tc, n};
+  if (!a.count(5)) return -1;
+  Arr A = a.arr(0, "A", kDLFloat, 32, kDevice), B = a.arr(1, "B", kDLFloat, 32, kDevice),
+      C = a.arr(2, "C", kDLFloat, 32, kDevice), P = a.arr(3, "indptr", kDLInt, 32, kDevice),
+      I = a.arr(4, "indices", kDLInt, 32, kDevice);
+  if (!a.ok) return -1;
+  const int64_t m = P.len - 1, nnz = A.len;
+  if (m < 0) return packed_fail("%s: indptr must have at least one entry", a.fn);
+  a.len(I, "indices", nnz);
+  if (!a.ok) return -1;
+  if (m == 0) return 0;
+  if (C.len % m != 0 || C.len == 0) return packed_fail("%s: C.shape[0]=%lld is not a multiple of m=%lld", a.fn, (long long)C.len, (long long)m);
+  const int64_t feat = C.len / m;
+  if (B.len % feat != 0) return packed_fail("%s: B.shape[0]=%lld is not a multiple of feat=%lld", a.fn, (long long)B.len, (long long)feat);
+  const int64_t ncols = B.len / feat;
+  if (!fits_i32(m) || !fits_i32(ncols) || !fits_i32(feat)) return packed_fail("%s: sizes exceed int32", a.fn);
+  DeviceGuard g;
+  if (g.enter(a.dev_id)) return forward(-1);
+  return forward(stir_csr_spmm_f32((int32_t)m, (int32_t)ncols, (int32_t)feat, nnz, (const float*)A.data,
+                                   (const float*)B.data, (float*)C.data, (const int32_t*)P.data,
+                                   (const int32_t*)I.data, g_stream));
+}
+
+int stir_packed_hyb_csrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.hyb_csrmm", v, tc, n};
+  if (n < 4 || (n - 4) % 3 != 0) return packed_fail("%s: num_args should be 2 + 3*buckets + 2", a.fn);
+  const int nk = (n - 4) / 3;
+  Arr B = a.arr(0, "B", kDLFloat, 32, kDevice), C = a.arr(1, "C", kDLFloat, 32, kDevice);
+  const int64_t feat = a.integer(n - 2, "feat"), parts = a.integer(n - 1, "num_col_parts");
+  if (!a.ok) return -1;
+  if (feat <= 0 || parts <= 0 || nk % parts != 0)
+    return packed_fail("%s: feat=%lld num_col_parts=%lld do not fit %d buckets", a.fn, (long long)feat, (long long)parts, nk);
+  if (B.len % feat != 0 || C.len % feat != 0) return packed_fail("%s: B/C lengths are not multiples of feat", a.fn);
+  const int nb = nk / (int)parts;
+  std::vector<const float*> Ak(nk);
+  std::vector<const int32_t*> Rk(nk), Ck(nk);
+  std::vector<int64_t> nrows(nk);
+  std::vector<int32_t> widths(nb, 0);
+  for (int k = 0; k < nk; ++k) {
+    Arr Aa = a.arr(2 + 3 * k, "A_k", kDLFloat, 32, kDevice), Rr = a.arr(3 + 3 * k, "rows_k", kDLInt, 32, kDevice),
+        Cc = a.arr(4 + 3 * k, "cols_k", kDLInt, 32, kDevice);
+    if (!a.ok) return -1;
+    a.len(Cc, "cols_k", Aa.len);
+    if (!a.ok) return -1;
+    nrows[k] = Rr.len;
+    Ak[k] = (const float*)Aa.data;
+    Rk[k] = (const int32_t*)Rr.data;
+    Ck[k] = (const int32_t*)Cc.data;
+    if (Rr.len > 0) {
+      if (Aa.len % Rr.len != 0) return packed_fail("%s: A_%d length is not a multiple of its row count", a.fn, k);
+      const int64_t w = Aa.len / Rr.len;
+      if (widths[k % nb] != 0 && widths[k % nb] != w)
+        return packed_fail("%s: bucket %d has width %lld in one partition and %d in another", a.fn, k % nb, (long long)w, widths[k % nb]);
+      widths[k % nb] = (int32_t)w;
+    } else if (Aa.len != 0) {
+      return packed_fail("%s: A_%d has slots but no rows", a.fn, k);
+    }
+  }
+  for (int b = 0; b < nb; ++b)
+    if (widths[b] == 0) widths[b] = b ? widths[b - 1] : 1;  // width of an empty bucket is immaterial
+  DeviceGuard g;
+  if (g.enter(a.dev_id)) return forward(-1);
+  HybKey key;
+  for (int k = 0; k < nk; ++k) {
+    key.ptrs.push_back((uintptr_t)Ak[k]);
+    key.ptrs.push_back((uintptr_t)Rk[k]);
+    key.ptrs.push_back((uintptr_t)Ck[k]);
+    key.nums.push_back(nrows[k]);
+  }
+  for (int b = 0; b < nb; ++b) key.nums.push_back(widths[b]);
+  key.nums.push_back(parts);
+  key.nums.push_back(a.dev_id);
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  if (!g_hyb_plan || !(key == g_hyb_key)) {
+    if (g_hyb_plan) stir_hyb_plan_destroy(g_hyb_plan);
+    g_hyb_plan = nullptr;
+    if (stir_hyb_plan_create(&g_hyb_plan, (int32_t)(C.len / feat), (int32_t)(B.len / feat), (int32_t)parts, nb,
+                             widths.data(), nrows.data(), Ak.data(), Rk.data(), Ck.data()))
+      return forward(-1);
+    g_hyb_key = key;
+  }
+  return forward(stir_hyb_spmm_f32(g_hyb_plan, (int32_t)feat, (const float*)B.data, (float*)C.data, g_stream));
+}
+
+static int sddmm_common(const char* fn, bool preproc, TVMValue* v, int* tc, int n) {
+  Args a{fn, v, tc, n};
+  if (!a.count(6)) return -1;
+  Arr A = a.arr(0, "A", kDLFloat, 32, kDevice), B = a.arr(1, "B", kDLFloat, 32, kDevice),
+      C = a.arr(2, "C", kDLFloat, 32, kDevice), P = a.arr(3, "indptr", kDLInt, 32, kDevice),
+      I = a.arr(4, "indices", kDLInt, 32, kDevice), M = a.arr(5, "mid", kDLInt, 32, kDevice);
+  if (!a.ok) return -1;
+  const int64_t m = P.len - 1, nnz = C.len;
+  if (m < 0) return packed_fail("%s: indptr must have at least one entry", fn);
+  a.len(I, "indices", nnz);
+  a.len(M, "mid", nnz);
+  if (!a.ok) return -1;
+  if (nnz == 0) return 0;
+  if (m == 0 || A.len % m != 0 || A.len == 0) return packed_fail("%s: A.shape[0] is not a multiple of m", fn);
+  const int64_t feat = A.len / m;
+  if (B.len % feat != 0) return packed_fail("%s: B.shape[0] is not a multiple of feat", fn);
+  if (!fits_i32(m) || !fits_i32(B.len / feat) || !fits_i32(feat)) return packed_fail("%s: sizes exceed int32", fn);
+  DeviceGuard g;
+  if (g.enter(a.dev_id)) return forward(-1);
+  if (preproc) return forward(stir_sddmm_preproc((int32_t)m, nnz, (const int32_t*)P.data, (int32_t*)M.data, g_stream));
+  return forward(stir_sddmm_f32((int32_t)m, (int32_t)(B.len / feat), (int32_t)feat, nnz, (const float*)A.data,
+                                (const float*)B.data, (float*)C.data, (const int32_t*)P.data,
+                                (const int32_t*)I.data, (const int32_t*)M.data, g_stream));
+}
+
+int stir_packed_sddmm_preproc(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return sddmm_common("sparsetir.sddmm_preproc", true, v, tc, n);
+}
+int stir_packed_sddmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return sddmm_common("sparsetir.sddmm", false, v, tc, n);
+}
+
+int stir_packed_bsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.bsrmm", v, tc, n};
+  if (!a.count(7)) return -1;
+  // the 16-bit type is read from A's dtype: float16 (kDLFloat/16) or bfloat16 (kDLBfloat/16)
+  const DLTensor* d0 = (tc[0] == kTVMDLTensorHandle || tc[0] == kTVMNDArrayHandle || tc[0] == kTVMOpaqueHandle)
+                           ? static_cast<const DLTensor*>(v[0].v_handle) : nullptr;
+  if (!d0) return packed_fail("%s: Expect arg[0] to be pointer", a.fn);
+  const bool bf = d0->dtype.code == kDLBfloat;
+  const uint8_t code = bf ? kDLBfloat : kDLFloat;
+  Arr A = a.arr(0, "A", code, 16, kDevice), X = a.arr(1, "X", code, 16, kDevice);
+  const DLTensor* d2 = (tc[2] == kTVMDLTensorHandle || tc[2] == kTVMNDArrayHandle || tc[2] == kTVMOpaqueHandle)
+                           ? static_cast<const DLTensor*>(v[2].v_handle) : nullptr;
+  if (!d2) return packed_fail("%s: Expect arg[2] to be pointer", a.fn);
+  const bool out32 = d2->dtype.code == kDLFloat && d2->dtype.bits == 32;
+  Arr Y = out32 ? a.arr(2, "Y", kDLFloat, 32, kDevice) : a.arr(2, "Y", code, 16, kDevice);
+  Arr P = a.arr(3, "indptr", kDLInt, 32, kDevice), I = a.arr(4, "indices", kDLInt, 32, kDevice);
+  const int64_t blk = a.integer(5, "blk"), feat = a.integer(6, "feat");
+  if (!a.ok) return -1;
+  const int64_t mb = P.len - 1, nnzb = I.len;
+  if (mb < 0 || blk <= 0 || feat <= 0) return packed_fail("%s: bad sizes", a.fn);
+  a.len(A, "A", nnzb * blk * blk);
+  a.len(Y, "Y", mb * blk * feat);
+  if (!a.ok) return -1;
+  if (X.len % (blk * feat) != 0) return packed_fail("%s: X.shape[0] is not a multiple of blk*feat", a.fn);
+  const int64_t nbk = X.len / (blk * feat);
+  if (!fits_i32(mb) || !fits_i32(nbk) || !fits_i32(blk) || !fits_i32(feat)) return packed_fail("%s: sizes exceed int32", a.fn);
+  DeviceGuard g;
+  if (g.enter(a.dev_id)) return forward(-1);
+  const int dt = bf ? STIR_BF16 : STIR_F16;
+  return forward(stir_bsr_spmm(dt, out32 ? STIR_F32 : dt, (int32_t)mb, (int32_t)nbk, (int32_t)blk, (int32_t)feat,
+                               nnzb, A.data, X.data, Y.data, (const int32_t*)P.data, (const int32_t*)I.data,
+                               g_stream));
+}
+
+int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.rgms", v, tc, n};
+  if (n < 5 || (n - 5) % 4 != 0) return packed_fail("%s: num_args should be 3 + 4*buckets + 2", a.fn);
+  const int nb = (n - 5) / 4;
+  Arr W = a.arr(0, "W", kDLFloat, 16, kDevice), X = a.arr(1, "X", kDLFloat, 16, kDevice),
+      Y = a.arr(2, "Y", kDLFloat, 32, kDevice);
+  const int64_t fin = a.integer(n - 2, "feat_in"), fout = a.integer(n - 1, "feat_out");
+  if (!a.ok) return -1;
+  if (fin <= 0 || fout <= 0 || W.len % (fin * fout) != 0 || X.len % fin != 0 || Y.len % fout != 0)
+    return packed_fail("%s: W/X/Y lengths do not fit feat_in=%lld feat_out=%lld", a.fn, (long long)fin, (long long)fout);
+  std::vector<const void*> Ak(nb);
+  std::vector<const int32_t*> Rk(nb), Ck(nb), Mk(nb);
+  std::vector<int64_t> groups(nb);
+  std::vector<int32_t> rb(nb, 1), cb(nb, 1);
+  for (int b = 0; b < nb; ++b) {
+    Arr Aa = a.arr(3 + 3 * b, "A_k", kDLFloat, 16, kDevice), Rr = a.arr(4 + 3 * b, "rows_k", kDLInt, 32, kDevice),
+        Cc = a.arr(5 + 3 * b, "cols_k", kDLInt, 32, kDevice), Mm = a.arr(3 + 3 * nb + b, "mids_k", kDLInt, 32, kDevice);
+    if (!a.ok) return -1;
+    a.len(Cc, "cols_k", Aa.len);
+    if (!a.ok) return -1;
+    groups[b] = Mm.len;
+    Ak[b] = Aa.data;
+    Rk[b] = (const int32_t*)Rr.data;
+    Ck[b] = (const int32_t*)Cc.data;
+    Mk[b] = (const int32_t*)Mm.data;
+    if (Mm.len > 0) {
+      if (Rr.len % Mm.len != 0 || Rr.len == 0 || Aa.len % Rr.len != 0)
+        return packed_fail("%s: bucket %d: rows/cols lengths are not multiples of the group count", a.fn, b);
+      rb[b] = (int32_t)(Rr.len / Mm.len);
+      cb[b] = (int32_t)(Aa.len / Rr.len);
+    } else if (Rr.len != 0 || Aa.len != 0) {
+      return packed_fail("%s: bucket %d has slots but no groups", a.fn, b);
+    }
+  }
+  DeviceGuard g;
+  if (g.enter(a.dev_id)) return forward(-1);
+  HybKey key;
+  for (int b = 0; b < nb; ++b) {
+    key.ptrs.push_back((uintptr_t)Ak[b]);
+    key.ptrs.push_back((uintptr_t)Rk[b]);
+    key.ptrs.push_back((uintptr_t)Ck[b]);
+    key.ptrs.push_back((uintptr_t)Mk[b]);
+    key.nums.push_back(groups[b]);
+    key.nums.push_back(rb[b]);
+    key.nums.push_back(cb[b]);
+  }
+  key.nums.push_back(a.dev_id);
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  if (!g_rgms_plan || !(key == g_rgms_key)) {
+    if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
+    g_rgms_plan = nullptr;
+    if (stir_rgms_plan_create(&g_rgms_plan, nb, rb.data(), cb.data(), groups.data(), Ak.data(), Rk.data(),
+                              Ck.data(), Mk.data()))
+      return forward(-1);
+    g_rgms_key = key;
+  }
+  return forward(stir_rgms_f16(g_rgms_plan, (int32_t)(Y.len / fout), (int32_t)(X.len / fin),
+                               (int32_t)(W.len / (fin * fout)), (int32_t)fin, (int32_t)fout, W.data, X.data,
+                               (float*)Y.data, g_stream));
+}
+
+// ----------------------------------------------------------------------------- format pass
+
+static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
+  Args a{fn, v, tc, n};
+  if (n < 7) return packed_fail("%s: num_args should be at least 7", fn);
+  const bool dev = a.on_device(2);
+  const Where w = dev ? kDevice : kHost;
+  const int64_t num_rows = a.integer(0, "num_rows"), num_cols = a.integer(1, "num_cols");
+  Arr P = a.arr(2, "indptr", kDLInt, 32, w), I = a.arr(3, "indices", kDLInt, 32, w);
+  const int64_t parts = a.integer(4, "num_col_parts");
+  Arr Bk = a.arr(5, "buckets", kDLInt, 32, kHost);
+  if (!a.ok) return -1;
+  if (!fits_i32(num_rows) || !fits_i32(num_cols) || parts <= 0 || !fits_i32(parts) || Bk.len <= 0)
+    return packed_fail("%s: bad sizes", fn);
+  a.len(P, "indptr", num_rows + 1);
+  if (!a.ok) return -1;
+  const int nb = (int)Bk.len;
+  const int64_t nk = parts * nb;
+  DeviceGuard g;
+  if (dev && g.enter(a.dev_id)) return forward(-1);
+  // the device path keeps its scratch between the sizing and the fill call
+  static thread_local void* ws = nullptr;
+  static thread_local size_t ws_bytes = 0;
+  if (!fill) {
+    if (!a.count(7)) return -1;
+    Arr N = a.arr(6, "nrows_out", kDLInt, 64, kHost);
+    if (!a.ok || !a.len(N, "nrows_out", nk)) return -1;
+    if (!dev)
+      return forward(stir_column_part_hyb_sizes((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
+                                                (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data,
+                                                nb, (int64_t*)N.data));
+    const size_t need = stir_column_part_hyb_device_workspace_bytes((int32_t)num_rows, (int32_t)parts, nb);
+    if (need > ws_bytes) {
+      if (ws) (void)hipFree(ws);
+      ws = nullptr;
+      ws_bytes = 0;
+      if (hipMalloc(&ws, need) != hipSuccess) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
+      ws_bytes = need;
+    }
+    return forward(stir_column_part_hyb_device_sizes((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
+                                                     (const int32_t*)I.data, (int32_t)parts,
+                                                     (const int32_t*)Bk.data, nb, ws, (int64_t*)N.data, g_stream));
+  }
+  if (!a.count(6 + 3 * (int)nk)) return -1;
+  std::vector<int32_t*> R(nk), C(nk), M(nk);
+  for (int64_t k = 0; k < nk; ++k) {
+    Arr r = a.arr(6 + 3 * (int)k, "rows_k", kDLInt, 32, w), c = a.arr(7 + 3 * (int)k, "cols_k", kDLInt, 32, w),
+        mk = a.arr(8 + 3 * (int)k, "mask_k", kDLInt, 32, w);
+    if (!a.ok) return -1;
+    const int64_t width = ((const int32_t*)Bk.data)[k % nb];
+    a.len(c, "cols_k", r.len * width);
+    a.len(mk, "mask_k", r.len * width);
+    if (!a.ok) return -1;
+    R[k] = (int32_t*)r.data;
+    C[k] = (int32_t*)c.data;
+    M[k] = (int32_t*)mk.data;
+  }
+  if (!dev)
+    return forward(stir_column_part_hyb_fill((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
+                                             (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data, nb,
+                                             R.data(), C.data(), M.data()));
+  if (!ws) return packed_fail("%s: call tir.sparse.ColumnPartHyb.sizes first on this thread", fn);
+  int rc = stir_column_part_hyb_device_fill((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
+                                            (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data, nb,
+                                            ws, R.data(), C.data(), M.data(), g_stream);
+  return forward(rc);
+}
+
+int stir_packed_column_part_hyb_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return hyb_format("tir.sparse.ColumnPartHyb.sizes", false, v, tc, n);
+}
+int stir_packed_column_part_hyb_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return hyb_format("tir.sparse.ColumnPartHyb.fill", true, v, tc, n);
+}
+
+static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
+  Args a{fn, v, tc, n};
+  if (n < 7) return packed_fail("%s: num_args should be at least 7", fn);
+  Arr P0 = a.arr(0, "csf_indptr_0", kDLInt, 32, kHost), I0 = a.arr(1, "csf_indices_0", kDLInt, 32, kHost),
+      P1 = a.arr(2, "csf_indptr_1", kDLInt, 32, kHost), I1 = a.arr(3, "csf_indices_1", kDLInt, 32, kHost),
+      RB = a.arr(4, "nnz_rows_bkt", kDLInt, 32, kHost), CB = a.arr(5, "nnz_cols_bkt", kDLInt, 32, kHost);
+  if (!a.ok) return -1;
+  if (RB.len != CB.len) return packed_fail("%s: Input nnz_rows and nnz_cols should have same length.", fn);
+  const int nb = (int)CB.len;
+  const int64_t rels = P0.len - 1;
+  if (rels < 0 || !fits_i32(rels)) return packed_fail("%s: csf_indptr_0 must have at least one entry", fn);
+  const int32_t *p0 = (const int32_t*)P0.data, *i0 = (const int32_t*)I0.data, *p1 = (const int32_t*)P1.data,
+                *i1 = (const int32_t*)I1.data, *rb = (const int32_t*)RB.data, *cb = (const int32_t*)CB.data;
+  if (!fill) {
+    if (!a.count(7)) return -1;
+    Arr G = a.arr(6, "groups_out", kDLInt, 64, kHost);
+    if (!a.ok || !a.len(G, "groups_out", nb)) return -1;
+    return forward(stir_csf_to_ell3d_sizes((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, (int64_t*)G.data));
+  }
+  if (!a.count(6 + 4 * nb)) return -1;
+  std::vector<int32_t*> OP(nb), R(nb), C(nb), M(nb);
+  for (int b = 0; b < nb; ++b) {
+    Arr op = a.arr(6 + 4 * b, "indptr_k", kDLInt, 32, kHost), r = a.arr(7 + 4 * b, "rows_k", kDLInt, 32, kHost),
+        c = a.arr(8 + 4 * b, "cols_k", kDLInt, 32, kHost), mk = a.arr(9 + 4 * b, "mask_k", kDLInt, 32, kHost);
+    if (!a.ok) return -1;
+    a.len(op, "indptr_k", rels + 1);
+    a.len(c, "cols_k", r.len * cb[b]);
+    a.len(mk, "mask_k", r.len * cb[b]);
+    if (!a.ok) return -1;
+    OP[b] = (int32_t*)op.data;
+    R[b] = (int32_t*)r.data;
+    C[b] = (int32_t*)c.data;
+    M[b] = (int32_t*)mk.data;
+  }
+  return forward(stir_csf_to_ell3d_fill((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, OP.data(), R.data(), C.data(),
+                                        M.data()));
+}
+
+int stir_packed_csf_to_ell3d_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return csf_format("tir.sparse.CSFToELL3D.sizes", false, v, tc, n);
+}
+int stir_packed_csf_to_ell3d_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return csf_format("tir.sparse.CSFToELL3D.fill", true, v, tc, n);
+}
+
+int stir_packed_condense_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"tir.sparse.ConDense.sizes", v, tc, n};
+  if (!a.count(6)) return -1;
+  Arr P = a.arr(0, "indptr", kDLInt, 32, kHost), I = a.arr(1, "indices", kDLInt, 32, kHost);
+  const int64_t t = a.integer(2, "t"), g = a.integer(3, "g");
+  Arr GP = a.arr(4, "group_indptr_out", kDLInt, 32, kHost), NG = a.arr(5, "num_groups_out", kDLInt, 64, kHost);
+  if (!a.ok) return -1;
+  const int64_t rows = P.len - 1;
+  if (rows < 0 || t <= 0 || g <= 0 || !fits_i32(t) || !fits_i32(g)) return packed_fail("%s: bad sizes", a.fn);
+  a.len(GP, "group_indptr_out", (rows + t - 1) / t + 1);
+  a.len(NG, "num_groups_out", 1);
+  if (!a.ok) return -1;
+  return forward(stir_condense_sizes((int32_t)rows, (const int32_t*)P.data, (const int32_t*)I.data, (int32_t)t,
+                                     (int32_t)g, (int32_t*)GP.data, (int64_t*)NG.data));
+}
+
+int stir_packed_condense_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"tir.sparse.ConDense.fill", v, tc, n};
+  if (!a.count(6)) return -1;
+  Arr P = a.arr(0, "indptr", kDLInt, 32, kHost), I = a.arr(1, "indices", kDLInt, 32, kHost);
+  const int64_t t = a.integer(2, "t"), g = a.integer(3, "g");
+  Arr TI = a.arr(4, "tile_indices_out", kDLInt, 32, kHost), MK = a.arr(5, "mask_out", kDLInt, 32, kHost);
+  if (!a.ok) return -1;
+  const int64_t rows = P.len - 1;
+  if (rows < 0 || t <= 0 || g <= 0 || !fits_i32(t) || !fits_i32(g)) return packed_fail("%s: bad sizes", a.fn);
+  if (TI.len % g != 0 || MK.len != TI.len * t) return packed_fail("%s: output lengths do not fit t and g", a.fn);
+  return forward(stir_condense_fill((int32_t)rows, (const int32_t*)P.data, (const int32_t*)I.data, (int32_t)t,
+                                    (int32_t)g, (int32_t*)TI.data, (int32_t*)MK.data));
+}
+
+// ------------------------------------------------------------------------------ registry
+
+struct PackedEntry {
+  const char* name;
+  TVMPackedCFunc fn;
+};
+static const PackedEntry kTable[] = {
+    {"sparsetir.csrmm", stir_packed_csrmm},
+    {"sparsetir.hyb_csrmm", stir_packed_hyb_csrmm},
+    {"sparsetir.sddmm_preproc", stir_packed_sddmm_preproc},
+    {"sparsetir.sddmm", stir_packed_sddmm},
+    {"sparsetir.bsrmm", stir_packed_bsrmm},
+    {"sparsetir.rgms", stir_packed_rgms},
+    {"tir.sparse.ColumnPartHyb.sizes", stir_packed_column_part_hyb_sizes},
+    {"tir.sparse.ColumnPartHyb.fill", stir_packed_column_part_hyb_fill},
+    {"tir.sparse.CSFToELL3D.sizes", stir_packed_csf_to_ell3d_sizes},
+    {"tir.sparse.CSFToELL3D.fill", stir_packed_csf_to_ell3d_fill},
+    {"tir.sparse.ConDense.sizes", stir_packed_condense_sizes},
+    {"tir.sparse.ConDense.fill", stir_packed_condense_fill},
+};
+static const int kTableSize = (int)(sizeof(kTable) / sizeof(kTable[0]));
+
+int stir_packed_count(void) { return kTableSize; }
+const char* stir_packed_name(int i) { return i >= 0 && i < kTableSize ? kTable[i].name : nullptr; }
+TVMPackedCFunc stir_packed_func(int i) { return i >= 0 && i < kTableSize ? kTable[i].fn : nullptr; }
+
+int stir_register_all(int (*create_from_cfunc)(TVMPackedCFunc, void*, TVMPackedCFuncFinalizer,
+                                               TVMFunctionHandle*),
+                      int (*register_global)(const char*, TVMFunctionHandle, int), int override) {
+  if (!create_from_cfunc || !register_global) return packed_fail("stir_register_all: null callback");
+  for (int i = 0; i < kTableSize; ++i) {
+    TVMFunctionHandle h = nullptr;
+    int rc = create_from_cfunc(kTable[i].fn, nullptr, nullptr, &h);
+    if (rc != 0) return rc;
+    rc = register_global(kTable[i].name, h, override);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
+}  // extern "C"

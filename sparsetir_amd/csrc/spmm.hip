@@ -6,6 +6,9 @@
 // step with fully coalesced 16-byte loads.  Column indices and values are fetched once per
 // wavefront with one coalesced load (lane l holds slot l of the 64-slot tile) and handed to
 // the lane groups through cross-lane reads, so no lane issues a redundant index load.
+#include <algorithm>
+#include <vector>
+
 #include "common.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -22,8 +25,12 @@ struct alignas(16) HybBucket {
   int32_t width;
   int32_t log2w;   // log2(width) when the bucket runs in slot-tile mode, else -1
   int32_t atomic;  // accumulate with atomics instead of storing
-  int32_t pad;
+  int32_t chunks;  // row mode: wave tiles per ELL row (each covers kRowChunk slots)
 };
+
+// Row mode splits an ELL row of an accumulating bucket into chunks of this many slots, one
+// wavefront each, so that a hub row does not serialise on a single wavefront.
+constexpr int kRowChunk = 256;
 
 __device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 
@@ -172,8 +179,10 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
       const int col = __shfl(my_col, sl, kWave);
       v[u] = __shfl(my_val, sl, kWave);
       const float* bp = B + (int64_t)col * feat + gl * 4;
+      // a slot of weight zero (padding) adds nothing: its row of B is not fetched
 #pragma unroll
-      for (int r = 0; r < REP; ++r) x[u][r] = ld4(bp + r * G * 4);
+      for (int r = 0; r < REP; ++r)
+        x[u][r] = v[u] != 0.f ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int u = 0; u < CH; ++u) {
@@ -199,7 +208,8 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
   }
 }
 
-// Row mode (any width): a wavefront owns one ELL row and walks it 64 slots at a time.
+// Row mode (any width): a wavefront owns one ELL row, or one kRowChunk-slot piece of it when
+// the bucket accumulates, and walks it 64 slots at a time.
 template <int G, int REP>
 __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int feat,
                                              const float* __restrict__ B, float* __restrict__ C,
@@ -207,15 +217,18 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
   constexpr int CH = G < 8 ? G : 8;
   const int g = lane / G, gl = lane % G;
   const int w = bk.width;
-  const int32_t* cols = bk.cols + t * w;
-  const float* vals = bk.A + t * w;
+  const int64_t row = bk.chunks > 1 ? t / bk.chunks : t;
+  const int s_begin = bk.chunks > 1 ? (int)(t % bk.chunks) * kRowChunk : 0;
+  const int s_end = bk.chunks > 1 ? min(w, s_begin + kRowChunk) : w;
+  const int32_t* cols = bk.cols + row * w;
+  const float* vals = bk.A + row * w;
   float4 acc[REP];
 #pragma unroll
   for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int c0 = 0; c0 < w; c0 += kWave) {
+  for (int c0 = s_begin; c0 < s_end; c0 += kWave) {
     const int s = c0 + lane;
-    const int my_col = s < w ? cols[s] : 0;
-    const float my_val = s < w ? vals[s] : 0.f;
+    const int my_col = s < s_end ? cols[s] : 0;
+    const float my_val = s < s_end ? vals[s] : 0.f;
 #pragma unroll 1
     for (int c = 0; c < G; c += CH) {
       float4 x[CH][REP];
@@ -224,12 +237,11 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
       for (int u = 0; u < CH; ++u) {
         const int sl = g * G + c + u;
         const int col = __shfl(my_col, sl, kWave);
-        v[u] = __shfl(my_val, sl, kWave);
+        v[u] = __shfl(my_val, sl, kWave);  // zero beyond s_end and on padding
         const float* bp = B + (int64_t)col * feat + gl * 4;
-        const bool live = c0 + sl < w;
 #pragma unroll
         for (int r = 0; r < REP; ++r)
-          x[u][r] = live ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+          x[u][r] = v[u] != 0.f ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int u = 0; u < CH; ++u)
@@ -238,7 +250,7 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
     }
   }
   reduce_groups<G, REP>(acc, kWave);
-  if (g == 0) write_row<G, REP>(C, bk.rows[t], feat, gl, acc, bk.atomic != 0);
+  if (g == 0) write_row<G, REP>(C, bk.rows[row], feat, gl, acc, bk.atomic != 0);
 }
 
 __device__ __forceinline__ int find_bucket(const HybBucket* __restrict__ table, int nb,
@@ -355,20 +367,25 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
   for (int b = 0; b < num_buckets; ++b)
     STIR_REQUIRE(bucket_widths[b] > 0, "hyb_plan_create: bucket width %d is not positive", bucket_widths[b]);
   const int total = num_col_parts * num_buckets;
-  HybBucket* host = new HybBucket[total > 0 ? 2 * total : 1];
-  HybBucket* host_rows = host + total;
-  int nk = 0;
-  int64_t tiles = 0, rows = 0;
   for (int k = 0; k < total; ++k) {
-    if (nrows[k] < 0) {
-      delete[] host;
-      return stir::fail("hyb_plan_create: nrows[%d] is negative", k);
-    }
-    if (nrows[k] == 0) continue;
-    if (!d_A[k] || !d_rows[k] || !d_cols[k]) {
-      delete[] host;
-      return stir::fail("hyb_plan_create: bucket %d has rows but a null array", k);
-    }
+    STIR_REQUIRE(nrows[k] >= 0, "hyb_plan_create: nrows[%d] is negative", k);
+    STIR_REQUIRE(nrows[k] == 0 || (d_A[k] && d_rows[k] && d_cols[k]),
+                 "hyb_plan_create: bucket %d has rows but a null array", k);
+  }
+  // Widest buckets first: their wavefronts run longest, so they are dispatched first and the
+  // launch does not end on a tail of hub rows.
+  std::vector<int> order;
+  for (int k = 0; k < total; ++k)
+    if (nrows[k] > 0) order.push_back(k);
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+    return bucket_widths[a % num_buckets] > bucket_widths[b % num_buckets];
+  });
+  const int nk = (int)order.size();
+  std::vector<HybBucket> host(nk > 0 ? 2 * nk : 1);
+  HybBucket* host_rows = host.data() + nk;
+  int64_t tiles = 0, rows = 0;
+  for (int q = 0; q < nk; ++q) {
+    const int k = order[q];
     const int b = k % num_buckets;
     const int w = bucket_widths[b];
     HybBucket e;
@@ -378,16 +395,16 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
     e.nrows = nrows[k];
     e.width = w;
     e.atomic = (num_col_parts > 1 || b == num_buckets - 1) ? 1 : 0;
-    e.pad = 0;
     const bool slot_mode = stir::is_pow2(w) && w <= kWave;
     e.log2w = slot_mode ? log2_exact(w) : -1;
+    e.chunks = (!slot_mode && e.atomic && w > kRowChunk) ? (int)stir::ceil_div(w, kRowChunk) : 1;
     e.tile_begin = tiles;
-    host[nk] = e;
-    tiles += slot_mode ? stir::ceil_div(nrows[k] * w, kWave) : nrows[k];
+    host[q] = e;
+    tiles += slot_mode ? stir::ceil_div(nrows[k] * w, kWave) : nrows[k] * e.chunks;
     e.tile_begin = rows;
-    host_rows[nk] = e;
+    e.chunks = 1;
+    host_rows[q] = e;
     rows += nrows[k];
-    ++nk;
   }
   stir_hyb_plan* p = new stir_hyb_plan();
   p->m = m;
@@ -404,12 +421,11 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
     e = hipMalloc(reinterpret_cast<void**>(&p->d_table_tiles), sizeof(HybBucket) * 2 * nk);
     if (e == hipSuccess) {
       p->d_table_rows = p->d_table_tiles + nk;
-      e = hipMemcpy(p->d_table_tiles, host, sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
+      e = hipMemcpy(p->d_table_tiles, host.data(), sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
       if (e == hipSuccess)
         e = hipMemcpy(p->d_table_rows, host_rows, sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
     }
   }
-  delete[] host;
   if (e != hipSuccess) {
     if (p->d_table_tiles) (void)hipFree(p->d_table_tiles);
     delete p;

@@ -1,0 +1,109 @@
+"""The TVM-PackedFunc entry points on device tensors: same results as the oracle / the
+operator objects, and the generated-stub style argument checks."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparsetir_amd as st
+from sparsetir_amd import datasets, ops, packed
+from sparsetir_amd._lib import SparseTIRError
+from helpers import random_csf, random_csr, sddmm_f64, spmm_f64
+
+pytestmark = pytest.mark.gpu
+
+
+def test_packed_csrmm_and_sddmm(dev):
+    m, n, feat = 700, 500, 64
+    indptr, indices = random_csr(m, n, 15000, 0, skew=1.0)
+    rng = np.random.default_rng(0)
+    vals = rng.random(len(indices), dtype=np.float32)
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    a2 = rng.standard_normal((m, feat), dtype=np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    c = torch.zeros(m * feat, device=dev)
+    packed.get_global_func("sparsetir.csrmm")(t(vals), t(x.ravel()), c, t(indptr), t(indices))
+    torch.cuda.synchronize()
+    want = spmm_f64(indptr, indices, vals, x)
+    scale = spmm_f64(indptr, indices, vals, np.abs(x))
+    assert np.all(np.abs(c.cpu().numpy().reshape(m, feat) - want) <= 1e-5 * scale + 1e-30)
+
+    out = torch.zeros(len(indices), device=dev)
+    mid = torch.zeros(len(indices), dtype=torch.int32, device=dev)
+    args = (t(a2.ravel()), t(x.ravel()), out, t(indptr), t(indices), mid)
+    packed.get_global_func("sparsetir.sddmm_preproc")(*args)
+    packed.get_global_func("sparsetir.sddmm")(*args)
+    torch.cuda.synchronize()
+    assert np.array_equal(mid.cpu().numpy(), oracle.sddmm_mid(indptr, len(indices)))
+    assert np.allclose(out.cpu().numpy(), sddmm_f64(indptr, indices, a2, x), rtol=1e-4, atol=1e-4)
+
+
+def test_packed_device_column_part_hyb_and_hyb_csrmm(dev):
+    m = n = 900
+    feat, parts, buckets = 128, 2, [1, 2, 4, 8, 16]
+    indptr, indices = random_csr(m, n, 20000, 1, skew=1.2)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    d_ptr, d_idx = t(indptr), t(indices)
+    b = np.asarray(buckets, np.int32)
+    nrows = np.zeros(parts * len(buckets), np.int64)
+    packed.get_global_func("tir.sparse.ColumnPartHyb.sizes")(m, n, d_ptr, d_idx, parts, b, nrows)
+    outs = []
+    for k, r in enumerate(nrows):
+        w = buckets[k % len(buckets)]
+        outs += [torch.empty(int(r), dtype=torch.int32, device=dev),
+                 torch.empty(int(r) * w, dtype=torch.int32, device=dev),
+                 torch.empty(int(r) * w, dtype=torch.int32, device=dev)]
+    packed.get_global_func("tir.sparse.ColumnPartHyb.fill")(m, n, d_ptr, d_idx, parts, b, *outs)
+    torch.cuda.synchronize()
+    rows, cols, mask = oracle.column_part_hyb(m, n, indptr, indices, parts, buckets)
+    triples = []
+    for p in range(parts):
+        for q in range(len(buckets)):
+            k = p * len(buckets) + q
+            assert np.array_equal(outs[3 * k].cpu().numpy(), rows[p][q])
+            assert np.array_equal(outs[3 * k + 1].cpu().numpy(), cols[p][q].ravel())
+            assert np.array_equal(outs[3 * k + 2].cpu().numpy(), mask[p][q].ravel())
+            triples += [outs[3 * k + 2].float(), outs[3 * k], outs[3 * k + 1]]
+    x = np.random.default_rng(1).standard_normal((n, feat), dtype=np.float32)
+    c = torch.zeros(m * feat, device=dev)
+    f = packed.get_global_func("sparsetir.hyb_csrmm")
+    f(t(x.ravel()), c, *triples, feat, parts)
+    torch.cuda.synchronize()
+    ones = np.ones(len(indices), np.float32)
+    want = spmm_f64(indptr, indices, ones, x)
+    scale = spmm_f64(indptr, indices, ones, np.abs(x))
+    assert np.all(np.abs(c.cpu().numpy().reshape(m, feat) - want) <= 1e-5 * scale + 1e-30)
+    with pytest.raises(SparseTIRError, match="num_args"):
+        f(t(x.ravel()), c, *triples[:-1], feat, parts)
+
+
+def test_packed_bsrmm_and_rgms_match_operator_objects(dev):
+    cfg = datasets.config4(seed=2, mb=8, nb=8, blk=32, density=0.3, feat=64)
+    a = torch.from_numpy(cfg["data"]).to(dev).half().reshape(-1)
+    x = torch.from_numpy(cfg["x"]).to(dev).half().reshape(-1)
+    ptr, idx = torch.from_numpy(cfg["indptr"]).to(dev), torch.from_numpy(cfg["indices"]).to(dev)
+    y1 = torch.zeros(8 * 32 * 64, dtype=torch.float16, device=dev)
+    y2 = torch.zeros_like(y1)
+    ops.build_bsrmm(8, 8, len(cfg["indices"]), 32, 64)(a, x, y1, ptr, idx)
+    packed.get_global_func("sparsetir.bsrmm")(a, x, y2, ptr, idx, 32, 64)
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2) and y1.abs().sum() > 0
+
+    R, n, fin, fout, group, buckets = 4, 200, 32, 32, 32, [1, 2, 4, 8]
+    csf = random_csf(R, n, 800, seed=3)
+    rb = [group // b for b in buckets]
+    iptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    rng = np.random.default_rng(3)
+    w = t(rng.standard_normal(R * fin * fout).astype(np.float16))
+    xx = t(rng.standard_normal(n * fin).astype(np.float16))
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float16).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(iptr[k]))))
+    ya = torch.zeros(n * fout, device=dev)
+    yb = torch.zeros(n * fout, device=dev)
+    ops.build_rgms(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols])(w, xx, ya, *triples, *mids)
+    packed.get_global_func("sparsetir.rgms")(w, xx, yb, *triples, *mids, fin, fout)
+    torch.cuda.synchronize()
+    assert torch.allclose(ya, yb, rtol=1e-5, atol=1e-5) and ya.abs().sum() > 0

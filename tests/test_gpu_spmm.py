@@ -186,7 +186,7 @@ def test_hyb_spmm_store_semantics_of_non_atomic_buckets(dev):
     last_rows = np.unique(triples[-1][1])
     other = np.setdiff1d(np.arange(m), last_rows)
     assert np.array_equal(twice[other], once[other])
-    assert np.allclose(twice[last_rows], 2 * once[last_rows], rtol=1e-6)
+    assert np.allclose(twice[last_rows], 2 * once[last_rows], rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.parametrize("feat", [32, 128])
