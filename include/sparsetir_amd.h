@@ -31,6 +31,9 @@ const char* stir_last_error(void);
 /* Library version string. */
 const char* stir_version(void);
 
+/* Element types of 16-bit / 32-bit floating-point operands. */
+enum { STIR_F16 = 0, STIR_BF16 = 1, STIR_F32 = 2 };
+
 /* ------------------------------------------------------------------ format pass (host) */
 
 /*
@@ -100,6 +103,39 @@ int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols,
                                      int32_t* const* d_col_indices, int32_t* const* d_mask,
                                      void* stream);
 
+/*
+ * Value rewrite for hyb: after _sizes and _fill (same workspace), gathers the CSR values into the
+ * per-bucket arrays, d_A[k][slot] = d_values[e] for the slot nonzero e was placed in, padding
+ * slots zero.  This is what the reference's "rewrite_A_k" preprocess blocks compute
+ * (tests/python/sparsetir/sparse_tir_composable_format_scripts.py:331-351); its example scripts
+ * feed the 0/1 mask instead (examples/spmm/bench_spmm.py:211-213), which handles unweighted
+ * graphs only.
+ */
+int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const int32_t* d_indptr,
+                                       const int32_t* d_indices, const float* d_values,
+                                       int32_t num_col_parts, const int32_t* buckets,
+                                       int32_t num_buckets, void* d_workspace, const int64_t* nrows,
+                                       float* const* d_A, void* stream);
+
+/*
+ * CSR -> BSR packing on the GPU (blk x blk blocks; m and n multiples of blk): the canonical BSR
+ * arrays that scipy's csr_matrix.tobsr hands the reference's example
+ * (examples/blocksparse/bsr_spmm.py:441-445) -- block columns ascending in each block row,
+ * absent entries of a stored block zero.  The CSR input must hold no duplicate entries.
+ * _sizes fills d_bsr_indptr (m/blk + 1) and *nnzb (host; synchronises the stream); _fill writes
+ * d_bsr_indices (nnzb) and d_bsr_data (nnzb*blk*blk of data_dtype: STIR_F32, STIR_F16 or
+ * STIR_BF16, converted from the fp32 values with round-to-nearest-even).  d_workspace holds
+ * stir_csr_to_bsr_workspace_bytes(...) bytes and must stay untouched between the two calls.
+ */
+size_t stir_csr_to_bsr_workspace_bytes(int32_t m, int32_t n, int32_t blk);
+int stir_csr_to_bsr_sizes(int32_t m, int32_t n, int32_t blk, const int32_t* d_indptr,
+                          const int32_t* d_indices, void* d_workspace, int32_t* d_bsr_indptr,
+                          int64_t* nnzb, void* stream);
+int stir_csr_to_bsr_fill(int32_t m, int32_t n, int32_t blk, const int32_t* d_indptr,
+                         const int32_t* d_indices, const float* d_values, void* d_workspace,
+                         const int32_t* d_bsr_indptr, int32_t* d_bsr_indices, void* d_bsr_data,
+                         int32_t data_dtype, int64_t nnzb, void* stream);
+
 /* ------------------------------------------------------------------------------ kernels */
 
 /*
@@ -151,7 +187,6 @@ int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float*
  * Y: mb*blk*feat.  dtype: STIR_F16 or STIR_BF16 for A and X; out_dtype: the same 16-bit
  * type or STIR_F32.  blk must be 16 or 32 and feat a multiple of 32.
  */
-enum { STIR_F16 = 0, STIR_BF16 = 1, STIR_F32 = 2 };
 int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk,
                   int32_t feat, int64_t nnzb, const void* d_A, const void* d_X, void* d_Y,
                   const int32_t* d_indptr, const int32_t* d_indices, void* stream);

@@ -1,14 +1,15 @@
 // BSR SpMM on the gfx950 matrix cores: Y[i-th block row] = sum over stored blocks p of
 // A_p (blk x blk) * X[indices[p]-th block of rows], 16-bit inputs, fp32 accumulation.
 //
-// A workgroup of four wavefronts owns one 32-row slice of a block row and a 128-wide slice
-// of the feature axis; wavefront w owns features [32w, 32w+32) and accumulates a 32x32 fp32
-// tile with v_mfma_f32_32x32x16_{f16,bf16}.  The A operand wants 8 consecutive k per lane,
-// which is exactly how a row of a stored block lies in memory, so it is loaded straight from
-// global memory (16 bytes per lane).  The X operand wants 8 consecutive k for one feature
-// column, but X is feature-contiguous, so the 32 x 128 tile of X goes through LDS: every
-// thread loads two adjacent k rows (16 bytes each), interleaves them into (k, k+1) pairs
-// and stores 32 bytes; a lane's MFMA operand is then four 4-byte LDS reads.
+// A workgroup of four wavefronts owns one 32-row slice of a block row and a 128*NT-wide slice
+// of the feature axis; a wavefront owns NT 32-feature tiles, each a 32x32 fp32 accumulator fed
+// by v_mfma_f32_32x32x16_{f16,bf16}.  The A operand wants 8 consecutive k per lane, which is
+// exactly how a row of a stored block lies in memory, so it is loaded straight from global
+// memory (16 bytes per lane).  The X operand wants 8 consecutive k for one feature column, but
+// X is feature-contiguous, so the 32 x TF tile of X goes through LDS: every thread loads two
+// adjacent k rows (16 bytes each), interleaves them into (k, k+1) pairs and stores 32 bytes; a
+// lane's MFMA operand is then four 4-byte LDS reads.  Tiles are double-buffered in LDS and the
+// next step's global loads are in flight while the current one is multiplied.
 #include <hip/hip_fp16.h>
 
 #include "common.h"
@@ -49,77 +50,136 @@ __device__ __forceinline__ uint16_t to16(float v) {
   }
 }
 
-// grid: (mb * (blk/32), ceil(feat/128)); block: 256 threads.
-template <bool BF16, int OUT>  // OUT: 0 = same 16-bit type as the inputs, 1 = fp32
-__global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, const uint16_t* __restrict__ A,
+// Workgroup -> (32-row slice, feature tile).  Workgroups are dispatched round-robin over the 8
+// XCDs, each with its own L2.  All slices of one feature tile read the same columns of X
+// (nb*blk rows x TF features), so when there are at least 8 feature tiles each XCD walks its own
+// feature tiles one after the other and that slice of X stays resident in its L2; with fewer
+// tiles the tile index is the fastest-varying one, which (for 1, 2 or 4 tiles) also pins a tile
+// to an XCD.
+__device__ __forceinline__ bool decode_tile(int64_t L, int64_t slices, int f_tiles, int64_t& slice,
+                                            int& f_tile) {
+  if (f_tiles >= 8) {
+    const int xcd = (int)(L & 7);
+    const int64_t slot = L >> 3;
+    f_tile = xcd + 8 * (int)(slot / slices);
+    slice = slot % slices;
+    return f_tile < f_tiles;
+  }
+  f_tile = (int)(L % f_tiles);
+  slice = L / f_tiles;
+  return slice < slices;
+}
+
+// 1-D grid (see decode_tile); block: 256 threads = 4 wavefronts; wavefront w owns features
+// [32*NT*w, 32*NT*(w+1)) of the TF = 128*NT wide tile and NT 32x32 accumulators.  The X tile of
+// step it+1 is fetched into registers while step it is multiplied out of LDS (two LDS buffers,
+// one barrier per step).
+template <bool BF16, int OUT, int NT, int S>  // OUT: 0 = same 16-bit type as the inputs, 1 = fp32
+__global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles,
+                                                       const uint16_t* __restrict__ A,
                                                        const uint16_t* __restrict__ X, void* __restrict__ Y,
                                                        const int32_t* __restrict__ indptr,
                                                        const int32_t* __restrict__ indices) {
-  __shared__ uint32_t xs[kTileK / 2][kTileF];  // [k pair][feature] -> (X[2kp][f], X[2kp+1][f])
+  constexpr int TF = kTileF * NT;
+  constexpr int FC = TF / 8;      // 8-feature chunks per tile row
+  constexpr int KPT = 256 / FC;   // k pairs covered by one pass of the 256 threads
+  __shared__ uint32_t xs[2][kTileK / 2][TF];  // [buffer][k pair][feature] -> (X[2kp][f], X[2kp+1][f])
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = lane & 31, h = lane >> 5;
+  int64_t slice;
+  int f_tile;
+  if (!decode_tile(blockIdx.x, slices, f_tiles, slice, f_tile)) return;
   const int sub = blk / 32;  // 32-row slices per block row
-  const int i = blockIdx.x / sub, bi0 = (blockIdx.x % sub) * 32;
-  const int f0 = blockIdx.y * kTileF;
-  // staging role: k pair kp, feature chunk fc (8 features)
-  const int kp = tid >> 4, fc = tid & 15;
+  const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * 32;
+  const int f0 = f_tile * TF;
+  const int kp0 = tid / FC, fc = tid % FC;
   const bool stage_live = f0 + fc * 8 < feat;  // feat is a multiple of 32, so chunks are whole
-  const bool wave_live = f0 + wave * 32 < feat;
 
-  f32x16 acc;
+  f32x16 acc[NT];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
-  const int p_begin = indptr[i], p_end = indptr[i + 1];
-  for (int p = p_begin; p < p_end; ++p) {
+  const int p_begin = indptr[i];
+  const int ksteps = blk / kTileK;
+  const int steps = (indptr[i + 1] - p_begin) * ksteps;
+
+  // Register ring of S prefetched steps: loads for step it+S are issued as soon as step it has
+  // been copied to LDS, so S tiles per wavefront are in flight while the matrix cores work.
+  u32x4 r0[S][NT], r1[S][NT], areg[S][2];
+  auto fetch = [&](int it, int s) {
+    const int p = p_begin + it / ksteps, k0 = (it % ksteps) * kTileK;
     const int64_t j = indices[p];
-    const uint16_t* ablk = A + (int64_t)p * blk * blk + (int64_t)(bi0 + n) * blk;
-    for (int k0 = 0; k0 < blk; k0 += kTileK) {
-      // ---- stage X[j*blk + k0 .. +32][f0 .. +128] as k pairs
-      u32x4 r0 = {0, 0, 0, 0}, r1 = {0, 0, 0, 0};
+    const uint16_t* ablk = A + (int64_t)p * blk * blk + (int64_t)(bi0 + n) * blk + k0;
+    areg[s][0] = *reinterpret_cast<const u32x4*>(ablk + 8 * h);       // k = k0 + 8h + (0..7)
+    areg[s][1] = *reinterpret_cast<const u32x4*>(ablk + 16 + 8 * h);  // k = k0 + 16 + 8h + (0..7)
+#pragma unroll
+    for (int q = 0; q < NT; ++q) {
+      r0[s][q] = r1[s][q] = u32x4{0, 0, 0, 0};
       if (stage_live) {
-        const uint16_t* xp = X + ((int64_t)j * blk + k0 + 2 * kp) * feat + f0 + fc * 8;
-        r0 = *reinterpret_cast<const u32x4*>(xp);
-        r1 = *reinterpret_cast<const u32x4*>(xp + feat);
+        const uint16_t* xp = X + ((int64_t)j * blk + k0 + 2 * (kp0 + KPT * q)) * feat + f0 + fc * 8;
+        r0[s][q] = *reinterpret_cast<const u32x4*>(xp);
+        r1[s][q] = *reinterpret_cast<const u32x4*>(xp + feat);
       }
-      // ---- A operand straight from global: rows bi0+n, k = k0 + 16*kk + 8h + (0..7)
-      u32x4 a0 = *reinterpret_cast<const u32x4*>(ablk + k0 + 8 * h);
-      u32x4 a1 = *reinterpret_cast<const u32x4*>(ablk + k0 + 16 + 8 * h);
-      u32x4 lo, hi;  // (k, k+1) pairs for features fc*8 + 0..3 and 4..7
+    }
+  };
+
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        lo[2 * q] = __builtin_amdgcn_perm(r1[q], r0[q], 0x05040100);      // low halves
-        lo[2 * q + 1] = __builtin_amdgcn_perm(r1[q], r0[q], 0x07060302);  // high halves
-        hi[2 * q] = __builtin_amdgcn_perm(r1[q + 2], r0[q + 2], 0x05040100);
-        hi[2 * q + 1] = __builtin_amdgcn_perm(r1[q + 2], r0[q + 2], 0x07060302);
-      }
-      __syncthreads();  // previous step's readers are done
-      *reinterpret_cast<u32x4*>(&xs[kp][fc * 8]) = lo;
-      *reinterpret_cast<u32x4*>(&xs[kp][fc * 8 + 4]) = hi;
-      __syncthreads();
-      if (wave_live) {
-        u32x4 b0, b1;
+  for (int s = 0; s < S; ++s)
+    if (s < steps) fetch(s, s);
+  for (int it0 = 0; it0 < steps; it0 += S) {
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          b0[d] = xs[4 * h + d][wave * 32 + n];
-          b1[d] = xs[8 + 4 * h + d][wave * 32 + n];
+    for (int s = 0; s < S; ++s) {
+      const int it = it0 + s;
+      if (it < steps) {  // uniform over the workgroup
+        const int buf = it & 1;
+        const u32x4 a0 = areg[s][0], a1 = areg[s][1];
+#pragma unroll
+        for (int q = 0; q < NT; ++q) {
+          u32x4 lo, hi;  // (k, k+1) pairs for features fc*8 + 0..3 and 4..7
+#pragma unroll
+          for (int d = 0; d < 2; ++d) {
+            lo[2 * d] = __builtin_amdgcn_perm(r1[s][q][d], r0[s][q][d], 0x05040100);      // low halves
+            lo[2 * d + 1] = __builtin_amdgcn_perm(r1[s][q][d], r0[s][q][d], 0x07060302);  // high halves
+            hi[2 * d] = __builtin_amdgcn_perm(r1[s][q][d + 2], r0[s][q][d + 2], 0x05040100);
+            hi[2 * d + 1] = __builtin_amdgcn_perm(r1[s][q][d + 2], r0[s][q][d + 2], 0x07060302);
+          }
+          *reinterpret_cast<u32x4*>(&xs[buf][kp0 + KPT * q][fc * 8]) = lo;
+          *reinterpret_cast<u32x4*>(&xs[buf][kp0 + KPT * q][fc * 8 + 4]) = hi;
         }
-        acc = mfma32<BF16>(a0, b0, acc);
-        acc = mfma32<BF16>(a1, b1, acc);
+        if (it + S < steps) fetch(it + S, s);
+        __syncthreads();  // tile `it` is complete; the other buffer's readers passed the previous barrier
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const int col = (wave * NT + t) * 32 + n;
+          u32x4 b0, b1;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            b0[d] = xs[buf][4 * h + d][col];
+            b1[d] = xs[buf][8 + 4 * h + d][col];
+          }
+          acc[t] = mfma32<BF16>(a0, b0, acc[t]);
+          acc[t] = mfma32<BF16>(a1, b1, acc[t]);
+        }
       }
     }
   }
-  if (!wave_live) return;
-  // acc[v] is row (v%4) + 4h + 8(v/4), column n of the 32x32 tile
+  // acc[t][v] is row (v%4) + 4h + 8(v/4), column n of the t-th 32x32 tile
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int row = (v & 3) + 4 * h + 8 * (v >> 2);
-    const int64_t off = ((int64_t)i * blk + bi0 + row) * feat + f0 + wave * 32 + n;
-    if constexpr (OUT == 1)
-      static_cast<float*>(Y)[off] = acc[v];
-    else
-      static_cast<uint16_t*>(Y)[off] = to16<BF16>(acc[v]);
+  for (int t = 0; t < NT; ++t) {
+    const int fcol = f0 + (wave * NT + t) * 32;
+    if (fcol >= feat) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = (v & 3) + 4 * h + 8 * (v >> 2);
+      const int64_t off = ((int64_t)i * blk + bi0 + row) * feat + fcol + n;
+      if constexpr (OUT == 1)
+        static_cast<float*>(Y)[off] = acc[t][v];
+      else
+        static_cast<uint16_t*>(Y)[off] = to16<BF16>(acc[t][v]);
+    }
   }
 }
 
@@ -135,20 +195,36 @@ extern "C" int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32
   STIR_REQUIRE(feat > 0 && feat % 32 == 0, "bsr_spmm: feat=%d must be a multiple of 32", feat);
   if (mb == 0) return 0;
   STIR_REQUIRE(d_X && d_Y && d_indptr && (nnzb == 0 || (d_A && d_indices)), "bsr_spmm: null pointer argument");
-  const int64_t gx = (int64_t)mb * (blk / 32);
-  STIR_REQUIRE(gx < (int64_t(1) << 31), "bsr_spmm: too many block rows for one launch");
-  dim3 grid((unsigned)gx, (unsigned)stir::ceil_div(feat, kTileF)), block(256);
+  const int64_t slices = (int64_t)mb * (blk / 32);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
-#define STIR_BSR(BF, OUT) \
-  hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT>), grid, block, 0, st, blk, feat, A, X, d_Y, d_indptr, d_indices)
+  // Two 32-wide accumulators per wavefront once the feature axis is wide enough to still yield
+  // several workgroups per CU.  One prefetched step is enough: measured on MI355X, deeper
+  // register rings (2-6 steps) change nothing, the kernel is bound by the traffic that misses
+  // the per-XCD L2, not by latency.
+  const int nt = (feat >= 1024) ? 2 : 1;
+  const int f_tiles = (int)stir::ceil_div(feat, kTileF * nt);
+  const int64_t blocks = f_tiles >= 8 ? 8 * stir::ceil_div(f_tiles, 8) * slices : (int64_t)f_tiles * slices;
+  STIR_REQUIRE(blocks < (int64_t(1) << 31), "bsr_spmm: too many tiles for one launch");
+  dim3 grid((unsigned)blocks), block(256);
+#define STIR_BSR_L(BF, OUT, NTV, SV)                                                                     \
+  hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, SV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
+                     A, X, d_Y, d_indptr, d_indices)
+#define STIR_BSR(BF, OUT)                  \
+  do {                                     \
+    if (nt == 2)                           \
+      STIR_BSR_L(BF, OUT, 2, 1);           \
+    else                                   \
+      STIR_BSR_L(BF, OUT, 1, 1);           \
+  } while (0)
   if (dtype == STIR_BF16) {
     if (out_dtype == STIR_F32) STIR_BSR(true, 1); else STIR_BSR(true, 0);
   } else {
     if (out_dtype == STIR_F32) STIR_BSR(false, 1); else STIR_BSR(false, 0);
   }
 #undef STIR_BSR
+#undef STIR_BSR_L
   STIR_LAUNCH_CHECK();
   return 0;
 }

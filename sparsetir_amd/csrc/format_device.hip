@@ -245,6 +245,34 @@ __global__ __launch_bounds__(256) void place_entries_kernel(int m, int P, int ps
   mask_tab[k][pos] = 1;
 }
 
+// Value rewrite: A_k[slot] = values[e] for every nonzero (padding slots stay zero), the
+// placement computed exactly as in place_entries_kernel.
+__global__ __launch_bounds__(256) void place_values_kernel(int m, int P, int psize, int NB, int64_t nnz,
+                                                           int32_t first,
+                                                           const int32_t* __restrict__ indptr,
+                                                           const int32_t* __restrict__ indices,
+                                                           const float* __restrict__ values,
+                                                           const int32_t* __restrict__ widths,
+                                                           const int32_t* __restrict__ lo_in,
+                                                           const int32_t* __restrict__ base_in,
+                                                           float* const* __restrict__ a_tab) {
+  const int64_t e = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= first + nnz) return;
+  const int col = indices[e];
+  const int p = col / psize;
+  int a = 0, b = m;
+  while (a < b) {
+    const int mid = a + ((b - a + 1) >> 1);
+    if ((int64_t)indptr[mid] <= e) a = mid; else b = mid - 1;
+  }
+  const int i = a;
+  const int lo = lo_in[(int64_t)p * m + i];
+  const int hi = p == P - 1 ? indptr[i + 1] : lo_in[(int64_t)(p + 1) * m + i];
+  const int beta = bucket_of_dev(widths, NB, hi - lo);
+  const int64_t pos = (int64_t)base_in[(int64_t)p * m + i] * widths[beta] + (e - lo);
+  a_tab[p * NB + beta][pos] = values[e];
+}
+
 int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t parts, const int32_t* buckets,
                int32_t nb) {
   STIR_REQUIRE(num_rows >= 0 && num_cols >= 0, "%s: bad matrix shape %d x %d", who, num_rows, num_cols);
@@ -342,6 +370,40 @@ int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols, const i
   hipLaunchKernelGGL(place_entries_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, m, P,
                      psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.lo, ws.base, ws.cols_tab,
                      ws.mask_tab);
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const int32_t* d_indptr,
+                                       const int32_t* d_indices, const float* d_values,
+                                       int32_t num_col_parts, const int32_t* buckets, int32_t num_buckets,
+                                       void* d_workspace, const int64_t* nrows, float* const* d_A,
+                                       void* stream) {
+  const char* who = "ColumnPartHyb(device values)";
+  if (check_args(who, num_rows, num_cols, num_col_parts, buckets, num_buckets)) return -1;
+  const int P = num_col_parts, NB = num_buckets, m = num_rows;
+  if (m == 0) return 0;
+  STIR_REQUIRE(d_indptr && d_workspace && nrows && d_A, "%s: null pointer argument", who);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Workspace ws = carve(d_workspace, m, P, NB);
+  int32_t ends[2];
+  STIR_HIP(hipMemcpyAsync(&ends[0], d_indptr, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  STIR_HIP(hipMemcpyAsync(&ends[1], d_indptr + m, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  // the A_k pointer table reuses the slot of the mask table (same size, no longer needed)
+  STIR_HIP(hipMemcpyAsync(ws.mask_tab, d_A, sizeof(void*) * size_t(P) * NB, hipMemcpyHostToDevice, st));
+  STIR_HIP(hipStreamSynchronize(st));
+  for (int k = 0; k < P * NB; ++k) {
+    STIR_REQUIRE(nrows[k] >= 0 && (nrows[k] == 0 || d_A[k]), "%s: bucket %d has rows but no array", who, k);
+    if (nrows[k] > 0)
+      STIR_HIP(hipMemsetAsync(d_A[k], 0, sizeof(float) * size_t(nrows[k]) * buckets[k % NB], st));
+  }
+  const int64_t nnz = (int64_t)ends[1] - ends[0];
+  if (nnz <= 0) return 0;
+  STIR_REQUIRE(d_indices && d_values, "%s: null pointer argument", who);
+  const int psize = (num_cols + P - 1) / P;
+  hipLaunchKernelGGL(place_values_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, m, P, psize,
+                     NB, nnz, ends[0], d_indptr, d_indices, d_values, ws.widths, ws.lo, ws.base,
+                     reinterpret_cast<float* const*>(ws.mask_tab));
   STIR_LAUNCH_CHECK();
   return 0;
 }

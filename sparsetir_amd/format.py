@@ -36,16 +36,22 @@ def _is_cuda_tensor(a):
     return hasattr(a, "is_cuda") and a.is_cuda
 
 
-def column_part_hyb(num_rows, num_cols, indptr_nd, indices_nd, num_col_parts, buckets):
+def column_part_hyb(num_rows, num_cols, indptr_nd, indices_nd, num_col_parts, buckets, values=None):
     """Partition a CSR matrix by columns and collect rows into ELL buckets by their number of
     nonzeros per partition.
 
     Returns ``(row_indices, col_indices, mask)``; each is a list over column partitions of
     lists over buckets of int32 arrays shaped ``(nrows,)``, ``(nrows, b)``, ``(nrows, b)``.
+
+    Extension (GPU path only): with ``values`` (float32 CUDA tensor aligned with ``indices``) a
+    fourth nested list is returned holding the per-bucket value arrays ``A_k`` of shape
+    ``(nrows, b)``, i.e. the result of the reference's "rewrite_A_k" preprocess blocks.
     """
     if _is_cuda_tensor(indptr_nd) or _is_cuda_tensor(indices_nd):
         return _column_part_hyb_device(num_rows, num_cols, indptr_nd, indices_nd,
-                                       num_col_parts, buckets)
+                                       num_col_parts, buckets, values)
+    if values is not None:
+        raise _lib.SparseTIRError("ColumnPartHyb: the value rewrite needs CUDA tensors")
     L = _lib.lib()
     indptr = _host_i32(indptr_nd, "indptr")
     indices = _host_i32(indices_nd, "indices")
@@ -69,7 +75,7 @@ def column_part_hyb(num_rows, num_cols, indptr_nd, indices_nd, num_col_parts, bu
     return nest(rows), nest(cols), nest(mask)
 
 
-def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, buckets):
+def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, buckets, values=None):
     import torch
 
     L = _lib.lib()
@@ -107,10 +113,73 @@ def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, 
             _lib.ptr_table([a.data_ptr() for a in rows]),
             _lib.ptr_table([a.data_ptr() for a in cols]),
             _lib.ptr_table([a.data_ptr() for a in mask]), stream))
+        avals = None
+        if values is not None:
+            if not _is_cuda_tensor(values) or values.dtype != torch.float32 or values.numel() != indices.numel():
+                raise _lib.SparseTIRError("ColumnPartHyb: values must be a float32 CUDA tensor aligned with indices")
+            values = values.contiguous()
+            avals = [torch.empty((int(nrows[k]), int(widths[k % nb])), dtype=torch.float32, device=dev)
+                     for k in range(nk)]
+            _lib.check(L.stir_column_part_hyb_device_values(
+                num_rows, num_cols, ctypes.c_void_p(indptr.data_ptr()),
+                ctypes.c_void_p(indices.data_ptr()), ctypes.c_void_p(values.data_ptr()),
+                num_col_parts, _vp(widths), nb, ctypes.c_void_p(ws.data_ptr()), _vp(nrows),
+                _lib.ptr_table([a.data_ptr() for a in avals]), stream))
         # the workspace is read by the fill kernels: keep it alive until they are done
         torch.cuda.current_stream().synchronize()
     nest = lambda xs: [[xs[p * nb + b] for b in range(nb)] for p in range(num_col_parts)]
+    if avals is not None:
+        return nest(rows), nest(cols), nest(mask), nest(avals)
     return nest(rows), nest(cols), nest(mask)
+
+
+def csr_to_bsr(indptr, indices, values, shape, blocksize, dtype=None):
+    """Pack a CSR matrix (CUDA tensors: int32 indptr/indices, float32 values, no duplicate
+    entries) into BSR with ``blocksize x blocksize`` blocks on the GPU.
+
+    Returns ``(bsr_indptr, bsr_indices, bsr_data)`` as CUDA tensors; block columns ascend in
+    each block row and ``bsr_data`` is ``(nnzb, blocksize, blocksize)`` of ``dtype``
+    (float32 by default, float16 / bfloat16 for direct use by the BSR SpMM operator) -- the
+    arrays ``scipy.sparse.csr_matrix.tobsr`` returns, which is how the reference's BSR example
+    builds its input (examples/blocksparse/bsr_spmm.py:441-445).
+    """
+    import torch
+
+    L = _lib.lib()
+    m, n = int(shape[0]), int(shape[1])
+    blk = int(blocksize)
+    dtype = torch.float32 if dtype is None else dtype
+    codes = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+    if dtype not in codes:
+        raise _lib.SparseTIRError("csr_to_bsr: dtype must be float32, float16 or bfloat16")
+    for t, name, dt in ((indptr, "indptr", torch.int32), (indices, "indices", torch.int32),
+                        (values, "values", torch.float32)):
+        if not _is_cuda_tensor(t):
+            raise _lib.SparseTIRError(f"csr_to_bsr: {name} must be a CUDA tensor")
+        if t.dtype != dt:
+            raise _lib.SparseTIRError(f"csr_to_bsr: {name} must be {dt}")
+    if indptr.numel() != m + 1 or values.numel() != indices.numel():
+        raise _lib.SparseTIRError("csr_to_bsr: array lengths do not fit the shape")
+    indptr, indices, values = indptr.contiguous(), indices.contiguous(), values.contiguous()
+    dev = indptr.device
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        ws = torch.empty(max(256, L.stir_csr_to_bsr_workspace_bytes(m, n, blk)), dtype=torch.uint8, device=dev)
+        if blk <= 0 or m % blk or n % blk:
+            raise _lib.SparseTIRError(f"csr_to_bsr: shape {m} x {n} is not a multiple of the block size {blk}")
+        bptr = torch.empty(m // blk + 1, dtype=torch.int32, device=dev)
+        nnzb = ctypes.c_int64(0)
+        p = lambda t: ctypes.c_void_p(t.data_ptr())
+        _lib.check(L.stir_csr_to_bsr_sizes(m, n, blk, p(indptr), p(indices), p(ws), p(bptr),
+                                           ctypes.byref(nnzb), stream))
+        bidx = torch.empty(nnzb.value, dtype=torch.int32, device=dev)
+        bdata = torch.empty((nnzb.value, blk, blk), dtype=dtype, device=dev)
+        _lib.check(L.stir_csr_to_bsr_fill(m, n, blk, p(indptr), p(indices), p(values), p(ws), p(bptr),
+                                          ctypes.c_void_p(bidx.data_ptr() if nnzb.value else 0),
+                                          ctypes.c_void_p(bdata.data_ptr() if nnzb.value else 0),
+                                          codes[dtype], nnzb.value, stream))
+        torch.cuda.current_stream().synchronize()
+    return bptr, bidx, bdata
 
 
 def condense(indptr_nd, indices_nd, t, g):

@@ -59,3 +59,73 @@ def test_device_column_part_hyb_rejects_unsorted_and_out_of_range(dev):
     bad = np.asarray([0, 50], np.int32)
     with pytest.raises(SparseTIRError, match="outside"):
         _device_hyb(dev, 2, 40, np.asarray([0, 1, 2], np.int32), bad, 2, [1, 2])
+
+
+def test_device_hyb_value_rewrite(dev):
+    """A_k gathered on the device equals the values placed by the decomposition's own index
+    arrays: A_k[r, s] = value of nonzero (rows_k[r], cols_k[r, s]) where mask is 1, else 0."""
+    import scipy.sparse as sp
+
+    m = n = 700
+    parts, buckets = 3, [1, 2, 4, 8]
+    indptr, indices = random_csr(m, n, 12000, 4, skew=1.1)
+    vals = np.random.default_rng(4).random(len(indices), dtype=np.float32) + 0.5
+    t = lambda a: torch.from_numpy(a).to(dev)
+    rows, cols, mask, avals = st.column_part_hyb(m, n, t(indptr), t(indices), parts, buckets, values=t(vals))
+    dense = sp.csr_matrix((vals, indices, indptr), shape=(m, n)).toarray()
+    for p in range(parts):
+        for b in range(len(buckets)):
+            r, c = rows[p][b].cpu().numpy(), cols[p][b].cpu().numpy()
+            k, a = mask[p][b].cpu().numpy(), avals[p][b].cpu().numpy()
+            if len(r) == 0:
+                continue
+            want = dense[np.repeat(r[:, None], c.shape[1], 1), c] * k
+            assert np.array_equal(a, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("m,n,blk,nnz,seed", [(256, 256, 32, 3000, 0), (4096, 4096, 32, 200000, 1),
+                                             (128, 512, 16, 900, 2), (64, 64, 64, 50, 3), (96, 160, 32, 0, 4),
+                                             (2048, 8192, 64, 100000, 5)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_device_csr_to_bsr_matches_scipy(dev, m, n, blk, nnz, seed, dtype):
+    import scipy.sparse as sp
+
+    indptr, indices = random_csr(m, n, nnz, seed, sort=(seed % 2 == 0), skew=0.5)
+    vals = np.random.default_rng(seed).standard_normal(len(indices)).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    bptr, bidx, bdata = st.csr_to_bsr(t(indptr), t(indices), t(vals), (m, n), blk, dtype)
+    ref = sp.csr_matrix((vals, indices, indptr), shape=(m, n)).tobsr((blk, blk))
+    ref.sort_indices()
+    assert np.array_equal(bptr.cpu().numpy(), ref.indptr.astype(np.int32))
+    assert np.array_equal(bidx.cpu().numpy(), ref.indices.astype(np.int32))
+    want = torch.from_numpy(ref.data.astype(np.float32)).to(dtype)
+    assert torch.equal(bdata.cpu(), want.reshape(bdata.shape))
+
+
+def test_device_csr_to_bsr_feeds_the_bsr_operator(dev):
+    from sparsetir_amd import ops
+    import scipy.sparse as sp
+
+    m = n = 1024
+    blk, feat = 32, 64
+    indptr, indices = random_csr(m, n, 30000, 9)
+    vals = (np.random.default_rng(9).standard_normal(len(indices)) * 0.1).astype(np.float32)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    bptr, bidx, bdata = st.csr_to_bsr(t(indptr), t(indices), t(vals), (m, n), blk, torch.float16)
+    x = torch.randn(n * feat, device=dev).half()
+    y = torch.zeros(m * feat, device=dev, dtype=torch.float32)
+    ops.build_bsrmm(m // blk, n // blk, bidx.numel(), blk, feat, torch.float16, torch.float32)(
+        bdata.reshape(-1), x, y, bptr, bidx)
+    torch.cuda.synchronize()
+    a16 = sp.csr_matrix((vals.astype(np.float16).astype(np.float64), indices, indptr), shape=(m, n))
+    want = a16 @ x.float().cpu().numpy().astype(np.float64).reshape(n, feat)
+    assert np.allclose(y.cpu().numpy().reshape(m, feat), want, rtol=2e-2, atol=1e-3)
+
+
+def test_device_csr_to_bsr_errors(dev):
+    z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
+    with pytest.raises(SparseTIRError, match="multiple"):
+        st.csr_to_bsr(z(101, torch.int32), z(0, torch.int32), z(0, torch.float32), (100, 64), 32)
+    with pytest.raises(SparseTIRError, match="outside"):
+        st.csr_to_bsr(torch.tensor([0, 1] + [1] * 31, dtype=torch.int32, device=dev),
+                      torch.tensor([99], dtype=torch.int32, device=dev), z(1, torch.float32), (32, 64), 32)
