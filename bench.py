@@ -75,6 +75,59 @@ def time_steps(fn, steps, warmup, torch):
     return wall, float(np.mean(dev_ms)) / 1e3, float(np.min(dev_ms)) / 1e3
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def side_kernels(torch, dev, ops, st, datasets, time_steps):
+    """BSR SpMM (config 4 and a scaled-up shape) and RGMS (config 5): time, flop rate against the
+    dense fp16 MFMA peak, algorithmic bytes against the HBM peak."""
+    out = {}
+
+    def bsr(tag, mb, nb, blk, density, feat, dtype):
+        cfg = datasets.config4(seed=3, mb=mb, nb=nb, blk=blk, density=density, feat=32)
+        nnzb = len(cfg["indices"])
+        a = torch.from_numpy(cfg["data"]).to(dev).to(dtype).reshape(-1)
+        x = torch.randn(nb * blk * feat, device=dev).to(dtype)
+        y = torch.zeros(mb * blk * feat, device=dev, dtype=dtype)
+        ip, ix = torch.from_numpy(cfg["indptr"]).to(dev), torch.from_numpy(cfg["indices"]).to(dev)
+        f = ops.build_bsrmm(mb, nb, nnzb, blk, feat, dtype)
+        _, d, _ = time_steps(lambda: f(a, x, y, ip, ix), 100, 5, torch)
+        flops = 2.0 * nnzb * blk * blk * feat
+        byts = 2.0 * nnzb * blk * blk + 4 * nnzb + 4 * (mb + 1) + 2.0 * nb * blk * feat + 2.0 * mb * blk * feat
+        out[tag] = {"us": d * 1e6, "tflops": flops / d / 1e12, "frac_of_mfma_peak": flops / d / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                    "alg_GBps": byts / d / 1e9, "frac_of_hbm_peak": byts / d / 1e9 / HBM_PEAK_GBS,
+                    "nnzb": nnzb, "shape": [mb * blk, nb * blk, feat], "blk": blk, "dtype": str(dtype).split(".")[-1]}
+
+    bsr("bsr_config4_f16", 128, 128, 32, 0.10, 512, torch.float16)
+    bsr("bsr_config4_bf16", 128, 128, 32, 0.10, 512, torch.bfloat16)
+    bsr("bsr_16384x16384_f4096_f16", 512, 512, 32, 0.10, 4096, torch.float16)
+
+    cfg = datasets.config5()
+    R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
+    buckets, group = cfg["buckets"], 256
+    rb = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"],
+                                            rb, buckets)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float16).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
+    f = ops.build_rgms(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols])
+    w = t(cfg["w"].astype(np.float16).ravel())
+    x = t(cfg["x"].astype(np.float16).ravel())
+    y = torch.zeros(n * fout, device=dev)
+    _, d, _ = time_steps(lambda: f(w, x, y, *triples, *mids), 10, 1, torch)
+    E = len(cfg["indices1"])
+    flops = 2.0 * E * fin * fout + 2.0 * E * fout
+    byts = 8.0 * E + 2.0 * n * fin + 2.0 * R * fin * fout + 4.0 * n * fout
+    out["rgms_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts / d / 1e9,
+                           "frac_of_hbm_peak": byts / d / 1e9 / HBM_PEAK_GBS, "edges": E,
+                           "ell_rows": int(sum(r.size for r in rows)),
+                           "atomic_GBps": sum(r.size for r in rows) * fout * 4.0 / d / 1e9}
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -236,6 +289,8 @@ def main():
         sd_bytes = nnz * 8.0 + 4.0 * (m + 1) + 4.0 * (m + n) * f2
         extra["sddmm_f64"] = {"gflops": 2.0 * nnz * f2 / w4 / 1e9, "ms": d4 * 1e3,
                               "alg_GBps": sd_bytes / d4 / 1e9, "preproc_ms": d3 * 1e3}
+        del a2, b2, out, mid
+        extra.update(side_kernels(torch, dev, ops, st, datasets, time_steps))
         result["extra"] = extra
 
     print(json.dumps(result), flush=True)

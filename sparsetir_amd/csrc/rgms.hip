@@ -25,11 +25,14 @@ struct alignas(16) RgmsBucket {
   const int32_t* cols;  // groups*rb*cb
   const int32_t* mids;  // groups
   int64_t groups;
-  int64_t group_begin;  // first group of this bucket in the fused launch
+  int64_t unit_begin;  // first work unit (one wavefront each) of this bucket in the fused launch
   int32_t rb, cb;
   int32_t log2cb;  // log2(cb) when cb is a power of two <= 32, else -1
-  int32_t pad;
+  int32_t chunks;  // work units per group: ceil(rb*cb / kChunkSlots)
 };
+
+// A wavefront processes this many consecutive slots of one group.
+constexpr int kChunkSlots = 128;
 
 constexpr int kMaxKK = 8;  // feat_in <= 128 keeps the X operand in registers
 
@@ -41,25 +44,19 @@ __device__ __forceinline__ void atomic_addf(float* p, float v) {
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// KK = feat_in / 16.  grid: one wavefront per group (4 per workgroup); feat_out tiles of 32
-// are walked inside.
-template <int KK>
-__global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict__ table, int nb,
-                                                   int64_t total_groups, int feat_out,
-                                                   const uint16_t* __restrict__ W,
-                                                   const uint16_t* __restrict__ X, float* __restrict__ Y) {
+// One group (one relation), one wavefront.  KK = feat_in / 16; LCB = log2(cb) for power-of-two
+// cb <= 32, else -1.  The group is processed in chunks of TI tiles (32 slots each): the chunk's
+// column ids, slot weights and row ids are fetched with a few coalesced loads (lane l holds slots
+// l, l+64, ...), then the X rows of all TI tiles are requested at once, so a chunk costs two
+// memory latencies instead of several per tile.
+template <int KK, int LCB>
+__device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int chunk, int feat_out,
+                                           const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
+                                           float* __restrict__ Y, int lane) {
   constexpr int FIN = KK * 16;
-  const int lane = threadIdx.x & 63;
+  constexpr int TI = KK <= 2 ? 4 : 2;  // tiles in flight
+  constexpr int MJ = TI / 2;           // 64-slot metadata registers per lane
   const int n = lane & 31, h = lane >> 5;
-  const int64_t gid = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if (gid >= total_groups) return;
-  int lo = 0, hi = nb - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (table[mid].group_begin <= gid) lo = mid; else hi = mid - 1;
-  }
-  const RgmsBucket bk = table[lo];
-  const int64_t g = gid - bk.group_begin;
   const int rel = bk.mids[g];
   const int gsize = bk.rb * bk.cb;
   const uint16_t* Ag = bk.A + g * gsize;
@@ -78,77 +75,149 @@ __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict_
         wf[kk][d] = (uint32_t)wp[0] | ((uint32_t)wp[feat_out] << 16);
       }
     }
-    for (int s0 = 0; s0 < gsize; s0 += 32) {
-      const int slot = s0 + n;  // this lane's slot as the A-operand row
-      const bool live = slot < gsize;
-      const int col = live ? colg[slot] : 0;
-      f32x16 acc;
+    float* yb = Y + nt + n;
+    const int s_end = min(gsize, (chunk + 1) * kChunkSlots);
+#pragma unroll 1
+    for (int s_base = chunk * kChunkSlots; s_base < s_end; s_base += 32 * TI) {
+      // ---- chunk metadata: slot s_base + 64j + lane lives in register j of this lane
+      int mcol[MJ], mrow[MJ];
+      float mw[MJ];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-      const uint16_t* xp = X + (int64_t)col * FIN + 8 * h;
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        const u32x4 xa = *reinterpret_cast<const u32x4*>(xp + 16 * kk);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, xa),
-                                                    __builtin_bit_cast(f16x8, wf[kk]), acc, 0, 0, 0);
+      for (int j = 0; j < MJ; ++j) {
+        const int sl = s_base + 64 * j + lane;
+        const bool live = sl < gsize;
+        mcol[j] = live ? colg[sl] : 0;
+        mw[j] = live ? half_bits_to_float(Ag[sl]) : 0.f;
+        // ELL rows of the chunk (power-of-two cb): row (s_base >> LCB) + 64j + lane
+        mrow[j] = 0;
+        if constexpr (LCB >= 0) {
+          const int r = (s_base >> LCB) + 64 * j + lane;
+          if (r < bk.rb) mrow[j] = rowg[r];
+        }
       }
-      // acc[v]: slot s0 + (v%4) + 4h + 8(v/4), output feature nt + n.  Scale by slot weight.
-      float wgt[16];
+      // ---- request the X rows of every tile of the chunk (tiles past the group read row 0)
+      u32x4 xa[TI][KK];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int sl = s0 + (v & 3) + 4 * h + 8 * (v >> 2);
-        wgt[v] = sl < gsize ? half_bits_to_float(Ag[sl]) : 0.f;
-        acc[v] *= wgt[v];
+      for (int t = 0; t < TI; ++t) {
+        const int col = __shfl(mcol[t >> 1], 32 * (t & 1) + n, kWave);
+        const uint16_t* xp = X + (int64_t)col * FIN + 8 * h;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) xa[t][kk] = *reinterpret_cast<const u32x4*>(xp + 16 * kk);
       }
-      float* yb = Y + nt + n;
-      if (bk.log2cb < 0 || bk.log2cb == 0) {
-        // one atomic per slot (zero-weight slots contribute nothing and are skipped)
+#pragma unroll
+      for (int t = 0; t < TI; ++t) {
+        const bool tile_live = s_base + 32 * t < gsize;  // uniform
+        // keep the tiles' instruction streams apart: interleaving them would hold every tile's
+        // accumulators, weights and row ids live at once
+        __builtin_amdgcn_sched_barrier(0);
+        f32x16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, xa[t][kk]),
+                                                      __builtin_bit_cast(f16x8, wf[kk]), acc, 0, 0, 0);
+        // acc[v]: slot 32t + (v%4) + 4h + 8(v/4) of the chunk, output feature nt + n.
+        // Scale by the slot weight (zero beyond the group).
+        float wgt[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int sl = s0 + (v & 3) + 4 * h + 8 * (v >> 2);
-          if (wgt[v] != 0.f) atomic_addf(yb + (int64_t)rowg[sl / bk.cb] * feat_out, acc[v]);
+          wgt[v] = __shfl(mw[t >> 1], 32 * (t & 1) + (v & 3) + 4 * h + 8 * (v >> 2), kWave);
+          acc[v] *= wgt[v];
         }
-      } else if (bk.log2cb == 1) {
+        // row id of ELL row q of the chunk; its register index j is a compile-time constant
+        auto row_of = [&](int q, int j) { return __shfl(mrow[j < MJ ? j : 0], q & 63, kWave); };
+        if constexpr (LCB < 0) {
+          // cb is not a power of two: one atomic per slot, row ids read directly
 #pragma unroll
-        for (int v = 0; v < 16; v += 2) {
-          const int sl = s0 + (v & 3) + 4 * h + 8 * (v >> 2);
-          if (sl < gsize) atomic_addf(yb + (int64_t)rowg[sl >> 1] * feat_out, acc[v] + acc[v + 1]);
-        }
-      } else {
-        // cb >= 4: the four registers of a quad belong to one ELL row
-        float q[4];
+          for (int v = 0; v < 16; ++v) {
+            const int sl = s_base + 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
+            if (wgt[v] != 0.f) atomic_addf(yb + (int64_t)rowg[sl / bk.cb] * feat_out, acc[v]);
+          }
+        } else if constexpr (LCB == 0) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) q[t] = (acc[4 * t] + acc[4 * t + 1]) + (acc[4 * t + 2] + acc[4 * t + 3]);
-        if (bk.log2cb == 2) {
+          for (int v = 0; v < 16; ++v) {
+            const int row = row_of(32 * t + (v & 3) + 4 * h + 8 * (v >> 2), t >> 1);
+            if (wgt[v] != 0.f) atomic_addf(yb + (int64_t)row * feat_out, acc[v]);
+          }
+        } else if constexpr (LCB == 1) {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int sl = s0 + 4 * h + 8 * t;
-            if (sl < gsize) atomic_addf(yb + (int64_t)rowg[sl >> 2] * feat_out, q[t]);
+          for (int v = 0; v < 16; v += 2) {
+            const int sl = 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
+            const int row = row_of(sl >> 1, t >> 2);
+            if (s_base + sl < gsize) atomic_addf(yb + (int64_t)row * feat_out, acc[v] + acc[v + 1]);
           }
         } else {
-          // cb >= 8: add the other half-wave's quad (slots 8t+4..8t+7 vs 8t..8t+3)
+          // cb >= 4: the four registers of a quad belong to one ELL row
+          float q4[4];
 #pragma unroll
-          for (int t = 0; t < 4; ++t) q[t] += __shfl_xor(q[t], 32, kWave);
-          if (bk.log2cb == 3) {
-            // four ELL rows per tile; half h writes rows 2h, 2h+1
+          for (int u = 0; u < 4; ++u) q4[u] = (acc[4 * u] + acc[4 * u + 1]) + (acc[4 * u + 2] + acc[4 * u + 3]);
+          if constexpr (LCB == 2) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-              const int tt = 2 * h + t;
-              const int sl = s0 + 8 * tt;
-              const float val = tt == 0 ? q[0] : tt == 1 ? q[1] : tt == 2 ? q[2] : q[3];
-              if (sl < gsize) atomic_addf(yb + (int64_t)rowg[sl >> 3] * feat_out, val);
+            for (int u = 0; u < 4; ++u) {
+              const int sl = 32 * t + 4 * h + 8 * u;
+              const int row = row_of(sl >> 2, 0);
+              if (s_base + sl < gsize) atomic_addf(yb + (int64_t)row * feat_out, q4[u]);
             }
-          } else if (bk.log2cb == 4) {
-            const float val = h == 0 ? q[0] + q[1] : q[2] + q[3];
-            const int sl = s0 + 16 * h;
-            if (sl < gsize) atomic_addf(yb + (int64_t)rowg[sl >> 4] * feat_out, val);
-          } else {  // cb == 32: the whole tile is one ELL row
-            const float val = (q[0] + q[1]) + (q[2] + q[3]);
-            if (h == 0) atomic_addf(yb + (int64_t)rowg[s0 >> 5] * feat_out, val);
+          } else {
+            // cb >= 8: add the other half-wave's quad (slots 8u+4..8u+7 vs 8u..8u+3)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) q4[u] += __shfl_xor(q4[u], 32, kWave);
+            if constexpr (LCB == 3) {
+              // four ELL rows per tile; half h writes rows 2h, 2h+1
+#pragma unroll
+              for (int u = 0; u < 2; ++u) {
+                const int tt = 2 * h + u;
+                const int sl = 32 * t + 8 * tt;
+                const float val = tt == 0 ? q4[0] : tt == 1 ? q4[1] : tt == 2 ? q4[2] : q4[3];
+                const int row = row_of(sl >> 3, 0);
+                if (s_base + sl < gsize) atomic_addf(yb + (int64_t)row * feat_out, val);
+              }
+            } else if constexpr (LCB == 4) {
+              const float val = h == 0 ? q4[0] + q4[1] : q4[2] + q4[3];
+              const int sl = 32 * t + 16 * h;
+              const int row = row_of(sl >> 4, 0);
+              if (s_base + sl < gsize) atomic_addf(yb + (int64_t)row * feat_out, val);
+            } else {  // cb == 32: the whole tile is one ELL row
+              const float val = (q4[0] + q4[1]) + (q4[2] + q4[3]);
+              const int row = row_of(t, 0);
+              if (h == 0 && tile_live) atomic_addf(yb + (int64_t)row * feat_out, val);
+            }
           }
         }
+        (void)tile_live;
       }
     }
+  }
+}
+
+// grid: one wavefront per work unit (kChunkSlots slots of one group), 4 per workgroup; feat_out
+// tiles of 32 are walked inside.
+template <int KK>
+__global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict__ table, int nb,
+                                                   int64_t total_units, int feat_out,
+                                                   const uint16_t* __restrict__ W,
+                                                   const uint16_t* __restrict__ X, float* __restrict__ Y) {
+  const int lane = threadIdx.x & 63;
+  const int64_t gid = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (gid >= total_units) return;
+  int lo = 0, hi = nb - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (table[mid].unit_begin <= gid) lo = mid; else hi = mid - 1;
+  }
+  const RgmsBucket bk = table[lo];
+  const int64_t unit = gid - bk.unit_begin;
+  const int64_t g = unit / bk.chunks;
+  const int chunk = (int)(unit % bk.chunks);
+  switch (bk.log2cb) {
+    case 0: rgms_group<KK, 0>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 1: rgms_group<KK, 1>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 2: rgms_group<KK, 2>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 3: rgms_group<KK, 3>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 4: rgms_group<KK, 4>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 5: rgms_group<KK, 5>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    default: rgms_group<KK, -1>(bk, g, chunk, feat_out, W, X, Y, lane); break;
   }
 }
 
@@ -157,7 +226,7 @@ __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict_
 struct stir_rgms_plan {
   int nk;
   RgmsBucket* d_table;
-  int64_t total_groups;
+  int64_t total_units;
 };
 
 extern "C" {
@@ -186,7 +255,7 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
     e.cols = d_cols[b];
     e.mids = d_mids[b];
     e.groups = groups[b];
-    e.group_begin = total;
+    e.unit_begin = total;
     e.rb = rows_bkt[b];
     e.cb = cols_bkt[b];
     e.log2cb = -1;
@@ -196,13 +265,13 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
       while ((1 << l) < cols_bkt[b]) ++l;
       e.log2cb = l;
     }
-    e.pad = 0;
+    e.chunks = (int32_t)stir::ceil_div((int64_t)rows_bkt[b] * cols_bkt[b], kChunkSlots);
     host[nk++] = e;
-    total += groups[b];
+    total += groups[b] * e.chunks;
   }
   stir_rgms_plan* p = new stir_rgms_plan();
   p->nk = nk;
-  p->total_groups = total;
+  p->total_units = total;
   p->d_table = nullptr;
   hipError_t err = hipSuccess;
   if (nk > 0) {
@@ -229,7 +298,7 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
   STIR_REQUIRE(feat_out > 0 && feat_out % 32 == 0, "rgms: feat_out=%d must be a multiple of 32", feat_out);
   if (plan->nk == 0) return 0;
   STIR_REQUIRE(d_W && d_X && d_Y, "rgms: null pointer argument");
-  const int64_t blocks = stir::ceil_div(plan->total_groups, 4);
+  const int64_t blocks = stir::ceil_div(plan->total_units, 4);
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "rgms: too many groups for one launch");
   dim3 grid((unsigned)blocks), block(256);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -238,7 +307,7 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
 #define STIR_RGMS(KK)                                                                              \
   case KK:                                                                                         \
     hipLaunchKernelGGL((rgms_kernel<KK>), grid, block, 0, st, plan->d_table, plan->nk,             \
-                       plan->total_groups, feat_out, W, X, d_Y);                                   \
+                       plan->total_units, feat_out, W, X, d_Y);                                   \
     break
   switch (feat_in / 16) {
     STIR_RGMS(1);

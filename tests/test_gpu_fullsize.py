@@ -1,0 +1,132 @@
+"""Parity at the full sizes of the headline configurations (config 3: 2.45M nodes / 61.9M edges;
+config 5: 100k nodes / 65 relations / 2M edges): bit-exact index arrays against the oracle, and
+size-independent properties for the numeric kernels (hyb equals CSR row-split on the same matrix,
+linearity, oracle agreement on row / edge samples)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparsetir_amd as st
+from sparsetir_amd import datasets, ops
+from helpers import rgms_f64, sddmm_f64, spmm_f64
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cfg3():
+    return datasets.config3()
+
+
+def test_config3_device_format_bit_exact(dev, cfg3):
+    g = cfg3
+    m, n, parts, buckets = g["m"], g["n"], 2, [1, 2, 4, 8, 16, 32]
+    t = lambda a: torch.from_numpy(a).to(dev)
+    rows, cols, mask = st.column_part_hyb(m, n, t(g["indptr"]), t(g["indices"]), parts, buckets)
+    want = oracle.column_part_hyb(m, n, g["indptr"], g["indices"], parts, buckets)
+    total = 0
+    for p in range(parts):
+        for b in range(len(buckets)):
+            assert np.array_equal(rows[p][b].cpu().numpy(), want[0][p][b])
+            assert np.array_equal(cols[p][b].cpu().numpy(), want[1][p][b])
+            assert np.array_equal(mask[p][b].cpu().numpy(), want[2][p][b])
+            total += int(want[2][p][b].sum())
+    assert total == len(g["indices"])  # every nonzero placed exactly once
+
+
+def test_config3_hyb_equals_csr_and_oracle_sample(dev, cfg3):
+    g = cfg3
+    m, n, feat = g["m"], g["n"], 128
+    parts, buckets = g["num_col_parts"], g["buckets"]
+    indptr, indices = g["indptr"], g["indices"]
+    nnz = len(indices)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    d_ptr, d_idx = t(indptr), t(indices)
+    vals = torch.rand(nnz, device=dev, generator=torch.Generator(device=dev).manual_seed(5)) + 0.5
+    rows, cols, mask, avals = st.column_part_hyb(m, n, d_ptr, d_idx, parts, buckets, values=vals)
+    triples, nrows = [], []
+    for p in range(parts):
+        for b in range(len(buckets)):
+            triples += [avals[p][b].reshape(-1), rows[p][b], cols[p][b].reshape(-1)]
+            nrows.append(int(rows[p][b].shape[0]))
+    del mask
+    x = torch.randn(n * feat, device=dev, generator=torch.Generator(device=dev).manual_seed(6))
+    hyb = ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)
+    csr = ops.build_csrmm(m, n, feat, nnz)
+    c_h = torch.zeros(m * feat, device=dev)
+    c_c = torch.empty(m * feat, device=dev)
+    hyb(x, c_h, *triples)
+    csr(vals, x, c_c, d_ptr, d_idx)
+    torch.cuda.synchronize()
+    deg = t(np.diff(indptr).astype(np.float32))
+    # |a| <= 1.5, |x| below ~6: summed magnitude per element is at most 9 * degree
+    tol = (1e-5 * 9.0 * deg.clamp(min=1.0)).repeat_interleave(feat)
+    assert bool(((c_h - c_c).abs() <= tol).all())
+    # linearity: hyb(2x) == 2 hyb(x) up to accumulation order
+    c2 = torch.zeros(m * feat, device=dev)
+    hyb(2 * x, c2, *triples)
+    assert bool(((c2 - 2 * c_h).abs() <= 2 * tol).all())
+    # oracle (serial CPU loop nest) on the first 20000 rows
+    r = 20000
+    sub_ptr, sub_idx = indptr[:r + 1], indices[:indptr[r]]
+    vh, xh = vals[:indptr[r]].cpu().numpy(), x.cpu().numpy().reshape(n, feat)
+    ref = oracle.csrmm(vh, xh, sub_ptr, sub_idx, feat)
+    scale = spmm_f64(sub_ptr, sub_idx, vh, np.abs(xh))
+    got = c_h[:r * feat].cpu().numpy().reshape(r, feat)
+    assert np.all(np.abs(got - ref) <= 2e-5 * scale + 1e-30)
+
+
+def test_config3_sddmm_edge_sample(dev, cfg3):
+    g = cfg3
+    m, n, feat = g["m"], g["n"], 64
+    indptr, indices = g["indptr"], g["indices"]
+    nnz = len(indices)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    a = torch.randn(m * feat, device=dev, generator=torch.Generator(device=dev).manual_seed(7))
+    b = torch.randn(n * feat, device=dev, generator=torch.Generator(device=dev).manual_seed(8))
+    out = torch.empty(nnz, device=dev)
+    mid = torch.empty(nnz, dtype=torch.int32, device=dev)
+    args = (a, b, out, t(indptr), t(indices), mid)
+    ops.build_sddmm_preproc(m, n, feat, nnz)(*args)
+    ops.build_sddmm(m, n, feat, nnz)(*args)
+    torch.cuda.synchronize()
+    rows = np.repeat(np.arange(m, dtype=np.int32), np.diff(indptr))
+    assert np.array_equal(mid.cpu().numpy(), rows)  # mid is the row of every nonzero
+    sel = np.random.default_rng(0).choice(nnz, 200000, replace=False)
+    ah = a.cpu().numpy().reshape(m, feat)[rows[sel]].astype(np.float64)
+    bh = b.cpu().numpy().reshape(n, feat)[indices[sel]].astype(np.float64)
+    want = np.einsum("ek,ek->e", ah, bh)
+    scale = np.einsum("ek,ek->e", np.abs(ah), np.abs(bh))
+    assert np.all(np.abs(out.cpu().numpy()[sel] - want) <= 1e-5 * scale)
+
+
+def test_config5_rgms_full(dev):
+    cfg = datasets.config5()
+    R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    buckets, group = cfg["buckets"], 256
+    rb = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    want_fmt = oracle.csf_to_ell3d(*csf, rb, buckets)
+    for q, arrs in enumerate((ptr, rows, cols, mask)):
+        for k in range(len(buckets)):
+            assert np.array_equal(arrs[k], want_fmt[q][k])
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float16).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
+    x16, w16 = cfg["x"].astype(np.float16), cfg["w"].astype(np.float16)
+    y = torch.zeros(n * fout, device=dev)
+    ops.build_rgms(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols])(
+        t(w16.ravel()), t(x16.ravel()), y, *triples, *mids)
+    torch.cuda.synchronize()
+    ones = np.ones(len(cfg["indices1"]), np.float32)
+    x32, w32 = x16.astype(np.float32), w16.astype(np.float32)
+    want = rgms_f64(*csf, ones, x32, w32, n)
+    scale = rgms_f64(*csf, ones, np.abs(x32), np.abs(w32), n)
+    got = y.cpu().numpy().reshape(n, fout)
+    assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30)
+    ref = oracle.rgms(w32, x32, ones, *csf, n)
+    assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-5 * scale + 1e-30)
