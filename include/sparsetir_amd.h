@@ -192,6 +192,18 @@ int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int3
                   const int32_t* d_indptr, const int32_t* d_indices, void* stream);
 
 /*
+ * SpMM over the condensed format of ConDense on MFMA ("TC-SpMM"), fp16 inputs, fp32
+ * accumulation; argument list [A, B, C, indptr, indices] of examples/spmm/bench_tc_spmm.py:650-656
+ * (operator :538-565).  A: nnzb*t*g (the 0/1 mask of ConDense as fp16, or edge weights),
+ * B: dense features, at least max(indices)+1 rows of feat, C: mb*t*feat of out_dtype (STIR_F16
+ * as in the reference, or STIR_F32), indptr: group_indptr (mb+1), indices: tile_indices
+ * (nnzb*g).  The MFMA path needs tile_size t = 32 and group_size g = 16.
+ */
+int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t group_size,
+                     int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,
+                     const int32_t* d_indptr, const int32_t* d_indices, void* stream);
+
+/*
  * RGMS (relational gather-matmul-scatter), fp16 inputs, fp32 accumulation and output,
  * on the ELL3D buckets produced by CSFToELL3D.  Mirrors the built operator of
  * examples/rgms/rgcn/bench_rgcn_tensorcore.py:838-851: W is [R, feat_in, feat_out], X is

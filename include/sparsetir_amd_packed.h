@@ -95,6 +95,8 @@ enum {
  *      examples/sddmm/bench_sddmm.py:106-115, 170-171
  * "sparsetir.bsrmm"          (A, X, Y, indptr, indices, blk, feat)    A, X f16 or bf16
  *      examples/blocksparse/bsr_spmm.py:427-433
+ * "sparsetir.tcspmm"         (A, B, C, indptr, indices, feat, tile_size, group_size)
+ *      examples/spmm/bench_tc_spmm.py:650-656
  * "sparsetir.rgms"           (W, X, Y, A_0, rows_0, cols_0, ..., mids_0, ..., feat_in, feat_out)
  *      examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
  *
@@ -117,6 +119,7 @@ int stir_packed_hyb_csrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_sddmm_preproc(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_sddmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_bsrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_tcspmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);

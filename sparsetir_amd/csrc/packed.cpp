@@ -332,6 +332,34 @@ int stir_packed_bsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
                                g_stream));
 }
 
+int stir_packed_tcspmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.tcspmm", v, tc, n};
+  if (!a.count(8)) return -1;
+  Arr A = a.arr(0, "A", kDLFloat, 16, kDevice), B = a.arr(1, "B", kDLFloat, 16, kDevice);
+  const DLTensor* d2 = (tc[2] == kTVMDLTensorHandle || tc[2] == kTVMNDArrayHandle || tc[2] == kTVMOpaqueHandle)
+                           ? static_cast<const DLTensor*>(v[2].v_handle) : nullptr;
+  if (!d2) return packed_fail("%s: Expect arg[2] to be pointer", a.fn);
+  const bool out32 = d2->dtype.code == kDLFloat && d2->dtype.bits == 32;
+  Arr C = a.arr(2, "C", kDLFloat, out32 ? 32 : 16, kDevice);
+  Arr P = a.arr(3, "indptr", kDLInt, 32, kDevice), I = a.arr(4, "indices", kDLInt, 32, kDevice);
+  const int64_t feat = a.integer(5, "feat"), t = a.integer(6, "tile_size"), g = a.integer(7, "group_size");
+  if (!a.ok) return -1;
+  const int64_t mb = P.len - 1;
+  if (mb < 0 || feat <= 0 || t <= 0 || g <= 0) return packed_fail("%s: bad sizes", a.fn);
+  if (I.len % g != 0) return packed_fail("%s: indices.shape[0] is not a multiple of group_size", a.fn);
+  const int64_t nnzb = I.len / g;
+  a.len(A, "A", nnzb * t * g);
+  a.len(C, "C", mb * t * feat);
+  if (!a.ok) return -1;
+  if (B.len % feat != 0) return packed_fail("%s: B.shape[0] is not a multiple of feat", a.fn);
+  if (!fits_i32(mb) || !fits_i32(feat) || !fits_i32(t) || !fits_i32(g)) return packed_fail("%s: sizes exceed int32", a.fn);
+  DeviceGuard guard;
+  if (guard.enter(a.dev_id)) return forward(-1);
+  return forward(stir_tc_spmm_f16(out32 ? STIR_F32 : STIR_F16, (int32_t)mb, (int32_t)t, (int32_t)g, (int32_t)feat,
+                                  nnzb, A.data, B.data, C.data, (const int32_t*)P.data, (const int32_t*)I.data,
+                                  g_stream));
+}
+
 int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   Args a{"sparsetir.rgms", v, tc, n};
   if (n < 5 || (n - 5) % 4 != 0) return packed_fail("%s: num_args should be 3 + 4*buckets + 2", a.fn);
@@ -555,6 +583,7 @@ static const PackedEntry kTable[] = {
     {"sparsetir.sddmm_preproc", stir_packed_sddmm_preproc},
     {"sparsetir.sddmm", stir_packed_sddmm},
     {"sparsetir.bsrmm", stir_packed_bsrmm},
+    {"sparsetir.tcspmm", stir_packed_tcspmm},
     {"sparsetir.rgms", stir_packed_rgms},
     {"tir.sparse.ColumnPartHyb.sizes", stir_packed_column_part_hyb_sizes},
     {"tir.sparse.ColumnPartHyb.fill", stir_packed_column_part_hyb_fill},

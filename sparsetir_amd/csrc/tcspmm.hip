@@ -1,0 +1,137 @@
+// SpMM on the gfx950 matrix cores over the condensed format of ConDense: the rows of the
+// sparse matrix are cut into tiles of t = 32 rows; inside a tile the distinct columns are
+// gathered g = 16 at a time into dense 32 x 16 blocks A[jo] (zero where the row has no entry):
+//   C[io*32 + ii, f] = sum over groups jo of tile io, ji < 16:  A[jo, ii, ji] * B[indices[jo, ji], f]
+// fp16 inputs, fp32 accumulation, fp16 or fp32 output.
+//
+// Same tiling as the BSR kernel: a workgroup of four wavefronts owns (row tile, 128 features),
+// a wavefront a 32x32 accumulator.  A step covers two groups (32 gathered rows of B): A[jo] is
+// already in MFMA A-operand order (a lane's 8 k values are contiguous), the 32 gathered rows of
+// B go through LDS, interleaved into (k, k+1) pairs on the way, double-buffered, with the next
+// step's gathers in flight during the multiply.
+#include "common.h"
+#include "../../include/sparsetir_amd.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTileF = 128;
+constexpr int kTile = 32;   // t
+constexpr int kGroup = 16;  // g
+
+template <int OUT>  // 0: fp16 output, 1: fp32 output
+__global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f_tiles,
+                                                     const uint16_t* __restrict__ A,
+                                                     const uint16_t* __restrict__ B, void* __restrict__ C,
+                                                     const int32_t* __restrict__ indptr,
+                                                     const int32_t* __restrict__ indices) {
+  __shared__ uint32_t xs[2][16][kTileF];  // [buffer][k pair][feature]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  const int f_tile = (int)(blockIdx.x % f_tiles);
+  const int64_t io = blockIdx.x / f_tiles;
+  if (io >= mb) return;
+  const int f0 = f_tile * kTileF;
+  const int kp = tid >> 4, fc = tid & 15;  // staging role: k pair, 8-feature chunk
+  const bool stage_live = f0 + fc * 8 < feat;
+
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+
+  const int64_t g_begin = indptr[io], g_end = indptr[io + 1];
+  const int64_t rows_total = (g_end - g_begin) * kGroup;  // gathered rows of B for this tile
+  const int steps = (int)((rows_total + 31) / 32);
+  const int32_t* rowlist = indices + g_begin * kGroup;
+
+  u32x4 r0, r1, a_next[2];
+  auto fetch = [&](int it) {
+    // A[jo][n][8h .. 8h+7] for the step's two groups (zero when the tile has an odd group count)
+    const int64_t jo = g_begin + 2 * it;
+    a_next[0] = *reinterpret_cast<const u32x4*>(A + (jo * kTile + n) * kGroup + 8 * h);
+    a_next[1] = u32x4{0, 0, 0, 0};
+    if (jo + 1 < g_end) a_next[1] = *reinterpret_cast<const u32x4*>(A + ((jo + 1) * kTile + n) * kGroup + 8 * h);
+    r0 = r1 = u32x4{0, 0, 0, 0};
+    const int64_t k = (int64_t)it * 32 + 2 * kp;
+    if (stage_live && k < rows_total) {
+      // k and k+1 belong to the same group (groups hold 16 rows), so both exist
+      const int64_t row_a = rowlist[k], row_b = rowlist[k + 1];
+      r0 = *reinterpret_cast<const u32x4*>(B + row_a * feat + f0 + fc * 8);
+      r1 = *reinterpret_cast<const u32x4*>(B + row_b * feat + f0 + fc * 8);
+    }
+  };
+
+  if (steps > 0) fetch(0);
+  for (int it = 0; it < steps; ++it) {
+    const int buf = it & 1;
+    const u32x4 a0 = a_next[0], a1 = a_next[1];
+    u32x4 lo, hi;
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      lo[2 * d] = __builtin_amdgcn_perm(r1[d], r0[d], 0x05040100);
+      lo[2 * d + 1] = __builtin_amdgcn_perm(r1[d], r0[d], 0x07060302);
+      hi[2 * d] = __builtin_amdgcn_perm(r1[d + 2], r0[d + 2], 0x05040100);
+      hi[2 * d + 1] = __builtin_amdgcn_perm(r1[d + 2], r0[d + 2], 0x07060302);
+    }
+    *reinterpret_cast<u32x4*>(&xs[buf][kp][fc * 8]) = lo;
+    *reinterpret_cast<u32x4*>(&xs[buf][kp][fc * 8 + 4]) = hi;
+    if (it + 1 < steps) fetch(it + 1);
+    __syncthreads();
+    const int col = wave * 32 + n;
+    u32x4 b0, b1;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      b0[d] = xs[buf][4 * h + d][col];      // rows 8h .. 8h+7 of the first group
+      b1[d] = xs[buf][8 + 4 * h + d][col];  // rows 8h .. 8h+7 of the second group
+    }
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a0), __builtin_bit_cast(f16x8, b0),
+                                                acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a1), __builtin_bit_cast(f16x8, b1),
+                                                acc, 0, 0, 0);
+  }
+  const int fcol = f0 + wave * 32;
+  if (fcol >= feat) return;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int row = (v & 3) + 4 * h + 8 * (v >> 2);
+    const int64_t off = (io * kTile + row) * feat + fcol + n;
+    if constexpr (OUT == 1) {
+      static_cast<float*>(C)[off] = acc[v];
+    } else {
+      const _Float16 hv = (_Float16)acc[v];
+      static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t group_size,
+                                int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,
+                                const int32_t* d_indptr, const int32_t* d_indices, void* stream) {
+  STIR_REQUIRE(out_dtype == STIR_F16 || out_dtype == STIR_F32, "tc_spmm: out_dtype must be STIR_F16 or STIR_F32");
+  STIR_REQUIRE(tile_size == kTile && group_size == kGroup,
+               "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t=32, g=16", tile_size, group_size);
+  STIR_REQUIRE(mb >= 0 && nnzb >= 0, "tc_spmm: bad sizes");
+  STIR_REQUIRE(feat > 0 && feat % 32 == 0, "tc_spmm: feat=%d must be a multiple of 32", feat);
+  if (mb == 0) return 0;
+  STIR_REQUIRE(d_B && d_C && d_indptr && (nnzb == 0 || (d_A && d_indices)), "tc_spmm: null pointer argument");
+  const int f_tiles = (int)stir::ceil_div(feat, kTileF);
+  const int64_t blocks = (int64_t)mb * f_tiles;
+  STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint16_t* A = static_cast<const uint16_t*>(d_A);
+  const uint16_t* B = static_cast<const uint16_t*>(d_B);
+  if (out_dtype == STIR_F32)
+    hipLaunchKernelGGL(tcspmm_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb, f_tiles, A,
+                       B, d_C, d_indptr, d_indices);
+  else
+    hipLaunchKernelGGL(tcspmm_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb, f_tiles, A,
+                       B, d_C, d_indptr, d_indices);
+  STIR_LAUNCH_CHECK();
+  return 0;
+}

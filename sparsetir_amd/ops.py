@@ -9,6 +9,7 @@ hand-written gfx950 kernel through the C ABI on torch's current stream:
   build_sddmm_preproc f(A, B, C, indptr, indices, mid)        examples/sddmm/bench_sddmm.py:106-115
   build_sddmm         f(A, B, C, indptr, indices, mid)        examples/sddmm/bench_sddmm.py:170-171
   build_bsrmm         f(A, X, Y, indptr, indices)             examples/blocksparse/bsr_spmm.py:427-433
+  build_tcspmm        f(A, B, C, indptr, indices)             examples/spmm/bench_tc_spmm.py:650-656
   build_rgms          f(W, X, Y, (A_k, rows_k, cols_k)..., mids_k...)
                                                                examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
 
@@ -217,6 +218,28 @@ class BsrMM(_Operator):
                                             _ptr(indptr), _ptr(indices), _stream()))
 
 
+class TcSpMM(_Operator):
+    """SpMM over the condensed (t x 1 tiles, g per group) format on the matrix cores."""
+    name = "tcspmm"
+
+    def __init__(self, mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=torch.float16):
+        self.mb, self.nnzb, self.feat = int(mb), int(nnzb), int(feat)
+        self.t, self.g, self.brows = int(tile_size), int(group_size), int(num_b_rows)
+        self.out_dtype = out_dtype
+        self.L = _lib.lib()
+
+    def __call__(self, *args):
+        f16, i32 = torch.float16, torch.int32
+        dev = self._check(args, [("A", f16, self.nnzb * self.t * self.g), ("B", f16, self.brows * self.feat),
+                                 ("C", self.out_dtype, self.mb * self.t * self.feat),
+                                 ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb * self.g)])
+        a, b, c, indptr, indices = args
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_tc_spmm_f16(_DT[self.out_dtype], self.mb, self.t, self.g, self.feat,
+                                               self.nnzb, _ptr(a), _ptr(b), _ptr(c), _ptr(indptr),
+                                               _ptr(indices), _stream()))
+
+
 class Rgms(_Operator):
     """RGMS on ELL3D buckets.  ``groups`` lists the group count of every bucket, ``rows_bkt`` /
     ``cols_bkt`` the ELL rows per group and slots per ELL row."""
@@ -294,6 +317,10 @@ def build_sddmm(m, n, feat, nnz):
 
 def build_bsrmm(mb, nb, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):
     return BsrMM(mb, nb, nnzb, blk, feat, dtype, out_dtype)
+
+
+def build_tcspmm(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=torch.float16):
+    return TcSpMM(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype)
 
 
 def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
