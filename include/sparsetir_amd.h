@@ -180,6 +180,13 @@ int stir_sddmm_preproc(int32_t m, int64_t nnz, const int32_t* d_indptr, int32_t*
 int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
                    const float* d_B, float* d_C, const int32_t* d_indptr,
                    const int32_t* d_indices, const int32_t* d_mid, void* stream);
+/* The same with every result scaled by its nonzero's value, C[e] = E[e] * <A[mid[e],:], B[indices[e],:]>
+ * (the form sampled dense-dense products take on a weighted graph; the reference's operator,
+ * examples/sddmm/bench_sddmm.py:32-55, is the E = 1 case). */
+int stir_sddmm_scaled_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
+                          const float* d_B, float* d_C, const int32_t* d_indptr,
+                          const int32_t* d_indices, const int32_t* d_mid, const float* d_edge_values,
+                          void* stream);
 
 /*
  * BSR SpMM on MFMA, 16-bit inputs, fp32 accumulation; argument list [A, X, Y, indptr,

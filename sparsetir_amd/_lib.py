@@ -38,6 +38,7 @@ SIGNATURES = {
     "stir_hyb_plan_destroy": (I32, [VP]),
     "stir_sddmm_preproc": (I32, [I32, I64, VP, VP, VP]),
     "stir_sddmm_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP]),
+    "stir_sddmm_scaled_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP, VP]),
     "stir_bsr_spmm": (I32, [I32, I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
     "stir_tc_spmm_f16": (I32, [I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),

@@ -37,7 +37,8 @@ template <int G, int REP>
 __global__ __launch_bounds__(256) void sddmm_kernel(int64_t nnz, int feat, const float* __restrict__ A,
                                                     const float* __restrict__ B, float* __restrict__ C,
                                                     const int32_t* __restrict__ indices,
-                                                    const int32_t* __restrict__ mid) {
+                                                    const int32_t* __restrict__ mid,
+                                                    const float* __restrict__ scale) {
   constexpr int CH = (G < 4 ? G : 4);  // nonzeros in flight per lane group (2 row loads each)
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -78,14 +79,15 @@ __global__ __launch_bounds__(256) void sddmm_kernel(int64_t nnz, int feat, const
       if (gl == c + u) out = p;
     }
   }
-  if (e < nnz) C[e] = out;
+  if (e < nnz) C[e] = scale ? out * scale[e] : out;
 }
 
 // Any feature width: one wavefront per 64 nonzeros, lanes stride over the features.
 __global__ __launch_bounds__(256) void sddmm_generic_kernel(int64_t nnz, int feat, const float* __restrict__ A,
                                                             const float* __restrict__ B, float* __restrict__ C,
                                                             const int32_t* __restrict__ indices,
-                                                            const int32_t* __restrict__ mid) {
+                                                            const int32_t* __restrict__ mid,
+                                                            const float* __restrict__ scale) {
   const int lane = threadIdx.x & 63;
   const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int64_t e0 = tile * kWave;
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(256) void sddmm_generic_kernel(int64_t nnz, int fea
     p = group_allreduce<64>(p);
     if (lane == j) out = p;
   }
-  if (lane < cnt) C[e0 + lane] = out;
+  if (lane < cnt) C[e0 + lane] = scale ? out * scale[e0 + lane] : out;
 }
 
 __global__ __launch_bounds__(256) void sddmm_preproc_kernel(int m, int64_t nnz,
@@ -136,10 +138,9 @@ int stir_sddmm_preproc(int32_t m, int64_t nnz, const int32_t* d_indptr, int32_t*
   return 0;
 }
 
-int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
-                   const float* d_B, float* d_C, const int32_t* d_indptr,
-                   const int32_t* d_indices, const int32_t* d_mid, void* stream) {
-  (void)d_indptr;  // part of the reference's argument list; rows come from mid
+static int sddmm_launch(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A, const float* d_B,
+                        float* d_C, const int32_t* d_indices, const int32_t* d_mid, const float* d_scale,
+                        void* stream) {
   STIR_REQUIRE(m >= 0 && n >= 0 && feat > 0 && nnz >= 0, "sddmm: bad sizes m=%d n=%d feat=%d", m, n, feat);
   if (nnz == 0) return 0;
   STIR_REQUIRE(d_A && d_B && d_C && d_indices && d_mid, "sddmm: null pointer argument");
@@ -147,8 +148,9 @@ int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float*
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "sddmm: nnz=%lld exceeds one launch", (long long)nnz);
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((unsigned)blocks), block(256);
-#define STIR_SDDMM(G, REP) \
-  hipLaunchKernelGGL((sddmm_kernel<G, REP>), grid, block, 0, st, nnz, feat, d_A, d_B, d_C, d_indices, d_mid)
+#define STIR_SDDMM(G, REP)                                                                             \
+  hipLaunchKernelGGL((sddmm_kernel<G, REP>), grid, block, 0, st, nnz, feat, d_A, d_B, d_C, d_indices, d_mid, \
+                     d_scale)
   switch (feat) {
     case 16: STIR_SDDMM(4, 1); break;
     case 32: STIR_SDDMM(8, 1); break;
@@ -157,11 +159,28 @@ int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float*
     case 256: STIR_SDDMM(64, 1); break;
     case 512: STIR_SDDMM(64, 2); break;
     default:
-      hipLaunchKernelGGL(sddmm_generic_kernel, grid, block, 0, st, nnz, feat, d_A, d_B, d_C, d_indices, d_mid);
+      hipLaunchKernelGGL(sddmm_generic_kernel, grid, block, 0, st, nnz, feat, d_A, d_B, d_C, d_indices, d_mid,
+                         d_scale);
   }
 #undef STIR_SDDMM
   STIR_LAUNCH_CHECK();
   return 0;
+}
+
+int stir_sddmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
+                   const float* d_B, float* d_C, const int32_t* d_indptr,
+                   const int32_t* d_indices, const int32_t* d_mid, void* stream) {
+  (void)d_indptr;  // part of the reference's argument list; rows come from mid
+  return sddmm_launch(m, n, feat, nnz, d_A, d_B, d_C, d_indices, d_mid, nullptr, stream);
+}
+
+int stir_sddmm_scaled_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const float* d_A,
+                          const float* d_B, float* d_C, const int32_t* d_indptr,
+                          const int32_t* d_indices, const int32_t* d_mid, const float* d_edge_values,
+                          void* stream) {
+  (void)d_indptr;
+  STIR_REQUIRE(nnz == 0 || d_edge_values, "sddmm_scaled: edge values are null");
+  return sddmm_launch(m, n, feat, nnz, d_A, d_B, d_C, d_indices, d_mid, d_edge_values, stream);
 }
 
 }  // extern "C"

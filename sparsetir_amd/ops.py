@@ -191,6 +191,19 @@ class Sddmm(SddmmPreproc):
                                              _stream()))
 
 
+class SddmmScaled(SddmmPreproc):
+    """C[e] = E[e] * <A[mid[e], :], B[indices[e], :]>: f(A, B, C, indptr, indices, mid, E)."""
+    name = "sddmm_scaled"
+
+    def __call__(self, *args):
+        dev = self._check(args, self._spec() + [("E", torch.float32, self.nnz)])
+        a, b, c, indptr, indices, mid, e = args
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_sddmm_scaled_f32(self.m, self.n, self.feat, self.nnz, _ptr(a), _ptr(b),
+                                                    _ptr(c), _ptr(indptr), _ptr(indices), _ptr(mid), _ptr(e),
+                                                    _stream()))
+
+
 _DT = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
 
 
@@ -313,6 +326,10 @@ def build_sddmm_preproc(m, n, feat, nnz):
 
 def build_sddmm(m, n, feat, nnz):
     return Sddmm(m, n, feat, nnz)
+
+
+def build_sddmm_scaled(m, n, feat, nnz):
+    return SddmmScaled(m, n, feat, nnz)
 
 
 def build_bsrmm(mb, nb, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):

@@ -66,3 +66,24 @@ def test_sddmm_config3_shape_small_scale(dev):
     assert np.array_equal(mid, rows)
     scale = np.einsum("ek,ek->e", np.abs(a).astype(np.float64)[rows], np.abs(b).astype(np.float64)[g["indices"]])
     assert np.all(np.abs(got - want) <= RTOL * scale + 1e-30)
+
+
+def test_sddmm_scaled_by_edge_values(dev):
+    m, n, feat = 400, 300, 64
+    indptr, indices = random_csr(m, n, 9000, 5, skew=1.0)
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((m, feat), dtype=np.float32)
+    b = rng.standard_normal((n, feat), dtype=np.float32)
+    e = rng.random(len(indices), dtype=np.float32)
+    t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+    nnz = len(indices)
+    c = torch.empty(nnz, device=dev)
+    mid = torch.empty(nnz, dtype=torch.int32, device=dev)
+    args = [t(a.ravel()), t(b.ravel()), c, t(indptr), t(indices), mid]
+    ops.build_sddmm_preproc(m, n, feat, nnz)(*args)
+    ops.build_sddmm_scaled(m, n, feat, nnz)(*args, t(e))
+    torch.cuda.synchronize()
+    want = sddmm_f64(indptr, indices, a, b) * e
+    rows = np.repeat(np.arange(m), np.diff(indptr))
+    scale = np.einsum("ek,ek->e", np.abs(a).astype(np.float64)[rows], np.abs(b).astype(np.float64)[indices]) * e
+    assert np.all(np.abs(c.cpu().numpy() - want) <= 2 * RTOL * scale + 1e-30)
