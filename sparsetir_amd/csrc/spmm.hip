@@ -41,13 +41,6 @@ __device__ __forceinline__ void fma4(float4& acc, float a, const float4& x) {
   acc.w = fmaf(a, x.w, acc.w);
 }
 
-__device__ __forceinline__ void atomic_add4(float* p, const float4& v) {
-  __hip_atomic_fetch_add(p + 0, v.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_fetch_add(p + 1, v.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_fetch_add(p + 2, v.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_fetch_add(p + 3, v.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // Sum `acc` over the lane groups whose group index differs in the bits [G, limit).
 template <int G, int REP>
 __device__ __forceinline__ void reduce_groups(float4 (&acc)[REP], int limit) {
@@ -65,16 +58,35 @@ __device__ __forceinline__ void reduce_groups(float4 (&acc)[REP], int limit) {
   }
 }
 
+// Store, or accumulate with atomics, the 4*G*REP features a lane group holds for output row
+// `row`.  A lane owns 4 consecutive floats, so issuing the atomics straight from the registers
+// would make every atomic instruction touch G addresses 16 bytes apart (4 cache lines per 32
+// lanes, 4 times over).  Instead the group's floats go through the wavefront's piece of LDS
+// (`stage`, 256*REP floats) and come back with lane l holding float k*G + l, so each atomic
+// instruction covers G consecutive floats.  LDS instructions of one wavefront execute in order,
+// no workgroup barrier is involved.
 template <int G, int REP>
-__device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int gl,
-                                          const float4 (&acc)[REP], bool atomic) {
-  float* base = C + row * feat + gl * 4;
+__device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int lane,
+                                          const float4 (&acc)[REP], bool atomic, float* stage) {
+  const int g = lane / G, gl = lane % G;
+  if (!atomic) {
+    float* base = C + row * feat + gl * 4;
+#pragma unroll
+    for (int r = 0; r < REP; ++r) *reinterpret_cast<float4*>(base + r * G * 4) = acc[r];
+    return;
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int r = 0; r < REP; ++r) *reinterpret_cast<float4*>(stage + (r * kWave + lane) * 4) = acc[r];
+  __builtin_amdgcn_wave_barrier();
+  float* base = C + row * feat + gl;
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
-    if (atomic)
-      atomic_add4(base + r * G * 4, acc[r]);
-    else
-      *reinterpret_cast<float4*>(base + r * G * 4) = acc[r];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float v = stage[(r * kWave + g * G) * 4 + k * G + gl];
+      __hip_atomic_fetch_add(base + r * G * 4 + k * G, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 
@@ -123,7 +135,7 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, const fl
     }
   }
   reduce_groups<G, REP>(acc, kWave);
-  if (g == 0) write_row<G, REP>(C, row, feat, gl, acc, false);
+  if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, false, nullptr);
 }
 
 // Any feature width: one wavefront per row, lane l owns features l, l+64, ...
@@ -149,7 +161,7 @@ __global__ __launch_bounds__(256) void csr_spmm_generic_kernel(int m, int feat, 
 template <int G, int REP, int LOG2W>
 __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, int feat,
                                               const float* __restrict__ B, float* __restrict__ C,
-                                              int lane) {
+                                              int lane, float* stage) {
   constexpr int W = 1 << LOG2W;
   constexpr int CH = G < 8 ? G : 8;  // gathers in flight per lane
   const int g = lane / G, gl = lane % G;
@@ -192,7 +204,7 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
         // end of an ELL row inside this lane group; for W <= CH this folds to a constant
         if (((c + u + 1) & (W - 1)) == 0) {
           const int out_row = __shfl(my_row, (g * G + c + u) >> LOG2W, kWave);
-          if (out_row >= 0) write_row<G, REP>(C, out_row, feat, gl, acc, atomic);
+          if (out_row >= 0) write_row<G, REP>(C, out_row, feat, lane, acc, atomic, stage);
 #pragma unroll
           for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
@@ -204,7 +216,7 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
     reduce_groups<G, REP>(acc, W);
     const int out_row = __shfl(my_row, (g * G) >> LOG2W, kWave);
     if (((g * G) & (W - 1)) == 0 && out_row >= 0)
-      write_row<G, REP>(C, out_row, feat, gl, acc, atomic);
+      write_row<G, REP>(C, out_row, feat, lane, acc, atomic, stage);
   }
 }
 
@@ -213,7 +225,7 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
 template <int G, int REP>
 __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int feat,
                                              const float* __restrict__ B, float* __restrict__ C,
-                                             int lane) {
+                                             int lane, float* stage) {
   constexpr int CH = G < 8 ? G : 8;
   const int g = lane / G, gl = lane % G;
   const int w = bk.width;
@@ -250,7 +262,7 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
     }
   }
   reduce_groups<G, REP>(acc, kWave);
-  if (g == 0) write_row<G, REP>(C, bk.rows[row], feat, gl, acc, bk.atomic != 0);
+  if (g == 0) write_row<G, REP>(C, bk.rows[row], feat, lane, acc, bk.atomic != 0, stage);
 }
 
 __device__ __forceinline__ int find_bucket(const HybBucket* __restrict__ table, int nb,
@@ -271,22 +283,24 @@ __global__ __launch_bounds__(256) void hyb_spmm_kernel(const HybBucket* __restri
                                                        int64_t total_tiles, int feat,
                                                        const float* __restrict__ B,
                                                        float* __restrict__ C) {
+  __shared__ float stage_all[4][kWave * 4 * REP];  // per-wavefront staging for atomic rows
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  float* stage = stage_all[wave];
   const int64_t tile = (int64_t)blockIdx.x * 4 + wave;
   if (tile >= total_tiles) return;
   const int k = find_bucket(table, nb, tile);
   const HybBucket bk = table[k];
   const int64_t t = tile - bk.tile_begin;
   switch (bk.log2w) {
-    case 0: hyb_slot_tile<G, REP, 0>(bk, t, feat, B, C, lane); break;
-    case 1: hyb_slot_tile<G, REP, 1>(bk, t, feat, B, C, lane); break;
-    case 2: hyb_slot_tile<G, REP, 2>(bk, t, feat, B, C, lane); break;
-    case 3: hyb_slot_tile<G, REP, 3>(bk, t, feat, B, C, lane); break;
-    case 4: hyb_slot_tile<G, REP, 4>(bk, t, feat, B, C, lane); break;
-    case 5: hyb_slot_tile<G, REP, 5>(bk, t, feat, B, C, lane); break;
-    case 6: hyb_slot_tile<G, REP, 6>(bk, t, feat, B, C, lane); break;
-    default: hyb_row_tile<G, REP>(bk, t, feat, B, C, lane); break;
+    case 0: hyb_slot_tile<G, REP, 0>(bk, t, feat, B, C, lane, stage); break;
+    case 1: hyb_slot_tile<G, REP, 1>(bk, t, feat, B, C, lane, stage); break;
+    case 2: hyb_slot_tile<G, REP, 2>(bk, t, feat, B, C, lane, stage); break;
+    case 3: hyb_slot_tile<G, REP, 3>(bk, t, feat, B, C, lane, stage); break;
+    case 4: hyb_slot_tile<G, REP, 4>(bk, t, feat, B, C, lane, stage); break;
+    case 5: hyb_slot_tile<G, REP, 5>(bk, t, feat, B, C, lane, stage); break;
+    case 6: hyb_slot_tile<G, REP, 6>(bk, t, feat, B, C, lane, stage); break;
+    default: hyb_row_tile<G, REP>(bk, t, feat, B, C, lane, stage); break;
   }
 }
 
