@@ -199,6 +199,17 @@ int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int3
                   const int32_t* d_indptr, const int32_t* d_indices, void* stream);
 
 /*
+ * Doubly-compressed BSR ("dbsrmm", examples/blocksparse/bsr_spmm.py:66-102): only nnz_rows block
+ * rows are stored; stored block row i is block row d_row_ids[i] of Y (the reference's indices_0;
+ * its indptr_0 is [0, nnz_rows]), d_indptr (nnz_rows+1) / d_indices index its blocks.  Block rows
+ * of Y that are not stored are left untouched.
+ */
+int stir_dbsr_spmm(int32_t dtype, int32_t out_dtype, int32_t nnz_rows, int32_t nb, int32_t blk,
+                   int32_t feat, int64_t nnzb, const void* d_A, const void* d_X, void* d_Y,
+                   const int32_t* d_row_ids, const int32_t* d_indptr, const int32_t* d_indices,
+                   void* stream);
+
+/*
  * SpMM over the condensed format of ConDense on MFMA ("TC-SpMM"), fp16 inputs, fp32
  * accumulation; argument list [A, B, C, indptr, indices] of examples/spmm/bench_tc_spmm.py:650-656
  * (operator :538-565).  A: nnzb*t*g (the 0/1 mask of ConDense as fp16, or edge weights),

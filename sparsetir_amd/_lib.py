@@ -40,6 +40,7 @@ SIGNATURES = {
     "stir_sddmm_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP]),
     "stir_sddmm_scaled_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP, VP]),
     "stir_bsr_spmm": (I32, [I32, I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
+    "stir_dbsr_spmm": (I32, [I32, I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP]),
     "stir_tc_spmm_f16": (I32, [I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),

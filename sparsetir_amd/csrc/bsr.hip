@@ -79,7 +79,8 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
                                                        const uint16_t* __restrict__ A,
                                                        const uint16_t* __restrict__ X, void* __restrict__ Y,
                                                        const int32_t* __restrict__ indptr,
-                                                       const int32_t* __restrict__ indices) {
+                                                       const int32_t* __restrict__ indices,
+                                                       const int32_t* __restrict__ row_ids) {
   constexpr int TF = kTileF * NT;
   constexpr int FC = TF / 8;      // 8-feature chunks per tile row
   constexpr int KPT = 256 / FC;   // k pairs covered by one pass of the 256 threads
@@ -102,6 +103,8 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
+  // doubly-compressed form: stored block row i is block row row_ids[i] of the output
+  const int i_out = row_ids ? row_ids[i] : i;
   const int p_begin = indptr[i];
   const int ksteps = blk / kTileK;
   const int steps = (indptr[i + 1] - p_begin) * ksteps;
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int row = (v & 3) + 4 * h + 8 * (v >> 2);
-      const int64_t off = ((int64_t)i * blk + bi0 + row) * feat + fcol + n;
+      const int64_t off = ((int64_t)i_out * blk + bi0 + row) * feat + fcol + n;
       if constexpr (OUT == 1)
         static_cast<float*>(Y)[off] = acc[t][v];
       else
@@ -185,9 +188,9 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
 
 }  // namespace
 
-extern "C" int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk,
-                             int32_t feat, int64_t nnzb, const void* d_A, const void* d_X, void* d_Y,
-                             const int32_t* d_indptr, const int32_t* d_indices, void* stream) {
+static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk, int32_t feat,
+                      int64_t nnzb, const void* d_A, const void* d_X, void* d_Y, const int32_t* d_indptr,
+                      const int32_t* d_indices, const int32_t* d_row_ids, void* stream) {
   STIR_REQUIRE(dtype == STIR_F16 || dtype == STIR_BF16, "bsr_spmm: dtype must be STIR_F16 or STIR_BF16");
   STIR_REQUIRE(out_dtype == dtype || out_dtype == STIR_F32, "bsr_spmm: out_dtype must equal dtype or be STIR_F32");
   STIR_REQUIRE(mb >= 0 && nb >= 0 && nnzb >= 0, "bsr_spmm: bad sizes mb=%d nb=%d", mb, nb);
@@ -210,7 +213,7 @@ extern "C" int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32
   dim3 grid((unsigned)blocks), block(256);
 #define STIR_BSR_L(BF, OUT, NTV, SV)                                                                     \
   hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, SV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
-                     A, X, d_Y, d_indptr, d_indices)
+                     A, X, d_Y, d_indptr, d_indices, d_row_ids)
 #define STIR_BSR(BF, OUT)                  \
   do {                                     \
     if (nt == 2)                           \
@@ -228,3 +231,23 @@ extern "C" int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32
   STIR_LAUNCH_CHECK();
   return 0;
 }
+
+extern "C" {
+
+int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk, int32_t feat,
+                  int64_t nnzb, const void* d_A, const void* d_X, void* d_Y, const int32_t* d_indptr,
+                  const int32_t* d_indices, void* stream) {
+  return bsr_launch(dtype, out_dtype, mb, nb, blk, feat, nnzb, d_A, d_X, d_Y, d_indptr, d_indices, nullptr,
+                    stream);
+}
+
+int stir_dbsr_spmm(int32_t dtype, int32_t out_dtype, int32_t nnz_rows, int32_t nb, int32_t blk,
+                   int32_t feat, int64_t nnzb, const void* d_A, const void* d_X, void* d_Y,
+                   const int32_t* d_row_ids, const int32_t* d_indptr, const int32_t* d_indices,
+                   void* stream) {
+  STIR_REQUIRE(nnz_rows == 0 || d_row_ids, "dbsr_spmm: row ids are null");
+  return bsr_launch(dtype, out_dtype, nnz_rows, nb, blk, feat, nnzb, d_A, d_X, d_Y, d_indptr, d_indices,
+                    d_row_ids, stream);
+}
+
+}  // extern "C"

@@ -9,6 +9,8 @@ hand-written gfx950 kernel through the C ABI on torch's current stream:
   build_sddmm_preproc f(A, B, C, indptr, indices, mid)        examples/sddmm/bench_sddmm.py:106-115
   build_sddmm         f(A, B, C, indptr, indices, mid)        examples/sddmm/bench_sddmm.py:170-171
   build_bsrmm         f(A, X, Y, indptr, indices)             examples/blocksparse/bsr_spmm.py:427-433
+  build_dbsrmm        f(A, X, Y, indptr_0, indices_0, indptr_1, indices_1)
+                                                               examples/blocksparse/bsr_spmm.py:66-102
   build_tcspmm        f(A, B, C, indptr, indices)             examples/spmm/bench_tc_spmm.py:650-656
   build_rgms          f(W, X, Y, (A_k, rows_k, cols_k)..., mids_k...)
                                                                examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
@@ -231,6 +233,31 @@ class BsrMM(_Operator):
                                             _ptr(indptr), _ptr(indices), _stream()))
 
 
+class DBsrMM(_Operator):
+    """Doubly-compressed BSR SpMM: f(A, X, Y, indptr_0, indices_0, indptr_1, indices_1), the
+    argument list of the reference's dbsrmm (examples/blocksparse/bsr_spmm.py:66-102)."""
+    name = "dbsrmm"
+
+    def __init__(self, mb, nb, nnz_rows, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):
+        self.mb, self.nb, self.nr, self.nnzb, self.blk, self.feat = map(int, (mb, nb, nnz_rows, nnzb, blk, feat))
+        self.dtype = dtype
+        self.out_dtype = dtype if out_dtype is None else out_dtype
+        self.L = _lib.lib()
+
+    def __call__(self, *args):
+        i32 = torch.int32
+        dev = self._check(args, [("A", self.dtype, self.nnzb * self.blk * self.blk),
+                                 ("X", self.dtype, self.nb * self.blk * self.feat),
+                                 ("Y", self.out_dtype, self.mb * self.blk * self.feat),
+                                 ("indptr_0", i32, 2), ("indices_0", i32, self.nr),
+                                 ("indptr_1", i32, self.nr + 1), ("indices_1", i32, self.nnzb)])
+        a, x, y, _, rows, indptr, indices = args
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_dbsr_spmm(_DT[self.dtype], _DT[self.out_dtype], self.nr, self.nb, self.blk,
+                                             self.feat, self.nnzb, _ptr(a), _ptr(x), _ptr(y), _ptr(rows),
+                                             _ptr(indptr), _ptr(indices), _stream()))
+
+
 class TcSpMM(_Operator):
     """SpMM over the condensed (t x 1 tiles, g per group) format on the matrix cores."""
     name = "tcspmm"
@@ -334,6 +361,10 @@ def build_sddmm_scaled(m, n, feat, nnz):
 
 def build_bsrmm(mb, nb, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):
     return BsrMM(mb, nb, nnzb, blk, feat, dtype, out_dtype)
+
+
+def build_dbsrmm(mb, nb, nnz_rows, nnzb, blk, feat, dtype=torch.float16, out_dtype=None):
+    return DBsrMM(mb, nb, nnz_rows, nnzb, blk, feat, dtype, out_dtype)
 
 
 def build_tcspmm(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=torch.float16):

