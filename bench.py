@@ -125,6 +125,31 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
                            "frac_of_hbm_peak": byts / d / 1e9 / HBM_PEAK_GBS, "edges": E,
                            "ell_rows": int(sum(r.size for r in rows)),
                            "atomic_GBps": sum(r.size for r in rows) * fout * 4.0 / d / 1e9}
+
+    # fp32 forms: ELL3D buckets with 32-slot groups (the reference's composable fp32 setting) and the
+    # CSF traversal; W is [R, fout, fin]
+    w32 = t(np.ascontiguousarray(cfg["w"].transpose(0, 2, 1)).ravel())
+    x32 = t(cfg["x"].ravel())
+    byts32 = 8.0 * E + 4.0 * n * fin + 4.0 * R * fin * fout + 4.0 * n * fout
+    rb32 = [32 // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"],
+                                            rb32, buckets)
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float32).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
+    f32 = ops.build_rgms_f32(n, n, R, fin, fout, rb32, buckets, [c.shape[0] for c in cols])
+    _, d, _ = time_steps(lambda: f32(w32, x32, y, *triples, *mids), 10, 1, torch)
+    out["rgms_f32_ell3d_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
+                                     "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
+                                     "ell_rows": int(sum(r.size for r in rows))}
+    csf = [t(cfg[k]) for k in ("indptr0", "indices0", "indptr1", "indices1")]
+    ones = torch.ones(E, device=dev)
+    fc = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E)
+    _, d, _ = time_steps(lambda: fc(ones, w32, x32, y, *csf), 10, 1, torch)
+    out["rgms_f32_csf_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
+                                   "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
+                                   "stored_rows": int(len(cfg["indices0"]))}
     return out
 
 

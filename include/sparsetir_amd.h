@@ -239,6 +239,37 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
                   float* d_Y, void* stream);
 int stir_rgms_plan_destroy(stir_rgms_plan* plan);
 
+/*
+ * RGMS in fp32 on ELL3D buckets: the composable fp32 operator of
+ * examples/rgms/rgcn/bench_rgcn_composable.py:186-225 (rgcn_hetero_forward of
+ * examples/rgms/rgcn/utils.py:55-87 after format_decompose).  As stir_rgms_f16, except that
+ * every array is fp32 and W is [R, feat_out, feat_in].  feat_in: a multiple of 4, at most 128;
+ * W and X 16-byte aligned.
+ */
+typedef struct stir_rgms_f32_plan stir_rgms_f32_plan;
+int stir_rgms_f32_plan_create(stir_rgms_f32_plan** plan, int32_t num_buckets, const int32_t* rows_bkt,
+                              const int32_t* cols_bkt, const int64_t* groups,
+                              const float* const* d_A, const int32_t* const* d_rows,
+                              const int32_t* const* d_cols, const int32_t* const* d_mids);
+int stir_rgms_f32(const stir_rgms_f32_plan* plan, int32_t m, int32_t n, int32_t num_rels,
+                  int32_t feat_in, int32_t feat_out, const float* d_W, const float* d_X,
+                  float* d_Y, void* stream);
+int stir_rgms_f32_plan_destroy(stir_rgms_f32_plan* plan);
+
+/*
+ * RGMS in fp32 straight from the CSF arrays (relation -> stored row -> column): the
+ * non-composable operator of examples/rgms/rgcn/bench_rgcn_non_composable.py:82-112, argument
+ * list [A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j] (:109).  A: nnz_j edge values,
+ * W: [R, feat_out, feat_in], X: [n, feat_in], Y: [m, feat_out] zero-filled by the caller and
+ * accumulated into with atomics (the schedule's atomic write-back, :89-90), indptr_i: R+1,
+ * indices_i: nnz_i output rows, indptr_j: nnz_i+1, indices_j: nnz_j.
+ */
+int stir_rgms_csf_f32(int32_t m, int32_t n, int32_t num_rels, int32_t feat_in, int32_t feat_out,
+                      int64_t nnz_i, int64_t nnz_j, const float* d_A, const float* d_W,
+                      const float* d_X, float* d_Y, const int32_t* d_indptr_i,
+                      const int32_t* d_indices_i, const int32_t* d_indptr_j,
+                      const int32_t* d_indices_j, void* stream);
+
 /* ----------------------------------------------------------------------- bandwidth probes */
 
 /*

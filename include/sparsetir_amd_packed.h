@@ -95,10 +95,16 @@ enum {
  *      examples/sddmm/bench_sddmm.py:106-115, 170-171
  * "sparsetir.bsrmm"          (A, X, Y, indptr, indices, blk, feat)    A, X f16 or bf16
  *      examples/blocksparse/bsr_spmm.py:427-433
+ * "sparsetir.dbsrmm"         (A, X, Y, indptr_0, indices_0, indptr_1, indices_1, blk, feat)
+ *      examples/blocksparse/bsr_spmm.py:66-102; only the block rows listed in indices_0 are stored
  * "sparsetir.tcspmm"         (A, B, C, indptr, indices, feat, tile_size, group_size)
  *      examples/spmm/bench_tc_spmm.py:650-656
  * "sparsetir.rgms"           (W, X, Y, A_0, rows_0, cols_0, ..., mids_0, ..., feat_in, feat_out)
- *      examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
+ *      examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852         fp16, W [R, feat_in, feat_out]
+ * "sparsetir.rgms_f32"       same argument list, every array fp32, W [R, feat_out, feat_in]
+ *      examples/rgms/rgcn/bench_rgcn_composable.py:208-221
+ * "sparsetir.rgms_csf"       (A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j, feat_in, feat_out)
+ *      examples/rgms/rgcn/bench_rgcn_non_composable.py:109         fp32, W [R, feat_out, feat_in]
  *
  * Format pass (host tensors, kDLCPU; the reference returns nested Array<NDArray>, which needs
  * libtvm objects, so here a sizing call is followed by a fill call into caller-made tensors):
@@ -119,8 +125,11 @@ int stir_packed_hyb_csrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_sddmm_preproc(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_sddmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_bsrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_dbsrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_tcspmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_rgms_f32(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_rgms_csf(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_csf_to_ell3d_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);

@@ -193,3 +193,33 @@ def rgms(W, X, A, indptr0, indices0, indptr1, indices1, m):
     lib().oracle_rgms(R, fin, fout, _p(Wf), _p(Xf), _p(Y), _p(A), _p(indptr0), _p(indices0),
                       _p(indptr1), _p(indices1))
     return Y.reshape(m, fout)
+
+
+def rgms_csf_f32(A, W, X, indptr_i, indices_i, indptr_j, indices_j, m):
+    """W: (R, fout, fin), X: (n, fin), A: (nnz_j,); returns Y (m, fout)."""
+    W, X, A = _f32(W), _f32(X), _f32(A).ravel()
+    R, fout, fin = W.shape
+    indptr_i, indices_i = _i32(indptr_i), _i32(indices_i)
+    indptr_j, indices_j = _i32(indptr_j), _i32(indices_j)
+    Y = np.zeros(m * fout, np.float32)
+    Wf, Xf = W.ravel(), X.ravel()
+    lib().oracle_rgms_csf_f32(R, fin, fout, _p(A), _p(Wf), _p(Xf), _p(Y), _p(indptr_i), _p(indices_i),
+                              _p(indptr_j), _p(indices_j))
+    return Y.reshape(m, fout)
+
+
+def rgms_ell3d_f32(W, X, buckets, m):
+    """``buckets``: list of (A (G, rb, cb) f32, rows (G, rb), cols (G, rb, cb), mids (G,)).
+    W: (R, fout, fin).  Returns Y (m, fout)."""
+    W, X = _f32(W), _f32(X)
+    R, fout, fin = W.shape
+    Y = np.zeros(m * fout, np.float32)
+    Wf, Xf = W.ravel(), X.ravel()
+    for A, rows, cols, mids in buckets:
+        G, rb, cb = cols.shape
+        if G == 0:
+            continue
+        A, rows, cols, mids = _f32(A).ravel(), _i32(rows).ravel(), _i32(cols).ravel(), _i32(mids).ravel()
+        lib().oracle_rgms_ell3d_f32(ctypes.c_int64(G), rb, cb, fin, fout, _p(A), _p(rows), _p(cols), _p(mids),
+                                    _p(Wf), _p(Xf), _p(Y))
+    return Y.reshape(m, fout)

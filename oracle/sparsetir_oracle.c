@@ -17,6 +17,8 @@
  *   oracle_sddmm_mid/_sddmm  tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:510-568
  *   oracle_bsrmm             tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:191-248
  *   oracle_rgms              examples/rgms/rgcn/bench_rgcn_tensorcore.py:564-609
+ *   oracle_rgms_csf_f32      tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:901-993
+ *   oracle_rgms_ell3d_f32    examples/rgms/rgcn/bench_rgcn_composable.py:168-206
  *
  * Pinning status (which independent check fixes each function):
  *   column_part_hyb  known-answer vectors traced by hand from format.cc, the reference
@@ -358,4 +360,42 @@ void oracle_rgms(int num_rels, int fin, int fout, const float* W, const float* X
       }
     }
   free(wx);
+}
+
+/* fp32 RGMS with W[r, fo, fi] on the CSF form, loop nest of the lowered rgcn_hetero_forward
+ * (tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:901-993; the product is
+ * evaluated left to right, A * W * X, :984-991).  The examples schedule the write-back as an
+ * atomic add into a zero-filled Y (examples/rgms/rgcn/bench_rgcn_non_composable.py:89-90,
+ * bench_rgcn_composable.py:196-197), so every relation accumulates. */
+void oracle_rgms_csf_f32(int num_rels, int fin, int fout, const float* A, const float* W, const float* X,
+                         float* Y, const int32_t* indptr_i, const int32_t* indices_i,
+                         const int32_t* indptr_j, const int32_t* indices_j) {
+  for (int fo = 0; fo < fout; ++fo)
+    for (int r = 0; r < num_rels; ++r)
+      for (int i = indptr_i[r]; i < indptr_i[r + 1]; ++i) {
+        float acc = 0.0f;
+        for (int j = indptr_j[i]; j < indptr_j[i + 1]; ++j)
+          for (int fi = 0; fi < fin; ++fi)
+            acc = acc + A[j] * W[((int64_t)r * fout + fo) * fin + fi] * X[(int64_t)indices_j[j] * fin + fi];
+        Y[(int64_t)indices_i[i] * fout + fo] = Y[(int64_t)indices_i[i] * fout + fo] + acc;
+      }
+}
+
+/* The same on one ELL3D bucket (groups x rb x cb, relation mids[g] per group), the decomposed
+ * form of examples/rgms/rgcn/bench_rgcn_composable.py:168-206; accumulates into Y. */
+void oracle_rgms_ell3d_f32(int64_t groups, int rb, int cb, int fin, int fout, const float* A,
+                           const int32_t* rows, const int32_t* cols, const int32_t* mids, const float* W,
+                           const float* X, float* Y) {
+  for (int64_t g = 0; g < groups; ++g)
+    for (int ii = 0; ii < rb; ++ii)
+      for (int fo = 0; fo < fout; ++fo) {
+        float acc = 0.0f;
+        for (int s = 0; s < cb; ++s) {
+          int64_t e = (g * rb + ii) * cb + s;
+          for (int fi = 0; fi < fin; ++fi)
+            acc = acc + A[e] * W[((int64_t)mids[g] * fout + fo) * fin + fi] * X[(int64_t)cols[e] * fin + fi];
+        }
+        int64_t y = (int64_t)rows[g * rb + ii] * fout + fo;
+        Y[y] = Y[y] + acc;
+      }
 }

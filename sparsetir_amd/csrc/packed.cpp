@@ -173,6 +173,8 @@ HybKey g_hyb_key;
 stir_hyb_plan* g_hyb_plan = nullptr;
 HybKey g_rgms_key;
 stir_rgms_plan* g_rgms_plan = nullptr;
+HybKey g_rgms_f32_key;
+stir_rgms_f32_plan* g_rgms_f32_plan = nullptr;
 
 }  // namespace
 
@@ -298,9 +300,12 @@ int stir_packed_sddmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   return sddmm_common("sparsetir.sddmm", false, v, tc, n);
 }
 
-int stir_packed_bsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
-  Args a{"sparsetir.bsrmm", v, tc, n};
-  if (!a.count(7)) return -1;
+// bsrmm (A, X, Y, indptr, indices, blk, feat) and dbsrmm (A, X, Y, indptr_0, indices_0, indptr_1,
+// indices_1, blk, feat) differ in the two leading index arrays of the doubly-compressed form
+static int packed_bsr_any(const char* name, bool doubly, TVMValue* v, int* tc, int n) {
+  Args a{name, v, tc, n};
+  const int x = doubly ? 2 : 0;  // index of the extra arguments
+  if (!a.count(7 + x)) return -1;
   // the 16-bit type is read from A's dtype: float16 (kDLFloat/16) or bfloat16 (kDLBfloat/16)
   const DLTensor* d0 = (tc[0] == kTVMDLTensorHandle || tc[0] == kTVMNDArrayHandle || tc[0] == kTVMOpaqueHandle)
                            ? static_cast<const DLTensor*>(v[0].v_handle) : nullptr;
@@ -313,13 +318,25 @@ int stir_packed_bsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   if (!d2) return packed_fail("%s: Expect arg[2] to be pointer", a.fn);
   const bool out32 = d2->dtype.code == kDLFloat && d2->dtype.bits == 32;
   Arr Y = out32 ? a.arr(2, "Y", kDLFloat, 32, kDevice) : a.arr(2, "Y", code, 16, kDevice);
-  Arr P = a.arr(3, "indptr", kDLInt, 32, kDevice), I = a.arr(4, "indices", kDLInt, 32, kDevice);
-  const int64_t blk = a.integer(5, "blk"), feat = a.integer(6, "feat");
+  Arr P0, I0;
+  if (doubly) {
+    P0 = a.arr(3, "indptr_0", kDLInt, 32, kDevice);
+    I0 = a.arr(4, "indices_0", kDLInt, 32, kDevice);
+  }
+  Arr P = a.arr(3 + x, doubly ? "indptr_1" : "indptr", kDLInt, 32, kDevice),
+      I = a.arr(4 + x, doubly ? "indices_1" : "indices", kDLInt, 32, kDevice);
+  const int64_t blk = a.integer(5 + x, "blk"), feat = a.integer(6 + x, "feat");
   if (!a.ok) return -1;
-  const int64_t mb = P.len - 1, nnzb = I.len;
+  const int64_t mb = P.len - 1, nnzb = I.len;  // stored block rows
   if (mb < 0 || blk <= 0 || feat <= 0) return packed_fail("%s: bad sizes", a.fn);
   a.len(A, "A", nnzb * blk * blk);
-  a.len(Y, "Y", mb * blk * feat);
+  if (doubly) {
+    a.len(P0, "indptr_0", 2);
+    a.len(I0, "indices_0", mb);
+    if (a.ok && Y.len % (blk * feat) != 0) return packed_fail("%s: Y.shape[0] is not a multiple of blk*feat", a.fn);
+  } else {
+    a.len(Y, "Y", mb * blk * feat);
+  }
   if (!a.ok) return -1;
   if (X.len % (blk * feat) != 0) return packed_fail("%s: X.shape[0] is not a multiple of blk*feat", a.fn);
   const int64_t nbk = X.len / (blk * feat);
@@ -327,9 +344,21 @@ int stir_packed_bsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   DeviceGuard g;
   if (g.enter(a.dev_id)) return forward(-1);
   const int dt = bf ? STIR_BF16 : STIR_F16;
+  if (doubly)
+    return forward(stir_dbsr_spmm(dt, out32 ? STIR_F32 : dt, (int32_t)mb, (int32_t)nbk, (int32_t)blk,
+                                  (int32_t)feat, nnzb, A.data, X.data, Y.data, (const int32_t*)I0.data,
+                                  (const int32_t*)P.data, (const int32_t*)I.data, g_stream));
   return forward(stir_bsr_spmm(dt, out32 ? STIR_F32 : dt, (int32_t)mb, (int32_t)nbk, (int32_t)blk, (int32_t)feat,
                                nnzb, A.data, X.data, Y.data, (const int32_t*)P.data, (const int32_t*)I.data,
                                g_stream));
+}
+
+int stir_packed_bsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return packed_bsr_any("sparsetir.bsrmm", false, v, tc, n);
+}
+
+int stir_packed_dbsrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return packed_bsr_any("sparsetir.dbsrmm", true, v, tc, n);
 }
 
 int stir_packed_tcspmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
@@ -360,11 +389,13 @@ int stir_packed_tcspmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
                                   g_stream));
 }
 
-int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
-  Args a{"sparsetir.rgms", v, tc, n};
+// fp16 (W [R, fin, fout]) and fp32 (W [R, fout, fin]) forms share the argument list
+static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int n) {
+  Args a{name, v, tc, n};
+  const int bits = f32 ? 32 : 16;
   if (n < 5 || (n - 5) % 4 != 0) return packed_fail("%s: num_args should be 3 + 4*buckets + 2", a.fn);
   const int nb = (n - 5) / 4;
-  Arr W = a.arr(0, "W", kDLFloat, 16, kDevice), X = a.arr(1, "X", kDLFloat, 16, kDevice),
+  Arr W = a.arr(0, "W", kDLFloat, bits, kDevice), X = a.arr(1, "X", kDLFloat, bits, kDevice),
       Y = a.arr(2, "Y", kDLFloat, 32, kDevice);
   const int64_t fin = a.integer(n - 2, "feat_in"), fout = a.integer(n - 1, "feat_out");
   if (!a.ok) return -1;
@@ -375,7 +406,7 @@ int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   std::vector<int64_t> groups(nb);
   std::vector<int32_t> rb(nb, 1), cb(nb, 1);
   for (int b = 0; b < nb; ++b) {
-    Arr Aa = a.arr(3 + 3 * b, "A_k", kDLFloat, 16, kDevice), Rr = a.arr(4 + 3 * b, "rows_k", kDLInt, 32, kDevice),
+    Arr Aa = a.arr(3 + 3 * b, "A_k", kDLFloat, bits, kDevice), Rr = a.arr(4 + 3 * b, "rows_k", kDLInt, 32, kDevice),
         Cc = a.arr(5 + 3 * b, "cols_k", kDLInt, 32, kDevice), Mm = a.arr(3 + 3 * nb + b, "mids_k", kDLInt, 32, kDevice);
     if (!a.ok) return -1;
     a.len(Cc, "cols_k", Aa.len);
@@ -408,6 +439,21 @@ int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   }
   key.nums.push_back(a.dev_id);
   std::lock_guard<std::mutex> lock(g_plan_mutex);
+  const int32_t mm = (int32_t)(Y.len / fout), nn = (int32_t)(X.len / fin), rr = (int32_t)(W.len / (fin * fout));
+  if (f32) {
+    if (!g_rgms_f32_plan || !(key == g_rgms_f32_key)) {
+      if (g_rgms_f32_plan) stir_rgms_f32_plan_destroy(g_rgms_f32_plan);
+      g_rgms_f32_plan = nullptr;
+      std::vector<const float*> Af(nb);
+      for (int b = 0; b < nb; ++b) Af[b] = (const float*)Ak[b];
+      if (stir_rgms_f32_plan_create(&g_rgms_f32_plan, nb, rb.data(), cb.data(), groups.data(), Af.data(),
+                                    Rk.data(), Ck.data(), Mk.data()))
+        return forward(-1);
+      g_rgms_f32_key = key;
+    }
+    return forward(stir_rgms_f32(g_rgms_f32_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, (const float*)W.data,
+                                 (const float*)X.data, (float*)Y.data, g_stream));
+  }
   if (!g_rgms_plan || !(key == g_rgms_key)) {
     if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
     g_rgms_plan = nullptr;
@@ -416,9 +462,42 @@ int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
       return forward(-1);
     g_rgms_key = key;
   }
-  return forward(stir_rgms_f16(g_rgms_plan, (int32_t)(Y.len / fout), (int32_t)(X.len / fin),
-                               (int32_t)(W.len / (fin * fout)), (int32_t)fin, (int32_t)fout, W.data, X.data,
+  return forward(stir_rgms_f16(g_rgms_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data, X.data,
                                (float*)Y.data, g_stream));
+}
+
+int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return packed_rgms_any("sparsetir.rgms", false, v, tc, n);
+}
+
+int stir_packed_rgms_f32(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  return packed_rgms_any("sparsetir.rgms_f32", true, v, tc, n);
+}
+
+int stir_packed_rgms_csf(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.rgms_csf", v, tc, n};
+  if (!a.count(10)) return -1;
+  Arr A = a.arr(0, "A", kDLFloat, 32, kDevice), W = a.arr(1, "W", kDLFloat, 32, kDevice),
+      X = a.arr(2, "X", kDLFloat, 32, kDevice), Y = a.arr(3, "Y", kDLFloat, 32, kDevice),
+      Pi = a.arr(4, "indptr_i", kDLInt, 32, kDevice), Ii = a.arr(5, "indices_i", kDLInt, 32, kDevice),
+      Pj = a.arr(6, "indptr_j", kDLInt, 32, kDevice), Ij = a.arr(7, "indices_j", kDLInt, 32, kDevice);
+  const int64_t fin = a.integer(8, "feat_in"), fout = a.integer(9, "feat_out");
+  if (!a.ok) return -1;
+  if (fin <= 0 || fout <= 0 || W.len % (fin * fout) != 0 || X.len % fin != 0 || Y.len % fout != 0)
+    return packed_fail("%s: W/X/Y lengths do not fit feat_in=%lld feat_out=%lld", a.fn, (long long)fin, (long long)fout);
+  const int64_t R = W.len / (fin * fout);
+  a.len(Pi, "indptr_i", R + 1);
+  a.len(Pj, "indptr_j", Ii.len + 1);
+  a.len(Ij, "indices_j", A.len);
+  if (!a.ok) return -1;
+  if (!fits_i32(Y.len / fout) || !fits_i32(X.len / fin) || !fits_i32(R)) return packed_fail("%s: sizes exceed int32", a.fn);
+  DeviceGuard g;
+  if (g.enter(a.dev_id)) return forward(-1);
+  return forward(stir_rgms_csf_f32((int32_t)(Y.len / fout), (int32_t)(X.len / fin), (int32_t)R, (int32_t)fin,
+                                   (int32_t)fout, Ii.len, A.len, (const float*)A.data, (const float*)W.data,
+                                   (const float*)X.data, (float*)Y.data, (const int32_t*)Pi.data,
+                                   (const int32_t*)Ii.data, (const int32_t*)Pj.data, (const int32_t*)Ij.data,
+                                   g_stream));
 }
 
 // ----------------------------------------------------------------------------- format pass
@@ -583,8 +662,11 @@ static const PackedEntry kTable[] = {
     {"sparsetir.sddmm_preproc", stir_packed_sddmm_preproc},
     {"sparsetir.sddmm", stir_packed_sddmm},
     {"sparsetir.bsrmm", stir_packed_bsrmm},
+    {"sparsetir.dbsrmm", stir_packed_dbsrmm},
     {"sparsetir.tcspmm", stir_packed_tcspmm},
     {"sparsetir.rgms", stir_packed_rgms},
+    {"sparsetir.rgms_f32", stir_packed_rgms_f32},
+    {"sparsetir.rgms_csf", stir_packed_rgms_csf},
     {"tir.sparse.ColumnPartHyb.sizes", stir_packed_column_part_hyb_sizes},
     {"tir.sparse.ColumnPartHyb.fill", stir_packed_column_part_hyb_fill},
     {"tir.sparse.CSFToELL3D.sizes", stir_packed_csf_to_ell3d_sizes},

@@ -14,6 +14,9 @@ hand-written gfx950 kernel through the C ABI on torch's current stream:
   build_tcspmm        f(A, B, C, indptr, indices)             examples/spmm/bench_tc_spmm.py:650-656
   build_rgms          f(W, X, Y, (A_k, rows_k, cols_k)..., mids_k...)
                                                                examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852
+  build_rgms_f32      same arguments in fp32, W [R, Fout, Fin]  examples/rgms/rgcn/bench_rgcn_composable.py:208-221
+  build_rgms_csf      f(A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j)
+                                                               examples/rgms/rgcn/bench_rgcn_non_composable.py:109
 
 Arrays are torch CUDA tensors (device memory and streams only).  Arguments are checked the
 way the reference's generated host stub checks DLTensors (src/tir/transforms/arg_binder.cc:152+):
@@ -285,6 +288,9 @@ class Rgms(_Operator):
     ``cols_bkt`` the ELL rows per group and slots per ELL row."""
     name = "rgms"
 
+    _in_dtype = torch.float16
+    _fns = ("stir_rgms_plan_create", "stir_rgms_f16", "stir_rgms_plan_destroy")
+
     def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
         self.m, self.n, self.R = int(m), int(n), int(num_rels)
         self.fin, self.fout = int(feat_in), int(feat_out)
@@ -296,7 +302,7 @@ class Rgms(_Operator):
         self._keep = None
 
     def _spec(self):
-        f16, f32, i32 = torch.float16, torch.float32, torch.int32
+        f16, f32, i32 = self._in_dtype, torch.float32, torch.int32
         spec = [("W", f16, self.R * self.fin * self.fout), ("X", f16, self.n * self.fin),
                 ("Y", f32, self.m * self.fout)]
         for k, g in enumerate(self.groups):
@@ -308,7 +314,7 @@ class Rgms(_Operator):
 
     def _drop_plan(self):
         if self._plan is not None:
-            self.L.stir_rgms_plan_destroy(self._plan)
+            getattr(self.L, self._fns[2])(self._plan)
             self._plan = None
 
     def __del__(self):
@@ -331,12 +337,43 @@ class Rgms(_Operator):
                 cb = (ctypes.c_int32 * nb)(*self.cb)
                 groups = (ctypes.c_int64 * nb)(*self.groups)
                 tab = lambda ts: _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in ts])
-                _lib.check(self.L.stir_rgms_plan_create(ctypes.byref(plan), nb, rb, cb, groups,
-                                                        tab(triples[0::3]), tab(triples[1::3]),
-                                                        tab(triples[2::3]), tab(mids)))
+                _lib.check(getattr(self.L, self._fns[0])(ctypes.byref(plan), nb, rb, cb, groups,
+                                                         tab(triples[0::3]), tab(triples[1::3]),
+                                                         tab(triples[2::3]), tab(mids)))
                 self._plan, self._key, self._keep = plan, key, rest
-            _lib.check(self.L.stir_rgms_f16(self._plan, self.m, self.n, self.R, self.fin, self.fout,
-                                            _ptr(w), _ptr(x), _ptr(y), _stream()))
+            _lib.check(getattr(self.L, self._fns[1])(self._plan, self.m, self.n, self.R, self.fin, self.fout,
+                                                     _ptr(w), _ptr(x), _ptr(y), _stream()))
+
+
+class RgmsF32(Rgms):
+    """fp32 RGMS on ELL3D buckets with W laid out [R, feat_out, feat_in]: the composable operator of
+    examples/rgms/rgcn/bench_rgcn_composable.py:208-221, same argument order as :class:`Rgms`."""
+    name = "rgms_f32"
+    _in_dtype = torch.float32
+    _fns = ("stir_rgms_f32_plan_create", "stir_rgms_f32", "stir_rgms_f32_plan_destroy")
+
+
+class RgmsCsf(_Operator):
+    """fp32 RGMS over the CSF arrays: f(A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j), the
+    non-composable operator of examples/rgms/rgcn/bench_rgcn_non_composable.py:82-112."""
+    name = "rgms_csf"
+
+    def __init__(self, m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j):
+        self.m, self.n, self.R = int(m), int(n), int(num_rels)
+        self.fin, self.fout, self.nnz_i, self.nnz_j = int(feat_in), int(feat_out), int(nnz_i), int(nnz_j)
+        self.L = _lib.lib()
+
+    def __call__(self, *args):
+        f32, i32 = torch.float32, torch.int32
+        dev = self._check(args, [("A", f32, self.nnz_j), ("W", f32, self.R * self.fout * self.fin),
+                                 ("X", f32, self.n * self.fin), ("Y", f32, self.m * self.fout),
+                                 ("indptr_i", i32, self.R + 1), ("indices_i", i32, self.nnz_i),
+                                 ("indptr_j", i32, self.nnz_i + 1), ("indices_j", i32, self.nnz_j)])
+        a, w, x, y, pi, ii, pj, ij = args
+        with torch.cuda.device(dev):
+            _lib.check(self.L.stir_rgms_csf_f32(self.m, self.n, self.R, self.fin, self.fout, self.nnz_i,
+                                                self.nnz_j, _ptr(a), _ptr(w), _ptr(x), _ptr(y), _ptr(pi),
+                                                _ptr(ii), _ptr(pj), _ptr(ij), _stream()))
 
 
 def build_csrmm(m, n, feat, nnz):
@@ -373,3 +410,11 @@ def build_tcspmm(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=to
 
 def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
     return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups)
+
+
+def build_rgms_f32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
+    return RgmsF32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups)
+
+
+def build_rgms_csf(m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j):
+    return RgmsCsf(m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j)

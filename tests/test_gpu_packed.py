@@ -107,3 +107,58 @@ def test_packed_bsrmm_and_rgms_match_operator_objects(dev):
     packed.get_global_func("sparsetir.rgms")(w, xx, yb, *triples, *mids, fin, fout)
     torch.cuda.synchronize()
     assert torch.allclose(ya, yb, rtol=1e-5, atol=1e-5) and ya.abs().sum() > 0
+
+
+def test_packed_dbsrmm_tcspmm_and_fp32_rgms_match_operator_objects(dev):
+    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    # doubly-compressed BSR
+    cfg = datasets.config4(seed=5, mb=10, nb=6, blk=32, density=0.2, feat=64)
+    counts = np.diff(cfg["indptr"])
+    keep = np.nonzero(counts > 0)[0].astype(np.int32)
+    ptr1 = np.concatenate([[0], np.cumsum(counts[keep])]).astype(np.int32)
+    a = t(cfg["data"]).half().reshape(-1)
+    x = t(cfg["x"]).half().reshape(-1)
+    idx_args = (t(np.asarray([0, len(keep)], np.int32)), t(keep), t(ptr1), t(cfg["indices"]))
+    y1 = torch.zeros(10 * 32 * 64, dtype=torch.float32, device=dev)
+    y2 = torch.zeros_like(y1)
+    ops.build_dbsrmm(10, 6, len(keep), len(cfg["indices"]), 32, 64, torch.float16, torch.float32)(a, x, y1, *idx_args)
+    packed.get_global_func("sparsetir.dbsrmm")(a, x, y2, *idx_args, 32, 64)
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2) and y1.abs().sum() > 0
+
+    # SpMM over the condensed format
+    m, n, feat = 300, 260, 64
+    indptr, indices = random_csr(m, n, 5000, 9, skew=1.0)
+    gptr, tiles, mask = st.condense(indptr, indices, 32, 16)
+    mb = len(gptr) - 1
+    rng = np.random.default_rng(9)
+    am, xm = t(mask.astype(np.float16).ravel()), t(rng.standard_normal(n * feat).astype(np.float16))
+    c1 = torch.zeros(mb * 32 * feat, dtype=torch.float16, device=dev)
+    c2 = torch.zeros_like(c1)
+    ops.build_tcspmm(mb, tiles.shape[0], feat, 32, 16, n)(am, xm, c1, t(gptr), t(tiles.ravel()))
+    packed.get_global_func("sparsetir.tcspmm")(am, xm, c2, t(gptr), t(tiles.ravel()), feat, 32, 16)
+    torch.cuda.synchronize()
+    assert torch.equal(c1, c2) and c1.float().abs().sum() > 0
+
+    # fp32 RGMS, both forms
+    R, n, fin, fout, group, buckets = 4, 200, 16, 24, 32, [1, 2, 4, 8]
+    csf = random_csf(R, n, 800, seed=6)
+    rb = [group // b for b in buckets]
+    iptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    w = t(rng.standard_normal(R * fout * fin).astype(np.float32))
+    xx = t(rng.standard_normal(n * fin).astype(np.float32))
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float32).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(iptr[k]))))
+    ya, yb, yc = (torch.zeros(n * fout, device=dev) for _ in range(3))
+    ops.build_rgms_f32(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols])(w, xx, ya, *triples, *mids)
+    packed.get_global_func("sparsetir.rgms_f32")(w, xx, yb, *triples, *mids, fin, fout)
+    ones = torch.ones(len(csf[3]), device=dev)
+    packed.get_global_func("sparsetir.rgms_csf")(ones, w, xx, yc, *[t(c) for c in csf], fin, fout)
+    torch.cuda.synchronize()
+    assert torch.allclose(ya, yb, rtol=1e-5, atol=1e-5) and ya.abs().sum() > 0
+    assert torch.allclose(ya, yc, rtol=1e-4, atol=1e-4)
+    with pytest.raises(SparseTIRError, match="indptr_j"):
+        packed.get_global_func("sparsetir.rgms_csf")(ones, w, xx, yc, t(csf[0]), t(csf[1]), t(csf[2][:-1]), t(csf[3]),
+                                                     fin, fout)

@@ -1,0 +1,140 @@
+"""GPU parity of the fp32 RGMS kernels (ELL3D buckets and CSF traversal, W[r, fo, fi]) against
+the oracle and the float64 closed form.  Tolerance: rtol 1e-5 on the result plus 1e-5 of the sum
+of term magnitudes (the kernel sums a row's X rows before multiplying by W, and adds rows into Y
+with atomics, so the order of the fp32 additions differs from the oracle's)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import sparsetir_amd as st
+from sparsetir_amd import datasets, ops
+from helpers import random_csf, rgms_f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(dev, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _check(got, want64, scale64, ref, what):
+    err = np.abs(got - want64)
+    assert np.all(err <= 1e-5 * np.abs(want64) + 1e-5 * scale64 + 1e-30), f"{what}: worst {err.max():.3e}"
+    assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(ref) + 2e-5 * scale64 + 1e-30), f"{what}: vs oracle"
+
+
+def _closed_forms(csf, a, x, w, m):
+    wt = np.ascontiguousarray(w.transpose(0, 2, 1))
+    return rgms_f64(*csf, a, x, wt, m), rgms_f64(*csf, np.abs(a), np.abs(x), np.abs(wt), m)
+
+
+@pytest.mark.parametrize("fin,fout", [(32, 32), (8, 12), (4, 4), (20, 40), (64, 96), (128, 32), (16, 70)])
+def test_rgms_csf_f32(dev, fin, fout):
+    R, n = 6, 300
+    csf = random_csf(R, n, 1500, seed=fin + fout)
+    rng = np.random.default_rng(fin)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
+    a = (0.5 + rng.random(len(csf[3]), dtype=np.float32))
+    a[::7] = 0.0  # zero-weight edges are skipped by the kernel
+    f = ops.build_rgms_csf(n, n, R, fin, fout, len(csf[1]), len(csf[3]))
+    y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
+    f(_t(dev, a), _t(dev, w.ravel()), _t(dev, x.ravel()), y, *[_t(dev, c) for c in csf])
+    torch.cuda.synchronize()
+    want, scale = _closed_forms(csf, a, x, w, n)
+    _check(y.cpu().numpy().reshape(n, fout), want, scale, oracle.rgms_csf_f32(a, w, x, *csf, n), f"csf {fin}x{fout}")
+
+
+def test_rgms_csf_f32_long_row_and_empty_relations(dev):
+    """One stored row with thousands of edges (several 64-edge passes of one tile), relations
+    without rows, a single stored row in the last relation."""
+    n, fin, fout, R = 5000, 32, 32, 5
+    rng = np.random.default_rng(3)
+    long_cols = np.sort(rng.choice(n, 3000, replace=False)).astype(np.int32)
+    p0 = np.asarray([0, 0, 3, 3, 3, 4], np.int32)
+    i0 = np.asarray([7, 9, 4000, 9], np.int32)
+    p1 = np.asarray([0, 2, 3002, 3003, 3005], np.int32)
+    i1 = np.concatenate([[1, 2], long_cols, [0], [4999, 17]]).astype(np.int32)
+    csf = (p0, i0, p1, i1)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
+    a = rng.standard_normal(len(i1)).astype(np.float32)
+    f = ops.build_rgms_csf(n, n, R, fin, fout, len(i0), len(i1))
+    y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
+    f(_t(dev, a), _t(dev, w.ravel()), _t(dev, x.ravel()), y, *[_t(dev, c) for c in csf])
+    torch.cuda.synchronize()
+    want, scale = _closed_forms(csf, a, x, w, n)
+    _check(y.cpu().numpy().reshape(n, fout), want, scale, oracle.rgms_csf_f32(a, w, x, *csf, n), "long row")
+
+
+def test_rgms_csf_f32_empty(dev):
+    f = ops.build_rgms_csf(10, 10, 3, 8, 8, 0, 0)
+    z = lambda dt, k=0: torch.zeros(k, dtype=dt, device=dev)
+    y = torch.full((80,), 3.0, dtype=torch.float32, device=dev)
+    f(z(torch.float32), z(torch.float32, 3 * 64), z(torch.float32, 80), y, z(torch.int32, 4), z(torch.int32),
+      z(torch.int32, 1), z(torch.int32))
+    torch.cuda.synchronize()
+    assert torch.all(y == 3.0)
+
+
+def _run_ell3d(dev, csf, n, x, w, group, buckets, weighted, seed=0):
+    R, fout, fin = w.shape
+    rows_bkt = [max(1, group // b) for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    rng = np.random.default_rng(seed)
+    triples, mids, bk = [], [], []
+    for b in range(len(buckets)):
+        a = mask[b].astype(np.float32)
+        if weighted:
+            a = a * (0.5 + rng.random(a.shape, dtype=np.float32))
+        mid = np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))
+        bk.append((a, rows[b], cols[b], mid))
+        triples += [_t(dev, a.ravel()), _t(dev, rows[b].ravel()), _t(dev, cols[b].ravel())]
+        mids.append(_t(dev, mid))
+    f = ops.build_rgms_f32(n, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols])
+    y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
+    f(_t(dev, w.ravel()), _t(dev, x.ravel()), y, *triples, *mids)
+    torch.cuda.synchronize()
+    return y.cpu().numpy().reshape(n, fout), bk
+
+
+@pytest.mark.parametrize("group,buckets,fin,fout,weighted", [
+    (32, [1, 2, 4, 8, 16], 32, 32, False),     # the reference's composable configuration
+    (256, [1, 2, 4, 8, 16], 32, 32, True),     # rb > 32: several tiles per group
+    (16, [1, 2, 4], 16, 40, True),
+    (12, [1, 3, 6], 48, 32, True),             # rb does not divide 32, cb not a power of two
+    (64, [2, 64], 64, 96, False),
+    (8, [1, 2], 4, 4, True),
+])
+def test_rgms_ell3d_f32(dev, group, buckets, fin, fout, weighted):
+    R, n = 5, 300
+    csf = random_csf(R, n, 900, seed=group)
+    rng = np.random.default_rng(group)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
+    got, bk = _run_ell3d(dev, csf, n, x, w, group, buckets, weighted)
+    ref = oracle.rgms_ell3d_f32(w, x, bk, n)
+    if not weighted:
+        ones = np.ones(len(csf[3]), np.float32)
+        want, scale = _closed_forms(csf, ones, x, w, n)
+        _check(got, want, scale, ref, f"ell3d group={group}")
+    else:
+        scale = oracle.rgms_ell3d_f32(np.abs(w), np.abs(x), [(np.abs(a), r, c, m) for a, r, c, m in bk], n)
+        assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(ref) + 2e-5 * scale + 1e-30)
+
+
+def test_rgms_f32_config5_reduced_both_forms_agree(dev):
+    cfg = datasets.config5(n=4000, num_rels=65, num_edges=40000)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    n = cfg["n"]
+    w = np.ascontiguousarray(cfg["w"].transpose(0, 2, 1))
+    got, bk = _run_ell3d(dev, csf, n, cfg["x"], w, 32, cfg["buckets"], False)
+    ones = np.ones(len(csf[3]), np.float32)
+    want, scale = _closed_forms(csf, ones, cfg["x"], w, n)
+    _check(got, want, scale, oracle.rgms_ell3d_f32(w, cfg["x"], bk, n), "config5 ell3d")
+    f = ops.build_rgms_csf(n, n, 65, 32, 32, len(csf[1]), len(csf[3]))
+    y = torch.zeros(n * 32, dtype=torch.float32, device=dev)
+    f(_t(dev, ones), _t(dev, w.ravel()), _t(dev, cfg["x"].ravel()), y, *[_t(dev, c) for c in csf])
+    torch.cuda.synchronize()
+    _check(y.cpu().numpy().reshape(n, 32), want, scale, oracle.rgms_csf_f32(ones, w, cfg["x"], *csf, n), "config5 csf")

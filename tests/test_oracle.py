@@ -272,3 +272,26 @@ def test_rgms_matches_float64():
     got = oracle.rgms(w, x, a, p0, i0, p1, i1, n)
     want = rgms_f64(p0, i0, p1, i1, a, x, w, n)
     assert_close(got, want, rtol=1e-5, atol=1e-4, what="rgms oracle")
+
+
+def test_rgms_fp32_forms_match_float64():
+    """fp32 RGMS with W[r, fo, fi] (feat_in != feat_out, so a transposed W fails), on the CSF
+    arrays and on the ELL3D buckets made from them; both against the float64 closed form."""
+    rels, n, fin, fout = 4, 40, 8, 12
+    p0, i0, p1, i1 = random_csf(rels, n, 400, 5)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((rels, fout, fin), dtype=np.float32)
+    a = rng.random(len(i1), dtype=np.float32)
+    want = rgms_f64(p0, i0, p1, i1, a, x, np.ascontiguousarray(w.transpose(0, 2, 1)), n)
+    got = oracle.rgms_csf_f32(a, w, x, p0, i0, p1, i1, n)
+    assert_close(got, want, rtol=1e-5, atol=1e-4, what="rgms csf fp32 oracle")
+    # ELL3D form with the 0/1 mask as weights == CSF form with unit weights
+    ones = np.ones(len(i1), np.float32)
+    want1 = rgms_f64(p0, i0, p1, i1, ones, x, np.ascontiguousarray(w.transpose(0, 2, 1)), n)
+    rows_bkt, cols_bkt = [4, 2, 1], [1, 2, 4]
+    ptr, rows, cols, mask = oracle.csf_to_ell3d(p0, i0, p1, i1, rows_bkt, cols_bkt)
+    bk = [(mask[b].astype(np.float32), rows[b], cols[b],
+           np.repeat(np.arange(rels, dtype=np.int32), np.diff(ptr[b]))) for b in range(3)]
+    got1 = oracle.rgms_ell3d_f32(w, x, bk, n)
+    assert_close(got1, want1, rtol=1e-5, atol=1e-4, what="rgms ell3d fp32 oracle")
