@@ -8,11 +8,13 @@
 // (p, beta).  Entry number t of the run lands at flat slot base * width + t; the slots from d
 // to rho * width are padding (col 0, mask 0); each of the rho ELL rows carries row id i.
 //
-// Passes: (0) validate (columns in range, ascending inside rows); (1) per (row, partition)
-// binary-search lo and build a per-wavefront histogram of rho per bucket; (2) exclusive scan of
-// the histograms along the rows for every (partition, bucket), which also yields the ELL row
-// counts; (3) per (row, partition) compute base from the scanned histogram plus the rank inside
-// the wavefront, write row ids and padding; (4) per nonzero, scatter the column id and mask.
+// Passes: (0) validate (columns in range; descents between neighbouring entries are counted and
+// compared with the descents found at row starts by pass 1, so rows ascend iff the counts agree);
+// (1) per (row, partition) binary-search lo and build a per-wavefront histogram of rho per
+// bucket; (2) exclusive scan of the histograms along the rows for every (partition, bucket),
+// which also yields the ELL row counts; (3) per (row, partition) compute base from the scanned
+// histogram plus the rank inside the wavefront, write row ids and padding; (4) scatter the
+// column ids and the mask, eight consecutive nonzeros per thread.
 #include <cstring>
 #include <vector>
 
@@ -26,15 +28,27 @@ using stir::kWave;
 struct Workspace {
   int32_t* lo;       // [P][m]   start of the (row, partition) run inside indices
   int32_t* base;     // [P][m]   first ELL row of the run inside its bucket
-  int32_t* hist;     // [P][W][NB] per-wavefront ELL-row counts, scanned in place
+  int32_t* hist;     // [P][NB][W] per-wavefront ELL-row counts, scanned in place
   int64_t* totals;   // [P][NB]
   int32_t* widths;   // [NB]
-  int32_t* status;   // [1] nonzero: input rejected
+  int32_t* coarse;   // [kCoarse] row that owns nonzero first + q * stride, stride = coarse_stride(nnz)
+  int32_t* status;   // [1 + 2 * kCountSlots] status bits; descents between neighbours; descents at row starts
   int32_t** rows_tab;  // [P*NB] output pointers
   int32_t** cols_tab;
   int32_t** mask_tab;
   size_t bytes;
 };
+
+// The two descent counts are kept as kCountSlots partial sums each (a workgroup adds to the slot
+// of its index), since atomics on a single address serialise; the host adds the slots up.
+constexpr int kCountSlots = 1024;
+constexpr int kStatusInts = 1 + 2 * kCountSlots;
+
+// Row lookup for the per-nonzero passes: the row of every stride-th nonzero is recorded while the
+// rows are counted, so a thread finds the row of its first nonzero with a binary search over the
+// few rows between two recorded ones instead of over all of indptr.
+constexpr int kCoarse = 65536;
+inline int64_t coarse_stride(int64_t nnz) { return nnz > kCoarse ? (nnz + kCoarse - 1) / kCoarse : 1; }
 
 size_t align_up(size_t x) { return (x + 255) & ~size_t(255); }
 
@@ -53,7 +67,8 @@ Workspace carve(void* p, int32_t m, int32_t P, int32_t NB) {
   w.hist = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(W > 0 ? W : 1) * NB));
   w.totals = reinterpret_cast<int64_t*>(take(sizeof(int64_t) * size_t(P) * NB));
   w.widths = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * NB));
-  w.status = reinterpret_cast<int32_t*>(take(sizeof(int32_t)));
+  w.coarse = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kCoarse));
+  w.status = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kStatusInts));
   w.rows_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * size_t(P) * NB));
   w.cols_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * size_t(P) * NB));
   w.mask_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * size_t(P) * NB));
@@ -61,7 +76,7 @@ Workspace carve(void* p, int32_t m, int32_t P, int32_t NB) {
   return w;
 }
 
-enum { kStatusRange = 1, kStatusUnsorted = 2 };
+enum { kStatusRange = 1, kStatusUnsorted = 2, kStatusIndptr = 4 };
 
 __device__ __forceinline__ int lower_bound_dev(const int32_t* a, int lo, int hi, int64_t key) {
   while (lo < hi) {
@@ -77,86 +92,172 @@ __device__ __forceinline__ int bucket_of_dev(const int32_t* widths, int nb, int 
   return k;
 }
 
-// (0) every column inside [0, num_cols); columns ascend inside each row
-__global__ __launch_bounds__(256) void validate_kernel(int m, int num_cols, int64_t nnz, int32_t first,
-                                                       const int32_t* __restrict__ indptr,
+// (0) every column inside [0, num_cols); counts the positions e whose successor holds a smaller
+// column.  Such a descent is legal only where e + 1 opens a row; count_kernel counts those, and the
+// rows ascend exactly when the two counts agree.  A thread checks kValidatePerThread consecutive
+// entries (vector loads when aligned) and the step to its neighbour's first entry.
+constexpr int kValidatePerThread = 16;
+__global__ __launch_bounds__(256) void validate_kernel(int num_cols, int64_t nnz, int32_t first,
                                                        const int32_t* __restrict__ indices,
                                                        int32_t* __restrict__ status) {
-  const int64_t e = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= first + nnz) return;
-  const int col = indices[e];
-  if (col < 0 || col >= num_cols) {
-    atomicOr(status, kStatusRange);
-    return;
+  constexpr int N = kValidatePerThread;
+  const int64_t end = first + nnz;
+  const int64_t e0 = first + ((int64_t)blockIdx.x * 256 + threadIdx.x) * N;
+  int v[N + 1];
+  const bool full = e0 + N <= end;
+  if (full && (reinterpret_cast<uintptr_t>(indices + e0) & 15) == 0) {
+#pragma unroll
+    for (int j = 0; j < N; j += 4) {
+      const int4 c = *reinterpret_cast<const int4*>(indices + e0 + j);
+      v[j] = c.x, v[j + 1] = c.y, v[j + 2] = c.z, v[j + 3] = c.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) v[j] = e0 + j < end ? indices[e0 + j] : 0;
   }
-  if (e + 1 < first + nnz && indices[e + 1] < col) {
-    // legal only when e+1 opens a row: some indptr entry equals e+1
-    const int r = lower_bound_dev(indptr, 0, m + 1, e + 1);
-    if (r > m || (int64_t)indptr[r] != e + 1) atomicOr(status, kStatusUnsorted);
+  // successor of the last entry: the next lane's first one; the wavefront's last lane reads it
+  v[N] = __shfl_down(v[0], 1, kWave);
+  if ((threadIdx.x & 63) == 63 && e0 + N < end) v[N] = indices[e0 + N];
+  int descents = 0;
+  bool bad = false;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    if (e0 + j < end) {
+      bad |= v[j] < 0 || v[j] >= num_cols;
+      if (e0 + j + 1 < end && v[j + 1] < v[j]) ++descents;
+    }
   }
+  __shared__ int block_descents;
+  if (threadIdx.x == 0) block_descents = 0;
+  __syncthreads();
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) descents += __shfl_xor(descents, off, kWave);
+  if ((threadIdx.x & 63) == 0 && descents) atomicAdd(&block_descents, descents);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_descents) atomicAdd(status + 1 + (blockIdx.x % kCountSlots), block_descents);
+  if (bad) atomicOr(status, kStatusRange);
 }
 
 // (1) lo per (row, partition) and per-wavefront histogram.  grid (ceil(m/256), P).
-__global__ __launch_bounds__(256) void count_kernel(int m, int psize, int NB, int64_t W,
+__global__ __launch_bounds__(256) void count_kernel(int m, int psize, int NB, int64_t W, int first, int64_t end,
+                                                    int64_t stride, int32_t* __restrict__ coarse,
                                                     const int32_t* __restrict__ indptr,
                                                     const int32_t* __restrict__ indices,
                                                     const int32_t* __restrict__ widths,
-                                                    int32_t* __restrict__ lo_out, int32_t* __restrict__ hist) {
+                                                    int32_t* __restrict__ lo_out, int32_t* __restrict__ hist,
+                                                    int32_t* __restrict__ status) {
   const int p = blockIdx.y;
   const int P = gridDim.y;
   const int i = blockIdx.x * 256 + threadIdx.x;
   const int lane = threadIdx.x & 63;
   const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   int d = 0;
+  bool boundary_descent = false;
   if (i < m) {
-    const int rs = indptr[i], re = indptr[i + 1];
+    int rs = indptr[i], re = indptr[i + 1];
+    if (re < rs || rs < first || re > end) {
+      if (p == 0) atomicOr(status, kStatusIndptr);
+      rs = re = first;
+    }
+    // a non-empty row that is not the last: does the next stored entry hold a smaller column?
+    if (p == 0 && re > rs && re < end) boundary_descent = indices[re] < indices[re - 1];
+    if (p == 0)
+      for (int64_t q = (rs - first + stride - 1) / stride; first + q * stride < re; ++q) coarse[q] = i;
     const int lo = p == 0 ? rs : lower_bound_dev(indices, rs, re, (int64_t)p * psize);
     const int hi = p == P - 1 ? re : lower_bound_dev(indices, lo, re, (int64_t)(p + 1) * psize);
     lo_out[(int64_t)p * m + i] = lo;
     d = hi - lo;
   }
   if (wave >= W) return;
+  if (p == 0) {
+    const unsigned long long bd = __ballot(boundary_descent);
+    if (lane == 0 && bd) atomicAdd(status + 1 + kCountSlots + (wave % kCountSlots), __popcll(bd));
+  }
   const int beta = bucket_of_dev(widths, NB, d);
   const int w = widths[beta];
   const int rho = d == 0 ? 0 : (d + w - 1) / w;
-  int32_t* h = hist + ((int64_t)p * W + wave) * NB;
+  int32_t* h = hist + (int64_t)p * NB * W + wave;  // [b][W]
   for (int b = 0; b < NB - 1; ++b) {
     const unsigned long long bal = __ballot(d > 0 && beta == b);
-    if (lane == 0) h[b] = __popcll(bal);
+    if (lane == 0) h[b * W] = __popcll(bal);
   }
   int tot = beta == NB - 1 ? rho : 0;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) tot += __shfl_xor(tot, off, kWave);
-  if (lane == 0) h[NB - 1] = tot;
+  if (lane == 0) h[(NB - 1) * W] = tot;
 }
 
-// (2) exclusive scan of hist[p][.][b] along the wavefront axis.  grid (NB, P), 256 threads.
-__global__ __launch_bounds__(256) void scan_kernel(int NB, int64_t W, int32_t* __restrict__ hist,
-                                                   int64_t* __restrict__ totals) {
-  __shared__ int64_t part[256];
+// (2) exclusive scan of hist[p][b][.] along the wavefront axis.  grid (NB, P), 1024 threads, each
+// owning one contiguous chunk.
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void scan_kernel(int NB, int64_t W, int32_t* __restrict__ hist,
+                                                            int64_t* __restrict__ totals) {
+  __shared__ int64_t part[kScanThreads];
   const int b = blockIdx.x, p = blockIdx.y;
-  int32_t* h = hist + (int64_t)p * W * NB + b;
-  const int64_t chunk = (W + 255) / 256;
-  const int64_t w0 = chunk * threadIdx.x, w1 = min(W, w0 + chunk);
+  int32_t* h = hist + ((int64_t)p * NB + b) * W;
+  const int64_t chunk = (W + kScanThreads - 1) / kScanThreads;
+  const int64_t w0 = min(W, chunk * threadIdx.x), w1 = min(W, w0 + chunk);
   int64_t sum = 0;
-  for (int64_t w = w0; w < w1; ++w) sum += h[w * NB];
+  for (int64_t w = w0; w < w1; ++w) sum += h[w];
   part[threadIdx.x] = sum;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int64_t run = 0;
-    for (int t = 0; t < 256; ++t) {
-      const int64_t v = part[t];
-      part[t] = run;
-      run += v;
+  // exclusive scan of the 1024 chunk sums by the first wavefront, 16 per lane
+  if (threadIdx.x < kWave) {
+    constexpr int PER = kScanThreads / kWave;
+    int64_t loc[PER];
+    int64_t tot = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      loc[j] = tot;
+      tot += part[threadIdx.x * PER + j];
     }
-    totals[(int64_t)p * NB + b] = run;
+    int64_t incl = tot;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const int64_t up = __shfl_up(incl, off, kWave);
+      if ((int)threadIdx.x >= off) incl += up;
+    }
+    const int64_t excl = incl - tot;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) part[threadIdx.x * PER + j] = excl + loc[j];
+    if (threadIdx.x == kWave - 1) totals[(int64_t)p * NB + b] = incl;
   }
   __syncthreads();
   int64_t run = part[threadIdx.x];
   for (int64_t w = w0; w < w1; ++w) {
-    const int32_t v = h[w * NB];
-    h[w * NB] = (int32_t)run;
+    const int32_t v = h[w];
+    h[w] = (int32_t)run;
     run += v;
+  }
+}
+
+// Spreads the items (lane, off), off < count[lane], evenly over the lanes: item number t (in lane
+// order, then off) goes to lane t % 64.  In every round all 64 lanes call f(owner, off, active)
+// together, so f may read other lanes' registers with __shfl(x, owner); lanes without an item in
+// the last round pass active = false (and owner 0) and must not store.
+template <class F>
+__device__ __forceinline__ void wave_fill(int count, int lane, F f) {
+  int incl = count;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int up = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += up;
+  }
+  const int excl = incl - count;
+  const int total = __shfl(incl, kWave - 1, kWave);
+  for (int t0 = 0; t0 < total; t0 += kWave) {
+    const int t = t0 + lane;
+    // owner: last lane whose exclusive prefix is <= t (lanes with count 0 share their prefix with
+    // the next lane and are never the last)
+    int lo = 0, hi = kWave - 1;
+#pragma unroll
+    for (int step = 0; step < 6; ++step) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (__shfl(excl, mid, kWave) <= t) lo = mid; else hi = mid - 1;
+    }
+    const int start = __shfl(excl, lo, kWave);
+    const bool active = t < total;
+    f(active ? lo : 0, active ? t - start : 0, active);
   }
 }
 
@@ -200,21 +301,148 @@ __global__ __launch_bounds__(256) void place_rows_kernel(int m, int NB, int64_t 
     if (lane >= off) incl += up;
   }
   if (beta == NB - 1) rank = incl - mine;
-  if (i >= m || d == 0) return;
-  const int64_t base = (int64_t)hist[((int64_t)p * W + wave) * NB + beta] + rank;
-  base_out[(int64_t)p * m + i] = (int32_t)base;
+  const bool live = i < m && d > 0;
+  int64_t base = 0;
+  if (live) {
+    base = (int64_t)hist[((int64_t)p * NB + beta) * W + wave] + rank;
+    base_out[(int64_t)p * m + i] = (int32_t)base;
+  }
   const int k = p * NB + beta;
-  int32_t* rows = rows_tab[k];
-  for (int j = 0; j < rho; ++j) rows[base + j] = i;
-  int32_t* cols = cols_tab[k];
-  int32_t* mask = mask_tab[k];
-  for (int64_t s = base * w + d; s < (base + rho) * w; ++s) {
-    cols[s] = 0;
-    mask[s] = 0;
+  // Row ids (rho per lane) and padding slots (rho * w - d per lane) are written by the whole
+  // wavefront: item t of the concatenated per-lane ranges goes to lane t % 64, which finds the
+  // owning lane by binary search over the exclusive prefix sums.  A row of the widest bucket with
+  // hundreds of ELL rows, or a wide row with hundreds of padding slots, costs its share of
+  // coalesced stores instead of a serial loop in one lane.
+  wave_fill(live ? rho : 0, lane, [&](int owner, int off, bool active) {
+    const int kk = __shfl(k, owner, kWave);
+    const int64_t b0 = __shfl(base, owner, kWave);
+    const int row = __shfl(i, owner, kWave);
+    if (active) rows_tab[kk][b0 + off] = row;
+  });
+  const int64_t pad0 = base * w + d;
+  wave_fill(live ? rho * w - d : 0, lane, [&](int owner, int off, bool active) {
+    const int kk = __shfl(k, owner, kWave);
+    const int64_t s = __shfl(pad0, owner, kWave) + off;
+    if (active) {
+      cols_tab[kk][s] = 0;
+      mask_tab[kk][s] = 0;
+    }
+  });
+}
+
+// (4) entry placement, two phases per wavefront over 512 consecutive nonzeros.  First a lane owns
+// kEntriesPerThread consecutive nonzeros: a binary search finds the row of the first, the others
+// follow by walking the row pointer; the slot of an entry is base * width + (position inside its
+// (row, partition) run), and the run's parameters are looked up again only when the row or the
+// partition changes.  The row pointers the wavefront needs -- the rows between the recorded rows
+// around its nonzeros -- are fetched into LDS with one coalesced load when they fit the window,
+// so the search and the walk touch no global memory.  The (bucket, slot) pairs go to the
+// wavefront's piece of LDS.  Then the lanes take the nonzeros in lane-strided order, so that
+// neighbouring lanes hold neighbouring nonzeros and -- inside a run -- neighbouring slots: the
+// scattered stores of a run coalesce.  f(k, slot, e) is called once for every nonzero e, k being
+// the (partition, bucket) index.
+constexpr int kEntriesPerThread = 8;
+constexpr int kStageStride = 72;  // LDS words between the j-th entries of lanes 0 and 64: 2-way conflicts at most
+constexpr int kRowWindow = 256;   // row pointers held in LDS per wavefront (plus one)
+constexpr int64_t kMaxSlots = int64_t(1) << 40;  // slot numbers are staged as 8 + 32 bits
+struct alignas(16) EntryStage {
+  int32_t kh[kEntriesPerThread * kStageStride];       // k * 256 + (slot >> 32), -1: no entry
+  uint32_t slot_lo[kEntriesPerThread * kStageStride];
+  int32_t ptr[kRowWindow + 1 + 3];
+};
+
+template <class F>
+__device__ __forceinline__ void for_each_entry_slot(int m, int P, int psize, int NB, int64_t nnz, int32_t first,
+                                                    const int32_t* __restrict__ indptr,
+                                                    const int32_t* __restrict__ indices,
+                                                    const int32_t* __restrict__ widths,
+                                                    const int32_t* __restrict__ lo_in,
+                                                    const int32_t* __restrict__ base_in,
+                                                    const int32_t* __restrict__ coarse, int64_t stride, F f) {
+  __shared__ EntryStage stage_all[4];
+  const int lane = threadIdx.x & 63;
+  EntryStage& st = stage_all[threadIdx.x >> 6];
+  const int64_t end = first + nnz;
+  const int64_t wave_e0 = first + ((int64_t)blockIdx.x * 256 + (threadIdx.x & ~63)) * kEntriesPerThread;
+  if (wave_e0 >= end) return;
+  // rows that can own the wavefront's nonzeros: [ra, rb]
+  const int64_t wave_last = min(end, wave_e0 + kWave * kEntriesPerThread) - 1;
+  const int64_t qa = (wave_e0 - first) / stride, qb = (wave_last - first) / stride;
+  const int ra = coarse[qa];
+  const int rb = (qb + 1) * stride < nnz ? coarse[qb + 1] : m - 1;
+  const bool windowed = rb - ra < kRowWindow;  // uniform
+  if (windowed) {
+#pragma unroll
+    for (int t = 0; t * kWave < kRowWindow + 1; ++t) {
+      const int r = ra + t * kWave + lane;
+      if (t * kWave + lane <= kRowWindow && r <= rb + 1) st.ptr[t * kWave + lane] = indptr[r];
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  auto ptr_at = [&](int r) -> int64_t { return windowed ? st.ptr[r - ra] : indptr[r]; };
+  const int64_t e0 = wave_e0 + lane * kEntriesPerThread;
+  if (e0 < end) {
+    int col[kEntriesPerThread];
+    if (e0 + kEntriesPerThread <= end && (reinterpret_cast<uintptr_t>(indices + e0) & 15) == 0) {
+      const int4 c0 = *reinterpret_cast<const int4*>(indices + e0);
+      const int4 c1 = *reinterpret_cast<const int4*>(indices + e0 + 4);
+      col[0] = c0.x, col[1] = c0.y, col[2] = c0.z, col[3] = c0.w;
+      col[4] = c1.x, col[5] = c1.y, col[6] = c1.z, col[7] = c1.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < kEntriesPerThread; ++j) col[j] = e0 + j < end ? indices[e0 + j] : 0;
+    }
+    // row that owns e0: last r in [ra, rb] with indptr[r] <= e0 (rows before it with the same
+    // offset are empty)
+    int a = ra, b = rb;
+    while (a < b) {
+      const int mid = a + ((b - a + 1) >> 1);
+      if (ptr_at(mid) <= e0) a = mid; else b = mid - 1;
+    }
+    int r = a;
+    int64_t row_end = ptr_at(r + 1);
+    int cur_p = -1, k = 0;
+    int64_t slot0 = 0;  // slot of entry e is slot0 + e
+#pragma unroll
+    for (int j = 0; j < kEntriesPerThread; ++j) {
+      const int64_t e = e0 + j;
+      const int at = j * kStageStride + lane;
+      if (e >= end) {
+        st.kh[at] = -1;
+        continue;
+      }
+      while (e >= row_end) {
+        ++r;
+        row_end = ptr_at(r + 1);
+        cur_p = -1;
+      }
+      const int p = col[j] / psize;
+      if (p != cur_p) {
+        cur_p = p;
+        const int lo = p == 0 ? (int)ptr_at(r) : lo_in[(int64_t)p * m + r];
+        const int hi = p == P - 1 ? (int)row_end : lo_in[(int64_t)(p + 1) * m + r];
+        const int beta = bucket_of_dev(widths, NB, hi - lo);
+        k = p * NB + beta;
+        slot0 = (int64_t)base_in[(int64_t)p * m + r] * widths[beta] - lo;
+      }
+      const int64_t slot = slot0 + e;
+      st.kh[at] = k * 256 + (int32_t)(slot >> 32);
+      st.slot_lo[at] = (uint32_t)slot;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kEntriesPerThread; ++j) st.kh[j * kStageStride + lane] = -1;
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int t = 0; t < kEntriesPerThread; ++t) {
+    const int n = t * kWave + lane;  // n-th nonzero of the wavefront: entry n % 8 of lane n / 8
+    const int at = (n % kEntriesPerThread) * kStageStride + n / kEntriesPerThread;
+    const int kh = st.kh[at];
+    if (kh >= 0) f(kh >> 8, ((int64_t)(kh & 255) << 32) | st.slot_lo[at], wave_e0 + n);
   }
 }
 
-// (4) one thread per nonzero: its slot is base * width + (position inside the run).
 __global__ __launch_bounds__(256) void place_entries_kernel(int m, int P, int psize, int NB, int64_t nnz,
                                                             int32_t first,
                                                             const int32_t* __restrict__ indptr,
@@ -222,27 +450,14 @@ __global__ __launch_bounds__(256) void place_entries_kernel(int m, int P, int ps
                                                             const int32_t* __restrict__ widths,
                                                             const int32_t* __restrict__ lo_in,
                                                             const int32_t* __restrict__ base_in,
+                                                            const int32_t* __restrict__ coarse, int64_t stride,
                                                             int32_t* const* __restrict__ cols_tab,
                                                             int32_t* const* __restrict__ mask_tab) {
-  const int64_t e = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= first + nnz) return;
-  const int col = indices[e];
-  const int p = col / psize;
-  // row that owns e: last r with indptr[r] <= e
-  int a = 0, b = m;
-  while (a < b) {
-    const int mid = a + ((b - a + 1) >> 1);
-    if ((int64_t)indptr[mid] <= e) a = mid; else b = mid - 1;
-  }
-  const int i = a;
-  const int lo = lo_in[(int64_t)p * m + i];
-  const int hi = p == P - 1 ? indptr[i + 1] : lo_in[(int64_t)(p + 1) * m + i];
-  const int d = hi - lo;
-  const int beta = bucket_of_dev(widths, NB, d);
-  const int64_t pos = (int64_t)base_in[(int64_t)p * m + i] * widths[beta] + (e - lo);
-  const int k = p * NB + beta;
-  cols_tab[k][pos] = col;
-  mask_tab[k][pos] = 1;
+  for_each_entry_slot(m, P, psize, NB, nnz, first, indptr, indices, widths, lo_in, base_in, coarse, stride,
+                      [&](int k, int64_t slot, int64_t e) {
+                        cols_tab[k][slot] = indices[e];
+                        mask_tab[k][slot] = 1;
+                      });
 }
 
 // Value rewrite: A_k[slot] = values[e] for every nonzero (padding slots stay zero), the
@@ -255,22 +470,10 @@ __global__ __launch_bounds__(256) void place_values_kernel(int m, int P, int psi
                                                            const int32_t* __restrict__ widths,
                                                            const int32_t* __restrict__ lo_in,
                                                            const int32_t* __restrict__ base_in,
+                                                           const int32_t* __restrict__ coarse, int64_t stride,
                                                            float* const* __restrict__ a_tab) {
-  const int64_t e = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= first + nnz) return;
-  const int col = indices[e];
-  const int p = col / psize;
-  int a = 0, b = m;
-  while (a < b) {
-    const int mid = a + ((b - a + 1) >> 1);
-    if ((int64_t)indptr[mid] <= e) a = mid; else b = mid - 1;
-  }
-  const int i = a;
-  const int lo = lo_in[(int64_t)p * m + i];
-  const int hi = p == P - 1 ? indptr[i + 1] : lo_in[(int64_t)(p + 1) * m + i];
-  const int beta = bucket_of_dev(widths, NB, hi - lo);
-  const int64_t pos = (int64_t)base_in[(int64_t)p * m + i] * widths[beta] + (e - lo);
-  a_tab[p * NB + beta][pos] = values[e];
+  for_each_entry_slot(m, P, psize, NB, nnz, first, indptr, indices, widths, lo_in, base_in, coarse, stride,
+                      [&](int k, int64_t slot, int64_t e) { a_tab[k][slot] = values[e]; });
 }
 
 int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t parts, const int32_t* buckets,
@@ -278,6 +481,7 @@ int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t part
   STIR_REQUIRE(num_rows >= 0 && num_cols >= 0, "%s: bad matrix shape %d x %d", who, num_rows, num_cols);
   STIR_REQUIRE(parts > 0 && parts <= 65535, "%s: num_col_parts=%d", who, parts);
   STIR_REQUIRE(nb > 0 && nb <= 65535 && buckets, "%s: empty bucket list", who);
+  STIR_REQUIRE((int64_t)parts * nb < (int64_t(1) << 22), "%s: %d partitions x %d buckets is too many", who, parts, nb);
   for (int b = 0; b < nb; ++b) STIR_REQUIRE(buckets[b] > 0, "%s: bucket width %d is not positive", who, buckets[b]);
   for (int b = 1; b < nb; ++b) STIR_REQUIRE(buckets[b - 1] <= buckets[b], "%s: bucket widths must ascend", who);
   return 0;
@@ -311,31 +515,41 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
   STIR_HIP(hipMemcpyAsync(&ends[0], d_indptr, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   STIR_HIP(hipMemcpyAsync(&ends[1], d_indptr + m, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   STIR_HIP(hipMemcpyAsync(ws.widths, buckets, sizeof(int32_t) * NB, hipMemcpyHostToDevice, st));
-  STIR_HIP(hipMemsetAsync(ws.status, 0, sizeof(int32_t), st));
+  STIR_HIP(hipMemsetAsync(ws.status, 0, sizeof(int32_t) * kStatusInts, st));
   STIR_HIP(hipStreamSynchronize(st));
   const int64_t nnz = (int64_t)ends[1] - ends[0];
   STIR_REQUIRE(ends[0] >= 0 && nnz >= 0, "%s: indptr is not a CSR row pointer", who);
   STIR_REQUIRE(nnz == 0 || (d_indices && num_cols > 0), "%s: nonzeros but no columns", who);
   const int psize = num_cols > 0 ? (num_cols + P - 1) / P : 1;
   if (nnz > 0) {
-    hipLaunchKernelGGL(validate_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, m,
-                       num_cols, nnz, ends[0], d_indptr, d_indices, ws.status);
+    hipLaunchKernelGGL(validate_kernel, dim3((unsigned)stir::ceil_div(nnz, 256 * kValidatePerThread)), dim3(256), 0, st, num_cols,
+                       nnz, ends[0], d_indices, ws.status);
     STIR_LAUNCH_CHECK();
   }
   dim3 grid((unsigned)stir::ceil_div(m, 256), (unsigned)P);
-  hipLaunchKernelGGL(count_kernel, grid, dim3(256), 0, st, m, psize, NB, W, d_indptr, d_indices,
-                     ws.widths, ws.lo, ws.hist);
+  hipLaunchKernelGGL(count_kernel, grid, dim3(256), 0, st, m, psize, NB, W, ends[0], (int64_t)ends[1],
+                     coarse_stride(nnz), ws.coarse, d_indptr,
+                     d_indices, ws.widths, ws.lo, ws.hist, ws.status);
   STIR_LAUNCH_CHECK();
-  hipLaunchKernelGGL(scan_kernel, dim3((unsigned)NB, (unsigned)P), dim3(256), 0, st, NB, W, ws.hist,
+  hipLaunchKernelGGL(scan_kernel, dim3((unsigned)NB, (unsigned)P), dim3(kScanThreads), 0, st, NB, W, ws.hist,
                      ws.totals);
   STIR_LAUNCH_CHECK();
-  int32_t status = 0;
-  STIR_HIP(hipMemcpyAsync(&status, ws.status, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  std::vector<int32_t> counts(kStatusInts, 0);
+  STIR_HIP(hipMemcpyAsync(counts.data(), ws.status, sizeof(int32_t) * kStatusInts, hipMemcpyDeviceToHost, st));
   STIR_HIP(hipMemcpyAsync(nrows, ws.totals, sizeof(int64_t) * size_t(P) * NB, hipMemcpyDeviceToHost, st));
   STIR_HIP(hipStreamSynchronize(st));
+  const int32_t status = counts[0];
+  int64_t descents = 0, row_start_descents = 0;
+  for (int k = 0; k < kCountSlots; ++k) {
+    descents += counts[1 + k];
+    row_start_descents += counts[1 + kCountSlots + k];
+  }
+  STIR_REQUIRE(!(status & kStatusIndptr), "%s: indptr is not a CSR row pointer (it decreases)", who);
   STIR_REQUIRE(!(status & kStatusRange), "%s: a column index lies outside [0, %d)", who, num_cols);
-  STIR_REQUIRE(!(status & kStatusUnsorted),
+  STIR_REQUIRE(descents == row_start_descents,
                "%s: column indices must ascend inside each row (use the host routine for unsorted rows)", who);
+  for (int k = 0; k < P * NB; ++k)
+    STIR_REQUIRE(nrows[k] < kMaxSlots / buckets[k % NB], "%s: bucket %d holds too many slots", who, k);
   return 0;
 }
 
@@ -367,9 +581,9 @@ int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols, const i
   hipLaunchKernelGGL(place_rows_kernel, grid, dim3(256), 0, st, m, NB, W, d_indptr, ws.widths, ws.lo,
                      ws.hist, ws.base, ws.rows_tab, ws.cols_tab, ws.mask_tab);
   STIR_LAUNCH_CHECK();
-  hipLaunchKernelGGL(place_entries_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, m, P,
-                     psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.lo, ws.base, ws.cols_tab,
-                     ws.mask_tab);
+  hipLaunchKernelGGL(place_entries_kernel, dim3((unsigned)stir::ceil_div(nnz, 256 * kEntriesPerThread)), dim3(256), 0, st, m, P,
+                     psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.lo, ws.base, ws.coarse,
+                     coarse_stride(nnz), ws.cols_tab, ws.mask_tab);
   STIR_LAUNCH_CHECK();
   return 0;
 }
@@ -401,9 +615,9 @@ int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const
   if (nnz <= 0) return 0;
   STIR_REQUIRE(d_indices && d_values, "%s: null pointer argument", who);
   const int psize = (num_cols + P - 1) / P;
-  hipLaunchKernelGGL(place_values_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, m, P, psize,
-                     NB, nnz, ends[0], d_indptr, d_indices, d_values, ws.widths, ws.lo, ws.base,
-                     reinterpret_cast<float* const*>(ws.mask_tab));
+  hipLaunchKernelGGL(place_values_kernel, dim3((unsigned)stir::ceil_div(nnz, 256 * kEntriesPerThread)), dim3(256), 0, st, m, P, psize,
+                     NB, nnz, ends[0], d_indptr, d_indices, d_values, ws.widths, ws.lo, ws.base, ws.coarse,
+                     coarse_stride(nnz), reinterpret_cast<float* const*>(ws.mask_tab));
   STIR_LAUNCH_CHECK();
   return 0;
 }

@@ -61,6 +61,43 @@ def test_device_column_part_hyb_rejects_unsorted_and_out_of_range(dev):
         _device_hyb(dev, 2, 40, np.asarray([0, 1, 2], np.int32), bad, 2, [1, 2])
 
 
+def test_device_column_part_hyb_single_descent_inside_a_row_is_rejected(dev):
+    """One swapped pair inside one row (every other row ascending, descents at row starts
+    everywhere) must be found; the same swap across a row boundary is legal."""
+    m, n = 400, 300
+    indptr, indices = random_csr(m, n, 6000, 11, skew=1.0)
+    row = int(np.argmax(np.diff(indptr) >= 3))
+    e = indptr[row]
+    bad = indices.copy()
+    bad[e], bad[e + 1] = indices[e + 1], indices[e]
+    with pytest.raises(SparseTIRError, match="ascend"):
+        _device_hyb(dev, m, n, indptr, bad, 2, [1, 2, 4])
+    with pytest.raises(SparseTIRError, match="row pointer"):
+        ptr = indptr.copy()
+        ptr[10] = ptr[11] + 1
+        _device_hyb(dev, m, n, ptr, indices, 2, [1, 2, 4])
+
+
+def test_device_column_part_hyb_mostly_empty_rows_and_offset_row_pointer(dev):
+    m, n = 6000, 500
+    indptr, indices = random_csr(m, n, 400, 12, skew=2.0)
+    got = _device_hyb(dev, m, n, indptr, indices, 3, [1, 2, 4])
+    want = oracle.column_part_hyb(m, n, indptr, indices, 3, [1, 2, 4])
+    for gq, wq in zip(got, want):
+        for gp, wp in zip(gq, wq):
+            for a, b in zip(gp, wp):
+                assert np.array_equal(a, b)
+    # a row pointer that does not start at zero: rows 100.. of a larger matrix, same indices array
+    big_ptr, big_idx = random_csr(900, 300, 20000, 13, skew=1.0)
+    sub = big_ptr[100:].copy()
+    got = _device_hyb(dev, 800, 300, sub, big_idx, 2, [1, 2, 4, 8])
+    want = oracle.column_part_hyb(800, 300, sub - sub[0], big_idx[sub[0]:], 2, [1, 2, 4, 8])
+    for gq, wq in zip(got, want):
+        for gp, wp in zip(gq, wq):
+            for a, b in zip(gp, wp):
+                assert np.array_equal(a, b)
+
+
 def test_device_hyb_value_rewrite(dev):
     """A_k gathered on the device equals the values placed by the decomposition's own index
     arrays: A_k[r, s] = value of nonzero (rows_k[r], cols_k[r, s]) where mask is 1, else 0."""
