@@ -27,7 +27,8 @@ using stir::kWave;
 
 struct Workspace {
   int32_t* lo;       // [P][m]   start of the (row, partition) run inside indices
-  int32_t* base;     // [P][m]   first ELL row of the run inside its bucket
+  int64_t* slot0;    // [P][m]   slot of the run's nonzero e is slot0 + e  (= first ELL row * width - lo)
+  int32_t* kb;       // [P][m]   bucket of the run
   int32_t* hist;     // [P][NB][W] per-wavefront ELL-row counts, scanned in place
   int64_t* totals;   // [P][NB]
   int32_t* widths;   // [NB]
@@ -63,7 +64,8 @@ Workspace carve(void* p, int32_t m, int32_t P, int32_t NB) {
     return r;
   };
   w.lo = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(m > 0 ? m : 1)));
-  w.base = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(m > 0 ? m : 1)));
+  w.slot0 = reinterpret_cast<int64_t*>(take(sizeof(int64_t) * size_t(P) * size_t(m > 0 ? m : 1)));
+  w.kb = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(m > 0 ? m : 1)));
   w.hist = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(W > 0 ? W : 1) * NB));
   w.totals = reinterpret_cast<int64_t*>(take(sizeof(int64_t) * size_t(P) * NB));
   w.widths = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * NB));
@@ -267,7 +269,8 @@ __global__ __launch_bounds__(256) void place_rows_kernel(int m, int NB, int64_t 
                                                          const int32_t* __restrict__ widths,
                                                          const int32_t* __restrict__ lo_in,
                                                          const int32_t* __restrict__ hist,
-                                                         int32_t* __restrict__ base_out,
+                                                         int64_t* __restrict__ slot0_out,
+                                                         int32_t* __restrict__ kb_out,
                                                          int32_t* const* __restrict__ rows_tab,
                                                          int32_t* const* __restrict__ cols_tab,
                                                          int32_t* const* __restrict__ mask_tab) {
@@ -277,9 +280,9 @@ __global__ __launch_bounds__(256) void place_rows_kernel(int m, int NB, int64_t 
   const int lane = threadIdx.x & 63;
   const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (wave >= W) return;
-  int d = 0;
+  int d = 0, lo = 0;
   if (i < m) {
-    const int lo = lo_in[(int64_t)p * m + i];
+    lo = lo_in[(int64_t)p * m + i];
     const int hi = p == P - 1 ? indptr[i + 1] : lo_in[(int64_t)(p + 1) * m + i];
     d = hi - lo;
   }
@@ -305,7 +308,10 @@ __global__ __launch_bounds__(256) void place_rows_kernel(int m, int NB, int64_t 
   int64_t base = 0;
   if (live) {
     base = (int64_t)hist[((int64_t)p * NB + beta) * W + wave] + rank;
-    base_out[(int64_t)p * m + i] = (int32_t)base;
+  }
+  if (i < m) {
+    slot0_out[(int64_t)p * m + i] = base * w - lo;
+    kb_out[(int64_t)p * m + i] = beta;
   }
   const int k = p * NB + beta;
   // Row ids (rho per lane) and padding slots (rho * w - d per lane) are written by the whole
@@ -319,6 +325,7 @@ __global__ __launch_bounds__(256) void place_rows_kernel(int m, int NB, int64_t 
     const int row = __shfl(i, owner, kWave);
     if (active) rows_tab[kk][b0 + off] = row;
   });
+  if (P == 1) return;  // one partition: the entry pass writes the padding with the entries
   const int64_t pad0 = base * w + d;
   wave_fill(live ? rho * w - d : 0, lane, [&](int owner, int off, bool active) {
     const int kk = __shfl(k, owner, kWave);
@@ -350,47 +357,89 @@ struct alignas(16) EntryStage {
   uint32_t slot_lo[kEntriesPerThread * kStageStride];
   int32_t ptr[kRowWindow + 1 + 3];
 };
+// One column partition: everything an entry needs is a function of its row, so the wavefront
+// tabulates it for the rows of its window instead.
+struct alignas(16) RowStage {
+  int32_t ptr[kRowWindow + 1 + 3];
+  int32_t k[kRowWindow];           // bucket of the row
+  uint32_t slot0_lo[kRowWindow];   // slot of entry e of the row is slot0 + e
+  int32_t slot0_hi[kRowWindow];
+  int32_t pad[kRowWindow];         // padding slots after the row's last entry
+};
 
-template <class F>
-__device__ __forceinline__ void for_each_entry_slot(int m, int P, int psize, int NB, int64_t nnz, int32_t first,
-                                                    const int32_t* __restrict__ indptr,
-                                                    const int32_t* __restrict__ indices,
-                                                    const int32_t* __restrict__ widths,
-                                                    const int32_t* __restrict__ lo_in,
-                                                    const int32_t* __restrict__ base_in,
-                                                    const int32_t* __restrict__ coarse, int64_t stride, F f) {
-  __shared__ EntryStage stage_all[4];
-  const int lane = threadIdx.x & 63;
-  EntryStage& st = stage_all[threadIdx.x >> 6];
-  const int64_t end = first + nnz;
-  const int64_t wave_e0 = first + ((int64_t)blockIdx.x * 256 + (threadIdx.x & ~63)) * kEntriesPerThread;
-  if (wave_e0 >= end) return;
-  // rows that can own the wavefront's nonzeros: [ra, rb]
-  const int64_t wave_last = min(end, wave_e0 + kWave * kEntriesPerThread) - 1;
-  const int64_t qa = (wave_e0 - first) / stride, qb = (wave_last - first) / stride;
-  const int ra = coarse[qa];
-  const int rb = (qb + 1) * stride < nnz ? coarse[qb + 1] : m - 1;
+constexpr int kGeneralTile = kWave * kEntriesPerThread;  // nonzeros per wavefront, general path
+constexpr int kSingleTile = kGeneralTile;
+
+// Output pointers of the first kLdsTable (partition, bucket) pairs, copied to LDS when a kernel
+// starts.  The memory counter of a wavefront retires loads and stores in order, so a pointer
+// fetched from global memory between two stores would wait for the first store to complete;
+// from LDS it does not.
+constexpr int kLdsTable = 256;
+template <class T>
+struct PtrTable {
+  T* lds[kLdsTable];
+  T* const* global;
+  int count;
+  __device__ __forceinline__ void load(T* const* tab, int n) {  // all threads of the workgroup
+    global = tab;
+    count = n;
+    for (int k = threadIdx.x; k < n && k < kLdsTable; k += blockDim.x) lds[k] = tab[k];
+  }
+  __device__ __forceinline__ T* at(int k) const { return k < kLdsTable ? lds[k] : global[k]; }
+};
+
+struct EntryArgs {
+  int m, P, psize, NB;
+  int64_t nnz;
+  int32_t first;
+  const int32_t* __restrict__ indptr;
+  const int32_t* __restrict__ indices;
+  const int32_t* __restrict__ widths;
+  const int64_t* __restrict__ slot0_in;
+  const int32_t* __restrict__ kb_in;
+  const int32_t* __restrict__ coarse;
+  int64_t stride;
+};
+
+// Rows that can own the nonzeros [e_first, e_last]: between the recorded rows around them.
+__device__ __forceinline__ void row_range(const EntryArgs& g, int64_t e_first, int64_t e_last, int& ra, int& rb) {
+  const int64_t qa = (e_first - g.first) / g.stride, qb = (e_last - g.first) / g.stride;
+  ra = g.coarse[qa];
+  rb = (qb + 1) * g.stride < g.nnz ? g.coarse[qb + 1] : g.m - 1;
+}
+
+// General path for the kGeneralTile nonzeros from tile_e0 on.
+template <bool SINGLE, class L, class F, class Z>
+__device__ __forceinline__ void place_general(const EntryArgs& g, EntryStage& st, int64_t tile_e0, int lane, L load,
+                                              F f, Z zero) {
+  const int m = g.m, NB = g.NB;
+  const int64_t end = g.first + g.nnz;
+  if (tile_e0 >= end) return;
+  const int64_t tile_last = min(end, tile_e0 + kGeneralTile) - 1;
+  int ra, rb;
+  row_range(g, tile_e0, tile_last, ra, rb);
   const bool windowed = rb - ra < kRowWindow;  // uniform
+  __builtin_amdgcn_wave_barrier();
   if (windowed) {
 #pragma unroll
     for (int t = 0; t * kWave < kRowWindow + 1; ++t) {
       const int r = ra + t * kWave + lane;
-      if (t * kWave + lane <= kRowWindow && r <= rb + 1) st.ptr[t * kWave + lane] = indptr[r];
+      if (t * kWave + lane <= kRowWindow && r <= rb + 1) st.ptr[t * kWave + lane] = g.indptr[r];
     }
   }
   __builtin_amdgcn_wave_barrier();
-  auto ptr_at = [&](int r) -> int64_t { return windowed ? st.ptr[r - ra] : indptr[r]; };
-  const int64_t e0 = wave_e0 + lane * kEntriesPerThread;
+  auto ptr_at = [&](int r) -> int64_t { return windowed ? st.ptr[r - ra] : g.indptr[r]; };
+  const int64_t e0 = tile_e0 + lane * kEntriesPerThread;
   if (e0 < end) {
     int col[kEntriesPerThread];
-    if (e0 + kEntriesPerThread <= end && (reinterpret_cast<uintptr_t>(indices + e0) & 15) == 0) {
-      const int4 c0 = *reinterpret_cast<const int4*>(indices + e0);
-      const int4 c1 = *reinterpret_cast<const int4*>(indices + e0 + 4);
+    if (e0 + kEntriesPerThread <= end && (reinterpret_cast<uintptr_t>(g.indices + e0) & 15) == 0) {
+      const int4 c0 = *reinterpret_cast<const int4*>(g.indices + e0);
+      const int4 c1 = *reinterpret_cast<const int4*>(g.indices + e0 + 4);
       col[0] = c0.x, col[1] = c0.y, col[2] = c0.z, col[3] = c0.w;
       col[4] = c1.x, col[5] = c1.y, col[6] = c1.z, col[7] = c1.w;
     } else {
 #pragma unroll
-      for (int j = 0; j < kEntriesPerThread; ++j) col[j] = e0 + j < end ? indices[e0 + j] : 0;
+      for (int j = 0; j < kEntriesPerThread; ++j) col[j] = e0 + j < end ? g.indices[e0 + j] : 0;
     }
     // row that owns e0: last r in [ra, rb] with indptr[r] <= e0 (rows before it with the same
     // offset are empty)
@@ -416,64 +465,172 @@ __device__ __forceinline__ void for_each_entry_slot(int m, int P, int psize, int
         row_end = ptr_at(r + 1);
         cur_p = -1;
       }
-      const int p = col[j] / psize;
+      const int p = col[j] / g.psize;
       if (p != cur_p) {
         cur_p = p;
-        const int lo = p == 0 ? (int)ptr_at(r) : lo_in[(int64_t)p * m + r];
-        const int hi = p == P - 1 ? (int)row_end : lo_in[(int64_t)(p + 1) * m + r];
-        const int beta = bucket_of_dev(widths, NB, hi - lo);
-        k = p * NB + beta;
-        slot0 = (int64_t)base_in[(int64_t)p * m + r] * widths[beta] - lo;
+        k = p * NB + g.kb_in[(int64_t)p * m + r];
+        slot0 = g.slot0_in[(int64_t)p * m + r];
       }
       const int64_t slot = slot0 + e;
       st.kh[at] = k * 256 + (int32_t)(slot >> 32);
       st.slot_lo[at] = (uint32_t)slot;
+      if (SINGLE && e + 1 == row_end) {
+        // one partition: the padding behind a row's last entry is written here (rare path:
+        // more rows around the wavefront's nonzeros than the window holds)
+        const int w = g.widths[k];
+        const int64_t stop = (slot + w) / w * w;
+        for (int64_t z = slot + 1; z < stop; ++z) zero(k, z);
+      }
     }
   } else {
 #pragma unroll
     for (int j = 0; j < kEntriesPerThread; ++j) st.kh[j * kStageStride + lane] = -1;
   }
   __builtin_amdgcn_wave_barrier();
+  int khs[kEntriesPerThread], src[kEntriesPerThread];
+  uint32_t lows[kEntriesPerThread];
 #pragma unroll
   for (int t = 0; t < kEntriesPerThread; ++t) {
-    const int n = t * kWave + lane;  // n-th nonzero of the wavefront: entry n % 8 of lane n / 8
+    const int n = t * kWave + lane;  // n-th nonzero of the tile: entry n % 8 of lane n / 8
     const int at = (n % kEntriesPerThread) * kStageStride + n / kEntriesPerThread;
-    const int kh = st.kh[at];
-    if (kh >= 0) f(kh >> 8, ((int64_t)(kh & 255) << 32) | st.slot_lo[at], wave_e0 + n);
+    khs[t] = st.kh[at];
+    lows[t] = st.slot_lo[at];
+    src[t] = khs[t] >= 0 ? load(tile_e0 + n) : 0;  // every load of the tile precedes its stores
+  }
+#pragma unroll
+  for (int t = 0; t < kEntriesPerThread; ++t)
+    if (khs[t] >= 0) f(khs[t] >> 8, ((int64_t)(khs[t] & 255) << 32) | lows[t], src[t]);
+}
+
+// One partition, rows [ra, rb] fit the window: fetch what the tile's nonzeros carry (lane-strided),
+// tabulate bucket and first slot per row, place the nonzeros, then zero the padding behind every
+// row whose last entry lies in the tile (so that a row's slots reach memory together).  All global
+// loads come before the first store.
+template <class L, class F, class Z>
+__device__ __forceinline__ void place_single(const EntryArgs& g, RowStage& rs, int64_t tile_e0, int64_t tile_last,
+                                             int ra, int rb, int lane, L load, F f, Z zero) {
+  const int nr = rb - ra + 1;
+  int src[kEntriesPerThread];
+#pragma unroll
+  for (int t = 0; t < kEntriesPerThread; ++t) {
+    const int64_t e = tile_e0 + t * kWave + lane;
+    src[t] = e <= tile_last ? load(e) : 0;
+  }
+#pragma unroll
+  for (int t = 0; t * kWave < kRowWindow; ++t) {
+    const int x = t * kWave + lane;
+    if (x < nr) {
+      const int lo = g.indptr[ra + x], hi = g.indptr[ra + x + 1];
+      const int beta = g.kb_in[ra + x];
+      const int64_t slot0 = g.slot0_in[ra + x];
+      const int d = hi - lo;
+      const int w = g.widths[beta];
+      rs.ptr[x] = lo;
+      if (x == nr - 1) rs.ptr[nr] = hi;
+      rs.k[x] = beta;
+      rs.slot0_lo[x] = (uint32_t)slot0;
+      rs.slot0_hi[x] = (int32_t)(slot0 >> 32);
+      const bool mine = d > 0 && hi - 1 >= tile_e0 && hi - 1 <= tile_last;
+      rs.pad[x] = mine ? (d + w - 1) / w * w - d : 0;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  int steps = 0;
+  while ((1 << steps) < nr) ++steps;
+  // window row of each of the lane's nonzeros: last x with ptr[x] <= e; the searches advance
+  // together so that their LDS reads overlap
+  int a[kEntriesPerThread], b[kEntriesPerThread];
+#pragma unroll
+  for (int t = 0; t < kEntriesPerThread; ++t) a[t] = 0, b[t] = nr - 1;
+  for (int it = 0; it < steps; ++it) {
+#pragma unroll
+    for (int t = 0; t < kEntriesPerThread; ++t) {
+      const int mid = (a[t] + b[t] + 1) >> 1;
+      if (rs.ptr[mid] <= tile_e0 + t * kWave + lane) a[t] = mid; else b[t] = mid - 1;
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kEntriesPerThread; ++t) {
+    const int64_t e = tile_e0 + t * kWave + lane;
+    if (e <= tile_last) {
+      const int64_t slot0 = ((int64_t)rs.slot0_hi[a[t]] << 32) | rs.slot0_lo[a[t]];
+      f(rs.k[a[t]], slot0 + e, src[t]);
+    }
+  }
+  for (int c = 0; c < nr; c += kWave) {
+    const int x = c + lane;
+    wave_fill(x < nr ? rs.pad[x] : 0, lane, [&](int owner, int off, bool active) {
+      const int xo = c + owner;
+      const int64_t slot0 = ((int64_t)rs.slot0_hi[xo] << 32) | rs.slot0_lo[xo];
+      if (active) zero(rs.k[xo], slot0 + rs.ptr[xo + 1] + off);
+    });
   }
 }
 
-__global__ __launch_bounds__(256) void place_entries_kernel(int m, int P, int psize, int NB, int64_t nnz,
-                                                            int32_t first,
-                                                            const int32_t* __restrict__ indptr,
-                                                            const int32_t* __restrict__ indices,
-                                                            const int32_t* __restrict__ widths,
-                                                            const int32_t* __restrict__ lo_in,
-                                                            const int32_t* __restrict__ base_in,
-                                                            const int32_t* __restrict__ coarse, int64_t stride,
-                                                            int32_t* const* __restrict__ cols_tab,
-                                                            int32_t* const* __restrict__ mask_tab) {
-  for_each_entry_slot(m, P, psize, NB, nnz, first, indptr, indices, widths, lo_in, base_in, coarse, stride,
-                      [&](int k, int64_t slot, int64_t e) {
-                        cols_tab[k][slot] = indices[e];
-                        mask_tab[k][slot] = 1;
-                      });
+// load(e) fetches what nonzero e carries (an int: its column, or the bits of its value),
+// f(k, slot, carried) stores it, zero(k, slot) clears a padding slot (one partition only).
+template <bool SINGLE, class L, class F, class Z>
+__device__ __forceinline__ void for_each_entry_slot(const EntryArgs& g, L load, F f, Z zero) {
+  // one piece of LDS per wavefront, viewed as either staging layout (the wavefronts of a
+  // workgroup may take different paths, so the pieces must not depend on the view)
+  union WaveStage {
+    EntryStage entry;
+    RowStage row;
+  };
+  __shared__ WaveStage stage_all[4];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t end = g.first + g.nnz;
+  if (SINGLE) {
+    const int64_t tile_e0 = g.first + ((int64_t)blockIdx.x * 4 + wave) * kSingleTile;
+    if (tile_e0 >= end) return;
+    const int64_t tile_last = min(end, tile_e0 + kSingleTile) - 1;
+    int ra, rb;
+    row_range(g, tile_e0, tile_last, ra, rb);
+    if (rb - ra < kRowWindow) {
+      place_single(g, stage_all[wave].row, tile_e0, tile_last, ra, rb, lane, load, f, zero);
+    } else {
+      for (int sub = 0; sub < kSingleTile / kGeneralTile; ++sub)
+        place_general<true>(g, stage_all[wave].entry, tile_e0 + (int64_t)sub * kGeneralTile, lane, load, f, zero);
+    }
+  } else {
+    const int64_t tile_e0 = g.first + ((int64_t)blockIdx.x * 4 + wave) * kGeneralTile;
+    place_general<false>(g, stage_all[wave].entry, tile_e0, lane, load, f, zero);
+  }
 }
 
-// Value rewrite: A_k[slot] = values[e] for every nonzero (padding slots stay zero), the
-// placement computed exactly as in place_entries_kernel.
-__global__ __launch_bounds__(256) void place_values_kernel(int m, int P, int psize, int NB, int64_t nnz,
-                                                           int32_t first,
-                                                           const int32_t* __restrict__ indptr,
-                                                           const int32_t* __restrict__ indices,
-                                                           const float* __restrict__ values,
-                                                           const int32_t* __restrict__ widths,
-                                                           const int32_t* __restrict__ lo_in,
-                                                           const int32_t* __restrict__ base_in,
-                                                           const int32_t* __restrict__ coarse, int64_t stride,
+template <bool SINGLE>
+__global__ __launch_bounds__(256) void place_entries_kernel(EntryArgs g, int32_t* const* __restrict__ cols_tab,
+                                                            int32_t* const* __restrict__ mask_tab) {
+  __shared__ PtrTable<int32_t> cols, mask;
+  cols.load(cols_tab, g.P * g.NB);
+  mask.load(mask_tab, g.P * g.NB);
+  __syncthreads();
+  for_each_entry_slot<SINGLE>(
+      g, [&](int64_t e) { return g.indices[e]; },
+      [&](int k, int64_t slot, int col) {
+        cols.at(k)[slot] = col;
+        mask.at(k)[slot] = 1;
+      },
+      [&](int k, int64_t slot) {
+        cols.at(k)[slot] = 0;
+        mask.at(k)[slot] = 0;
+      });
+}
+
+// Value rewrite: A_k[slot] = values[e] for every nonzero, zero in the padding slots, the
+// placement computed exactly as in place_entries_kernel.  (With several partitions the padding
+// is cleared beforehand instead.)
+template <bool SINGLE>
+__global__ __launch_bounds__(256) void place_values_kernel(EntryArgs g, const float* __restrict__ values,
                                                            float* const* __restrict__ a_tab) {
-  for_each_entry_slot(m, P, psize, NB, nnz, first, indptr, indices, widths, lo_in, base_in, coarse, stride,
-                      [&](int k, int64_t slot, int64_t e) { a_tab[k][slot] = values[e]; });
+  __shared__ PtrTable<float> out;
+  out.load(a_tab, g.P * g.NB);
+  __syncthreads();
+  for_each_entry_slot<SINGLE>(
+      g, [&](int64_t e) { return __float_as_int(values[e]); },
+      [&](int k, int64_t slot, int bits) { out.at(k)[slot] = __int_as_float(bits); },
+      [&](int k, int64_t slot) { out.at(k)[slot] = 0.f; });
 }
 
 int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t parts, const int32_t* buckets,
@@ -579,11 +736,16 @@ int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols, const i
   const int psize = (num_cols + P - 1) / P;
   dim3 grid((unsigned)stir::ceil_div(m, 256), (unsigned)P);
   hipLaunchKernelGGL(place_rows_kernel, grid, dim3(256), 0, st, m, NB, W, d_indptr, ws.widths, ws.lo,
-                     ws.hist, ws.base, ws.rows_tab, ws.cols_tab, ws.mask_tab);
+                     ws.hist, ws.slot0, ws.kb, ws.rows_tab, ws.cols_tab, ws.mask_tab);
   STIR_LAUNCH_CHECK();
-  hipLaunchKernelGGL(place_entries_kernel, dim3((unsigned)stir::ceil_div(nnz, 256 * kEntriesPerThread)), dim3(256), 0, st, m, P,
-                     psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.lo, ws.base, ws.coarse,
-                     coarse_stride(nnz), ws.cols_tab, ws.mask_tab);
+  const EntryArgs ea{m, P, psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.slot0, ws.kb, ws.coarse,
+                     coarse_stride(nnz)};
+  if (P == 1)
+    hipLaunchKernelGGL(place_entries_kernel<true>, dim3((unsigned)stir::ceil_div(nnz, 4 * kSingleTile)), dim3(256), 0,
+                       st, ea, ws.cols_tab, ws.mask_tab);
+  else
+    hipLaunchKernelGGL(place_entries_kernel<false>, dim3((unsigned)stir::ceil_div(nnz, 4 * kGeneralTile)), dim3(256),
+                       0, st, ea, ws.cols_tab, ws.mask_tab);
   STIR_LAUNCH_CHECK();
   return 0;
 }
@@ -608,16 +770,23 @@ int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const
   STIR_HIP(hipStreamSynchronize(st));
   for (int k = 0; k < P * NB; ++k) {
     STIR_REQUIRE(nrows[k] >= 0 && (nrows[k] == 0 || d_A[k]), "%s: bucket %d has rows but no array", who, k);
-    if (nrows[k] > 0)
+    // several partitions: padding slots are cleared here; with one the entry pass writes them
+    if (nrows[k] > 0 && P > 1)
       STIR_HIP(hipMemsetAsync(d_A[k], 0, sizeof(float) * size_t(nrows[k]) * buckets[k % NB], st));
   }
   const int64_t nnz = (int64_t)ends[1] - ends[0];
   if (nnz <= 0) return 0;
   STIR_REQUIRE(d_indices && d_values, "%s: null pointer argument", who);
   const int psize = (num_cols + P - 1) / P;
-  hipLaunchKernelGGL(place_values_kernel, dim3((unsigned)stir::ceil_div(nnz, 256 * kEntriesPerThread)), dim3(256), 0, st, m, P, psize,
-                     NB, nnz, ends[0], d_indptr, d_indices, d_values, ws.widths, ws.lo, ws.base, ws.coarse,
-                     coarse_stride(nnz), reinterpret_cast<float* const*>(ws.mask_tab));
+  float* const* a_tab = reinterpret_cast<float* const*>(ws.mask_tab);
+  const EntryArgs ea{m, P, psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.slot0, ws.kb, ws.coarse,
+                     coarse_stride(nnz)};
+  if (P == 1)
+    hipLaunchKernelGGL(place_values_kernel<true>, dim3((unsigned)stir::ceil_div(nnz, 4 * kSingleTile)), dim3(256), 0,
+                       st, ea, d_values, a_tab);
+  else
+    hipLaunchKernelGGL(place_values_kernel<false>, dim3((unsigned)stir::ceil_div(nnz, 4 * kGeneralTile)), dim3(256),
+                       0, st, ea, d_values, a_tab);
   STIR_LAUNCH_CHECK();
   return 0;
 }

@@ -29,6 +29,11 @@ def _device_hyb(dev, m, n, indptr, indices, parts, buckets):
     (50, 7, 300, 7, [1, 2, 4], 7),
     (63, 63, 900, 2, [1, 2, 4, 8], 8),
     (65, 200, 5000, 3, [1, 2], 9),
+    # one partition, tiles with few rows next to tiles with hundreds (both placement paths in
+    # one workgroup)
+    (20000, 500, 30000, 1, [1, 2, 4, 8], 10),
+    (50000, 500, 70000, 1, [1, 2, 4, 8], 11),
+    (2000, 2000, 150000, 1, [1, 2, 4, 8, 16, 32], 12),
 ])
 def test_device_column_part_hyb_bit_exact(dev, m, n, nnz, parts, buckets, seed):
     indptr, indices = random_csr(m, n, nnz, seed, skew=1.1)
