@@ -82,3 +82,42 @@ def test_rgms_config5_reduced(dev):
     csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
     got, x32, w32, av = _run(dev, csf, cfg["m"], cfg["n"], cfg["x"], cfg["w"], 256, cfg["buckets"], False)
     _check(got, csf, av, x32, w32, cfg["m"], "config5 reduced")
+
+
+@pytest.mark.parametrize("group,buckets", [(256, [1, 2, 4, 8, 16]), (32, [1, 2, 4, 8, 16, 32]), (48, [1, 3, 4, 16])])
+def test_rgms_staged_accumulation(dev, group, buckets):
+    """Enough ELL rows for the scatter-free path (results staged per ELL row, then summed per
+    output row); a bucket with a width that is not a power of two still goes through atomics in
+    the same launch.  Called twice on one operator: the second call reuses the index."""
+    cfg = datasets.config5(n=20000, num_rels=9, num_edges=200000, seed=7)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    got, x32, w32, av = _run(dev, csf, cfg["m"], cfg["n"], cfg["x"], cfg["w"], group, buckets, True)
+    _check(got, csf, av, x32, w32, cfg["m"], f"staged group={group}")
+
+
+def test_rgms_staged_repeat_calls_accumulate(dev):
+    cfg = datasets.config5(n=20000, num_rels=5, num_edges=150000, seed=8)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    R, fin, fout, buckets, group = 5, 32, 32, [1, 2, 4, 8], 64
+    rows_bkt = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    triples, mids = [], []
+    for b in range(len(buckets)):
+        triples += [t(mask[b].astype(np.float16).ravel()), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    f = ops.build_rgms(cfg["m"], cfg["n"], R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols])
+    w, x = t(cfg["w"].astype(np.float16).ravel()), t(cfg["x"].astype(np.float16).ravel())
+    y = torch.zeros(cfg["m"] * fout, dtype=torch.float32, device=dev)
+    f(w, x, y, *triples, *mids)
+    once = y.clone()
+    f(w, x, y, *triples, *mids)   # Y is accumulated into, as with the atomic path
+    torch.cuda.synchronize()
+    assert once.abs().sum() > 0
+    assert torch.allclose(y, 2 * once, rtol=1e-6, atol=1e-6)
+    y2 = torch.zeros_like(y)
+    f(w, x, y2, *triples, *mids)
+    torch.cuda.synchronize()
+    # the staged sums are formed in a fixed order except for output rows that span several
+    # chunks of the reduce kernel, whose partial sums meet in atomics
+    assert torch.allclose(y2, once, rtol=1e-6, atol=1e-6)

@@ -138,3 +138,4 @@ def test_rgms_f32_config5_reduced_both_forms_agree(dev):
     f(_t(dev, ones), _t(dev, w.ravel()), _t(dev, cfg["x"].ravel()), y, *[_t(dev, c) for c in csf])
     torch.cuda.synchronize()
     _check(y.cpu().numpy().reshape(n, 32), want, scale, oracle.rgms_csf_f32(ones, w, cfg["x"], *csf, n), "config5 csf")
+
