@@ -87,3 +87,22 @@ def test_sddmm_scaled_by_edge_values(dev):
     rows = np.repeat(np.arange(m), np.diff(indptr))
     scale = np.einsum("ek,ek->e", np.abs(a).astype(np.float64)[rows], np.abs(b).astype(np.float64)[indices]) * e
     assert np.all(np.abs(c.cpu().numpy() - want) <= 2 * RTOL * scale + 1e-30)
+
+
+def test_sddmm_preproc_empty_row_runs_and_hub_rows(dev):
+    """Row lookup where 512 consecutive nonzeros span thousands of rows (long runs of empty rows:
+    the per-nonzero fallback) and where one row holds thousands of nonzeros."""
+    rng = np.random.default_rng(21)
+    deg = np.zeros(40000, np.int64)
+    deg[rng.choice(40000, 300, replace=False)] = rng.integers(1, 6, 300)   # sparse region
+    deg[100] = 5000                                                         # hub
+    deg[20000:20400] = rng.integers(0, 40, 400)                             # dense region
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    nnz = int(indptr[-1])
+    pre = ops.build_sddmm_preproc(40000, 10, 16, nnz)
+    mid = torch.full((nnz,), -7, dtype=torch.int32, device=dev)
+    z = lambda k, dt=torch.float32: torch.zeros(k, dtype=dt, device=dev)
+    pre(z(40000 * 16), z(10 * 16), z(nnz), torch.from_numpy(indptr).to(dev), z(nnz, torch.int32), mid)
+    torch.cuda.synchronize()
+    assert np.array_equal(mid.cpu().numpy(), np.repeat(np.arange(40000), deg))
+    assert np.array_equal(mid.cpu().numpy(), oracle.sddmm_mid(indptr, nnz))
