@@ -72,7 +72,13 @@ __device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int l
   if (!atomic) {
     float* base = C + row * feat + gl * 4;
 #pragma unroll
-    for (int r = 0; r < REP; ++r) *reinterpret_cast<float4*>(base + r * G * 4) = acc[r];
+    for (int r = 0; r < REP; ++r) {
+      float* q = base + r * G * 4;
+      __builtin_nontemporal_store(acc[r].x, q);
+      __builtin_nontemporal_store(acc[r].y, q + 1);
+      __builtin_nontemporal_store(acc[r].z, q + 2);
+      __builtin_nontemporal_store(acc[r].w, q + 3);
+    }
     return;
   }
   __builtin_amdgcn_wave_barrier();
@@ -112,8 +118,8 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, const fl
 
   for (int base = start; base < end; base += kWave) {
     const int p = base + lane;
-    const int my_col = p < end ? indices[p] : 0;
-    const float my_val = p < end ? A[p] : 0.f;
+    const int my_col = p < end ? __builtin_nontemporal_load(indices + p) : 0;
+    const float my_val = p < end ? __builtin_nontemporal_load(A + p) : 0.f;
     const int cnt = min(kWave, end - base);
     for (int j0 = 0; j0 < cnt; j0 += NG * UNROLL) {
       float4 x[UNROLL][REP];
@@ -168,8 +174,9 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
   const int64_t slot0 = t * kWave;
   const int64_t nslots = bk.nrows << LOG2W;
   const int64_t s = slot0 + lane;
-  const int my_col = s < nslots ? bk.cols[s] : 0;
-  const float my_val = s < nslots ? bk.A[s] : 0.f;
+  // index and weight arrays are read once: non-temporal, so they do not displace rows of B
+  const int my_col = s < nslots ? __builtin_nontemporal_load(bk.cols + s) : 0;
+  const float my_val = s < nslots ? __builtin_nontemporal_load(bk.A + s) : 0.f;
   constexpr int ROWS = kWave >> LOG2W;  // ELL rows per tile
   const int64_t row0 = slot0 >> LOG2W;
   int my_row = -1;
@@ -239,8 +246,8 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
   for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
   for (int c0 = s_begin; c0 < s_end; c0 += kWave) {
     const int s = c0 + lane;
-    const int my_col = s < s_end ? cols[s] : 0;
-    const float my_val = s < s_end ? vals[s] : 0.f;
+    const int my_col = s < s_end ? __builtin_nontemporal_load(cols + s) : 0;
+    const float my_val = s < s_end ? __builtin_nontemporal_load(vals + s) : 0.f;
 #pragma unroll 1
     for (int c = 0; c < G; c += CH) {
       float4 x[CH][REP];
