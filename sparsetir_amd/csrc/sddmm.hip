@@ -46,8 +46,9 @@ __global__ __launch_bounds__(256) void sddmm_kernel(int64_t nnz, int feat, const
   if (e0 >= nnz) return;
   const int g = lane / G, gl = lane % G;
   const int64_t e = e0 + lane;
-  const int my_row = e < nnz ? mid[e] : 0;
-  const int my_col = e < nnz ? indices[e] : 0;
+  // streamed once: non-temporal, so they do not displace feature rows in the caches
+  const int my_row = e < nnz ? __builtin_nontemporal_load(mid + e) : 0;
+  const int my_col = e < nnz ? __builtin_nontemporal_load(indices + e) : 0;
   float out = 0.f;
 #pragma unroll
   for (int c = 0; c < G; c += CH) {
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(256) void sddmm_kernel(int64_t nnz, int feat, const
       if (gl == c + u) out = p;
     }
   }
-  if (e < nnz) C[e] = scale ? out * scale[e] : out;
+  if (e < nnz) __builtin_nontemporal_store(scale ? out * __builtin_nontemporal_load(scale + e) : out, C + e);
 }
 
 // Any feature width: one wavefront per 64 nonzeros, lanes stride over the features.
