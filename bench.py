@@ -78,6 +78,34 @@ def time_steps(fn, steps, warmup, torch):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
+def config2_sweep(torch, dev, ops, st, datasets, time_steps):
+    """Config 2: hyb SpMM (2 column partitions, widths 1..512) against CSR row-split on the
+    169k-node graph, feature widths 32/64/128/256."""
+    g = datasets.config2()
+    m, n, nnz = g["m"], g["n"], len(g["indices"])
+    parts, buckets = g["num_col_parts"], g["buckets"]
+    d_ptr, d_idx = torch.from_numpy(g["indptr"]).to(dev), torch.from_numpy(g["indices"]).to(dev)
+    rows, cols, mask = st.column_part_hyb(m, n, d_ptr, d_idx, parts, buckets)
+    triples, nrows = [], []
+    for p in range(parts):
+        for b in range(len(buckets)):
+            triples += [mask[p][b].reshape(-1).float(), rows[p][b], cols[p][b].reshape(-1)]
+            nrows.append(int(rows[p][b].shape[0]))
+    ones = torch.ones(nnz, device=dev)
+    out = {"nodes": m, "edges": nnz, "num_col_parts": parts}
+    for feat in (32, 64, 128, 256):
+        x = torch.randn(n * feat, device=dev)
+        c = torch.zeros(m * feat, device=dev)
+        hyb = ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)
+        csr = ops.build_csrmm(m, n, feat, nnz)
+        _, dh, _ = time_steps(lambda: hyb(x, c, *triples), 50, 5, torch)
+        _, dc, _ = time_steps(lambda: csr(ones, x, c, d_ptr, d_idx), 50, 5, torch)
+        byts = 8.0 * nnz + 4.0 * (m + 1) + 4.0 * n * feat + 4.0 * m * feat
+        out[f"feat{feat}"] = {"hyb_us": dh * 1e6, "csr_us": dc * 1e6, "hyb_gflops": 2.0 * nnz * feat / dh / 1e9,
+                              "hyb_alg_GBps": byts / dh / 1e9}
+    return out
+
+
 def side_kernels(torch, dev, ops, st, datasets, time_steps):
     """BSR SpMM (config 4 and a scaled-up shape) and RGMS (config 5): time, flop rate against the
     dense fp16 MFMA peak, algorithmic bytes against the HBM peak."""
@@ -327,6 +355,7 @@ def main():
         del edge
         del a2, b2, out, mid
         extra.update(side_kernels(torch, dev, ops, st, datasets, time_steps))
+        extra["config2_hyb_vs_csr"] = config2_sweep(torch, dev, ops, st, datasets, time_steps)
         result["extra"] = extra
 
     print(json.dumps(result), flush=True)

@@ -9,7 +9,7 @@ import torch
 import oracle
 import sparsetir_amd as st
 from sparsetir_amd import datasets, ops
-from helpers import rgms_f64, sddmm_f64, spmm_f64
+from helpers import rgms_f64, spmm_f64
 
 pytestmark = pytest.mark.gpu
 
