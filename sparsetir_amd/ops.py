@@ -45,9 +45,22 @@ class _Operator:
     entry_name = "main"
 
     def _check(self, args, spec):
-        """spec: list of (label, dtype, length)."""
+        """spec: list of (label, dtype, length).  Returns the device all arrays live on."""
         if len(args) != len(spec):
             raise _lib.SparseTIRError(f"{self.name}: num_args should be {len(spec)}")
+        first = args[0]
+        if isinstance(first, torch.Tensor) and first.is_cuda:
+            idx = first.get_device()
+            for t, (_, dtype, length) in zip(args, spec):
+                # one combined test per array; anything odd is diagnosed by the slow path below
+                if not (isinstance(t, torch.Tensor) and t.dtype == dtype and t.ndim == 1
+                        and t.shape[0] == length and t.is_contiguous() and t.get_device() == idx):
+                    break
+            else:
+                return first.device
+        return self._check_slow(args, spec)
+
+    def _check_slow(self, args, spec):
         dev = None
         for i, (t, (label, dtype, length)) in enumerate(zip(args, spec)):
             if not isinstance(t, torch.Tensor):
@@ -121,6 +134,7 @@ class HybCsrMM(_Operator):
         self._plan = None
         self._key = None
         self._keep = None
+        self._spec_cache = None
 
     def _spec(self):
         f32, i32 = torch.float32, torch.int32
@@ -144,7 +158,9 @@ class HybCsrMM(_Operator):
             pass
 
     def __call__(self, *args):
-        dev = self._check(args, self._spec())
+        if self._spec_cache is None:
+            self._spec_cache = self._spec()
+        dev = self._check(args, self._spec_cache)
         b, c, triples = args[0], args[1], args[2:]
         key = (dev,) + tuple(t.data_ptr() for t in triples)
         with torch.cuda.device(dev):
@@ -300,6 +316,7 @@ class Rgms(_Operator):
         self._plan = None
         self._key = None
         self._keep = None
+        self._spec_cache = None
 
     def _spec(self):
         f16, f32, i32 = self._in_dtype, torch.float32, torch.int32
@@ -324,7 +341,9 @@ class Rgms(_Operator):
             pass
 
     def __call__(self, *args):
-        dev = self._check(args, self._spec())
+        if self._spec_cache is None:
+            self._spec_cache = self._spec()
+        dev = self._check(args, self._spec_cache)
         w, x, y, rest = args[0], args[1], args[2], args[3:]
         nb = len(self.groups)
         triples, mids = rest[:3 * nb], rest[3 * nb:]
