@@ -97,25 +97,15 @@ __device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int l
 }
 
 // ----------------------------------------------------------------------------- CSR SpMM
-// One wavefront per row; the 64/G lane groups take the row's nonzeros round-robin and
-// their partial sums are combined with cross-lane adds at the end.
+// Partial sum of A[p] * B[indices[p], :] over p in [start, end) for one wavefront: the 64/G lane
+// groups take the nonzeros round-robin; the caller combines the groups.
 template <int G, int REP>
-__global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, const float* __restrict__ A,
-                                                       const float* __restrict__ B,
-                                                       float* __restrict__ C,
-                                                       const int32_t* __restrict__ indptr,
-                                                       const int32_t* __restrict__ indices) {
+__device__ __forceinline__ void csr_accumulate(float4 (&acc)[REP], int start, int end, int feat,
+                                               const float* __restrict__ A, const float* __restrict__ B,
+                                               const int32_t* __restrict__ indices, int lane) {
   constexpr int NG = kWave / G;
   constexpr int UNROLL = 4;
-  const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= m) return;
   const int g = lane / G, gl = lane % G;
-  const int start = indptr[row], end = indptr[row + 1];
-  float4 acc[REP];
-#pragma unroll
-  for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-
   for (int base = start; base < end; base += kWave) {
     const int p = base + lane;
     const int my_col = p < end ? __builtin_nontemporal_load(indices + p) : 0;
@@ -140,8 +130,90 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, const fl
         for (int r = 0; r < REP; ++r) fma4(acc[r], v[u], x[u][r]);
     }
   }
+}
+
+// Rows with more nonzeros than this are not left to a single wavefront (a 17k-entry hub row
+// costs one wavefront milliseconds): the row kernel only clears them and csr_long_rows_kernel,
+// launched after it, adds them up in pieces of kLongPiece nonzeros.
+constexpr int kLongRow = 256;
+constexpr int kLongPiece = 256;
+
+// One wavefront per row.  With split_long the rows above kLongRow are zero-filled here.
+template <int G, int REP>
+__global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, int split_long,
+                                                       const float* __restrict__ A,
+                                                       const float* __restrict__ B,
+                                                       float* __restrict__ C,
+                                                       const int32_t* __restrict__ indptr,
+                                                       const int32_t* __restrict__ indices) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= m) return;
+  const int g = lane / G;
+  const int start = indptr[row], end = indptr[row + 1];
+  float4 acc[REP];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (!(split_long && end - start > kLongRow)) csr_accumulate<G, REP>(acc, start, end, feat, A, B, indices, lane);
   reduce_groups<G, REP>(acc, kWave);
   if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, false, nullptr);
+}
+
+// last r in [0, m] with indptr[r] <= q; all lanes pass the same q and get the same answer
+// (64 probes per step narrow the range 64-fold)
+__device__ __forceinline__ int wave_last_row(const int32_t* __restrict__ indptr, int m, int64_t q, int lane) {
+  int lo = 0, hi = m;
+  while (hi > lo) {
+    const int span = hi - lo;
+    const int pos = lo + (int)(((int64_t)span * (lane + 1) + kWave - 1) / kWave);  // in (lo, hi], ascending
+    const int cnt = __popcll(__ballot((int64_t)indptr[pos] <= q));
+    const int new_lo = cnt ? __shfl(pos, cnt - 1, kWave) : lo;
+    const int new_hi = cnt < kWave ? __shfl(pos, cnt, kWave) - 1 : hi;
+    lo = new_lo;
+    hi = new_hi;
+  }
+  return lo;
+}
+
+// One wavefront per kLongPiece consecutive nonzeros: the parts of rows longer than kLongRow that
+// fall into the piece are summed and added to C (cleared by csr_spmm_kernel) with atomics.
+// Pieces that touch no long row -- nearly all of them -- end after looking at their rows.
+template <int G, int REP>
+__global__ __launch_bounds__(256) void csr_long_rows_kernel(int m, int feat, int64_t first, int64_t nnz,
+                                                            const float* __restrict__ A,
+                                                            const float* __restrict__ B,
+                                                            float* __restrict__ C,
+                                                            const int32_t* __restrict__ indptr,
+                                                            const int32_t* __restrict__ indices) {
+  __shared__ float stage_all[4][kWave * 4 * REP];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t p0 = first + ((int64_t)blockIdx.x * 4 + wave) * kLongPiece;
+  const int64_t end_all = first + nnz;
+  if (p0 >= end_all) return;
+  const int64_t p1 = min(end_all, p0 + kLongPiece);
+  const int ra = wave_last_row(indptr, m, p0, lane);
+  const int rb = wave_last_row(indptr, m, p1 - 1, lane);
+  const int g = lane / G;
+  for (int r0 = ra; r0 <= rb; r0 += kWave) {
+    const int r = r0 + lane;
+    int rs = 0, re = 0;
+    if (r <= rb && r < m) rs = indptr[r], re = indptr[r + 1];
+    uint64_t todo = __ballot(re - rs > kLongRow);
+    while (todo) {
+      const int src = __ffsll((long long)todo) - 1;
+      todo &= todo - 1;
+      const int row = r0 + src;
+      const int64_t s = max((int64_t)__shfl(rs, src, kWave), p0);
+      const int64_t e = min((int64_t)__shfl(re, src, kWave), p1);
+      float4 acc[REP];
+#pragma unroll
+      for (int q = 0; q < REP; ++q) acc[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+      csr_accumulate<G, REP>(acc, (int)s, (int)e, feat, A, B, indices, lane);
+      reduce_groups<G, REP>(acc, kWave);
+      if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, true, stage_all[wave]);
+    }
+  }
 }
 
 // Any feature width: one wavefront per row, lane l owns features l, l+64, ...
@@ -363,8 +435,18 @@ int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const flo
   STIR_REQUIRE(d_B && d_C && d_indptr && (nnz == 0 || (d_A && d_indices)), "csr_spmm: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((unsigned)stir::ceil_div(m, 4)), block(256);
-#define STIR_CSR(G, REP) \
-  hipLaunchKernelGGL((csr_spmm_kernel<G, REP>), grid, block, 0, st, m, feat, d_A, d_B, d_C, d_indptr, d_indices)
+  // Hub rows are split over many wavefronts by a second launch; a matrix this small cannot hold
+  // a row long enough to matter against the extra launch.
+  const int split_long = nnz >= (int64_t(1) << 18) ? 1 : 0;
+  dim3 pieces((unsigned)stir::ceil_div(stir::ceil_div(nnz, kLongPiece), 4));
+#define STIR_CSR(G, REP)                                                                                   \
+  {                                                                                                        \
+    hipLaunchKernelGGL((csr_spmm_kernel<G, REP>), grid, block, 0, st, m, feat, split_long, d_A, d_B, d_C,  \
+                       d_indptr, d_indices);                                                               \
+    if (split_long)                                                                                        \
+      hipLaunchKernelGGL((csr_long_rows_kernel<G, REP>), pieces, block, 0, st, m, feat, (int64_t)0, nnz, d_A,   \
+                         d_B, d_C, d_indptr, d_indices);                                                   \
+  }
   switch (feat) {
     case 32: STIR_CSR(8, 1); break;
     case 64: STIR_CSR(16, 1); break;

@@ -81,6 +81,25 @@ def test_csr_spmm_long_row(dev):
     _check(got, indptr, indices, vals, x, "long row")
 
 
+@pytest.mark.parametrize("feat", [32, 128, 512])
+def test_csr_spmm_hub_rows_are_split(dev, feat):
+    """Enough nonzeros for the second launch that adds up rows longer than 256 entries in
+    256-entry pieces: hub rows of different lengths (piece boundaries inside, at the start and at
+    the end of rows), rows just below and above the limit, the output pre-filled with NaN."""
+    m, n = 4500, 40000
+    rng = np.random.default_rng(feat)
+    deg = rng.integers(0, 120, m)
+    for row, d in [(0, 257), (1, 256), (2, 2049), (7, 30000), (8, 2560), (1500, 12345), (m - 1, 5000)]:
+        deg[row] = d
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    assert indptr[-1] >= 1 << 18
+    indices = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
+    vals = (rng.random(len(indices), dtype=np.float32) - 0.3)
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    got = _run_csr(dev, indptr, indices, vals, x, feat)
+    _check(got, indptr, indices, vals, x, f"hub rows feat={feat}")
+
+
 def test_csr_spmm_argument_checks(dev):
     f = ops.build_csrmm(4, 4, 32, 3)
     z = lambda k, dt=torch.float32: torch.zeros(k, dtype=dt, device=dev)
