@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; scaled by a
 # plain copy of known size), keyed by workload signature.  None when not measured.
 MEASURED_TRAFFIC = {
-    # profiles/hyb_spmm_config3_uniform.md: FETCH_SIZE 15,740,117 KiB x 2.0 + WRITE_SIZE 1,266,962 KiB x 1.0
+    # profiles/hyb_spmm_config3_uniform.md: FETCH_SIZE 15,737,890 KiB x 2.0 + WRITE_SIZE 1,266,963 KiB x 1.0
     "uniform/p1/b1-2-4-8-16-32-64-128-256-512/f128/s1.0": 33.53e9,
 }
 
