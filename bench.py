@@ -154,6 +154,20 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
                            "ell_rows": int(sum(r.size for r in rows)),
                            "accumulation": "staged per ELL row, summed per output row (no atomics)"}
 
+    # SpMM over the condensed format (t = 32, g = 16) on the config-2 graph, fp16 in, fp32 out
+    g2 = datasets.config2()
+    gptr, tiles, cmask = st.condense(g2["indptr"], g2["indices"], 32, 16)
+    mb2, nnzb2, f2 = len(gptr) - 1, tiles.shape[0], 128
+    tc = ops.build_tcspmm(mb2, nnzb2, f2, 32, 16, g2["n"], torch.float32)
+    a2, b2 = t(cmask.astype(np.float16).ravel()), torch.randn(g2["n"] * f2, device=dev).half()
+    c2 = torch.zeros(mb2 * 32 * f2, device=dev)
+    gp, ti = t(gptr), t(tiles.ravel())
+    _, d, _ = time_steps(lambda: tc(a2, b2, c2, gp, ti), 50, 5, torch)
+    nnz2 = len(g2["indices"])
+    out["tcspmm_config2_feat128"] = {"us": d * 1e6, "useful_gflops": 2.0 * nnz2 * f2 / d / 1e9,
+                                     "mfma_tflops": 2.0 * nnzb2 * 32 * 16 * f2 / d / 1e12, "groups": int(nnzb2),
+                                     "mask_density": float(nnz2) / (nnzb2 * 32 * 16)}
+
     # fp32 forms: ELL3D buckets with 32-slot groups (the reference's composable fp32 setting) and the
     # CSF traversal; W is [R, fout, fin]
     w32 = t(np.ascontiguousarray(cfg["w"].transpose(0, 2, 1)).ravel())

@@ -234,3 +234,17 @@ def test_hyb_spmm_empty_and_degenerate(dev):
     x = np.ones((n, 32), np.float32)
     got, _ = _run_hyb(dev, m, n, 32, 2, [1, 2], triples, x)
     assert np.all(got == 0)
+
+
+def test_time_evaluator_protocol(dev):
+    """One discarded call, then the mean of `number` launches between device events
+    (the reference's f.time_evaluator(f.entry_name, dev, number=N), src/runtime/profiling.cc:742-797)."""
+    g = datasets.config1()
+    m, n, feat, nnz = g["m"], g["n"], g["feat"], len(g["indices"])
+    f = ops.build_csrmm(m, n, feat, nnz)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    c = torch.zeros(m * feat, device=dev)
+    secs = f.time_evaluator(number=20)(t(g["values"]), t(g["x"].ravel()), c, t(g["indptr"]), t(g["indices"]))
+    assert 0 < secs < 1e-2
+    assert f.entry_name == "main"
+    _check(c.cpu().numpy().reshape(m, feat), g["indptr"], g["indices"], g["values"], g["x"], "after timing")
