@@ -16,6 +16,7 @@
 // histogram plus the rank inside the wavefront, write row ids and padding; (4) scatter the
 // column ids and the mask, eight consecutive nonzeros per thread.
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "common.h"
@@ -71,9 +72,10 @@ Workspace carve(void* p, int32_t m, int32_t P, int32_t NB) {
   w.widths = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * NB));
   w.coarse = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kCoarse));
   w.status = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kStatusInts));
-  w.rows_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * size_t(P) * NB));
-  w.cols_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * size_t(P) * NB));
-  w.mask_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * size_t(P) * NB));
+  // the three pointer tables are contiguous so that one copy fills them
+  w.rows_tab = reinterpret_cast<int32_t**>(take(sizeof(void*) * 3 * size_t(P) * NB));
+  w.cols_tab = w.rows_tab ? w.rows_tab + size_t(P) * NB : nullptr;
+  w.mask_tab = w.rows_tab ? w.rows_tab + 2 * size_t(P) * NB : nullptr;
   w.bytes = off;
   return w;
 }
@@ -633,6 +635,36 @@ __global__ __launch_bounds__(256) void place_values_kernel(EntryArgs g, const fl
       [&](int k, int64_t slot) { out.at(k)[slot] = 0.f; });
 }
 
+// indptr[0] and indptr[m] as read by the sizing call, remembered per (workspace, indptr) so that
+// the fill calls for the same matrix need no device round trip of their own.
+struct EndsEntry {
+  const void* workspace;
+  const void* indptr;
+  int32_t num_rows;
+  int32_t ends[2];
+};
+std::mutex g_ends_mutex;
+EndsEntry g_ends[8];
+int g_ends_next = 0;
+
+void remember_ends(const void* ws, const void* indptr, int32_t m, const int32_t (&ends)[2]) {
+  std::lock_guard<std::mutex> lock(g_ends_mutex);
+  for (EndsEntry& e : g_ends)
+    if (e.workspace == ws) e.workspace = nullptr;  // the workspace now describes another matrix
+  g_ends[g_ends_next] = EndsEntry{ws, indptr, m, {ends[0], ends[1]}};
+  g_ends_next = (g_ends_next + 1) % 8;
+}
+
+bool recall_ends(const void* ws, const void* indptr, int32_t m, int32_t (&ends)[2]) {
+  std::lock_guard<std::mutex> lock(g_ends_mutex);
+  for (const EndsEntry& e : g_ends)
+    if (e.workspace == ws && e.indptr == indptr && e.num_rows == m) {
+      ends[0] = e.ends[0], ends[1] = e.ends[1];
+      return true;
+    }
+  return false;
+}
+
 int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t parts, const int32_t* buckets,
                int32_t nb) {
   STIR_REQUIRE(num_rows >= 0 && num_cols >= 0, "%s: bad matrix shape %d x %d", who, num_rows, num_cols);
@@ -707,6 +739,7 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
                "%s: column indices must ascend inside each row (use the host routine for unsorted rows)", who);
   for (int k = 0; k < P * NB; ++k)
     STIR_REQUIRE(nrows[k] < kMaxSlots / buckets[k % NB], "%s: bucket %d holds too many slots", who, k);
+  remember_ends(d_workspace, d_indptr, m, ends);
   return 0;
 }
 
@@ -724,13 +757,18 @@ int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols, const i
   Workspace ws = carve(d_workspace, m, P, NB);
   const int64_t W = stir::ceil_div(m, kWave);
   int32_t ends[2];
-  STIR_HIP(hipMemcpyAsync(&ends[0], d_indptr, sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  STIR_HIP(hipMemcpyAsync(&ends[1], d_indptr + m, sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  const size_t tab = sizeof(void*) * size_t(P) * NB;
-  STIR_HIP(hipMemcpyAsync(ws.rows_tab, d_row_indices, tab, hipMemcpyHostToDevice, st));
-  STIR_HIP(hipMemcpyAsync(ws.cols_tab, d_col_indices, tab, hipMemcpyHostToDevice, st));
-  STIR_HIP(hipMemcpyAsync(ws.mask_tab, d_mask, tab, hipMemcpyHostToDevice, st));
-  STIR_HIP(hipStreamSynchronize(st));
+  const bool known = recall_ends(d_workspace, d_indptr, m, ends);
+  if (!known) {
+    STIR_HIP(hipMemcpyAsync(&ends[0], d_indptr, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    STIR_HIP(hipMemcpyAsync(&ends[1], d_indptr + m, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  }
+  const size_t pnb = size_t(P) * NB;
+  std::vector<int32_t*> tabs(3 * pnb);
+  std::copy(d_row_indices, d_row_indices + pnb, tabs.begin());
+  std::copy(d_col_indices, d_col_indices + pnb, tabs.begin() + pnb);
+  std::copy(d_mask, d_mask + pnb, tabs.begin() + 2 * pnb);
+  STIR_HIP(hipMemcpyAsync(ws.rows_tab, tabs.data(), sizeof(void*) * 3 * pnb, hipMemcpyHostToDevice, st));
+  STIR_HIP(hipStreamSynchronize(st));  // `tabs` and `ends` are host stack/heap of this call
   const int64_t nnz = (int64_t)ends[1] - ends[0];
   if (nnz <= 0) return 0;
   const int psize = (num_cols + P - 1) / P;
@@ -763,8 +801,10 @@ int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const
   hipStream_t st = static_cast<hipStream_t>(stream);
   Workspace ws = carve(d_workspace, m, P, NB);
   int32_t ends[2];
-  STIR_HIP(hipMemcpyAsync(&ends[0], d_indptr, sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  STIR_HIP(hipMemcpyAsync(&ends[1], d_indptr + m, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  if (!recall_ends(d_workspace, d_indptr, m, ends)) {
+    STIR_HIP(hipMemcpyAsync(&ends[0], d_indptr, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    STIR_HIP(hipMemcpyAsync(&ends[1], d_indptr + m, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  }
   // the A_k pointer table reuses the slot of the mask table (same size, no longer needed)
   STIR_HIP(hipMemcpyAsync(ws.mask_tab, d_A, sizeof(void*) * size_t(P) * NB, hipMemcpyHostToDevice, st));
   STIR_HIP(hipStreamSynchronize(st));

@@ -101,11 +101,19 @@ def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, 
             num_rows, num_cols, ctypes.c_void_p(indptr.data_ptr()),
             ctypes.c_void_p(indices.data_ptr()), num_col_parts, _vp(widths), nb,
             ctypes.c_void_p(ws.data_ptr()), _vp(nrows), stream))
-        rows = [torch.empty(int(nrows[k]), dtype=torch.int32, device=dev) for k in range(nk)]
-        cols = [torch.empty((int(nrows[k]), int(widths[k % nb])), dtype=torch.int32, device=dev)
-                for k in range(nk)]
-        mask = [torch.empty((int(nrows[k]), int(widths[k % nb])), dtype=torch.int32, device=dev)
-                for k in range(nk)]
+        # one allocation per kind, the buckets are 256-byte aligned views into it
+        def carve(dtype, shapes):
+            offs, total = [], 0
+            for shp in shapes:
+                offs.append(total)
+                total += (int(np.prod(shp)) + 63) // 64 * 64
+            pool = torch.empty(max(total, 1), dtype=dtype, device=dev)
+            return [pool[o:o + int(np.prod(shp))].view(shp) for o, shp in zip(offs, shapes)]
+
+        wide = [(int(nrows[k]), int(widths[k % nb])) for k in range(nk)]
+        rows = carve(torch.int32, [(int(nrows[k]),) for k in range(nk)])
+        cols = carve(torch.int32, wide)
+        mask = carve(torch.int32, wide)
         _lib.check(L.stir_column_part_hyb_device_fill(
             num_rows, num_cols, ctypes.c_void_p(indptr.data_ptr()),
             ctypes.c_void_p(indices.data_ptr()), num_col_parts, _vp(widths), nb,
@@ -118,8 +126,7 @@ def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, 
             if not _is_cuda_tensor(values) or values.dtype != torch.float32 or values.numel() != indices.numel():
                 raise _lib.SparseTIRError("ColumnPartHyb: values must be a float32 CUDA tensor aligned with indices")
             values = values.contiguous()
-            avals = [torch.empty((int(nrows[k]), int(widths[k % nb])), dtype=torch.float32, device=dev)
-                     for k in range(nk)]
+            avals = carve(torch.float32, wide)
             _lib.check(L.stir_column_part_hyb_device_values(
                 num_rows, num_cols, ctypes.c_void_p(indptr.data_ptr()),
                 ctypes.c_void_p(indices.data_ptr()), ctypes.c_void_p(values.data_ptr()),
