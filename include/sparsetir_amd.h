@@ -81,8 +81,9 @@ int stir_condense_fill(int32_t n, const int32_t* indptr, const int32_t* indices,
 
 /*
  * ColumnPartHyb on the GPU, bit-exact with the host routine above for CSR input whose
- * column indices ascend within each row (the reference runs this on the CPU only,
- * src/sparse/format.cc:58-59; unsorted rows are reported as an error here).
+ * column indices ascend within each row, and for any column order when num_col_parts is 1
+ * (the reference runs this on the CPU only, src/sparse/format.cc:58-59; unsorted rows with
+ * several partitions are reported as an error here).
  * d_workspace must hold stir_column_part_hyb_device_workspace_bytes(...) bytes and must
  * stay untouched between the _sizes and the _fill call.  _sizes synchronises the stream
  * to return nrows on the host; _fill writes device arrays through host tables of

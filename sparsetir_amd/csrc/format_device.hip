@@ -735,7 +735,8 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
   }
   STIR_REQUIRE(!(status & kStatusIndptr), "%s: indptr is not a CSR row pointer (it decreases)", who);
   STIR_REQUIRE(!(status & kStatusRange), "%s: a column index lies outside [0, %d)", who, num_cols);
-  STIR_REQUIRE(descents == row_start_descents,
+  // with one partition a run is the whole row whatever the order of its columns
+  STIR_REQUIRE(P == 1 || descents == row_start_descents,
                "%s: column indices must ascend inside each row (use the host routine for unsorted rows)", who);
   for (int k = 0; k < P * NB; ++k)
     STIR_REQUIRE(nrows[k] < kMaxSlots / buckets[k % NB], "%s: bucket %d holds too many slots", who, k);

@@ -57,6 +57,18 @@ def test_device_column_part_hyb_config2(dev):
     assert np.array_equal(decode_hyb(*got), coo_pairs(g["indptr"], g["indices"]))
 
 
+def test_device_column_part_hyb_one_partition_takes_unsorted_rows(dev):
+    """With one partition a (row, partition) run is the whole row, so the column order inside
+    rows does not matter: same arrays as the sequential routine."""
+    for m, n, nnz, buckets, seed in [(50, 40, 600, [1, 2, 4], 3), (3000, 900, 90000, [1, 2, 4, 8, 16, 32], 4)]:
+        indptr, indices = random_csr(m, n, nnz, seed, sort=False, skew=1.0)
+        got = _device_hyb(dev, m, n, indptr, indices, 1, buckets)
+        want = oracle.column_part_hyb(m, n, indptr, indices, 1, buckets)
+        for gq, wq in zip(got, want):
+            for a, b in zip(gq[0], wq[0]):
+                assert np.array_equal(a, b)
+
+
 def test_device_column_part_hyb_rejects_unsorted_and_out_of_range(dev):
     indptr, indices = random_csr(50, 40, 600, 3, sort=False)
     with pytest.raises(SparseTIRError, match="ascend"):
