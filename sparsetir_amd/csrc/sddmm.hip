@@ -62,8 +62,10 @@ __global__ __launch_bounds__(256) void sddmm_kernel(int64_t nnz, int feat, const
       const float* bp = B + (int64_t)col * feat + gl * 4;
 #pragma unroll
       for (int q = 0; q < REP; ++q) {
-        a[u][q] = ld4(ap + q * G * 4);
-        b[u][q] = ld4(bp + q * G * 4);
+        // feat below 4*G*REP: the lanes beyond feat / 4 hold padding
+        const bool live = gl * 4 + q * G * 4 < feat;
+        a[u][q] = live ? ld4(ap + q * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        b[u][q] = live ? ld4(bp + q * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     }
 #pragma unroll
@@ -208,13 +210,19 @@ static int sddmm_launch(int32_t m, int32_t n, int32_t feat, int64_t nnz, const f
 #define STIR_SDDMM(G, REP)                                                                             \
   hipLaunchKernelGGL((sddmm_kernel<G, REP>), grid, block, 0, st, nnz, feat, d_A, d_B, d_C, d_indices, d_mid, \
                      d_scale)
-  switch (feat) {
-    case 16: STIR_SDDMM(4, 1); break;
-    case 32: STIR_SDDMM(8, 1); break;
-    case 64: STIR_SDDMM(16, 1); break;
-    case 128: STIR_SDDMM(32, 1); break;
-    case 256: STIR_SDDMM(64, 1); break;
-    case 512: STIR_SDDMM(64, 2); break;
+  // feature widths that are a multiple of 4 take the vectorised kernel with the smallest lane
+  // group that covers them; anything else the generic one
+  int cls = -1;
+  if (feat % 4 == 0 && feat <= 512)
+    for (cls = 0; (16 << cls) < feat; ++cls) {
+    }
+  switch (cls) {
+    case 0: STIR_SDDMM(4, 1); break;
+    case 1: STIR_SDDMM(8, 1); break;
+    case 2: STIR_SDDMM(16, 1); break;
+    case 3: STIR_SDDMM(32, 1); break;
+    case 4: STIR_SDDMM(64, 1); break;
+    case 5: STIR_SDDMM(64, 2); break;
     default:
       hipLaunchKernelGGL(sddmm_generic_kernel, grid, block, 0, st, nnz, feat, d_A, d_B, d_C, d_indices, d_mid,
                          d_scale);

@@ -73,6 +73,7 @@ __device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int l
     float* base = C + row * feat + gl * 4;
 #pragma unroll
     for (int r = 0; r < REP; ++r) {
+      if (gl * 4 + r * G * 4 >= feat) continue;  // feat below 4*G*REP: this lane's float4 is padding
       float* q = base + r * G * 4;
       __builtin_nontemporal_store(acc[r].x, q);
       __builtin_nontemporal_store(acc[r].y, q + 1);
@@ -91,7 +92,8 @@ __device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int l
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const float v = stage[(r * kWave + g * G) * 4 + k * G + gl];
-      __hip_atomic_fetch_add(base + r * G * 4 + k * G, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (r * G * 4 + k * G + gl < feat)
+        __hip_atomic_fetch_add(base + r * G * 4 + k * G, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -122,7 +124,7 @@ __device__ __forceinline__ void csr_accumulate(float4 (&acc)[REP], int start, in
         const float* bp = B + (int64_t)col * feat + gl * 4;
 #pragma unroll
         for (int r = 0; r < REP; ++r)
-          x[u][r] = (j < cnt) ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+          x[u][r] = (j < cnt && gl * 4 + r * G * 4 < feat) ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u)
@@ -273,7 +275,8 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
       // a slot of weight zero (padding) adds nothing: its row of B is not fetched
 #pragma unroll
       for (int r = 0; r < REP; ++r)
-        x[u][r] = v[u] != 0.f ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        x[u][r] = (v[u] != 0.f && gl * 4 + r * G * 4 < feat) ? ld4(bp + r * G * 4)
+                                                             : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int u = 0; u < CH; ++u) {
@@ -332,7 +335,8 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
         const float* bp = B + (int64_t)col * feat + gl * 4;
 #pragma unroll
         for (int r = 0; r < REP; ++r)
-          x[u][r] = v[u] != 0.f ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+          x[u][r] = (v[u] != 0.f && gl * 4 + r * G * 4 < feat) ? ld4(bp + r * G * 4)
+                                                             : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int u = 0; u < CH; ++u)
@@ -408,6 +412,14 @@ __global__ __launch_bounds__(256) void hyb_spmm_generic_kernel(const HybBucket* 
   }
 }
 
+// 0..5: lane groups of 4, 8, 16, 32, 64 lanes and 64 lanes x 2 float4 cover feat; -1: generic kernel
+int vector_class(int feat) {
+  if (feat % 4 != 0 || feat > 512) return -1;
+  int c = 0;
+  while ((16 << c) < feat) ++c;
+  return c;
+}
+
 int log2_exact(int64_t x) {
   int l = 0;
   while ((int64_t(1) << l) < x) ++l;
@@ -447,12 +459,15 @@ int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const flo
       hipLaunchKernelGGL((csr_long_rows_kernel<G, REP>), pieces, block, 0, st, m, feat, (int64_t)0, nnz, d_A,   \
                          d_B, d_C, d_indptr, d_indices);                                                   \
   }
-  switch (feat) {
-    case 32: STIR_CSR(8, 1); break;
-    case 64: STIR_CSR(16, 1); break;
-    case 128: STIR_CSR(32, 1); break;
-    case 256: STIR_CSR(64, 1); break;
-    case 512: STIR_CSR(64, 2); break;
+  // feature widths that are a multiple of 4 take the vectorised kernel with the smallest lane
+  // group that covers them (lanes beyond feat / 4 idle); anything else the generic one
+  switch (vector_class(feat)) {
+    case 0: STIR_CSR(4, 1); break;
+    case 1: STIR_CSR(8, 1); break;
+    case 2: STIR_CSR(16, 1); break;
+    case 3: STIR_CSR(32, 1); break;
+    case 4: STIR_CSR(64, 1); break;
+    case 5: STIR_CSR(64, 2); break;
     default:
       hipLaunchKernelGGL(csr_spmm_generic_kernel, grid, block, 0, st, m, feat, d_A, d_B, d_C, d_indptr, d_indices);
   }
@@ -552,12 +567,13 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
 #define STIR_HYB(G, REP)                                                                        \
   hipLaunchKernelGGL((hyb_spmm_kernel<G, REP>), grid, block, 0, st, plan->d_table_tiles, plan->nk, \
                      plan->total_tiles, feat, d_B, d_C)
-  switch (feat) {
-    case 32: STIR_HYB(8, 1); break;
-    case 64: STIR_HYB(16, 1); break;
-    case 128: STIR_HYB(32, 1); break;
-    case 256: STIR_HYB(64, 1); break;
-    case 512: STIR_HYB(64, 2); break;
+  switch (vector_class(feat)) {
+    case 0: STIR_HYB(4, 1); break;
+    case 1: STIR_HYB(8, 1); break;
+    case 2: STIR_HYB(16, 1); break;
+    case 3: STIR_HYB(32, 1); break;
+    case 4: STIR_HYB(64, 1); break;
+    case 5: STIR_HYB(64, 2); break;
     default: {
       const int64_t rb = stir::ceil_div(plan->total_rows, 4);
       STIR_REQUIRE(rb < (int64_t(1) << 31), "hyb_spmm: %lld rows exceed one launch", (long long)plan->total_rows);

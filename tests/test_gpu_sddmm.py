@@ -26,7 +26,7 @@ def _run(dev, indptr, indices, a, b, feat):
     return c.cpu().numpy(), mid.cpu().numpy()
 
 
-@pytest.mark.parametrize("feat", [16, 32, 64, 128, 256, 512, 40, 3])
+@pytest.mark.parametrize("feat", [16, 32, 64, 128, 256, 512, 40, 3, 4, 96, 384, 260])
 def test_sddmm_feature_widths(dev, feat):
     m, n = 901, 1203
     indptr, indices = random_csr(m, n, 25000, feat, skew=1.1)

@@ -46,7 +46,7 @@ def test_csr_spmm_config1(dev):
     assert np.all(np.abs(got - ref) <= 2 * RTOL * scale)
 
 
-@pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 48, 20, 1])
+@pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 48, 20, 1, 4, 16, 96, 384, 260, 516])
 def test_csr_spmm_feature_widths(dev, feat):
     m, n = 1003, 777
     indptr, indices = random_csr(m, n, 30000, feat, skew=1.2)
@@ -81,7 +81,7 @@ def test_csr_spmm_long_row(dev):
     _check(got, indptr, indices, vals, x, "long row")
 
 
-@pytest.mark.parametrize("feat", [32, 128, 512])
+@pytest.mark.parametrize("feat", [32, 128, 512, 96])
 def test_csr_spmm_hub_rows_are_split(dev, feat):
     """Enough nonzeros for the second launch that adds up rows longer than 256 entries in
     256-entry pieces: hub rows of different lengths (piece boundaries inside, at the start and at
@@ -165,7 +165,7 @@ def _hyb_as_coo(triples_np):
     return np.concatenate(rr), np.concatenate(cc), np.concatenate(vv)
 
 
-@pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 96, 7])
+@pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 96, 7, 4, 16, 40, 384])
 @pytest.mark.parametrize("parts,buckets", [(1, [1, 2, 4, 8, 16, 32]), (2, [1, 2, 4, 8, 16, 32, 64, 128, 256, 512]),
                                            (4, [2, 3, 7]), (3, [1])])
 def test_hyb_spmm_matches_oracle(dev, feat, parts, buckets):
