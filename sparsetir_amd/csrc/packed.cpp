@@ -75,6 +75,11 @@ struct Args {
                   name, code, bits, d->dtype.code, d->dtype.bits, d->dtype.lanes);
       return a;
     }
+    if (d->shape[0] < 0) {
+      ok = false;
+      packed_fail("%s: %s.shape[0]=%lld is negative", fn, name, (long long)d->shape[0]);
+      return a;
+    }
     if (d->strides && d->shape[0] > 1 && d->strides[0] != 1) {
       ok = false;
       packed_fail("%s: %s.strides: expected to be compact array", fn, name);
