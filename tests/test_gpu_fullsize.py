@@ -130,3 +130,51 @@ def test_config5_rgms_full(dev):
     assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30)
     ref = oracle.rgms(w32, x32, ones, *csf, n)
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-5 * scale + 1e-30)
+
+
+def test_offsets_beyond_2_to_31_elements(dev):
+    """X with 2.3e9 floats (9.2 GB): rows of X that start beyond the 2^31-th element must be
+    reached with 64-bit offsets by the CSR, hyb and SDDMM kernels.  Checked against torch's own
+    gathers on the device."""
+    n, feat, m = 18_000_000, 128, 2048
+    assert n * feat > 2**31
+    gen = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn(n * feat, device=dev, generator=gen)
+    rng = np.random.default_rng(11)
+    deg = rng.integers(1, 40, m)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    # most columns near the end of X, a few near the start
+    cols = [np.sort(rng.choice(np.concatenate([np.arange(n - 200000, n), np.arange(0, 1000)]), d, replace=False))
+            for d in deg]
+    indices = np.concatenate(cols).astype(np.int32)
+    nnz = len(indices)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    d_ptr, d_idx = t(indptr), t(indices)
+    vals = torch.rand(nnz, device=dev, generator=gen) + 0.5
+    rowid = torch.repeat_interleave(torch.arange(m, device=dev), t(deg.astype(np.int64)))
+    want = torch.zeros(m, feat, device=dev, dtype=torch.float64)
+    want.index_add_(0, rowid, (x.view(n, feat)[d_idx.long()] * vals[:, None]).double())
+    scale = torch.zeros(m, feat, device=dev, dtype=torch.float64)
+    scale.index_add_(0, rowid, (x.view(n, feat)[d_idx.long()] * vals[:, None]).abs().double())
+
+    c = torch.empty(m * feat, device=dev)
+    ops.build_csrmm(m, n, feat, nnz)(vals, x, c, d_ptr, d_idx)
+    assert torch.all((c.view(m, feat).double() - want).abs() <= 1e-5 * scale + 1e-30)
+
+    buckets = [1, 2, 4, 8, 16, 32, 64]
+    rows, cols_k, mask, avals = st.column_part_hyb(m, n, d_ptr, d_idx, 1, buckets, values=vals)
+    triples = [a for b in range(len(buckets)) for a in (avals[0][b].reshape(-1), rows[0][b], cols_k[0][b].reshape(-1))]
+    c2 = torch.zeros(m * feat, device=dev)
+    ops.build_hyb_csrmm(m, n, feat, 1, buckets, [int(r.shape[0]) for r in rows[0]])(x, c2, *triples)
+    assert torch.all((c2.view(m, feat).double() - want).abs() <= 1e-5 * scale + 1e-30)
+
+    a = torch.randn(m * feat, device=dev, generator=gen)
+    out = torch.empty(nnz, device=dev)
+    mid = torch.empty(nnz, dtype=torch.int32, device=dev)
+    args = (a, x, out, d_ptr, d_idx, mid)
+    ops.build_sddmm_preproc(m, n, feat, nnz)(*args)
+    ops.build_sddmm(m, n, feat, nnz)(*args)
+    torch.cuda.synchronize()
+    ref = (a.view(m, feat)[rowid].double() * x.view(n, feat)[d_idx.long()].double()).sum(1)
+    mag = (a.view(m, feat)[rowid].double() * x.view(n, feat)[d_idx.long()].double()).abs().sum(1)
+    assert torch.all((out.double() - ref).abs() <= 1e-5 * mag + 1e-30)
