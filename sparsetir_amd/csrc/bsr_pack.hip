@@ -7,6 +7,7 @@
 // ascending order are the block column indices, and a nonzero's block position is its block
 // row's offset plus the number of set bits below its block column.
 #include "common.h"
+#include "row_lookup.h"
 #include "../../include/sparsetir_amd.h"
 
 namespace {
@@ -43,28 +44,39 @@ PackWs carve(void* p, int64_t mb, int64_t W) {
   return w;
 }
 
-__device__ __forceinline__ int row_of(const int32_t* indptr, int m, int64_t e) {
-  int a = 0, b = m;  // last r with indptr[r] <= e
-  while (a < b) {
-    const int mid = a + ((b - a + 1) >> 1);
-    if ((int64_t)indptr[mid] <= e) a = mid; else b = mid - 1;
-  }
-  return a;
-}
+constexpr int kPackPerLane = 8;  // a wavefront owns 64 * kPackPerLane consecutive nonzeros
 
+// Sets the bit of every nonzero's block.  Neighbouring lanes hold neighbouring nonzeros, which
+// mostly fall into the same block: only the first lane of a run of equal (word, bit) acts, and it
+// reads the word first and skips the atomic when the bit is already there -- a block of 1024
+// nonzeros costs a handful of atomics instead of 1024 on one address.
 __global__ __launch_bounds__(256) void mark_kernel(int m, int n, int blk, int64_t W, int64_t nnz, int32_t first,
                                                    const int32_t* __restrict__ indptr,
                                                    const int32_t* __restrict__ indices,
                                                    uint32_t* __restrict__ bits, int32_t* __restrict__ status) {
-  const int64_t e = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= first + nnz) return;
-  const int col = indices[e];
-  if (col < 0 || col >= n) {
-    atomicOr(status, 1);
-    return;
-  }
-  const int I = row_of(indptr, m, e) / blk, J = col / blk;
-  atomicOr(&bits[(int64_t)I * W + (J >> 5)], 1u << (J & 31));
+  __shared__ int32_t win_all[4][stir::kRowLookupWindow];
+  const int lane = threadIdx.x & 63;
+  const int64_t end = first + nnz;
+  const int64_t e0 = first + ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (kWave * kPackPerLane);
+  if (e0 >= end) return;
+  const int64_t e_last = min(end, e0 + kWave * kPackPerLane) - 1;
+  stir::for_each_nonzero_row<kPackPerLane>(indptr, m, e0, e_last, win_all[threadIdx.x >> 6], lane,
+                                           [&](int64_t e, int row, int, bool live) {
+    int64_t key = -1;  // (word index, bit); -1: nothing to set
+    if (live) {
+      const int col = indices[e];
+      if (col < 0 || col >= n)
+        atomicOr(status, 1);
+      else
+        key = (((int64_t)(row / blk) * W + (col / blk >> 5)) << 5) | (col / blk & 31);
+    }
+    const int64_t before = __shfl_up(key, 1, kWave);
+    if (key >= 0 && (lane == 0 || before != key)) {
+      uint32_t* word = &bits[key >> 5];
+      const uint32_t bit = 1u << (key & 31);
+      if (!(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit)) atomicOr(word, bit);
+    }
+  });
 }
 
 // One wavefront per block row: popcount per word, exclusive prefix over the words.
@@ -159,14 +171,21 @@ __global__ __launch_bounds__(256) void scatter_kernel(int m, int blk, int64_t W,
                                                       const uint32_t* __restrict__ bits,
                                                       const int32_t* __restrict__ wprefix,
                                                       const int32_t* __restrict__ bsr_indptr, T* __restrict__ data) {
-  const int64_t e = first + (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= first + nnz) return;
-  const int col = indices[e];
-  const int row = row_of(indptr, m, e);
-  const int I = row / blk, J = col / blk;
-  const int64_t cell = (int64_t)I * W + (J >> 5);
-  const int64_t pos = (int64_t)bsr_indptr[I] + wprefix[cell] + __popc(bits[cell] & ((1u << (J & 31)) - 1u));
-  data[(pos * blk + (row - I * blk)) * blk + (col - J * blk)] = convert<T>(values[e]);
+  __shared__ int32_t win_all[4][stir::kRowLookupWindow];
+  const int lane = threadIdx.x & 63;
+  const int64_t end = first + nnz;
+  const int64_t e0 = first + ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (kWave * kPackPerLane);
+  if (e0 >= end) return;
+  const int64_t e_last = min(end, e0 + kWave * kPackPerLane) - 1;
+  stir::for_each_nonzero_row<kPackPerLane>(indptr, m, e0, e_last, win_all[threadIdx.x >> 6], lane,
+                                           [&](int64_t e, int row, int, bool live) {
+    if (!live) return;
+    const int col = indices[e];
+    const int I = row / blk, J = col / blk;
+    const int64_t cell = (int64_t)I * W + (J >> 5);
+    const int64_t pos = (int64_t)bsr_indptr[I] + wprefix[cell] + __popc(bits[cell] & ((1u << (J & 31)) - 1u));
+    data[(pos * blk + (row - I * blk)) * blk + (col - J * blk)] = convert<T>(values[e]);
+  });
 }
 
 int check(const char* who, int32_t m, int32_t n, int32_t blk) {
@@ -216,7 +235,7 @@ int stir_csr_to_bsr_sizes(int32_t m, int32_t n, int32_t blk, const int32_t* d_in
   STIR_HIP(hipMemsetAsync(ws.bits, 0, size_t(mb) * size_t(W > 0 ? W : 1) * 4, st));
   STIR_HIP(hipMemsetAsync(ws.status, 0, 4, st));
   if (nnz > 0) {
-    hipLaunchKernelGGL(mark_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, m, n, blk, W, nnz,
+    hipLaunchKernelGGL(mark_kernel, dim3((unsigned)stir::ceil_div(nnz, 4 * kWave * kPackPerLane)), dim3(256), 0, st, m, n, blk, W, nnz,
                        first, d_indptr, d_indices, ws.bits, ws.status);
     STIR_LAUNCH_CHECK();
   }
@@ -257,7 +276,7 @@ int stir_csr_to_bsr_fill(int32_t m, int32_t n, int32_t blk, const int32_t* d_ind
                      ws.bits, ws.wprefix, d_bsr_indptr, d_bsr_indices);
   STIR_LAUNCH_CHECK();
   if (nnz > 0) {
-    dim3 grid((unsigned)stir::ceil_div(nnz, 256)), block(256);
+    dim3 grid((unsigned)stir::ceil_div(nnz, 4 * kWave * kPackPerLane)), block(256);
 #define STIR_SCATTER(T)                                                                                    \
   hipLaunchKernelGGL((scatter_kernel<T>), grid, block, 0, st, m, blk, W, nnz, first, d_indptr, d_indices,  \
                      d_values, ws.bits, ws.wprefix, d_bsr_indptr, static_cast<T*>(d_bsr_data))

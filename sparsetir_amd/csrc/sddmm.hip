@@ -8,6 +8,7 @@
 // of a group keeps the result of the group's j-th nonzero, so the 64 results leave with one
 // coalesced store.
 #include "common.h"
+#include "row_lookup.h"
 #include "../../include/sparsetir_amd.h"
 
 namespace {
@@ -108,76 +109,21 @@ __global__ __launch_bounds__(256) void sddmm_generic_kernel(int64_t nnz, int fea
   if (lane < cnt) C[e0 + lane] = scale ? out * scale[e0 + lane] : out;
 }
 
-// Row lookup mid[e] = upper_bound(indptr, e) - 1 for 512 consecutive nonzeros per wavefront.
-// The rows of the first and the last nonzero are found by the whole wavefront (64 probes of
-// indptr per step narrow the range 64-fold, so a few dependent loads replace the ~log2(m) of a
-// per-nonzero binary search); the row pointers in between go to LDS with one coalesced load and
-// every nonzero is then located there.  A span with more rows than the window holds (long runs
-// of empty rows) falls back to a per-nonzero search between the two rows.
+// Row lookup mid[e] = upper_bound(indptr, e) - 1, 512 consecutive nonzeros per wavefront.
 constexpr int kMidPerLane = 8;
-constexpr int kMidWindow = 512;
-
-// last r in [0, m] with indptr[r] <= q; all lanes pass the same q and get the same answer
-__device__ __forceinline__ int wave_last_row(const int32_t* __restrict__ indptr, int m, int64_t q, int lane) {
-  int lo = 0, hi = m;  // indptr[lo] <= q, the answer lies in [lo, hi]
-  while (hi > lo) {
-    const int span = hi - lo;
-    const int pos = lo + (int)(((int64_t)span * (lane + 1) + kWave - 1) / kWave);  // in (lo, hi], ascending
-    const bool le = (int64_t)indptr[pos] <= q;
-    const int cnt = __popcll(__ballot(le));  // the predicate is true for the first cnt lanes
-    const int new_lo = cnt ? __shfl(pos, cnt - 1, kWave) : lo;
-    const int new_hi = cnt < kWave ? __shfl(pos, cnt, kWave) - 1 : hi;
-    lo = new_lo;
-    hi = new_hi;
-  }
-  return lo;
-}
 
 __global__ __launch_bounds__(256) void sddmm_preproc_kernel(int m, int64_t nnz,
                                                             const int32_t* __restrict__ indptr,
                                                             int32_t* __restrict__ mid) {
-  __shared__ int32_t win_all[4][kMidWindow + 1];
+  __shared__ int32_t win_all[4][stir::kRowLookupWindow];
   const int lane = threadIdx.x & 63;
-  int32_t* win = win_all[threadIdx.x >> 6];
   const int64_t e0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (kWave * kMidPerLane);
   if (e0 >= nnz) return;
   const int64_t e_last = min(nnz, e0 + kWave * kMidPerLane) - 1;
-  const int ra = wave_last_row(indptr, m, e0, lane);
-  const int rb = wave_last_row(indptr, m, e_last, lane);
-  const int nr = rb - ra + 1;
-  if (nr <= kMidWindow) {
-    for (int x = lane; x < nr; x += kWave) win[x] = indptr[ra + x];
-    __builtin_amdgcn_wave_barrier();
-    int steps = 0;
-    while ((1 << steps) < nr) ++steps;
-    int a[kMidPerLane], b[kMidPerLane];
-#pragma unroll
-    for (int t = 0; t < kMidPerLane; ++t) a[t] = 0, b[t] = nr - 1;
-    for (int it = 0; it < steps; ++it) {
-#pragma unroll
-      for (int t = 0; t < kMidPerLane; ++t) {
-        const int c = (a[t] + b[t] + 1) >> 1;
-        if ((int64_t)win[c] <= e0 + t * kWave + lane) a[t] = c; else b[t] = c - 1;
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < kMidPerLane; ++t) {
-      const int64_t e = e0 + t * kWave + lane;
-      if (e <= e_last) mid[e] = ra + a[t];
-    }
-  } else {
-#pragma unroll 1
-    for (int t = 0; t < kMidPerLane; ++t) {
-      const int64_t e = e0 + t * kWave + lane;
-      if (e > e_last) continue;
-      int a = ra, b = rb;
-      while (a < b) {
-        const int c = a + ((b - a + 1) >> 1);
-        if ((int64_t)indptr[c] <= e) a = c; else b = c - 1;
-      }
-      mid[e] = a;
-    }
-  }
+  stir::for_each_nonzero_row<kMidPerLane>(indptr, m, e0, e_last, win_all[threadIdx.x >> 6], lane,
+                                          [&](int64_t e, int row, int, bool live) {
+                                            if (live) mid[e] = row;
+                                          });
 }
 
 }  // namespace

@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "common.h"
+#include "row_lookup.h"
 #include "../../include/sparsetir_amd.h"
 
 namespace {
@@ -161,22 +162,6 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, int spli
   if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, false, nullptr);
 }
 
-// last r in [0, m] with indptr[r] <= q; all lanes pass the same q and get the same answer
-// (64 probes per step narrow the range 64-fold)
-__device__ __forceinline__ int wave_last_row(const int32_t* __restrict__ indptr, int m, int64_t q, int lane) {
-  int lo = 0, hi = m;
-  while (hi > lo) {
-    const int span = hi - lo;
-    const int pos = lo + (int)(((int64_t)span * (lane + 1) + kWave - 1) / kWave);  // in (lo, hi], ascending
-    const int cnt = __popcll(__ballot((int64_t)indptr[pos] <= q));
-    const int new_lo = cnt ? __shfl(pos, cnt - 1, kWave) : lo;
-    const int new_hi = cnt < kWave ? __shfl(pos, cnt, kWave) - 1 : hi;
-    lo = new_lo;
-    hi = new_hi;
-  }
-  return lo;
-}
-
 // One wavefront per kLongPiece consecutive nonzeros: the parts of rows longer than kLongRow that
 // fall into the piece are summed and added to C (cleared by csr_spmm_kernel) with atomics.
 // Pieces that touch no long row -- nearly all of them -- end after looking at their rows.
@@ -194,8 +179,8 @@ __global__ __launch_bounds__(256) void csr_long_rows_kernel(int m, int feat, int
   const int64_t end_all = first + nnz;
   if (p0 >= end_all) return;
   const int64_t p1 = min(end_all, p0 + kLongPiece);
-  const int ra = wave_last_row(indptr, m, p0, lane);
-  const int rb = wave_last_row(indptr, m, p1 - 1, lane);
+  const int ra = stir::wave_last_row(indptr, m, p0, lane);
+  const int rb = stir::wave_last_row(indptr, m, p1 - 1, lane);
   const int g = lane / G;
   for (int r0 = ra; r0 <= rb; r0 += kWave) {
     const int r = r0 + lane;
