@@ -238,6 +238,10 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
 int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
                   int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
                   float* d_Y, void* stream);
+/* The same with bf16 W, X and slot weights (the reference has an fp16 example only). */
+int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
+                   int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
+                   float* d_Y, void* stream);
 int stir_rgms_plan_destroy(stir_rgms_plan* plan);
 
 /*

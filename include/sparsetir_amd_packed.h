@@ -100,7 +100,7 @@ enum {
  * "sparsetir.tcspmm"         (A, B, C, indptr, indices, feat, tile_size, group_size)
  *      examples/spmm/bench_tc_spmm.py:650-656
  * "sparsetir.rgms"           (W, X, Y, A_0, rows_0, cols_0, ..., mids_0, ..., feat_in, feat_out)
- *      examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852         fp16, W [R, feat_in, feat_out]
+ *      examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-852         fp16 or bf16, W [R, feat_in, feat_out]
  * "sparsetir.rgms_f32"       same argument list, every array fp32, W [R, feat_out, feat_in]
  *      examples/rgms/rgcn/bench_rgcn_composable.py:208-221
  * "sparsetir.rgms_csf"       (A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j, feat_in, feat_out)

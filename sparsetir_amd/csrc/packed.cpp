@@ -398,9 +398,15 @@ int stir_packed_tcspmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
 static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int n) {
   Args a{name, v, tc, n};
   const int bits = f32 ? 32 : 16;
+  // the 16-bit form takes float16 or bfloat16, read from W's dtype
+  const DLTensor* d0 = (n > 0 && (tc[0] == kTVMDLTensorHandle || tc[0] == kTVMNDArrayHandle ||
+                                  tc[0] == kTVMOpaqueHandle))
+                           ? static_cast<const DLTensor*>(v[0].v_handle) : nullptr;
+  const bool bf = !f32 && d0 && d0->dtype.code == kDLBfloat;
+  const uint8_t fcode = bf ? kDLBfloat : kDLFloat;
   if (n < 5 || (n - 5) % 4 != 0) return packed_fail("%s: num_args should be 3 + 4*buckets + 2", a.fn);
   const int nb = (n - 5) / 4;
-  Arr W = a.arr(0, "W", kDLFloat, bits, kDevice), X = a.arr(1, "X", kDLFloat, bits, kDevice),
+  Arr W = a.arr(0, "W", fcode, bits, kDevice), X = a.arr(1, "X", fcode, bits, kDevice),
       Y = a.arr(2, "Y", kDLFloat, 32, kDevice);
   const int64_t fin = a.integer(n - 2, "feat_in"), fout = a.integer(n - 1, "feat_out");
   if (!a.ok) return -1;
@@ -411,7 +417,7 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
   std::vector<int64_t> groups(nb);
   std::vector<int32_t> rb(nb, 1), cb(nb, 1);
   for (int b = 0; b < nb; ++b) {
-    Arr Aa = a.arr(3 + 3 * b, "A_k", kDLFloat, bits, kDevice), Rr = a.arr(4 + 3 * b, "rows_k", kDLInt, 32, kDevice),
+    Arr Aa = a.arr(3 + 3 * b, "A_k", fcode, bits, kDevice), Rr = a.arr(4 + 3 * b, "rows_k", kDLInt, 32, kDevice),
         Cc = a.arr(5 + 3 * b, "cols_k", kDLInt, 32, kDevice), Mm = a.arr(3 + 3 * nb + b, "mids_k", kDLInt, 32, kDevice);
     if (!a.ok) return -1;
     a.len(Cc, "cols_k", Aa.len);
@@ -467,8 +473,8 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
       return forward(-1);
     g_rgms_key = key;
   }
-  return forward(stir_rgms_f16(g_rgms_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data, X.data,
-                               (float*)Y.data, g_stream));
+  return forward((bf ? stir_rgms_bf16 : stir_rgms_f16)(g_rgms_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data,
+                                                       X.data, (float*)Y.data, g_stream));
 }
 
 int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {

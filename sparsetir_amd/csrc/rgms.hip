@@ -19,6 +19,7 @@ namespace {
 using stir::kWave;
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -40,8 +41,23 @@ constexpr int kChunkSlots = 128;
 
 constexpr int kMaxKK = 8;  // feat_in <= 128 keeps the X operand in registers
 
-__device__ __forceinline__ float half_bits_to_float(uint16_t b) {
-  return (float)__builtin_bit_cast(_Float16, b);
+// 16-bit storage type of W, X and the slot weights: fp16, or bf16 with BF16
+template <bool BF16>
+__device__ __forceinline__ float bits_to_float(uint16_t b) {
+  if constexpr (BF16)
+    return __uint_as_float((uint32_t)b << 16);
+  else
+    return (float)__builtin_bit_cast(_Float16, b);
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
 }
 
 __device__ __forceinline__ void atomic_addf(float* p, float v) {
@@ -53,7 +69,7 @@ __device__ __forceinline__ void atomic_addf(float* p, float v) {
 // column ids, slot weights and row ids are fetched with a few coalesced loads (lane l holds slots
 // l, l+64, ...), then the X rows of all TI tiles are requested at once, so a chunk costs two
 // memory latencies instead of several per tile.
-template <int KK, int LCB>
+template <int KK, int LCB, bool BF16>
 __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int chunk, int feat_out,
                                            const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
                                            float* __restrict__ Y, float* __restrict__ Z, int lane) {
@@ -101,7 +117,7 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
         const int sl = s_base + 64 * j + lane;
         const bool live = sl < gsize;
         mcol[j] = live ? colg[sl] : 0;
-        mw[j] = live ? half_bits_to_float(Ag[sl]) : 0.f;
+        mw[j] = live ? bits_to_float<BF16>(Ag[sl]) : 0.f;
         // ELL rows of the chunk (power-of-two cb): row (s_base >> LCB) + 64j + lane
         mrow[j] = 0;
         if constexpr (LCB >= 0) {
@@ -129,8 +145,7 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
         for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk)
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, xa[t][kk]),
-                                                      __builtin_bit_cast(f16x8, wf[kk]), acc, 0, 0, 0);
+          acc = mfma32<BF16>(xa[t][kk], wf[kk], acc);
         // acc[v]: slot 32t + (v%4) + 4h + 8(v/4) of the chunk, output feature nt + n.
         // Scale by the slot weight (zero beyond the group).
         float wgt[16];
@@ -208,7 +223,7 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
 
 // grid: one wavefront per work unit (kChunkSlots slots of one group), 4 per workgroup; feat_out
 // tiles of 32 are walked inside.
-template <int KK>
+template <int KK, bool BF16>
 __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict__ table, int nb,
                                                    int64_t total_units, int feat_out,
                                                    const uint16_t* __restrict__ W,
@@ -227,13 +242,13 @@ __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict_
   const int64_t g = unit / bk.chunks;
   const int chunk = (int)(unit % bk.chunks);
   switch (bk.log2cb) {
-    case 0: rgms_group<KK, 0>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 1: rgms_group<KK, 1>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 2: rgms_group<KK, 2>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 3: rgms_group<KK, 3>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 4: rgms_group<KK, 4>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 5: rgms_group<KK, 5>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    default: rgms_group<KK, -1>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 0: rgms_group<KK, 0, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 1: rgms_group<KK, 1, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 2: rgms_group<KK, 2, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 3: rgms_group<KK, 3, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 4: rgms_group<KK, 4, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 5: rgms_group<KK, 5, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    default: rgms_group<KK, -1, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
   }
 }
 
@@ -322,9 +337,9 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   return 0;
 }
 
-int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
-                  int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X, float* d_Y,
-                  void* stream) {
+static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
+                       int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X, float* d_Y,
+                       void* stream) {
   STIR_REQUIRE(plan, "rgms: plan is null");
   STIR_REQUIRE(m >= 0 && n >= 0 && num_rels >= 0, "rgms: bad sizes");
   STIR_REQUIRE(feat_in > 0 && feat_in % 16 == 0 && feat_in <= 16 * kMaxKK,
@@ -348,8 +363,12 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
   }
 #define STIR_RGMS(KK)                                                                              \
   case KK:                                                                                         \
-    hipLaunchKernelGGL((rgms_kernel<KK>), grid, block, 0, st, plan->d_table, plan->nk,             \
-                       plan->total_units, feat_out, W, X, d_Y, Z);                                \
+    if (bf16)                                                                                      \
+      hipLaunchKernelGGL((rgms_kernel<KK, true>), grid, block, 0, st, plan->d_table, plan->nk,     \
+                         plan->total_units, feat_out, W, X, d_Y, Z);                              \
+    else                                                                                           \
+      hipLaunchKernelGGL((rgms_kernel<KK, false>), grid, block, 0, st, plan->d_table, plan->nk,    \
+                         plan->total_units, feat_out, W, X, d_Y, Z);                              \
     break
   switch (feat_in / 16) {
     STIR_RGMS(1);
@@ -365,6 +384,16 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
   STIR_LAUNCH_CHECK();
   if (Z) return stir::dest_reduce(mp->dest, feat_out, d_Y, st);
   return 0;
+}
+
+int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels, int32_t feat_in,
+                  int32_t feat_out, const void* d_W, const void* d_X, float* d_Y, void* stream) {
+  return rgms_launch(false, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
+}
+
+int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels, int32_t feat_in,
+                   int32_t feat_out, const void* d_W, const void* d_X, float* d_Y, void* stream) {
+  return rgms_launch(true, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
 }
 
 int stir_rgms_plan_destroy(stir_rgms_plan* plan) {

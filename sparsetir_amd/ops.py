@@ -307,7 +307,13 @@ class Rgms(_Operator):
     _in_dtype = torch.float16
     _fns = ("stir_rgms_plan_create", "stir_rgms_f16", "stir_rgms_plan_destroy")
 
-    def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
+    def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=None):
+        if dtype is not None and self._in_dtype is torch.float16:
+            if dtype not in (torch.float16, torch.bfloat16):
+                raise _lib.SparseTIRError("rgms: dtype must be torch.float16 or torch.bfloat16")
+            if dtype is torch.bfloat16:  # same kernel on the bf16 matrix-core instruction
+                self._in_dtype = dtype
+                self._fns = ("stir_rgms_plan_create", "stir_rgms_bf16", "stir_rgms_plan_destroy")
         self.m, self.n, self.R = int(m), int(n), int(num_rels)
         self.fin, self.fout = int(feat_in), int(feat_out)
         self.rb, self.cb = [int(v) for v in rows_bkt], [int(v) for v in cols_bkt]
@@ -427,8 +433,8 @@ def build_tcspmm(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=to
     return TcSpMM(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype)
 
 
-def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
-    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups)
+def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=torch.float16):
+    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype)
 
 
 def build_rgms_f32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):

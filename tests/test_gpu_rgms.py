@@ -121,3 +121,29 @@ def test_rgms_staged_repeat_calls_accumulate(dev):
     # the staged sums are formed in a fixed order except for output rows that span several
     # chunks of the reduce kernel, whose partial sums meet in atomics
     assert torch.allclose(y2, once, rtol=1e-6, atol=1e-6)
+
+
+def test_rgms_bf16(dev):
+    """bf16 W, X and slot weights through the same kernel (bf16 MFMA), fp32 accumulate and output."""
+    R, n, fin, fout, group, buckets = 5, 300, 32, 64, 32, [1, 2, 4, 8]
+    csf = random_csf(R, n, 900, seed=31)
+    rng = np.random.default_rng(31)
+    rows_bkt = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    x = torch.from_numpy(rng.standard_normal((n, fin), dtype=np.float32)).to(dev).bfloat16()
+    w = torch.from_numpy(rng.standard_normal((R, fin, fout), dtype=np.float32) * 0.1).to(dev).bfloat16()
+    triples, mids = [], []
+    for b in range(len(buckets)):
+        triples += [t(mask[b].astype(np.float32).ravel()).bfloat16(), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    f = ops.build_rgms(n, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols], dtype=torch.bfloat16)
+    y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
+    f(w.reshape(-1), x.reshape(-1), y, *triples, *mids)
+    y2 = torch.zeros_like(y)
+    from sparsetir_amd import packed
+    packed.get_global_func("sparsetir.rgms")(w.reshape(-1), x.reshape(-1), y2, *triples, *mids, fin, fout)
+    torch.cuda.synchronize()
+    av = np.ones(len(csf[3]), np.float32)
+    _check(y.cpu().numpy().reshape(n, fout), csf, av, x.float().cpu().numpy(), w.float().cpu().numpy(), n, "bf16")
+    assert torch.allclose(y, y2, rtol=1e-5, atol=1e-5)
