@@ -80,17 +80,18 @@ int stir_condense_fill(int32_t n, const int32_t* indptr, const int32_t* indices,
 /* ---------------------------------------------------------------- format pass (device) */
 
 /*
- * ColumnPartHyb on the GPU, bit-exact with the host routine above for CSR input whose
- * column indices ascend within each row, and for any column order when num_col_parts is 1
- * (the reference runs this on the CPU only, src/sparse/format.cc:58-59; unsorted rows with
- * several partitions are reported as an error here).
- * d_workspace must hold stir_column_part_hyb_device_workspace_bytes(...) bytes and must
- * stay untouched between the _sizes and the _fill call.  _sizes synchronises the stream
- * to return nrows on the host; _fill writes device arrays through host tables of
- * device pointers (k = part*num_buckets + bucket).
+ * ColumnPartHyb on the GPU, bit-exact with the host routine above (the reference runs this on
+ * the CPU only, src/sparse/format.cc:58-59).  CSR rows whose entries are ordered by column
+ * partition -- ascending columns in particular -- take the fast path; other input is first
+ * regrouped by (row, partition) with a stable sort, which keeps the order the sequential
+ * routine produces.  d_workspace must hold
+ * stir_column_part_hyb_device_workspace_bytes(num_rows, num_col_parts, num_buckets, nnz) bytes
+ * and must stay untouched between the _sizes and the _fill / _values calls.  _sizes
+ * synchronises the stream to return nrows on the host; _fill writes device arrays through host
+ * tables of device pointers (k = part*num_buckets + bucket).
  */
 size_t stir_column_part_hyb_device_workspace_bytes(int32_t num_rows, int32_t num_col_parts,
-                                                   int32_t num_buckets);
+                                                   int32_t num_buckets, int64_t nnz);
 int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols,
                                       const int32_t* d_indptr, const int32_t* d_indices,
                                       int32_t num_col_parts, const int32_t* buckets,

@@ -25,7 +25,7 @@ SIGNATURES = {
     "stir_csf_to_ell3d_fill": (I32, [I32, VP, VP, VP, VP, VP, VP, I32, VP, VP, VP, VP]),
     "stir_condense_sizes": (I32, [I32, VP, VP, I32, I32, VP, VP]),
     "stir_condense_fill": (I32, [I32, VP, VP, I32, I32, VP, VP]),
-    "stir_column_part_hyb_device_workspace_bytes": (SZ, [I32, I32, I32]),
+    "stir_column_part_hyb_device_workspace_bytes": (SZ, [I32, I32, I32, I64]),
     "stir_column_part_hyb_device_sizes": (I32, [I32, I32, VP, VP, I32, VP, I32, VP, VP, VP]),
     "stir_column_part_hyb_device_fill": (I32, [I32, I32, VP, VP, I32, VP, I32, VP, VP, VP, VP, VP]),
     "stir_column_part_hyb_device_values": (I32, [I32, I32, VP, VP, VP, I32, VP, I32, VP, VP, VP, VP]),

@@ -19,7 +19,10 @@
 #include <mutex>
 #include <vector>
 
+#include <hipcub/hipcub.hpp>
+
 #include "common.h"
+#include "row_lookup.h"
 #include "../../include/sparsetir_amd.h"
 
 namespace {
@@ -38,13 +41,17 @@ struct Workspace {
   int32_t** rows_tab;  // [P*NB] output pointers
   int32_t** cols_tab;
   int32_t** mask_tab;
-  size_t bytes;
+  size_t bytes;       // of the regions above
+  // Behind them, with several partitions: the nonzeros regrouped by (row, partition) for
+  // matrices whose rows are not ordered by partition -- column ids idx2[nnz] and their source
+  // positions perm[nnz], see permuted_tail().
 };
 
 // The two descent counts are kept as kCountSlots partial sums each (a workgroup adds to the slot
 // of its index), since atomics on a single address serialise; the host adds the slots up.
 constexpr int kCountSlots = 1024;
-constexpr int kStatusInts = 1 + 2 * kCountSlots;
+constexpr int kStatusInts = 2 + 2 * kCountSlots;  // status bits, 2 x kCountSlots counters, permuted flag
+constexpr int kPermutedAt = 1 + 2 * kCountSlots;
 
 // Row lookup for the per-nonzero passes: the row of every stride-th nonzero is recorded while the
 // rows are counted, so a thread finds the row of its first nonzero with a binary search over the
@@ -96,12 +103,13 @@ __device__ __forceinline__ int bucket_of_dev(const int32_t* widths, int nb, int 
   return k;
 }
 
-// (0) every column inside [0, num_cols); counts the positions e whose successor holds a smaller
-// column.  Such a descent is legal only where e + 1 opens a row; count_kernel counts those, and the
-// rows ascend exactly when the two counts agree.  A thread checks kValidatePerThread consecutive
+// (0) every column inside [0, num_cols); counts the positions e whose successor lies in an
+// earlier column partition.  Such a descent is legal only where e + 1 opens a row; count_kernel
+// counts those, and the rows are ordered by partition -- all the closed form needs -- exactly
+// when the two counts agree.  A thread checks kValidatePerThread consecutive
 // entries (vector loads when aligned) and the step to its neighbour's first entry.
 constexpr int kValidatePerThread = 16;
-__global__ __launch_bounds__(256) void validate_kernel(int num_cols, int64_t nnz, int32_t first,
+__global__ __launch_bounds__(256) void validate_kernel(int num_cols, int psize, int64_t nnz, int32_t first,
                                                        const int32_t* __restrict__ indices,
                                                        int32_t* __restrict__ status) {
   constexpr int N = kValidatePerThread;
@@ -128,7 +136,7 @@ __global__ __launch_bounds__(256) void validate_kernel(int num_cols, int64_t nnz
   for (int j = 0; j < N; ++j) {
     if (e0 + j < end) {
       bad |= v[j] < 0 || v[j] >= num_cols;
-      if (e0 + j + 1 < end && v[j + 1] < v[j]) ++descents;
+      if (e0 + j + 1 < end && v[j + 1] / psize < v[j] / psize) ++descents;
     }
   }
   __shared__ int block_descents;
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(256) void count_kernel(int m, int psize, int NB, in
       rs = re = first;
     }
     // a non-empty row that is not the last: does the next stored entry hold a smaller column?
-    if (p == 0 && re > rs && re < end) boundary_descent = indices[re] < indices[re - 1];
+    if (p == 0 && re > rs && re < end) boundary_descent = indices[re] / psize < indices[re - 1] / psize;
     if (p == 0)
       for (int64_t q = (rs - first + stride - 1) / stride; first + q * stride < re; ++q) coarse[q] = i;
     const int lo = p == 0 ? rs : lower_bound_dev(indices, rs, re, (int64_t)p * psize);
@@ -401,7 +409,21 @@ struct EntryArgs {
   const int32_t* __restrict__ kb_in;
   const int32_t* __restrict__ coarse;
   int64_t stride;
+  // several partitions: flag (device) saying that the rows were not ordered by partition, and
+  // then the regrouped column ids and their source positions, indexed like `indices`
+  const int32_t* permuted;
+  const int32_t* idx2;
+  const int32_t* perm;
 };
+
+// The view of the matrix the placement kernels walk: the caller's arrays, or the regrouped ones.
+__device__ __forceinline__ EntryArgs effective(EntryArgs g) {
+  if (g.permuted && *g.permuted)
+    g.indices = g.idx2;
+  else
+    g.perm = nullptr;
+  return g;
+}
 
 // Rows that can own the nonzeros [e_first, e_last]: between the recorded rows around them.
 __device__ __forceinline__ void row_range(const EntryArgs& g, int64_t e_first, int64_t e_last, int& ra, int& rb) {
@@ -602,8 +624,9 @@ __device__ __forceinline__ void for_each_entry_slot(const EntryArgs& g, L load, 
 }
 
 template <bool SINGLE>
-__global__ __launch_bounds__(256) void place_entries_kernel(EntryArgs g, int32_t* const* __restrict__ cols_tab,
+__global__ __launch_bounds__(256) void place_entries_kernel(EntryArgs g_in, int32_t* const* __restrict__ cols_tab,
                                                             int32_t* const* __restrict__ mask_tab) {
+  const EntryArgs g = effective(g_in);
   __shared__ PtrTable<int32_t> cols, mask;
   cols.load(cols_tab, g.P * g.NB);
   mask.load(mask_tab, g.P * g.NB);
@@ -624,13 +647,14 @@ __global__ __launch_bounds__(256) void place_entries_kernel(EntryArgs g, int32_t
 // placement computed exactly as in place_entries_kernel.  (With several partitions the padding
 // is cleared beforehand instead.)
 template <bool SINGLE>
-__global__ __launch_bounds__(256) void place_values_kernel(EntryArgs g, const float* __restrict__ values,
+__global__ __launch_bounds__(256) void place_values_kernel(EntryArgs g_in, const float* __restrict__ values,
                                                            float* const* __restrict__ a_tab) {
+  const EntryArgs g = effective(g_in);
   __shared__ PtrTable<float> out;
   out.load(a_tab, g.P * g.NB);
   __syncthreads();
   for_each_entry_slot<SINGLE>(
-      g, [&](int64_t e) { return __float_as_int(values[e]); },
+      g, [&](int64_t e) { return __float_as_int(values[g.perm ? g.perm[e] : e]); },
       [&](int k, int64_t slot, int bits) { out.at(k)[slot] = __int_as_float(bits); },
       [&](int k, int64_t slot) { out.at(k)[slot] = 0.f; });
 }
@@ -665,6 +689,84 @@ bool recall_ends(const void* ws, const void* indptr, int32_t m, int32_t (&ends)[
   return false;
 }
 
+// ---- rows that are not ordered by partition: regroup the nonzeros by (row, partition), stably
+size_t tail_bytes(int32_t P, int64_t nnz) { return P > 1 && nnz > 0 ? 2 * align_up(sizeof(int32_t) * size_t(nnz)) : 0; }
+
+struct PermutedTail {
+  int32_t* idx2;
+  int32_t* perm;
+};
+PermutedTail permuted_tail(void* workspace, const Workspace& ws, int64_t nnz) {
+  char* base = static_cast<char*>(workspace) + ws.bytes;
+  return PermutedTail{reinterpret_cast<int32_t*>(base),
+                      reinterpret_cast<int32_t*>(base + align_up(sizeof(int32_t) * size_t(nnz)))};
+}
+
+__global__ __launch_bounds__(256) void perm_keys_kernel(int m, int P, int psize, int64_t nnz, int32_t first,
+                                                        const int32_t* __restrict__ indptr,
+                                                        const int32_t* __restrict__ indices,
+                                                        uint32_t* __restrict__ keys, int32_t* __restrict__ vals) {
+  __shared__ int32_t win_all[4][stir::kRowLookupWindow];
+  const int lane = threadIdx.x & 63;
+  const int64_t end = first + nnz;
+  const int64_t e0 = first + ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (kWave * 8);
+  if (e0 >= end) return;
+  const int64_t e_last = min(end, e0 + kWave * 8) - 1;
+  stir::for_each_nonzero_row<8>(indptr, m, e0, e_last, win_all[threadIdx.x >> 6], lane,
+                                [&](int64_t e, int row, int, bool live) {
+    if (!live) return;
+    keys[e - first] = (uint32_t)row * (uint32_t)P + (uint32_t)(indices[e] / psize);
+    vals[e - first] = (int32_t)e;
+  });
+}
+
+__global__ __launch_bounds__(256) void perm_gather_kernel(int64_t nnz, const int32_t* __restrict__ indices,
+                                                          const int32_t* __restrict__ perm,
+                                                          int32_t* __restrict__ idx2) {
+  const int64_t s = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (s < nnz) idx2[s] = indices[perm[s]];
+}
+
+// Fills tail.perm (source position of the s-th nonzero in the regrouped order) and tail.idx2 (its
+// column).  Scratch for the keys and the sort is allocated and freed here: this is the slow path.
+int build_permutation(const char* who, int m, int P, int psize, int64_t nnz, int32_t first,
+                      const int32_t* d_indptr, const int32_t* d_indices, const PermutedTail& tail,
+                      hipStream_t st) {
+  STIR_REQUIRE((int64_t)m * P < (int64_t(1) << 32), "%s: %d rows x %d partitions is too large for unsorted rows",
+               who, m, P);
+  STIR_REQUIRE(nnz < (int64_t(1) << 31), "%s: too many nonzeros for unsorted rows", who);
+  int end_bit = 1;
+  while (end_bit < 32 && (int64_t(1) << end_bit) < (int64_t)m * P) ++end_bit;
+  size_t sort_bytes = 0;
+  hipError_t err = hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, (const uint32_t*)nullptr,
+                                                      (uint32_t*)nullptr, (const int32_t*)nullptr,
+                                                      (int32_t*)nullptr, (int)nnz, 0, end_bit, st);
+  uint32_t* keys = nullptr;  // keys, sorted keys, source positions
+  void* d_sort = nullptr;
+  if (err == hipSuccess) err = hipMalloc(reinterpret_cast<void**>(&keys), sizeof(uint32_t) * 3 * size_t(nnz));
+  if (err == hipSuccess) err = hipMalloc(&d_sort, sort_bytes ? sort_bytes : 16);
+  if (err == hipSuccess) {
+    uint32_t* keys_sorted = keys + nnz;
+    int32_t* vals = reinterpret_cast<int32_t*>(keys + 2 * nnz);
+    hipLaunchKernelGGL(perm_keys_kernel, dim3((unsigned)stir::ceil_div(nnz, 4 * kWave * 8)), dim3(256), 0, st, m, P,
+                       psize, nnz, first, d_indptr, d_indices, keys, vals);
+    err = hipGetLastError();
+    if (err == hipSuccess)
+      err = hipcub::DeviceRadixSort::SortPairs(d_sort, sort_bytes, (const uint32_t*)keys, keys_sorted,
+                                               (const int32_t*)vals, tail.perm, (int)nnz, 0, end_bit, st);
+    if (err == hipSuccess) {
+      hipLaunchKernelGGL(perm_gather_kernel, dim3((unsigned)stir::ceil_div(nnz, 256)), dim3(256), 0, st, nnz,
+                         d_indices, tail.perm, tail.idx2);
+      err = hipGetLastError();
+    }
+    if (err == hipSuccess) err = hipStreamSynchronize(st);
+  }
+  if (keys) (void)hipFree(keys);
+  if (d_sort) (void)hipFree(d_sort);
+  STIR_REQUIRE(err == hipSuccess, "%s: regrouping unsorted rows failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
 int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t parts, const int32_t* buckets,
                int32_t nb) {
   STIR_REQUIRE(num_rows >= 0 && num_cols >= 0, "%s: bad matrix shape %d x %d", who, num_rows, num_cols);
@@ -681,9 +783,9 @@ int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t part
 extern "C" {
 
 size_t stir_column_part_hyb_device_workspace_bytes(int32_t num_rows, int32_t num_col_parts,
-                                                   int32_t num_buckets) {
-  if (num_rows < 0 || num_col_parts <= 0 || num_buckets <= 0) return 0;
-  return carve(nullptr, num_rows, num_col_parts, num_buckets).bytes;
+                                                   int32_t num_buckets, int64_t nnz) {
+  if (num_rows < 0 || num_col_parts <= 0 || num_buckets <= 0 || nnz < 0) return 0;
+  return carve(nullptr, num_rows, num_col_parts, num_buckets).bytes + tail_bytes(num_col_parts, nnz);
 }
 
 int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const int32_t* d_indptr,
@@ -712,7 +814,7 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
   const int psize = num_cols > 0 ? (num_cols + P - 1) / P : 1;
   if (nnz > 0) {
     hipLaunchKernelGGL(validate_kernel, dim3((unsigned)stir::ceil_div(nnz, 256 * kValidatePerThread)), dim3(256), 0, st, num_cols,
-                       nnz, ends[0], d_indices, ws.status);
+                       psize, nnz, ends[0], d_indices, ws.status);
     STIR_LAUNCH_CHECK();
   }
   dim3 grid((unsigned)stir::ceil_div(m, 256), (unsigned)P);
@@ -735,9 +837,24 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
   }
   STIR_REQUIRE(!(status & kStatusIndptr), "%s: indptr is not a CSR row pointer (it decreases)", who);
   STIR_REQUIRE(!(status & kStatusRange), "%s: a column index lies outside [0, %d)", who, num_cols);
-  // with one partition a run is the whole row whatever the order of its columns
-  STIR_REQUIRE(P == 1 || descents == row_start_descents,
-               "%s: column indices must ascend inside each row (use the host routine for unsorted rows)", who);
+  // With one partition a run is the whole row whatever the order of its columns.  With several,
+  // rows that are not ordered by partition are regrouped by (row, partition) -- stably, so every
+  // run keeps the CSR order of its entries as in the sequential routine -- and counted again.
+  if (P > 1 && descents != row_start_descents) {
+    const PermutedTail tail = permuted_tail(d_workspace, ws, nnz);
+    if (build_permutation(who, m, P, psize, nnz, ends[0], d_indptr, d_indices, tail, st)) return -1;
+    const int32_t one = 1;
+    STIR_HIP(hipMemcpyAsync(ws.status + kPermutedAt, &one, sizeof(one), hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(count_kernel, grid, dim3(256), 0, st, m, psize, NB, W, ends[0], (int64_t)ends[1],
+                       coarse_stride(nnz), ws.coarse, d_indptr, tail.idx2 - ends[0], ws.widths, ws.lo, ws.hist,
+                       ws.status);
+    STIR_LAUNCH_CHECK();
+    hipLaunchKernelGGL(scan_kernel, dim3((unsigned)NB, (unsigned)P), dim3(kScanThreads), 0, st, NB, W, ws.hist,
+                       ws.totals);
+    STIR_LAUNCH_CHECK();
+    STIR_HIP(hipMemcpyAsync(nrows, ws.totals, sizeof(int64_t) * size_t(P) * NB, hipMemcpyDeviceToHost, st));
+    STIR_HIP(hipStreamSynchronize(st));
+  }
   for (int k = 0; k < P * NB; ++k)
     STIR_REQUIRE(nrows[k] < kMaxSlots / buckets[k % NB], "%s: bucket %d holds too many slots", who, k);
   remember_ends(d_workspace, d_indptr, m, ends);
@@ -777,8 +894,10 @@ int stir_column_part_hyb_device_fill(int32_t num_rows, int32_t num_cols, const i
   hipLaunchKernelGGL(place_rows_kernel, grid, dim3(256), 0, st, m, NB, W, d_indptr, ws.widths, ws.lo,
                      ws.hist, ws.slot0, ws.kb, ws.rows_tab, ws.cols_tab, ws.mask_tab);
   STIR_LAUNCH_CHECK();
+  const PermutedTail tail = permuted_tail(d_workspace, ws, nnz);
   const EntryArgs ea{m, P, psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.slot0, ws.kb, ws.coarse,
-                     coarse_stride(nnz)};
+                     coarse_stride(nnz), P > 1 ? ws.status + kPermutedAt : nullptr,
+                     P > 1 ? tail.idx2 - ends[0] : nullptr, P > 1 ? tail.perm - ends[0] : nullptr};
   if (P == 1)
     hipLaunchKernelGGL(place_entries_kernel<true>, dim3((unsigned)stir::ceil_div(nnz, 4 * kSingleTile)), dim3(256), 0,
                        st, ea, ws.cols_tab, ws.mask_tab);
@@ -820,8 +939,10 @@ int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const
   STIR_REQUIRE(d_indices && d_values, "%s: null pointer argument", who);
   const int psize = (num_cols + P - 1) / P;
   float* const* a_tab = reinterpret_cast<float* const*>(ws.mask_tab);
+  const PermutedTail tail = permuted_tail(d_workspace, ws, nnz);
   const EntryArgs ea{m, P, psize, NB, nnz, ends[0], d_indptr, d_indices, ws.widths, ws.slot0, ws.kb, ws.coarse,
-                     coarse_stride(nnz)};
+                     coarse_stride(nnz), P > 1 ? ws.status + kPermutedAt : nullptr,
+                     P > 1 ? tail.idx2 - ends[0] : nullptr, P > 1 ? tail.perm - ends[0] : nullptr};
   if (P == 1)
     hipLaunchKernelGGL(place_values_kernel<true>, dim3((unsigned)stir::ceil_div(nnz, 4 * kSingleTile)), dim3(256), 0,
                        st, ea, d_values, a_tab);

@@ -542,7 +542,7 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
       return forward(stir_column_part_hyb_sizes((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
                                                 (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data,
                                                 nb, (int64_t*)N.data));
-    const size_t need = stir_column_part_hyb_device_workspace_bytes((int32_t)num_rows, (int32_t)parts, nb);
+    const size_t need = stir_column_part_hyb_device_workspace_bytes((int32_t)num_rows, (int32_t)parts, nb, I.len);
     if (need > ws_bytes) {
       if (ws) (void)hipFree(ws);
       ws = nullptr;

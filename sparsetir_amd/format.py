@@ -94,7 +94,7 @@ def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, 
     nk = num_col_parts * nb
     with torch.cuda.device(dev):
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-        ws_bytes = L.stir_column_part_hyb_device_workspace_bytes(num_rows, num_col_parts, nb)
+        ws_bytes = L.stir_column_part_hyb_device_workspace_bytes(num_rows, num_col_parts, nb, indices.numel())
         ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
         nrows = np.zeros(max(nk, 1), np.int64)
         _lib.check(L.stir_column_part_hyb_device_sizes(

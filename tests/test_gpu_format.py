@@ -69,30 +69,72 @@ def test_device_column_part_hyb_one_partition_takes_unsorted_rows(dev):
                 assert np.array_equal(a, b)
 
 
-def test_device_column_part_hyb_rejects_unsorted_and_out_of_range(dev):
-    indptr, indices = random_csr(50, 40, 600, 3, sort=False)
-    with pytest.raises(SparseTIRError, match="ascend"):
-        _device_hyb(dev, 50, 40, indptr, indices, 2, [1, 2, 4])
+def _assert_same(got, want):
+    for gq, wq in zip(got, want):
+        for gp, wp in zip(gq, wq):
+            for a, b in zip(gp, wp):
+                assert a.shape == b.shape and np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("m,n,nnz,parts,buckets,seed", [
+    (50, 40, 600, 2, [1, 2, 4], 3),
+    (3000, 900, 90000, 4, [1, 2, 4, 8, 16, 32], 4),
+    (700, 5000, 40000, 16, [1, 2, 4, 8], 5),
+    (20000, 300, 30000, 3, [1, 2], 6),
+])
+def test_device_column_part_hyb_unsorted_rows_with_partitions(dev, m, n, nnz, parts, buckets, seed):
+    """Rows in arbitrary column order and several partitions: the device pass regroups the
+    nonzeros by (row, partition) with a stable sort and must give the sequential routine's arrays
+    (every run keeps the CSR order of its entries)."""
+    indptr, indices = random_csr(m, n, nnz, seed, sort=False, skew=1.0)
+    got = _device_hyb(dev, m, n, indptr, indices, parts, buckets)
+    _assert_same(got, oracle.column_part_hyb(m, n, indptr, indices, parts, buckets))
+
+
+def test_device_column_part_hyb_one_swapped_pair(dev):
+    """One swapped pair inside one row, across a partition boundary (every other row ascending):
+    the regrouping path must be taken -- found through the descent counts -- and be bit-exact."""
+    m, n, parts, buckets = 400, 300, 2, [1, 2, 4]
+    indptr, indices = random_csr(m, n, 6000, 11, skew=1.0)
+    psize = (n + parts - 1) // parts
+    for row in range(m):
+        seg = indices[indptr[row]:indptr[row + 1]]
+        cut = np.searchsorted(seg, psize)
+        if 0 < cut < len(seg):
+            e = indptr[row] + cut
+            break
+    swapped = indices.copy()
+    swapped[e - 1], swapped[e] = indices[e], indices[e - 1]
+    got = _device_hyb(dev, m, n, indptr, swapped, parts, buckets)
+    want = oracle.column_part_hyb(m, n, indptr, swapped, parts, buckets)
+    _assert_same(got, want)
+
+
+def test_device_column_part_hyb_unsorted_value_rewrite(dev):
+    m, n, parts, buckets = 600, 500, 3, [1, 2, 4, 8]
+    indptr, indices = random_csr(m, n, 12000, 14, sort=False, skew=1.0)
+    vals = np.random.default_rng(14).random(len(indices), dtype=np.float32) + 0.5
+    t = lambda a: torch.from_numpy(a).to(dev)
+    rows, cols, mask, avals = st.column_part_hyb(m, n, t(indptr), t(indices), parts, buckets, values=t(vals))
+    import scipy.sparse as sp
+    dense = sp.csr_matrix((vals, indices, indptr), shape=(m, n)).toarray()
+    for p in range(parts):
+        for b in range(len(buckets)):
+            r, c = rows[p][b].cpu().numpy(), cols[p][b].cpu().numpy()
+            k, a = mask[p][b].cpu().numpy(), avals[p][b].cpu().numpy()
+            if len(r):
+                assert np.array_equal(a, (dense[np.repeat(r[:, None], c.shape[1], 1), c] * k).astype(np.float32))
+
+
+def test_device_column_part_hyb_rejects_bad_input(dev):
     bad = np.asarray([0, 50], np.int32)
     with pytest.raises(SparseTIRError, match="outside"):
         _device_hyb(dev, 2, 40, np.asarray([0, 1, 2], np.int32), bad, 2, [1, 2])
-
-
-def test_device_column_part_hyb_single_descent_inside_a_row_is_rejected(dev):
-    """One swapped pair inside one row (every other row ascending, descents at row starts
-    everywhere) must be found; the same swap across a row boundary is legal."""
-    m, n = 400, 300
-    indptr, indices = random_csr(m, n, 6000, 11, skew=1.0)
-    row = int(np.argmax(np.diff(indptr) >= 3))
-    e = indptr[row]
-    bad = indices.copy()
-    bad[e], bad[e + 1] = indices[e + 1], indices[e]
-    with pytest.raises(SparseTIRError, match="ascend"):
-        _device_hyb(dev, m, n, indptr, bad, 2, [1, 2, 4])
+    indptr, indices = random_csr(400, 300, 6000, 11, skew=1.0)
     with pytest.raises(SparseTIRError, match="row pointer"):
         ptr = indptr.copy()
         ptr[10] = ptr[11] + 1
-        _device_hyb(dev, m, n, ptr, indices, 2, [1, 2, 4])
+        _device_hyb(dev, 400, 300, ptr, indices, 2, [1, 2, 4])
 
 
 def test_device_column_part_hyb_mostly_empty_rows_and_offset_row_pointer(dev):
