@@ -91,6 +91,19 @@ def test_device_column_part_hyb_unsorted_rows_with_partitions(dev, m, n, nnz, pa
     _assert_same(got, oracle.column_part_hyb(m, n, indptr, indices, parts, buckets))
 
 
+def test_device_column_part_hyb_partition_ordered_rows(dev):
+    """Columns shuffled inside every (row, partition) run but the runs in partition order: the
+    fast path applies (its row searches only compare partitions) and must stay bit-exact."""
+    m, n, parts, buckets = 800, 640, 4, [1, 2, 4, 8, 16]
+    indptr, indices = random_csr(m, n, 30000, 21, sort=False, skew=1.0)
+    psize = (n + parts - 1) // parts
+    for i in range(m):
+        seg = indices[indptr[i]:indptr[i + 1]]
+        seg[:] = seg[np.argsort(seg // psize, kind="stable")]
+    got = _device_hyb(dev, m, n, indptr, indices, parts, buckets)
+    _assert_same(got, oracle.column_part_hyb(m, n, indptr, indices, parts, buckets))
+
+
 def test_device_column_part_hyb_one_swapped_pair(dev):
     """One swapped pair inside one row, across a partition boundary (every other row ascending):
     the regrouping path must be taken -- found through the descent counts -- and be bit-exact."""
