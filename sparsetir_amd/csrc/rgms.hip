@@ -11,7 +11,9 @@
 #include <vector>
 
 #include "common.h"
+#include <cstdlib>
 #include "dest_index.h"
+#include "rgms_tiles.h"
 #include "../../include/sparsetir_amd.h"
 
 namespace {
@@ -267,6 +269,9 @@ struct stir_rgms_plan {
   std::vector<stir::DestBucket> staged;
   int64_t staged_rows;
   stir::DestIndex dest;
+  std::vector<stir::TileBucket> tile_buckets;
+  int64_t slots;
+  stir::TileIndex tiles;
 };
 
 extern "C" {
@@ -280,6 +285,8 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   int nk = 0;
   int64_t total = 0, staged_rows = 0;
   std::vector<stir::DestBucket> staged;
+  std::vector<stir::TileBucket> tile_buckets;
+  int64_t slots = 0;
   for (int b = 0; b < num_buckets; ++b) {
     if (rows_bkt[b] <= 0 || cols_bkt[b] <= 0 || groups[b] < 0) {
       delete[] host;
@@ -315,6 +322,8 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
     }
     host[nk++] = e;
     total += groups[b] * e.chunks;
+    tile_buckets.push_back(stir::TileBucket{e.A, e.rows, e.cols, e.mids, e.groups, e.rb, e.cb});
+    slots += e.groups * e.rb * e.cb;
   }
   stir_rgms_plan* p = new stir_rgms_plan();
   p->nk = nk;
@@ -322,6 +331,8 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   p->d_table = nullptr;
   p->staged = staged;
   p->staged_rows = staged_rows;
+  p->tile_buckets = tile_buckets;
+  p->slots = slots;
   hipError_t err = hipSuccess;
   if (nk > 0) {
     err = hipMalloc(reinterpret_cast<void**>(&p->d_table), sizeof(RgmsBucket) * nk);
@@ -356,6 +367,11 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
   // the plan's staging state is filled in by the first launch (plans are not shared between
   // host threads)
   stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
+  static const bool legacy = getenv("STIR_RGMS_LEGACY") != nullptr;
+  if (!legacy && mp->slots >= 65536 && mp->slots < (int64_t(1) << 31)) {
+    if (stir::tile_index_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, st)) return -1;
+    return stir::tile_rgms_launch(bf16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
+  }
   float* Z = nullptr;
   if (mp->staged_rows >= kStagingMinRows) {
     if (stir::dest_index_prepare(mp->dest, mp->staged, m, feat_out, st)) return -1;
@@ -400,6 +416,7 @@ int stir_rgms_plan_destroy(stir_rgms_plan* plan) {
   if (!plan) return 0;
   if (plan->d_table) (void)hipFree(plan->d_table);
   stir::dest_index_free(plan->dest);
+  stir::tile_index_free(plan->tiles);
   delete plan;
   return 0;
 }

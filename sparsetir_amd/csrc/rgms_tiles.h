@@ -1,0 +1,44 @@
+// Destination-tiled RGMS for large ELL3D inputs: no atomics and no staging matrix.
+//
+// The slots of all buckets are re-indexed once per plan as "edges" (source row, relation,
+// destination row, address of the slot weight) sorted by (destination tile of 32 rows, relation,
+// row inside the tile).  A wavefront owns a tile: it keeps the tile's 32 x 32 fp32 block of Y in
+// MFMA accumulators, walks the tile's edges 32 at a time and writes Y once at the end.  Tiles with
+// very many edges are cut into several units whose results are added with atomics.
+#pragma once
+#include <cstdint>
+#include <vector>
+
+#include "common.h"
+
+namespace stir {
+
+struct TileBucket {
+  const uint16_t* A;    // device: slot weights (16-bit), groups*rb*cb
+  const int32_t* rows;  // device: groups*rb
+  const int32_t* cols;  // device: groups*rb*cb
+  const int32_t* mids;  // device: groups
+  int64_t groups;
+  int32_t rb, cb;
+};
+
+struct TileIndex {
+  int32_t m = -1, n = -1, num_rels = -1;  // what the index was built for
+  int64_t edges = 0;                      // slots of all buckets
+  int64_t units = 0;
+  void* d_edges = nullptr;  // edges x 16 bytes, sorted
+  void* d_units = nullptr;  // units x 16 bytes
+  void* d_wpack = nullptr;  // W in MFMA operand order, rewritten by every launch
+  size_t wpack_bytes = 0;
+};
+
+// Builds the index on `stream` (synchronises; allocates).  A no-op when it already exists for
+// the same m, n and num_rels.  Fails when a row id, column id or relation id is out of range.
+int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
+                       int32_t num_rels, hipStream_t stream);
+// Y += RGMS(W, X) over the indexed edges.  W: [R, feat_in, feat_out], X: [n, feat_in], 16-bit.
+int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W,
+                     const void* d_X, float* d_Y, hipStream_t stream);
+void tile_index_free(TileIndex& ix);
+
+}  // namespace stir

@@ -1,0 +1,522 @@
+// Destination-tiled RGMS declared in rgms_tiles.h: index construction and the MFMA kernel.
+//
+// Per step a wavefront takes the next 32 edges of its tile (sorted by relation, then row):
+//   stage 1  T[e, :] = X[src_e, :] @ W[rel_e]      one MFMA chain per distinct relation of the
+//                                                  step; the rows of other relations enter as zeros
+//   stage 2  Ytile  += S @ T                       S[i, e] = weight_e if edge e ends in row i
+// The gathered X rows are the stage-1 A operand straight from global memory (lane (e, h) loads 8
+// consecutive input features of its edge).  T leaves stage 1 in accumulator layout, which is the
+// B-operand layout of stage 2 up to a fixed permutation of the edge index; S is laid out with the
+// same permutation.  T is split into two (fp16) or three (bf16) 16-bit terms so that stage 2
+// keeps fp32 accuracy.  S is assembled in a per-wavefront LDS tile: the lane of edge e stores
+// weight_e at (row_e, e), every lane reads its operand row, then the entry is cleared again.
+#include "rgms_tiles.h"
+
+#include <hipcub/hipcub.hpp>
+
+namespace stir {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) uint16_t GlobalU16;  // a global-memory load, not a flat one
+
+struct alignas(16) DevBucket {
+  const uint16_t* A;
+  const int32_t* rows;
+  const int32_t* cols;
+  const int32_t* mids;
+  int64_t slot_begin;  // first slot of the bucket in the numbering over all buckets
+  int32_t rb, cb;
+};
+
+struct alignas(16) Edge {
+  int32_t src;         // row of X
+  uint32_t w_lo, w_hi;  // device address of the 16-bit slot weight
+  uint32_t rel_dl;     // relation << 5 | destination row inside its tile
+};
+
+struct alignas(16) Unit {
+  int64_t edge_begin;
+  int32_t edge_count;
+  int32_t tile_flag;  // tile << 1 | 1 when the tile has several units (atomic write-back)
+};
+
+constexpr int kTileRows = 32;
+constexpr int kStepEdges = 32;
+constexpr int kMaxKK = 8;
+
+__device__ __forceinline__ int bucket_of(const DevBucket* __restrict__ tab, int nb, int64_t q) {
+  int lo = 0, hi = nb - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (tab[mid].slot_begin <= q) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// key = (destination tile, relation, row inside the tile), value = slot
+__global__ __launch_bounds__(256) void edge_keys_kernel(const DevBucket* __restrict__ tab, int nb, int64_t slots, int m,
+                                                        int num_rels, uint64_t* __restrict__ keys,
+                                                        int32_t* __restrict__ vals, int32_t* __restrict__ bad) {
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (q >= slots) return;
+  const DevBucket bk = tab[bucket_of(tab, nb, q)];
+  const int64_t local = q - bk.slot_begin;
+  const int64_t gs = (int64_t)bk.rb * bk.cb;
+  const int64_t g = local / gs;
+  const int r = (int)((local - g * gs) / bk.cb);
+  int dest = bk.rows[g * bk.rb + r];
+  int rel = bk.mids[g];
+  if ((unsigned)dest >= (unsigned)m || (unsigned)rel >= (unsigned)num_rels) {
+    *bad = 1;
+    dest = rel = 0;
+  }
+  keys[q] = ((((uint64_t)(dest >> 5)) * num_rels + rel) << 5) | (uint64_t)(dest & 31);
+  vals[q] = (int32_t)q;
+}
+
+__global__ __launch_bounds__(256) void edge_records_kernel(const DevBucket* __restrict__ tab, int nb, int64_t slots,
+                                                           int n, int num_rels, const uint64_t* __restrict__ keys,
+                                                           const int32_t* __restrict__ vals, Edge* __restrict__ edges,
+                                                           int32_t* __restrict__ bad) {
+  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (p >= slots) return;
+  const int64_t q = vals[p];
+  const DevBucket bk = tab[bucket_of(tab, nb, q)];
+  const int64_t local = q - bk.slot_begin;
+  int src = bk.cols[local];
+  if ((unsigned)src >= (unsigned)n) {
+    *bad = 2;
+    src = 0;
+  }
+  const uint64_t key = keys[p];
+  const uint64_t addr = reinterpret_cast<uint64_t>(bk.A + local);
+  Edge e;
+  e.src = src;
+  e.w_lo = (uint32_t)addr;
+  e.w_hi = (uint32_t)(addr >> 32);
+  e.rel_dl = (uint32_t)(((key >> 5) % (uint64_t)num_rels) << 5) | (uint32_t)(key & 31);
+  edges[p] = e;
+}
+
+// begin[t] = first sorted edge of tile t (t = tiles gives the edge count)
+__global__ __launch_bounds__(256) void tile_bounds_kernel(const uint64_t* __restrict__ keys, int64_t slots,
+                                                          int64_t tiles, int num_rels, int64_t* __restrict__ begin) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t > tiles) return;
+  const uint64_t target = ((uint64_t)t * num_rels) << 5;
+  int64_t lo = 0, hi = slots;
+  while (lo < hi) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (keys[mid] < target) lo = mid + 1; else hi = mid;
+  }
+  begin[t] = lo;
+}
+
+// A tile of up to 1.5 * cap steps is one unit; longer ones are cut into units of cap steps.
+__device__ __forceinline__ int units_of(int64_t edges, int cap) {
+  const int64_t steps = (edges + kStepEdges - 1) / kStepEdges;
+  if (steps == 0) return 0;
+  if (steps <= cap + cap / 2) return 1;
+  return (int)((steps + cap - 1) / cap);
+}
+
+__global__ __launch_bounds__(256) void unit_count_kernel(const int64_t* __restrict__ begin, int64_t tiles, int cap,
+                                                         int32_t* __restrict__ count) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t > tiles) return;
+  count[t] = t < tiles ? units_of(begin[t + 1] - begin[t], cap) : 0;
+}
+
+__global__ __launch_bounds__(256) void unit_fill_kernel(const int64_t* __restrict__ begin,
+                                                        const int32_t* __restrict__ unit_begin, int64_t tiles, int cap,
+                                                        Unit* __restrict__ units) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= tiles) return;
+  const int64_t e0 = begin[t], e1 = begin[t + 1];
+  const int nu = units_of(e1 - e0, cap);
+  const int64_t per = nu == 1 ? e1 - e0 : (int64_t)cap * kStepEdges;
+  for (int u = 0; u < nu; ++u) {
+    Unit un;
+    un.edge_begin = e0 + u * per;
+    un.edge_count = (int32_t)min(per, e1 - un.edge_begin);
+    un.tile_flag = (int32_t)(t << 1) | (nu > 1 ? 1 : 0);
+    units[unit_begin[t] + u] = un;
+  }
+}
+
+// W[rel][16kk + 8h + 2d (+1)][32nt + n] -> operand word d of lane (n, h), one wavefront per
+// (rel, nt, kk)
+__global__ __launch_bounds__(256) void pack_w_kernel(const uint16_t* __restrict__ W, u32x4* __restrict__ Wp,
+                                                     int64_t frags, int kk_count, int feat_out) {
+  const int lane = threadIdx.x & 63, n = lane & 31, h = lane >> 5;
+  const int64_t f = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (f >= frags) return;
+  const int ntiles = feat_out / 32;
+  const int kk = (int)(f % kk_count);
+  const int nt = (int)((f / kk_count) % ntiles);
+  const int64_t rel = f / ((int64_t)kk_count * ntiles);
+  const uint16_t* w = W + (rel * kk_count * 16 + 16 * kk + 8 * h) * feat_out + 32 * nt + n;
+  u32x4 v;
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+    v[d] = (uint32_t)w[(int64_t)(2 * d) * feat_out] | ((uint32_t)w[(int64_t)(2 * d + 1) * feat_out] << 16);
+  Wp[f * 64 + lane] = v;
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+}
+
+// acc += S-operand @ (8 rows of T held as fp32 in t[0..7]), T split into 16-bit terms whose sum
+// carries at least 21 significant bits.
+template <bool BF16>
+__device__ __forceinline__ f32x16 stage2(u32x4 sa, const float* t, f32x16 acc) {
+  if constexpr (BF16) {
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = t[i];
+#pragma unroll
+    for (int term = 0; term < 3; ++term) {
+      u32x4 b;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t lo = __float_as_uint(r[2 * d]), hi = __float_as_uint(r[2 * d + 1]);
+        b[d] = __builtin_amdgcn_perm(hi, lo, 0x07060302);  // the two upper halves (truncation)
+        r[2 * d] -= __uint_as_float(lo & 0xffff0000u);
+        r[2 * d + 1] -= __uint_as_float(hi & 0xffff0000u);
+      }
+      acc = mfma32<true>(sa, b, acc);
+    }
+  } else {
+    typedef __fp16 h2 __attribute__((ext_vector_type(2)));
+    u32x4 bh, bl;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const h2 hi = __builtin_amdgcn_cvt_pkrtz(t[2 * d], t[2 * d + 1]);
+      const h2 lo = __builtin_amdgcn_cvt_pkrtz(t[2 * d] - (float)hi[0], t[2 * d + 1] - (float)hi[1]);
+      bh[d] = __builtin_bit_cast(uint32_t, hi);
+      bl[d] = __builtin_bit_cast(uint32_t, lo);
+    }
+    acc = mfma32<false>(sa, bh, acc);
+    acc = mfma32<false>(sa, bl, acc);
+  }
+  return acc;
+}
+
+constexpr int kSStride = 40;  // 16-bit elements per row of the S tile (32 used; 80-byte rows)
+
+// One wavefront per unit, 4 per workgroup; no workgroup barrier is used, so wavefronts without a
+// unit leave at once.  KK = feat_in / 16.
+template <int KK, bool BF16>
+__global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__ units, int64_t n_units,
+                                                        const Edge* __restrict__ edges, int m, int feat_out,
+                                                        const u32x4* __restrict__ Wp, const uint16_t* __restrict__ X,
+                                                        float* __restrict__ Y) {
+  constexpr int FIN = KK * 16;
+  constexpr int PW = KK <= 4 ? 2 : 1;  // relations whose W fragments are requested together
+  __shared__ __attribute__((aligned(16))) uint16_t s_all[4][kTileRows * kSStride];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t uid = (int64_t)blockIdx.x * 4 + wave;
+  if (uid >= n_units) return;
+  uint16_t* S = s_all[wave];
+  {
+    uint32_t* s32 = reinterpret_cast<uint32_t*>(S);
+#pragma unroll
+    for (int k = 0; k < kTileRows * kSStride / 2 / 64; ++k) s32[lane + 64 * k] = 0;
+  }
+  const Unit u = units[uid];
+  const int mrow = lane & 31, h = lane >> 5;
+  const int ntiles = feat_out / 32;
+  // Step row e sits at column j of the S tile such that lane (i, h) finds the 8 edges of its
+  // stage-2 operand word c at columns 16c + 8h .. +8: these are the rows (t%4) + 4h + 8(2c + t/4)
+  // that stage 1 leaves in accumulator registers 8c + t of the lanes of half h.
+  const int jcol = 16 * (mrow >> 4) + 8 * ((mrow >> 2) & 1) + 4 * ((mrow >> 3) & 1) + (mrow & 3);
+  const int64_t e_end = u.edge_begin + u.edge_count;
+  const int tile = u.tile_flag >> 1;
+
+  for (int nti = 0; nti < ntiles; ++nti) {
+    f32x16 acc2;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc2[v] = 0.f;
+    // lanes past the last edge repeat it with weight zero
+    Edge next = edges[min(u.edge_begin + mrow, e_end - 1)];
+#pragma unroll 1
+    for (int64_t e0 = u.edge_begin; e0 < e_end; e0 += kStepEdges) {
+      const Edge cur = next;
+      const int left = (int)min((int64_t)kStepEdges, e_end - e0);  // uniform
+      const bool live = mrow < left;
+      const int rel = (int)(cur.rel_dl >> 5), dl = (int)(cur.rel_dl & 31);
+      // the first PW runs of equal relation (the step is sorted by relation)
+      int r[PW], pos = 0;
+#pragma unroll
+      for (int q = 0; q < PW; ++q) {
+        r[q] = -1;
+        if (pos < kStepEdges) {
+          r[q] = __builtin_amdgcn_readlane(rel, pos);
+          pos += __popcll(__ballot(rel == r[q]) & 0xffffffffull);
+        }
+      }
+      // every load of the step is requested here; the next step's records go last, so that
+      // waiting for the operands leaves them in flight
+      u32x4 xa[KK], wf[PW][KK];
+      const uint16_t* xp = X + (int64_t)cur.src * FIN + 8 * h;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) xa[kk] = *reinterpret_cast<const u32x4*>(xp + 16 * kk);
+      const uint16_t wbits = *reinterpret_cast<const GlobalU16*>(((uint64_t)cur.w_hi << 32) | cur.w_lo);
+#pragma unroll
+      for (int q = 0; q < PW; ++q) {
+        if (r[q] >= 0) {
+          const u32x4* w = Wp + ((int64_t)r[q] * ntiles + nti) * KK * 64 + lane;
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) wf[q][kk] = w[kk * 64];
+        }
+      }
+      next = edges[min(e0 + kStepEdges + mrow, e_end - 1)];  // the last step re-reads the last record
+
+      // ---- stage 1
+      f32x16 acc1;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc1[v] = 0.f;
+      auto add_run = [&](int rq, const u32x4* w) {
+        const bool sel = rel == rq;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          u32x4 a;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) a[d] = sel ? xa[kk][d] : 0u;
+          acc1 = mfma32<BF16>(a, w[kk], acc1);
+        }
+      };
+#pragma unroll
+      for (int q = 0; q < PW; ++q)
+        if (r[q] >= 0) add_run(r[q], wf[q]);
+      while (pos < kStepEdges) {  // steps with more than PW relations: one at a time
+        const int rq = __builtin_amdgcn_readlane(rel, pos);
+        pos += __popcll(__ballot(rel == rq) & 0xffffffffull);
+        const u32x4* w = Wp + ((int64_t)rq * ntiles + nti) * KK * 64 + lane;
+        u32x4 wl[KK];
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) wl[kk] = w[kk * 64];
+        add_run(rq, wl);
+      }
+
+      // ---- stage 2
+      if (h == 0) S[dl * kSStride + jcol] = live ? wbits : (uint16_t)0;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      const u32x4 sa0 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 8 * h);
+      u32x4 sa1 = {0u, 0u, 0u, 0u};
+      if (left > 16) sa1 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 16 + 8 * h);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (h == 0) S[dl * kSStride + jcol] = 0;
+      float t[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) t[v] = acc1[v];
+      acc2 = stage2<BF16>(sa0, t, acc2);
+      if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
+    }
+
+    // ---- write back: acc2[v] is row (v%4) + 4h + 8(v/4) of the tile, output feature 32 nti + lane%32
+    float* ybase = Y + ((int64_t)tile * kTileRows + 4 * h) * feat_out + 32 * nti + mrow;
+    const int rows_left = m - (tile * kTileRows + 4 * h);  // rows v%4 + 8(v/4) below this count exist
+    if (u.tile_flag & 1) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int rr = (v & 3) + 8 * (v >> 2);
+        if (rr < rows_left)
+          __hip_atomic_fetch_add(ybase + (int64_t)rr * feat_out, acc2[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else {
+      float old[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int rr = (v & 3) + 8 * (v >> 2);
+        old[v] = rr < rows_left ? ybase[(int64_t)rr * feat_out] : 0.f;
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int rr = (v & 3) + 8 * (v >> 2);
+        if (rr < rows_left) ybase[(int64_t)rr * feat_out] = old[v] + acc2[v];
+      }
+    }
+  }
+}
+
+struct DevBuf {
+  void* p = nullptr;
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+  hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16); }
+  template <typename T>
+  T* as() const { return static_cast<T*>(p); }
+};
+
+int bit_length(uint64_t x) {
+  int b = 0;
+  while (x) ++b, x >>= 1;
+  return b;
+}
+
+}  // namespace
+
+void tile_index_free(TileIndex& ix) {
+  if (ix.d_edges) (void)hipFree(ix.d_edges);
+  if (ix.d_units) (void)hipFree(ix.d_units);
+  if (ix.d_wpack) (void)hipFree(ix.d_wpack);
+  ix = TileIndex();
+}
+
+int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
+                       int32_t num_rels, hipStream_t stream) {
+  if (ix.m == m && ix.n == n && ix.num_rels == num_rels) return 0;
+  STIR_REQUIRE(num_rels > 0 && num_rels < (1 << 26), "rgms: num_rels=%d out of range", num_rels);
+  if (ix.d_edges) STIR_HIP(hipFree(ix.d_edges));
+  if (ix.d_units) STIR_HIP(hipFree(ix.d_units));
+  ix.d_edges = ix.d_units = nullptr;
+  ix.m = -1;
+  ix.edges = ix.units = 0;
+  std::vector<DevBucket> host;
+  int64_t slots = 0;
+  for (const TileBucket& b : buckets) {
+    if (b.groups == 0) continue;
+    host.push_back(DevBucket{b.A, b.rows, b.cols, b.mids, slots, b.rb, b.cb});
+    slots += b.groups * b.rb * b.cb;
+  }
+  STIR_REQUIRE(slots < (int64_t(1) << 31), "rgms: %lld slots exceed the edge index", (long long)slots);
+  if (slots == 0 || m == 0) {
+    ix.m = m, ix.n = n, ix.num_rels = num_rels;
+    return 0;
+  }
+  const int nb = (int)host.size();
+  const int64_t tiles = ceil_div(m, kTileRows);
+  const int end_bit = bit_length((((uint64_t)tiles * num_rels) << 5) - 1);
+  int dev = 0, cus = 256;
+  STIR_HIP(hipGetDevice(&dev));
+  STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  // units of about total steps / (8 per CU), at least 16 steps: tiles are cut only when the
+  // launch would otherwise leave most of the chip idle
+  const int64_t steps_bound = slots / kStepEdges + tiles;
+  const int cap = (int)std::max<int64_t>(16, ceil_div(steps_bound, (int64_t)cus * 8));
+
+  size_t sort_bytes = 0, scan_bytes = 0;
+  STIR_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, (const uint64_t*)nullptr, (uint64_t*)nullptr,
+                                              (const int32_t*)nullptr, (int32_t*)nullptr, (int)slots, 0, end_bit,
+                                              stream));
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, scan_bytes, (const int32_t*)nullptr, (int32_t*)nullptr,
+                                            (int)(tiles + 1), stream));
+  DevBuf tab, keys_in, keys, vals_in, vals, tmp, bad, begin, count, ubegin;
+  STIR_HIP(tab.alloc(sizeof(DevBucket) * host.size()));
+  STIR_HIP(keys_in.alloc(sizeof(uint64_t) * size_t(slots)));
+  STIR_HIP(keys.alloc(sizeof(uint64_t) * size_t(slots)));
+  STIR_HIP(vals_in.alloc(sizeof(int32_t) * size_t(slots)));
+  STIR_HIP(vals.alloc(sizeof(int32_t) * size_t(slots)));
+  STIR_HIP(tmp.alloc(std::max(sort_bytes, scan_bytes)));
+  STIR_HIP(bad.alloc(sizeof(int32_t)));
+  STIR_HIP(begin.alloc(sizeof(int64_t) * size_t(tiles + 1)));
+  STIR_HIP(count.alloc(sizeof(int32_t) * size_t(tiles + 1)));
+  STIR_HIP(ubegin.alloc(sizeof(int32_t) * size_t(tiles + 1)));
+  DevBuf edges;
+  STIR_HIP(edges.alloc(sizeof(Edge) * size_t(slots)));
+
+  STIR_HIP(hipMemcpyAsync(tab.p, host.data(), sizeof(DevBucket) * host.size(), hipMemcpyHostToDevice, stream));
+  STIR_HIP(hipMemsetAsync(bad.p, 0, sizeof(int32_t), stream));
+  const dim3 block(256);
+  const dim3 slot_grid((unsigned)ceil_div(slots, 256)), tile_grid((unsigned)ceil_div(tiles + 1, 256));
+  hipLaunchKernelGGL(edge_keys_kernel, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, m, num_rels,
+                     keys_in.as<uint64_t>(), vals_in.as<int32_t>(), bad.as<int32_t>());
+  STIR_LAUNCH_CHECK();
+  STIR_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, sort_bytes, keys_in.as<const uint64_t>(), keys.as<uint64_t>(),
+                                              vals_in.as<const int32_t>(), vals.as<int32_t>(), (int)slots, 0,
+                                              end_bit, stream));
+  hipLaunchKernelGGL(edge_records_kernel, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, n, num_rels,
+                     keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<Edge>(), bad.as<int32_t>());
+  STIR_LAUNCH_CHECK();
+  hipLaunchKernelGGL(tile_bounds_kernel, tile_grid, block, 0, stream, keys.as<const uint64_t>(), slots, tiles,
+                     num_rels, begin.as<int64_t>());
+  STIR_LAUNCH_CHECK();
+  hipLaunchKernelGGL(unit_count_kernel, tile_grid, block, 0, stream, begin.as<const int64_t>(), tiles, cap,
+                     count.as<int32_t>());
+  STIR_LAUNCH_CHECK();
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(tmp.p, scan_bytes, count.as<const int32_t>(), ubegin.as<int32_t>(),
+                                            (int)(tiles + 1), stream));
+  int32_t h_bad = 0, h_units = 0;
+  STIR_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+  STIR_HIP(hipMemcpyAsync(&h_units, ubegin.as<int32_t>() + tiles, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+  STIR_HIP(hipStreamSynchronize(stream));
+  if (h_bad == 1) return fail("rgms: a row id lies outside [0, %d) or a relation id outside [0, %d)", m, num_rels);
+  if (h_bad == 2) return fail("rgms: a column id lies outside [0, %d)", n);
+  DevBuf units;
+  STIR_HIP(units.alloc(sizeof(Unit) * size_t(h_units)));
+  hipLaunchKernelGGL(unit_fill_kernel, tile_grid, block, 0, stream, begin.as<const int64_t>(),
+                     ubegin.as<const int32_t>(), tiles, cap, units.as<Unit>());
+  STIR_LAUNCH_CHECK();
+  STIR_HIP(hipStreamSynchronize(stream));
+  ix.d_edges = edges.p, edges.p = nullptr;
+  ix.d_units = units.p, units.p = nullptr;
+  ix.edges = slots;
+  ix.units = h_units;
+  ix.m = m, ix.n = n, ix.num_rels = num_rels;
+  return 0;
+}
+
+int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
+                     float* d_Y, hipStream_t stream) {
+  STIR_REQUIRE(ix.m >= 0, "rgms: the edge index has not been built");
+  if (ix.units == 0) return 0;
+  STIR_REQUIRE(feat_in % 16 == 0 && feat_in / 16 <= kMaxKK && feat_out % 32 == 0, "rgms: unsupported feature sizes");
+  const int kk_count = feat_in / 16;
+  const int64_t frags = (int64_t)ix.num_rels * (feat_out / 32) * kk_count;
+  const size_t need = size_t(frags) * 64 * sizeof(u32x4);
+  if (need > ix.wpack_bytes) {
+    if (ix.d_wpack) STIR_HIP(hipFree(ix.d_wpack));
+    ix.d_wpack = nullptr;
+    ix.wpack_bytes = 0;
+    STIR_HIP(hipMalloc(&ix.d_wpack, need));
+    ix.wpack_bytes = need;
+  }
+  u32x4* Wp = static_cast<u32x4*>(ix.d_wpack);
+  hipLaunchKernelGGL(pack_w_kernel, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream,
+                     static_cast<const uint16_t*>(d_W), Wp, frags, kk_count, feat_out);
+  STIR_LAUNCH_CHECK();
+  const dim3 grid((unsigned)ceil_div(ix.units, 4)), block(256);
+  const Unit* units = static_cast<const Unit*>(ix.d_units);
+  const Edge* edges = static_cast<const Edge*>(ix.d_edges);
+  const uint16_t* X = static_cast<const uint16_t*>(d_X);
+#define STIR_TILES(KKV)                                                                                          \
+  case KKV:                                                                                                      \
+    if (bf16)                                                                                                    \
+      hipLaunchKernelGGL((rgms_tile_kernel<KKV, true>), grid, block, 0, stream, units, ix.units, edges, ix.m,    \
+                         feat_out, Wp, X, d_Y);                                                                  \
+    else                                                                                                         \
+      hipLaunchKernelGGL((rgms_tile_kernel<KKV, false>), grid, block, 0, stream, units, ix.units, edges, ix.m,   \
+                         feat_out, Wp, X, d_Y);                                                                  \
+    break
+  switch (kk_count) {
+    STIR_TILES(1);
+    STIR_TILES(2);
+    STIR_TILES(3);
+    STIR_TILES(4);
+    STIR_TILES(5);
+    STIR_TILES(6);
+    STIR_TILES(7);
+    STIR_TILES(8);
+  }
+#undef STIR_TILES
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace stir

@@ -147,3 +147,82 @@ def test_rgms_bf16(dev):
     av = np.ones(len(csf[3]), np.float32)
     _check(y.cpu().numpy().reshape(n, fout), csf, av, x.float().cpu().numpy(), w.float().cpu().numpy(), n, "bf16")
     assert torch.allclose(y, y2, rtol=1e-5, atol=1e-5)
+
+
+def _csf_from_pairs(pairs, n):
+    """CSF from one (dst, src) array pair per relation (duplicates removed, sorted)."""
+    indptr0, indices0, indptr1, indices1, nnz = [0], [], [0], [], 0
+    for dst, src in pairs:
+        key = np.unique(dst.astype(np.int64) * n + src)
+        dst, src = key // n, key % n
+        rows, counts = np.unique(dst, return_counts=True)
+        indptr0.append(indptr0[-1] + len(rows))
+        indices0.append(rows)
+        indptr1.append(nnz + np.cumsum(counts))
+        indices1.append(src)
+        nnz += len(src)
+    i32 = lambda parts: np.concatenate([np.atleast_1d(p) for p in parts]).astype(np.int32)
+    return i32(indptr0), i32(indices0), i32(indptr1), i32(indices1)
+
+
+@pytest.mark.parametrize("fin,fout,group,buckets,bf16", [
+    (32, 32, 256, [1, 2, 4, 8, 16], False),
+    (16, 64, 64, [1, 2, 4, 64], False),
+    (48, 32, 48, [1, 3, 4, 16], False),
+    (128, 32, 32, [2, 8, 32], False),
+    (32, 64, 64, [1, 4, 16], True),
+])
+def test_rgms_tiled_hub_rows(dev, fin, fout, group, buckets, bf16):
+    """Destination-tiled path (64k slots and more): output rows not a multiple of 32, one row that
+    receives thousands of edges in three relations (its tile is cut into several units that meet
+    in atomics), relations without edges, widths that are not powers of two."""
+    n, R = 5001, 7
+    rng = np.random.default_rng(fin + fout)
+    pairs = []
+    for r in range(R):
+        e = 0 if r == 3 else 20000
+        dst, src = rng.integers(0, n, e), rng.integers(0, n, e)
+        if r in (0, 1, 5):
+            hub = rng.choice(n, 3000, replace=False)
+            dst = np.concatenate([dst, np.full(3000, 77)])
+            src = np.concatenate([src, hub])
+        pairs.append((dst, src))
+    csf = _csf_from_pairs(pairs, n)
+    rows_bkt = [max(1, group // b) for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    assert sum(mk.size for mk in mask) >= 65536
+    tdt = torch.bfloat16 if bf16 else torch.float16
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    x = t(rng.standard_normal((n, fin), dtype=np.float32)).to(tdt)
+    w = t(rng.standard_normal((R, fin, fout), dtype=np.float32) * 0.1).to(tdt)
+    triples, mids, wts = [], [], []
+    for b in range(len(buckets)):
+        a = t(mask[b].astype(np.float32) * (0.5 + rng.random(mask[b].shape, dtype=np.float32))).to(tdt)
+        wts.append(a.float().cpu().numpy())
+        triples += [a.reshape(-1), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    f = ops.build_rgms(n, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols], dtype=tdt)
+    y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
+    f(w.reshape(-1), x.reshape(-1), y, *triples, *mids)
+    torch.cuda.synchronize()
+    # closed form in float64 straight from the ELL3D arrays: Y[row] += a * X[col] @ W[rel]
+    x64, w64 = x.double().cpu().numpy(), w.double().cpu().numpy()
+    want, scale = np.zeros((n, fout)), np.zeros((n, fout))
+    for b in range(len(buckets)):
+        G, rb, cb = cols[b].shape
+        rel = np.repeat(np.arange(R), np.diff(ptr[b]))
+        for r in range(R):
+            g = np.nonzero(rel == r)[0]
+            if len(g) == 0:
+                continue
+            a = wts[b][g].reshape(-1, cb).astype(np.float64)
+            c = cols[b][g].reshape(-1, cb)
+            agg = np.einsum("es,esk->ek", a, x64[c])
+            agg_abs = np.einsum("es,esk->ek", a, np.abs(x64[c]))
+            dest = rows[b][g].reshape(-1)
+            np.add.at(want, dest, agg @ w64[r])
+            np.add.at(scale, dest, agg_abs @ np.abs(w64[r]))
+    got = y.cpu().numpy().reshape(n, fout).astype(np.float64)
+    err = np.abs(got - want)
+    assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), f"worst {err.max():.3e}"
+    assert np.abs(want[77]).max() > 0
