@@ -21,6 +21,10 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
 # Packed fp32 VALU ops are kept off for every device translation unit.
 DEVICE = [f"--offload-arch={ARCH}", "-munsafe-fp-atomics",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Per-file additions.  The destination-tiled RGMS kernel chains MFMAs through ordinary vector
+# registers (one accumulator feeds the next stage's operand); with the accumulator-register form
+# the compiler copies both accumulators between the two register files on every step.
+EXTRA = {"rgms_tiles.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources():
@@ -31,7 +35,7 @@ def _compile(src):
     obj = os.path.join(OBJ, os.path.basename(src) + ".o")
     cmd = [HIPCC] + COMMON
     if src.endswith(".hip"):
-        cmd += DEVICE + ["-x", "hip"]
+        cmd += DEVICE + EXTRA.get(os.path.basename(src), []) + ["-x", "hip"]
     cmd += ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     return src, obj, r.returncode, r.stdout + r.stderr

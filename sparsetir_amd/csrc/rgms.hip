@@ -8,11 +8,11 @@
 // are loaded once per group and stay in registers.  The 32x32 fp32 result tile is scaled by
 // the slot weights, summed over the slots of each ELL row inside the wavefront (register adds
 // plus one cross-half exchange) and added to Y with one fp32 atomic per (ELL row, feature).
+// This kernel serves small inputs; from kTileMinSlots slots on, the destination-tiled kernel of
+// rgms_tiles.hip (no atomics) takes over.
 #include <vector>
 
 #include "common.h"
-#include <cstdlib>
-#include "dest_index.h"
 #include "rgms_tiles.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -32,7 +32,6 @@ struct alignas(16) RgmsBucket {
   const int32_t* mids;  // groups
   int64_t groups;
   int64_t unit_begin;  // first work unit (one wavefront each) of this bucket in the fused launch
-  int64_t row_begin;   // first row of the bucket in the staging matrix (buckets with log2cb >= 0)
   int32_t rb, cb;
   int32_t log2cb;  // log2(cb) when cb is a power of two <= 32, else -1
   int32_t chunks;  // work units per group: ceil(rb*cb / kChunkSlots)
@@ -74,7 +73,7 @@ __device__ __forceinline__ void atomic_addf(float* p, float v) {
 template <int KK, int LCB, bool BF16>
 __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int chunk, int feat_out,
                                            const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
-                                           float* __restrict__ Y, float* __restrict__ Z, int lane) {
+                                           float* __restrict__ Y, int lane) {
   constexpr int FIN = KK * 16;
   constexpr int TI = KK <= 2 ? 4 : 2;  // tiles in flight
   constexpr int MJ = TI / 2;           // 64-slot metadata registers per lane
@@ -98,16 +97,8 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
       }
     }
     float* yb = Y + nt + n;
-    // staging rows of this group (power-of-two cb): row q of the group is zb + q * feat_out
-    float* zb = (LCB >= 0 && Z) ? Z + (bk.row_begin + g * bk.rb) * feat_out + nt + n : nullptr;
-    // result of ELL row q of the group, output row `row`: a plain store to the staging matrix
-    // (every row, zeros included: the matrix is not cleared), else an atomic add to Y
-    auto emit = [&](int q, int row, float v) {
-      if (zb)
-        zb[(int64_t)q * feat_out] = v;
-      else
-        atomic_addf(yb + (int64_t)row * feat_out, v);
-    };
+    // result of an ELL row with output row `row`
+    auto emit = [&](int row, float v) { atomic_addf(yb + (int64_t)row * feat_out, v); };
     const int s_end = min(gsize, (chunk + 1) * kChunkSlots);
 #pragma unroll 1
     for (int s_base = chunk * kChunkSlots; s_base < s_end; s_base += 32 * TI) {
@@ -170,14 +161,14 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
           for (int v = 0; v < 16; ++v) {
             const int sl = 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
             const int row = row_of(sl, t >> 1);
-            if (zb ? s_base + sl < gsize : wgt[v] != 0.f) emit(s_base + sl, row, wgt[v] != 0.f ? acc[v] : 0.f);
+            if (wgt[v] != 0.f) emit(row, acc[v]);
           }
         } else if constexpr (LCB == 1) {
 #pragma unroll
           for (int v = 0; v < 16; v += 2) {
             const int sl = 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
             const int row = row_of(sl >> 1, t >> 2);
-            if (s_base + sl < gsize) emit((s_base + sl) >> 1, row, acc[v] + acc[v + 1]);
+            if (s_base + sl < gsize) emit(row, acc[v] + acc[v + 1]);
           }
         } else {
           // cb >= 4: the four registers of a quad belong to one ELL row
@@ -189,7 +180,7 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
             for (int u = 0; u < 4; ++u) {
               const int sl = 32 * t + 4 * h + 8 * u;
               const int row = row_of(sl >> 2, 0);
-              if (s_base + sl < gsize) emit((s_base + sl) >> 2, row, q4[u]);
+              if (s_base + sl < gsize) emit(row, q4[u]);
             }
           } else {
             // cb >= 8: add the other half-wave's quad (slots 8u+4..8u+7 vs 8u..8u+3)
@@ -203,17 +194,17 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
                 const int sl = 32 * t + 8 * tt;
                 const float val = tt == 0 ? q4[0] : tt == 1 ? q4[1] : tt == 2 ? q4[2] : q4[3];
                 const int row = row_of(sl >> 3, 0);
-                if (s_base + sl < gsize) emit((s_base + sl) >> 3, row, val);
+                if (s_base + sl < gsize) emit(row, val);
               }
             } else if constexpr (LCB == 4) {
               const float val = h == 0 ? q4[0] + q4[1] : q4[2] + q4[3];
               const int sl = 32 * t + 16 * h;
               const int row = row_of(sl >> 4, 0);
-              if (s_base + sl < gsize) emit((s_base + sl) >> 4, row, val);
+              if (s_base + sl < gsize) emit(row, val);
             } else {  // cb == 32: the whole tile is one ELL row
               const float val = (q4[0] + q4[1]) + (q4[2] + q4[3]);
               const int row = row_of(t, 0);
-              if (h == 0 && tile_live) emit((s_base >> 5) + t, row, val);
+              if (h == 0 && tile_live) emit(row, val);
             }
           }
         }
@@ -229,8 +220,7 @@ template <int KK, bool BF16>
 __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict__ table, int nb,
                                                    int64_t total_units, int feat_out,
                                                    const uint16_t* __restrict__ W,
-                                                   const uint16_t* __restrict__ X, float* __restrict__ Y,
-                                                   float* __restrict__ Z) {
+                                                   const uint16_t* __restrict__ X, float* __restrict__ Y) {
   const int lane = threadIdx.x & 63;
   const int64_t gid = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   if (gid >= total_units) return;
@@ -244,31 +234,28 @@ __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict_
   const int64_t g = unit / bk.chunks;
   const int chunk = (int)(unit % bk.chunks);
   switch (bk.log2cb) {
-    case 0: rgms_group<KK, 0, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 1: rgms_group<KK, 1, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 2: rgms_group<KK, 2, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 3: rgms_group<KK, 3, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 4: rgms_group<KK, 4, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    case 5: rgms_group<KK, 5, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
-    default: rgms_group<KK, -1, BF16>(bk, g, chunk, feat_out, W, X, Y, Z, lane); break;
+    case 0: rgms_group<KK, 0, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 1: rgms_group<KK, 1, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 2: rgms_group<KK, 2, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 3: rgms_group<KK, 3, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 4: rgms_group<KK, 4, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 5: rgms_group<KK, 5, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    default: rgms_group<KK, -1, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
   }
 }
 
 }  // namespace
 
-// Below this many ELL rows the atomics cost less than a second launch.
-constexpr int64_t kStagingMinRows = 32768;
+// From this many slots on the destination-tiled kernel is used (its index is built by the first
+// launch); below, one launch of the atomic kernel costs less.
+constexpr int64_t kTileMinSlots = 8192;
 
 struct stir_rgms_plan {
   int nk;
   RgmsBucket* d_table;
   int64_t total_units;
-  // scatter-free accumulation: buckets with power-of-two cb write their rows to a staging
-  // matrix that a second kernel adds up per output row; index and matrix are made by the first
-  // launch (they need m and feat_out) and kept
-  std::vector<stir::DestBucket> staged;
-  int64_t staged_rows;
-  stir::DestIndex dest;
+  // destination-tiled path: the edge index is made by the first launch (it needs m, n and
+  // num_rels) and kept
   std::vector<stir::TileBucket> tile_buckets;
   int64_t slots;
   stir::TileIndex tiles;
@@ -283,8 +270,7 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   STIR_REQUIRE(plan && num_buckets > 0, "rgms_plan_create: bad arguments");
   RgmsBucket* host = new RgmsBucket[num_buckets];
   int nk = 0;
-  int64_t total = 0, staged_rows = 0;
-  std::vector<stir::DestBucket> staged;
+  int64_t total = 0;
   std::vector<stir::TileBucket> tile_buckets;
   int64_t slots = 0;
   for (int b = 0; b < num_buckets; ++b) {
@@ -314,12 +300,6 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
       e.log2cb = l;
     }
     e.chunks = (int32_t)stir::ceil_div((int64_t)rows_bkt[b] * cols_bkt[b], kChunkSlots);
-    e.row_begin = 0;
-    if (e.log2cb >= 0) {
-      e.row_begin = staged_rows;
-      staged.push_back(stir::DestBucket{e.rows, groups[b] * rows_bkt[b], staged_rows});
-      staged_rows += groups[b] * rows_bkt[b];
-    }
     host[nk++] = e;
     total += groups[b] * e.chunks;
     tile_buckets.push_back(stir::TileBucket{e.A, e.rows, e.cols, e.mids, e.groups, e.rb, e.cb});
@@ -329,8 +309,6 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   p->nk = nk;
   p->total_units = total;
   p->d_table = nullptr;
-  p->staged = staged;
-  p->staged_rows = staged_rows;
   p->tile_buckets = tile_buckets;
   p->slots = slots;
   hipError_t err = hipSuccess;
@@ -364,27 +342,21 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* W = static_cast<const uint16_t*>(d_W);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
-  // the plan's staging state is filled in by the first launch (plans are not shared between
-  // host threads)
-  stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
-  static const bool legacy = getenv("STIR_RGMS_LEGACY") != nullptr;
-  if (!legacy && mp->slots >= 65536 && mp->slots < (int64_t(1) << 31)) {
+  if (plan->slots >= kTileMinSlots && plan->slots < (int64_t(1) << 31)) {
+    // the plan's edge index and packed copy of W are filled in by the launches: a plan serves
+    // one call at a time
+    stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
     if (stir::tile_index_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, st)) return -1;
     return stir::tile_rgms_launch(bf16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
-  }
-  float* Z = nullptr;
-  if (mp->staged_rows >= kStagingMinRows) {
-    if (stir::dest_index_prepare(mp->dest, mp->staged, m, feat_out, st)) return -1;
-    Z = mp->dest.d_Z;
   }
 #define STIR_RGMS(KK)                                                                              \
   case KK:                                                                                         \
     if (bf16)                                                                                      \
       hipLaunchKernelGGL((rgms_kernel<KK, true>), grid, block, 0, st, plan->d_table, plan->nk,     \
-                         plan->total_units, feat_out, W, X, d_Y, Z);                              \
+                         plan->total_units, feat_out, W, X, d_Y);                              \
     else                                                                                           \
       hipLaunchKernelGGL((rgms_kernel<KK, false>), grid, block, 0, st, plan->d_table, plan->nk,    \
-                         plan->total_units, feat_out, W, X, d_Y, Z);                              \
+                         plan->total_units, feat_out, W, X, d_Y);                              \
     break
   switch (feat_in / 16) {
     STIR_RGMS(1);
@@ -398,7 +370,6 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
   }
 #undef STIR_RGMS
   STIR_LAUNCH_CHECK();
-  if (Z) return stir::dest_reduce(mp->dest, feat_out, d_Y, st);
   return 0;
 }
 
@@ -415,7 +386,6 @@ int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num
 int stir_rgms_plan_destroy(stir_rgms_plan* plan) {
   if (!plan) return 0;
   if (plan->d_table) (void)hipFree(plan->d_table);
-  stir::dest_index_free(plan->dest);
   stir::tile_index_free(plan->tiles);
   delete plan;
   return 0;

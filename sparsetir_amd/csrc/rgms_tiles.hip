@@ -47,6 +47,7 @@ struct alignas(16) Unit {
 constexpr int kTileRows = 32;
 constexpr int kStepEdges = 32;
 constexpr int kMaxKK = 8;
+constexpr int kUnitWaves = 4;  // wavefronts that share a unit
 
 __device__ __forceinline__ int bucket_of(const DevBucket* __restrict__ tab, int nb, int64_t q) {
   int lo = 0, hi = nb - 1;
@@ -215,20 +216,22 @@ __device__ __forceinline__ f32x16 stage2(u32x4 sa, const float* t, f32x16 acc) {
 
 constexpr int kSStride = 40;  // 16-bit elements per row of the S tile (32 used; 80-byte rows)
 
-// One wavefront per unit, 4 per workgroup; no workgroup barrier is used, so wavefronts without a
-// unit leave at once.  KK = feat_in / 16.
+// One workgroup per unit.  Its four wavefronts take the unit's steps in turn (wavefront w the
+// steps w, w + 4, ...: more wavefronts in flight per tile, since a step costs a full memory
+// round trip), each with its own accumulator tile; the four tiles are added through LDS and the
+// workgroup writes the 32 rows of Y once.  KK = feat_in / 16.
 template <int KK, bool BF16>
-__global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__ units, int64_t n_units,
+__global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__ units,
                                                         const Edge* __restrict__ edges, int m, int feat_out,
                                                         const u32x4* __restrict__ Wp, const uint16_t* __restrict__ X,
                                                         float* __restrict__ Y) {
   constexpr int FIN = KK * 16;
   constexpr int PW = KK <= 4 ? 2 : 1;  // relations whose W fragments are requested together
-  __shared__ __attribute__((aligned(16))) uint16_t s_all[4][kTileRows * kSStride];
+  __shared__ __attribute__((aligned(16))) uint16_t s_all[kUnitWaves][kTileRows * kSStride];
+  __shared__ float partial[kUnitWaves][16 * 64];  // [wavefront][accumulator register][lane]
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t uid = (int64_t)blockIdx.x * 4 + wave;
-  if (uid >= n_units) return;
+  const int64_t uid = blockIdx.x;
   uint16_t* S = s_all[wave];
   {
     uint32_t* s32 = reinterpret_cast<uint32_t*>(S);
@@ -250,10 +253,13 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc2[v] = 0.f;
     // lanes past the last edge repeat it with weight zero
-    Edge next = edges[min(u.edge_begin + mrow, e_end - 1)];
+    constexpr int64_t kStride = kUnitWaves * kStepEdges;  // edges between a wavefront's steps
+    Edge next = edges[min(u.edge_begin + wave * kStepEdges + mrow, e_end - 1)];
+    Edge after = edges[min(u.edge_begin + wave * kStepEdges + kStride + mrow, e_end - 1)];
 #pragma unroll 1
-    for (int64_t e0 = u.edge_begin; e0 < e_end; e0 += kStepEdges) {
+    for (int64_t e0 = u.edge_begin + wave * kStepEdges; e0 < e_end; e0 += kStride) {
       const Edge cur = next;
+      next = after;
       const int left = (int)min((int64_t)kStepEdges, e_end - e0);  // uniform
       const bool live = mrow < left;
       const int rel = (int)(cur.rel_dl >> 5), dl = (int)(cur.rel_dl & 31);
@@ -267,8 +273,9 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
           pos += __popcll(__ballot(rel == r[q]) & 0xffffffffull);
         }
       }
-      // every load of the step is requested here; the next step's records go last, so that
-      // waiting for the operands leaves them in flight
+      // every load of the step is requested here; the records of the step after the next go
+      // last, so that waiting for the operands leaves them in flight (loads retire in order, so
+      // they have until the next step's operands are waited for)
       u32x4 xa[KK], wf[PW][KK];
       const uint16_t* xp = X + (int64_t)cur.src * FIN + 8 * h;
 #pragma unroll
@@ -282,7 +289,7 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
           for (int kk = 0; kk < KK; ++kk) wf[q][kk] = w[kk * 64];
         }
       }
-      next = edges[min(e0 + kStepEdges + mrow, e_end - 1)];  // the last step re-reads the last record
+      after = edges[min(e0 + 2 * kStride + mrow, e_end - 1)];  // past the end: the last record again
 
       // ---- stage 1
       f32x16 acc1;
@@ -328,29 +335,36 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
       if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
     }
 
-    // ---- write back: acc2[v] is row (v%4) + 4h + 8(v/4) of the tile, output feature 32 nti + lane%32
-    float* ybase = Y + ((int64_t)tile * kTileRows + 4 * h) * feat_out + 32 * nti + mrow;
-    const int rows_left = m - (tile * kTileRows + 4 * h);  // rows v%4 + 8(v/4) below this count exist
-    if (u.tile_flag & 1) {
+    // ---- add the four tiles and write back.  acc2[v] of lane (n, h) is row (v%4) + 4h + 8(v/4)
+    // of the tile, output feature 32 nti + n.
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int rr = (v & 3) + 8 * (v >> 2);
-        if (rr < rows_left)
-          __hip_atomic_fetch_add(ybase + (int64_t)rr * feat_out, acc2[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    } else {
-      float old[16];
+    for (int v = 0; v < 16; ++v) partial[wave][v * 64 + lane] = acc2[v];
+    const bool atomic = u.tile_flag & 1;
+    float yold[4];  // requested before the barrier
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int rr = (v & 3) + 8 * (v >> 2);
-        old[v] = rr < rows_left ? ybase[(int64_t)rr * feat_out] : 0.f;
-      }
+    for (int k = 0; k < 4; ++k) {
+      const int elem = threadIdx.x + 256 * k;
+      const int64_t yrow = (int64_t)tile * kTileRows + (elem >> 5);
+      yold[k] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + (elem & 31)] : 0.f;
+    }
+    __syncthreads();
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int rr = (v & 3) + 8 * (v >> 2);
-        if (rr < rows_left) ybase[(int64_t)rr * feat_out] = old[v] + acc2[v];
+    for (int k = 0; k < 4; ++k) {
+      const int elem = threadIdx.x + 256 * k, row = elem >> 5, col = elem & 31;
+      const int at = ((row & 3) + 4 * (row >> 3)) * 64 + col + 32 * ((row >> 2) & 1);
+      float sum = partial[0][at];
+#pragma unroll
+      for (int w = 1; w < kUnitWaves; ++w) sum += partial[w][at];
+      const int64_t yrow = (int64_t)tile * kTileRows + row;
+      if (yrow < m) {
+        float* y = Y + yrow * feat_out + 32 * nti + col;
+        if (atomic)
+          __hip_atomic_fetch_add(y, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+          *y = yold[k] + sum;
       }
     }
+    if (nti + 1 < ntiles) __syncthreads();  // the partial sums are rewritten by the next pass
   }
 }
 
@@ -406,10 +420,10 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   int dev = 0, cus = 256;
   STIR_HIP(hipGetDevice(&dev));
   STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  // units of about total steps / (8 per CU), at least 16 steps: tiles are cut only when the
-  // launch would otherwise leave most of the chip idle
+  // units (one workgroup each) of about total steps / (8 per CU), at least 16 steps: tiles are
+  // cut only when the launch would otherwise leave most of the chip idle
   const int64_t steps_bound = slots / kStepEdges + tiles;
-  const int cap = (int)std::max<int64_t>(16, ceil_div(steps_bound, (int64_t)cus * 8));
+  const int cap = (int)std::max<int64_t>(16, kUnitWaves * ceil_div(steps_bound, (int64_t)cus * 8));
 
   size_t sort_bytes = 0, scan_bytes = 0;
   STIR_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, (const uint64_t*)nullptr, (uint64_t*)nullptr,
@@ -491,17 +505,17 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   hipLaunchKernelGGL(pack_w_kernel, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream,
                      static_cast<const uint16_t*>(d_W), Wp, frags, kk_count, feat_out);
   STIR_LAUNCH_CHECK();
-  const dim3 grid((unsigned)ceil_div(ix.units, 4)), block(256);
+  const dim3 grid((unsigned)ix.units), block(64 * kUnitWaves);
   const Unit* units = static_cast<const Unit*>(ix.d_units);
   const Edge* edges = static_cast<const Edge*>(ix.d_edges);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
 #define STIR_TILES(KKV)                                                                                          \
   case KKV:                                                                                                      \
     if (bf16)                                                                                                    \
-      hipLaunchKernelGGL((rgms_tile_kernel<KKV, true>), grid, block, 0, stream, units, ix.units, edges, ix.m,    \
+      hipLaunchKernelGGL((rgms_tile_kernel<KKV, true>), grid, block, 0, stream, units, edges, ix.m,    \
                          feat_out, Wp, X, d_Y);                                                                  \
     else                                                                                                         \
-      hipLaunchKernelGGL((rgms_tile_kernel<KKV, false>), grid, block, 0, stream, units, ix.units, edges, ix.m,   \
+      hipLaunchKernelGGL((rgms_tile_kernel<KKV, false>), grid, block, 0, stream, units, edges, ix.m,   \
                          feat_out, Wp, X, d_Y);                                                                  \
     break
   switch (kk_count) {

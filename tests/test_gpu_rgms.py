@@ -85,17 +85,16 @@ def test_rgms_config5_reduced(dev):
 
 
 @pytest.mark.parametrize("group,buckets", [(256, [1, 2, 4, 8, 16]), (32, [1, 2, 4, 8, 16, 32]), (48, [1, 3, 4, 16])])
-def test_rgms_staged_accumulation(dev, group, buckets):
-    """Enough ELL rows for the scatter-free path (results staged per ELL row, then summed per
-    output row); a bucket with a width that is not a power of two still goes through atomics in
-    the same launch.  Called twice on one operator: the second call reuses the index."""
+def test_rgms_tiled_accumulation(dev, group, buckets):
+    """Enough slots for the destination-tiled kernel (edges re-indexed by 32-row output tile, no
+    atomics), bucket widths that are not powers of two included."""
     cfg = datasets.config5(n=20000, num_rels=9, num_edges=200000, seed=7)
     csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
     got, x32, w32, av = _run(dev, csf, cfg["m"], cfg["n"], cfg["x"], cfg["w"], group, buckets, True)
-    _check(got, csf, av, x32, w32, cfg["m"], f"staged group={group}")
+    _check(got, csf, av, x32, w32, cfg["m"], f"tiled group={group}")
 
 
-def test_rgms_staged_repeat_calls_accumulate(dev):
+def test_rgms_tiled_repeat_calls_accumulate(dev):
     cfg = datasets.config5(n=20000, num_rels=5, num_edges=150000, seed=8)
     csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
     R, fin, fout, buckets, group = 5, 32, 32, [1, 2, 4, 8], 64
@@ -111,16 +110,15 @@ def test_rgms_staged_repeat_calls_accumulate(dev):
     y = torch.zeros(cfg["m"] * fout, dtype=torch.float32, device=dev)
     f(w, x, y, *triples, *mids)
     once = y.clone()
-    f(w, x, y, *triples, *mids)   # Y is accumulated into, as with the atomic path
+    f(w, x, y, *triples, *mids)   # Y is accumulated into, as with the atomic kernel; the index is reused
     torch.cuda.synchronize()
     assert once.abs().sum() > 0
     assert torch.allclose(y, 2 * once, rtol=1e-6, atol=1e-6)
     y2 = torch.zeros_like(y)
     f(w, x, y2, *triples, *mids)
     torch.cuda.synchronize()
-    # the staged sums are formed in a fixed order except for output rows that span several
-    # chunks of the reduce kernel, whose partial sums meet in atomics
-    assert torch.allclose(y2, once, rtol=1e-6, atol=1e-6)
+    # every tile is summed in a fixed order by one workgroup: repeatable bit for bit
+    assert torch.equal(y2, once)
 
 
 def test_rgms_bf16(dev):
@@ -173,7 +171,7 @@ def _csf_from_pairs(pairs, n):
     (32, 64, 64, [1, 4, 16], True),
 ])
 def test_rgms_tiled_hub_rows(dev, fin, fout, group, buckets, bf16):
-    """Destination-tiled path (64k slots and more): output rows not a multiple of 32, one row that
+    """Destination-tiled path: output rows not a multiple of 32, one row that
     receives thousands of edges in three relations (its tile is cut into several units that meet
     in atomics), relations without edges, widths that are not powers of two."""
     n, R = 5001, 7
@@ -190,7 +188,7 @@ def test_rgms_tiled_hub_rows(dev, fin, fout, group, buckets, bf16):
     csf = _csf_from_pairs(pairs, n)
     rows_bkt = [max(1, group // b) for b in buckets]
     ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
-    assert sum(mk.size for mk in mask) >= 65536
+    assert sum(mk.size for mk in mask) >= 8192
     tdt = torch.bfloat16 if bf16 else torch.float16
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     x = t(rng.standard_normal((n, fin), dtype=np.float32)).to(tdt)
