@@ -152,7 +152,7 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     out["rgms_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts / d / 1e9,
                            "frac_of_hbm_peak": byts / d / 1e9 / HBM_PEAK_GBS, "edges": E,
                            "ell_rows": int(sum(r.size for r in rows)),
-                           "accumulation": "staged per ELL row, summed per output row (no atomics)"}
+                           "accumulation": "32-row output tiles, written once (no atomics)"}
 
     # SpMM over the condensed format (t = 32, g = 16) on the config-2 graph, fp16 in, fp32 out
     g2 = datasets.config2()
