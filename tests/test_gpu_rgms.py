@@ -224,3 +224,91 @@ def test_rgms_tiled_hub_rows(dev, fin, fout, group, buckets, bf16):
     err = np.abs(got - want)
     assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), f"worst {err.max():.3e}"
     assert np.abs(want[77]).max() > 0
+
+
+def _tiled_case(dev, pairs, m, n, R, fin, fout, group, buckets, seed):
+    """Runs the fp16 operator on CSF built from (dst, src) pairs; returns (got, want, scale)."""
+    csf = _csf_from_pairs(pairs, n)
+    rows_bkt = [max(1, group // b) for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    rng = np.random.default_rng(seed)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    x = t(rng.standard_normal((n, fin), dtype=np.float32)).half()
+    w = t(rng.standard_normal((R, fin, fout), dtype=np.float32) * 0.1).half()
+    triples, mids = [], []
+    for b in range(len(buckets)):
+        triples += [t(mask[b].astype(np.float16).ravel()), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    f = ops.build_rgms(m, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols])
+    y = torch.zeros(m * fout, dtype=torch.float32, device=dev)
+    f(w.reshape(-1), x.reshape(-1), y, *triples, *mids)
+    torch.cuda.synchronize()
+    ones = np.ones(len(csf[3]), np.float32)
+    x32, w32 = x.float().cpu().numpy(), w.float().cpu().numpy()
+    want = rgms_f64(*csf, ones, x32, w32, m)
+    scale = rgms_f64(*csf, ones, np.abs(x32), np.abs(w32), m)
+    return y.cpu().numpy().reshape(m, fout), want, scale, (f, w, x, triples, mids, slots_of(mask))
+
+
+def slots_of(mask):
+    return sum(mk.size for mk in mask)
+
+
+def test_rgms_tiled_few_output_rows(dev):
+    """Five output rows, 12000 edges from 4000 sources: one tile of 32 rows cut into many units
+    that meet in atomics; m != n."""
+    m, n, R = 5, 4000, 3
+    rng = np.random.default_rng(5)
+    pairs = [(rng.integers(0, m, 6000), rng.integers(0, n, 6000)) for _ in range(R)]
+    got, want, scale, info = _tiled_case(dev, pairs, m, n, R, 32, 32, 32, [8, 32], 5)
+    assert info[-1] >= 8192
+    assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30)
+
+
+def test_rgms_tiled_sparse_rows_and_empty_tiles(dev):
+    """Edges end in two narrow bands of a large row range: most tiles have no edge and get no
+    unit; the rows in between stay untouched (checked with a non-zero Y)."""
+    m, n, R = 100_000, 3000, 4
+    rng = np.random.default_rng(6)
+    pairs = []
+    for r in range(R):
+        dst = np.concatenate([rng.integers(40, 140, 2500), rng.integers(99_900, m, 2500)])
+        pairs.append((dst, rng.integers(0, n, 5000)))
+    got, want, scale, info = _tiled_case(dev, pairs, m, n, R, 32, 32, 64, [1, 2, 4, 8, 16, 64], 6)
+    assert info[-1] >= 8192
+    assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30)
+    f, w, x, triples, mids, _ = info
+    y = torch.full((m * 32,), 3.0, dtype=torch.float32, device=dev)
+    f(w.reshape(-1), x.reshape(-1), y, *triples, *mids)
+    torch.cuda.synchronize()
+    y = y.cpu().numpy().reshape(m, 32)
+    assert np.all(y[200:99_000] == 3.0)
+    assert np.all(np.abs(y - 3.0 - want) <= 2e-2 * np.abs(want) + 1e-5 * (scale + 3.0) + 1e-30)
+
+
+def test_rgms_tiled_rejects_ids_out_of_range(dev):
+    """The index is built by the first launch: a row id >= m or a column id >= n fails it."""
+    m = n = 3000
+    rng = np.random.default_rng(7)
+    pairs = [(rng.integers(0, m, 6000), rng.integers(0, n, 6000)) for _ in range(2)]
+    csf = _csf_from_pairs(pairs, n)
+    buckets, rows_bkt = [1, 4, 16], [16, 4, 1]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    assert slots_of(mask) >= 8192
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    for what in ("row", "col"):
+        triples, mids = [], []
+        for b in range(len(buckets)):
+            r, c = rows[b].copy(), cols[b].copy()
+            if b == 1 and what == "row":
+                r.ravel()[3] = m
+            if b == 1 and what == "col":
+                c.ravel()[3] = n + 7
+            triples += [t(mask[b].astype(np.float16).ravel()), t(r.ravel()), t(c.ravel())]
+            mids.append(t(np.repeat(np.arange(2, dtype=np.int32), np.diff(ptr[b]))))
+        f = ops.build_rgms(m, n, 2, 32, 32, rows_bkt, buckets, [c.shape[0] for c in cols])
+        x = torch.zeros(n * 32, dtype=torch.float16, device=dev)
+        w = torch.zeros(2 * 32 * 32, dtype=torch.float16, device=dev)
+        y = torch.zeros(m * 32, dtype=torch.float32, device=dev)
+        with pytest.raises(Exception, match="outside"):
+            f(w, x, y, *triples, *mids)
