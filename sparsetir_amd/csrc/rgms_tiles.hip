@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
 #pragma unroll
       for (int q = 0; q < PW; ++q) {
         if (r[q] >= 0) {
-          const u32x4* w = Wp + ((int64_t)r[q] * ntiles + nti) * KK * 64 + lane;
+          const u32x4* w = Wp + (uint32_t)((r[q] * ntiles + nti) * (KK * 64) + lane);
 #pragma unroll
           for (int kk = 0; kk < KK; ++kk) wf[q][kk] = w[kk * 64];
         }
@@ -305,13 +305,19 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
           acc1 = mfma32<BF16>(a, w[kk], acc1);
         }
       };
+      if (pos >= kStepEdges && (PW == 1 || r[PW - 1] < 0) && r[0] >= 0 && (PW == 1 || r[1] < 0)) {
+        // one relation in the whole step: nothing to mask
 #pragma unroll
-      for (int q = 0; q < PW; ++q)
-        if (r[q] >= 0) add_run(r[q], wf[q]);
+        for (int kk = 0; kk < KK; ++kk) acc1 = mfma32<BF16>(xa[kk], wf[0][kk], acc1);
+      } else {
+#pragma unroll
+        for (int q = 0; q < PW; ++q)
+          if (r[q] >= 0) add_run(r[q], wf[q]);
+      }
       while (pos < kStepEdges) {  // steps with more than PW relations: one at a time
         const int rq = __builtin_amdgcn_readlane(rel, pos);
         pos += __popcll(__ballot(rel == rq) & 0xffffffffull);
-        const u32x4* w = Wp + ((int64_t)rq * ntiles + nti) * KK * 64 + lane;
+        const u32x4* w = Wp + (uint32_t)((rq * ntiles + nti) * (KK * 64) + lane);
         u32x4 wl[KK];
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) wl[kk] = w[kk * 64];
@@ -493,6 +499,7 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   STIR_REQUIRE(feat_in % 16 == 0 && feat_in / 16 <= kMaxKK && feat_out % 32 == 0, "rgms: unsupported feature sizes");
   const int kk_count = feat_in / 16;
   const int64_t frags = (int64_t)ix.num_rels * (feat_out / 32) * kk_count;
+  STIR_REQUIRE(frags < (int64_t(1) << 25), "rgms: W of %lld operand fragments exceeds the 32-bit fragment offsets", (long long)frags);
   const size_t need = size_t(frags) * 64 * sizeof(u32x4);
   if (need > ix.wpack_bytes) {
     if (ix.d_wpack) STIR_HIP(hipFree(ix.d_wpack));
