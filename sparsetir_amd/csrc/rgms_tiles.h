@@ -1,4 +1,5 @@
-// Destination-tiled RGMS for large ELL3D inputs: no atomics and no staging matrix.
+// Destination-tiled RGMS for ELL3D inputs that are not tiny: every 32-row tile of Y is summed in
+// registers and written once, without atomics.
 //
 // The slots of all buckets are re-indexed once per plan as "edges" (source row, relation,
 // destination row, address of the slot weight) sorted by (destination tile of 32 rows, relation,
