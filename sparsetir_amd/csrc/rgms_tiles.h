@@ -3,9 +3,10 @@
 //
 // The slots of all buckets are re-indexed once per plan as "edges" (source row, relation,
 // destination row, address of the slot weight) sorted by (destination tile of 32 rows, relation,
-// row inside the tile).  A wavefront owns a tile: it keeps the tile's 32 x 32 fp32 block of Y in
-// MFMA accumulators, walks the tile's edges 32 at a time and writes Y once at the end.  Tiles with
-// very many edges are cut into several units whose results are added with atomics.
+// row inside the tile).  A workgroup owns a tile: its four wavefronts walk the tile's edges 32 at
+// a time, each with a 32 x 32 fp32 block of partial sums in MFMA accumulators; the blocks are added
+// through LDS and the tile's rows of Y are written once.  Tiles with very many edges are cut into
+// several units whose results are added with atomics.
 #pragma once
 #include <cstdint>
 #include <vector>
