@@ -71,10 +71,12 @@ __device__ __forceinline__ bool decode_tile(int64_t L, int64_t slices, int f_til
 }
 
 // 1-D grid (see decode_tile); block: 256 threads = 4 wavefronts; wavefront w owns features
-// [32*NT*w, 32*NT*(w+1)) of the TF = 128*NT wide tile and NT 32x32 accumulators.  The X tile of
+// [32*NT*w, 32*NT*(w+1)) of the TF = 128*NT wide tile and RS*NT 32x32 accumulators.  The X tile of
 // step it+1 is fetched into registers while step it is multiplied out of LDS (two LDS buffers,
-// one barrier per step).
-template <bool BF16, int OUT, int NT, int S>  // OUT: 0 = same 16-bit type as the inputs, 1 = fp32
+// one barrier per step).  RS = 2 (blocks of 64 rows and more): a workgroup takes two adjacent
+// 32-row slices of a block row, so every X fragment read from LDS feeds two MFMAs and the X tile
+// is fetched once for 64 rows.
+template <bool BF16, int OUT, int NT, int S, int RS>  // OUT: 0 = same 16-bit type as the inputs, 1 = fp32
 __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles,
                                                        const uint16_t* __restrict__ A,
                                                        const uint16_t* __restrict__ X, void* __restrict__ Y,
@@ -91,17 +93,19 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
   int64_t slice;
   int f_tile;
   if (!decode_tile(blockIdx.x, slices, f_tiles, slice, f_tile)) return;
-  const int sub = blk / 32;  // 32-row slices per block row
-  const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * 32;
+  const int sub = blk / (32 * RS);  // slices of 32*RS rows per block row
+  const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * (32 * RS);
   const int f0 = f_tile * TF;
   const int kp0 = tid / FC, fc = tid % FC;
   const bool stage_live = f0 + fc * 8 < feat;  // feat is a multiple of 32, so chunks are whole
 
-  f32x16 acc[NT];
+  f32x16 acc[RS][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
+  for (int rs = 0; rs < RS; ++rs)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[rs][t][v] = 0.f;
 
   // doubly-compressed form: stored block row i is block row row_ids[i] of the output
   const int i_out = row_ids ? row_ids[i] : i;
@@ -111,13 +115,16 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
 
   // Register ring of S prefetched steps: loads for step it+S are issued as soon as step it has
   // been copied to LDS, so S tiles per wavefront are in flight while the matrix cores work.
-  u32x4 r0[S][NT], r1[S][NT], areg[S][2];
+  u32x4 r0[S][NT], r1[S][NT], areg[S][RS][2];
   auto fetch = [&](int it, int s) {
     const int p = p_begin + it / ksteps, k0 = (it % ksteps) * kTileK;
     const int64_t j = indices[p];
-    const uint16_t* ablk = A + (int64_t)p * blk * blk + (int64_t)(bi0 + n) * blk + k0;
-    areg[s][0] = *reinterpret_cast<const u32x4*>(ablk + 8 * h);       // k = k0 + 8h + (0..7)
-    areg[s][1] = *reinterpret_cast<const u32x4*>(ablk + 16 + 8 * h);  // k = k0 + 16 + 8h + (0..7)
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs) {
+      const uint16_t* ablk = A + (int64_t)p * blk * blk + (int64_t)(bi0 + 32 * rs + n) * blk + k0;
+      areg[s][rs][0] = *reinterpret_cast<const u32x4*>(ablk + 8 * h);       // k = k0 + 8h + (0..7)
+      areg[s][rs][1] = *reinterpret_cast<const u32x4*>(ablk + 16 + 8 * h);  // k = k0 + 16 + 8h + (0..7)
+    }
 #pragma unroll
     for (int q = 0; q < NT; ++q) {
       r0[s][q] = r1[s][q] = u32x4{0, 0, 0, 0};
@@ -138,7 +145,9 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
       const int it = it0 + s;
       if (it < steps) {  // uniform over the workgroup
         const int buf = it & 1;
-        const u32x4 a0 = areg[s][0], a1 = areg[s][1];
+        u32x4 a0[RS], a1[RS];
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs) a0[rs] = areg[s][rs][0], a1[rs] = areg[s][rs][1];
 #pragma unroll
         for (int q = 0; q < NT; ++q) {
           u32x4 lo, hi;  // (k, k+1) pairs for features fc*8 + 0..3 and 4..7
@@ -163,25 +172,31 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
             b0[d] = xs[buf][4 * h + d][col];
             b1[d] = xs[buf][8 + 4 * h + d][col];
           }
-          acc[t] = mfma32<BF16>(a0, b0, acc[t]);
-          acc[t] = mfma32<BF16>(a1, b1, acc[t]);
+#pragma unroll
+          for (int rs = 0; rs < RS; ++rs) {
+            acc[rs][t] = mfma32<BF16>(a0[rs], b0, acc[rs][t]);
+            acc[rs][t] = mfma32<BF16>(a1[rs], b1, acc[rs][t]);
+          }
         }
       }
     }
   }
-  // acc[t][v] is row (v%4) + 4h + 8(v/4), column n of the t-th 32x32 tile
+  // acc[rs][t][v] is row 32 rs + (v%4) + 4h + 8(v/4), column n of the t-th 32x32 tile
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int fcol = f0 + (wave * NT + t) * 32;
-    if (fcol >= feat) continue;
+  for (int rs = 0; rs < RS; ++rs) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = (v & 3) + 4 * h + 8 * (v >> 2);
-      const int64_t off = ((int64_t)i_out * blk + bi0 + row) * feat + fcol + n;
-      if constexpr (OUT == 1)
-        static_cast<float*>(Y)[off] = acc[t][v];
-      else
-        static_cast<uint16_t*>(Y)[off] = to16<BF16>(acc[t][v]);
+    for (int t = 0; t < NT; ++t) {
+      const int fcol = f0 + (wave * NT + t) * 32;
+      if (fcol >= feat) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = 32 * rs + (v & 3) + 4 * h + 8 * (v >> 2);
+        const int64_t off = ((int64_t)i_out * blk + bi0 + row) * feat + fcol + n;
+        if constexpr (OUT == 1)
+          static_cast<float*>(Y)[off] = acc[rs][t][v];
+        else
+          static_cast<uint16_t*>(Y)[off] = to16<BF16>(acc[rs][t][v]);
+      }
     }
   }
 }
@@ -198,7 +213,9 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   STIR_REQUIRE(feat > 0 && feat % 32 == 0, "bsr_spmm: feat=%d must be a multiple of 32", feat);
   if (mb == 0) return 0;
   STIR_REQUIRE(d_X && d_Y && d_indptr && (nnzb == 0 || (d_A && d_indices)), "bsr_spmm: null pointer argument");
-  const int64_t slices = (int64_t)mb * (blk / 32);
+  // two 32-row slices per workgroup when the block height allows it
+  const int rs = (blk % 64 == 0) ? 2 : 1;
+  const int64_t slices = (int64_t)mb * (blk / (32 * rs));
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
@@ -211,15 +228,16 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   const int64_t blocks = f_tiles >= 8 ? 8 * stir::ceil_div(f_tiles, 8) * slices : (int64_t)f_tiles * slices;
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "bsr_spmm: too many tiles for one launch");
   dim3 grid((unsigned)blocks), block(256);
-#define STIR_BSR_L(BF, OUT, NTV, SV)                                                                     \
-  hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, SV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
+#define STIR_BSR_L(BF, OUT, NTV, RSV)                                                                      \
+  hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, 1, RSV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
                      A, X, d_Y, d_indptr, d_indices, d_row_ids)
-#define STIR_BSR(BF, OUT)                  \
-  do {                                     \
-    if (nt == 2)                           \
-      STIR_BSR_L(BF, OUT, 2, 1);           \
-    else                                   \
-      STIR_BSR_L(BF, OUT, 1, 1);           \
+#define STIR_BSR(BF, OUT)                                                          \
+  do {                                                                             \
+    if (nt == 2) {                                                                 \
+      if (rs == 2) STIR_BSR_L(BF, OUT, 2, 2); else STIR_BSR_L(BF, OUT, 2, 1);      \
+    } else {                                                                       \
+      if (rs == 2) STIR_BSR_L(BF, OUT, 1, 2); else STIR_BSR_L(BF, OUT, 1, 1);      \
+    }                                                                              \
   } while (0)
   if (dtype == STIR_BF16) {
     if (out_dtype == STIR_F32) STIR_BSR(true, 1); else STIR_BSR(true, 0);

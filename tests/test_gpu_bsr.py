@@ -67,6 +67,18 @@ def test_bsr_block64_and_empty_rows(dev):
     assert np.all(got == 0)
 
 
+@pytest.mark.parametrize("blk,feat,dtype,out32", [
+    (64, 1056, torch.bfloat16, False),   # two slices per workgroup, two accumulators per wavefront
+    (128, 160, torch.float16, True),     # two slices per workgroup, four k steps per block
+    (96, 64, torch.float16, False),      # 96 rows: one slice per workgroup
+])
+def test_bsr_tall_blocks(dev, blk, feat, dtype, out32):
+    """Blocks of 64 rows and more: a workgroup takes two 32-row slices when blk is a multiple of 64."""
+    cfg = datasets.config4(seed=blk, mb=5, nb=6, blk=blk, density=0.35, feat=feat)
+    got, a32, x32 = _run(dev, cfg, dtype, torch.float32 if out32 else None)
+    _check(got, cfg, a32, x32, not out32, f"blk={blk} feat={feat} {dtype}")
+
+
 def test_bsr_rejects_unsupported(dev):
     z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
     f = ops.build_bsrmm(1, 1, 1, 16, 32)
