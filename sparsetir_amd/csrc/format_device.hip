@@ -35,6 +35,7 @@ struct Workspace {
   int32_t* kb;       // [P][m]   bucket of the run
   int32_t* hist;     // [P][NB][W] per-wavefront ELL-row counts, scanned in place
   int64_t* totals;   // [P][NB]
+  int64_t* tile_sums;  // [P][NB][ceil(W / kScanTile)] sums, then offsets, of the scan tiles of hist
   int32_t* widths;   // [NB]
   int32_t* coarse;   // [kCoarse] row that owns nonzero first + q * stride, stride = coarse_stride(nnz)
   int32_t* status;   // [1 + 2 * kCountSlots] status bits; descents between neighbours; descents at row starts
@@ -76,6 +77,7 @@ Workspace carve(void* p, int32_t m, int32_t P, int32_t NB) {
   w.kb = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(m > 0 ? m : 1)));
   w.hist = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(P) * size_t(W > 0 ? W : 1) * NB));
   w.totals = reinterpret_cast<int64_t*>(take(sizeof(int64_t) * size_t(P) * NB));
+  w.tile_sums = reinterpret_cast<int64_t*>(take(sizeof(int64_t) * size_t(P) * NB * size_t(W / 4096 + 1)));
   w.widths = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * NB));
   w.coarse = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kCoarse));
   w.status = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * kStatusInts));
@@ -199,47 +201,105 @@ __global__ __launch_bounds__(256) void count_kernel(int m, int psize, int NB, in
   if (lane == 0) h[(NB - 1) * W] = tot;
 }
 
-// (2) exclusive scan of hist[p][b][.] along the wavefront axis.  grid (NB, P), 1024 threads, each
-// owning one contiguous chunk.
-constexpr int kScanThreads = 1024;
-__global__ __launch_bounds__(kScanThreads) void scan_kernel(int NB, int64_t W, int32_t* __restrict__ hist,
-                                                            int64_t* __restrict__ totals) {
-  __shared__ int64_t part[kScanThreads];
-  const int b = blockIdx.x, p = blockIdx.y;
-  int32_t* h = hist + ((int64_t)p * NB + b) * W;
-  const int64_t chunk = (W + kScanThreads - 1) / kScanThreads;
-  const int64_t w0 = min(W, chunk * threadIdx.x), w1 = min(W, w0 + chunk);
-  int64_t sum = 0;
-  for (int64_t w = w0; w < w1; ++w) sum += h[w];
-  part[threadIdx.x] = sum;
+// (2) exclusive scan of hist[p][b][.] along the wavefront axis, in three launches: sums of tiles
+// of kScanTile entries, an exclusive scan of the tile sums of every (p, b) row by one workgroup,
+// and the scan inside every tile started from its offset.
+constexpr int kScanTile = 4096;  // 256 threads x 16 consecutive entries
+constexpr int kScanPer = kScanTile / 256;
+
+__device__ __forceinline__ int64_t block_sum_256(int64_t v, int64_t* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  if (lane == 0) red[wave] = v;
   __syncthreads();
-  // exclusive scan of the 1024 chunk sums by the first wavefront, 16 per lane
-  if (threadIdx.x < kWave) {
-    constexpr int PER = kScanThreads / kWave;
-    int64_t loc[PER];
-    int64_t tot = 0;
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+// grid (tiles, P * NB)
+__global__ __launch_bounds__(256) void scan_tile_sums_kernel(int64_t W, int64_t tiles,
+                                                             const int32_t* __restrict__ hist,
+                                                             int64_t* __restrict__ tile_sums) {
+  __shared__ int64_t red[4];
+  const int32_t* h = hist + (int64_t)blockIdx.y * W;
+  const int64_t w0 = (int64_t)blockIdx.x * kScanTile;
+  int64_t sum = 0;
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      loc[j] = tot;
-      tot += part[threadIdx.x * PER + j];
+  for (int k = 0; k < kScanPer; ++k) {
+    const int64_t w = w0 + threadIdx.x + 256 * k;
+    if (w < W) sum += h[w];
+  }
+  sum = block_sum_256(sum, red);
+  if (threadIdx.x == 0) tile_sums[(int64_t)blockIdx.y * tiles + blockIdx.x] = sum;
+}
+
+// grid (P * NB), 256 threads: tile sums -> exclusive offsets, row total
+__global__ __launch_bounds__(256) void scan_tile_offsets_kernel(int64_t tiles, int64_t* __restrict__ tile_sums,
+                                                                int64_t* __restrict__ totals) {
+  __shared__ int64_t part[256];
+  int64_t* ts = tile_sums + (int64_t)blockIdx.x * tiles;
+  int64_t carry = 0;
+  for (int64_t t0 = 0; t0 < tiles; t0 += 256) {
+    const int64_t t = t0 + threadIdx.x;
+    const int64_t v = t < tiles ? ts[t] : 0;
+    part[threadIdx.x] = v;
+    __syncthreads();
+    // Hillis-Steele inclusive scan of 256 values
+    for (int off = 1; off < 256; off <<= 1) {
+      const int64_t up = (int)threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+      __syncthreads();
+      part[threadIdx.x] += up;
+      __syncthreads();
     }
-    int64_t incl = tot;
+    if (t < tiles) ts[t] = carry + part[threadIdx.x] - v;
+    carry += part[255];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) totals[blockIdx.x] = carry;
+}
+
+// grid (tiles, P * NB): exclusive scan inside the tile; a thread owns kScanPer consecutive entries,
+// moved through LDS so that global accesses stay coalesced
+__global__ __launch_bounds__(256) void scan_apply_kernel(int64_t W, int64_t tiles, int32_t* __restrict__ hist,
+                                                         const int64_t* __restrict__ tile_sums) {
+  __shared__ int32_t tile[256][kScanPer + 1];
+  __shared__ int64_t part[256];
+  int32_t* h = hist + (int64_t)blockIdx.y * W;
+  const int64_t w0 = (int64_t)blockIdx.x * kScanTile;
 #pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const int64_t up = __shfl_up(incl, off, kWave);
-      if ((int)threadIdx.x >= off) incl += up;
-    }
-    const int64_t excl = incl - tot;
-#pragma unroll
-    for (int j = 0; j < PER; ++j) part[threadIdx.x * PER + j] = excl + loc[j];
-    if (threadIdx.x == kWave - 1) totals[(int64_t)p * NB + b] = incl;
+  for (int k = 0; k < kScanPer; ++k) {
+    const int e = threadIdx.x + 256 * k;
+    const int64_t w = w0 + e;
+    tile[e / kScanPer][e % kScanPer] = w < W ? h[w] : 0;
   }
   __syncthreads();
-  int64_t run = part[threadIdx.x];
-  for (int64_t w = w0; w < w1; ++w) {
-    const int32_t v = h[w];
-    h[w] = (int32_t)run;
-    run += v;
+  int32_t v[kScanPer];
+  int64_t sum = 0;
+#pragma unroll
+  for (int k = 0; k < kScanPer; ++k) {
+    v[k] = tile[threadIdx.x][k];
+    sum += v[k];
+  }
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  for (int off = 1; off < 256; off <<= 1) {
+    const int64_t up = (int)threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+    __syncthreads();
+    part[threadIdx.x] += up;
+    __syncthreads();
+  }
+  int64_t run = tile_sums[(int64_t)blockIdx.y * tiles + blockIdx.x] + part[threadIdx.x] - sum;
+#pragma unroll
+  for (int k = 0; k < kScanPer; ++k) {
+    tile[threadIdx.x][k] = (int32_t)run;
+    run += v[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kScanPer; ++k) {
+    const int e = threadIdx.x + 256 * k;
+    const int64_t w = w0 + e;
+    if (w < W) h[w] = tile[e / kScanPer][e % kScanPer];
   }
 }
 
@@ -778,6 +838,22 @@ int check_args(const char* who, int32_t num_rows, int32_t num_cols, int32_t part
   return 0;
 }
 
+// Scans hist in place (exclusive, per (partition, bucket) row) and leaves the row totals in
+// ws.totals.
+int scan_hist(const Workspace& ws, int P, int NB, int64_t W, hipStream_t st) {
+  const int64_t tiles = stir::ceil_div(W, kScanTile);
+  STIR_REQUIRE(tiles < (int64_t(1) << 31), "ColumnPartHyb(device): too many rows for the scan");
+  const dim3 grid((unsigned)tiles, (unsigned)(P * NB));
+  hipLaunchKernelGGL(scan_tile_sums_kernel, grid, dim3(256), 0, st, W, tiles, ws.hist, ws.tile_sums);
+  STIR_LAUNCH_CHECK();
+  hipLaunchKernelGGL(scan_tile_offsets_kernel, dim3((unsigned)(P * NB)), dim3(256), 0, st, tiles, ws.tile_sums,
+                     ws.totals);
+  STIR_LAUNCH_CHECK();
+  hipLaunchKernelGGL(scan_apply_kernel, grid, dim3(256), 0, st, W, tiles, ws.hist, ws.tile_sums);
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -822,9 +898,7 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
                      coarse_stride(nnz), ws.coarse, d_indptr,
                      d_indices, ws.widths, ws.lo, ws.hist, ws.status);
   STIR_LAUNCH_CHECK();
-  hipLaunchKernelGGL(scan_kernel, dim3((unsigned)NB, (unsigned)P), dim3(kScanThreads), 0, st, NB, W, ws.hist,
-                     ws.totals);
-  STIR_LAUNCH_CHECK();
+  if (scan_hist(ws, P, NB, W, st)) return -1;
   std::vector<int32_t> counts(kStatusInts, 0);
   STIR_HIP(hipMemcpyAsync(counts.data(), ws.status, sizeof(int32_t) * kStatusInts, hipMemcpyDeviceToHost, st));
   STIR_HIP(hipMemcpyAsync(nrows, ws.totals, sizeof(int64_t) * size_t(P) * NB, hipMemcpyDeviceToHost, st));
@@ -849,9 +923,7 @@ int stir_column_part_hyb_device_sizes(int32_t num_rows, int32_t num_cols, const 
                        coarse_stride(nnz), ws.coarse, d_indptr, tail.idx2 - ends[0], ws.widths, ws.lo, ws.hist,
                        ws.status);
     STIR_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_kernel, dim3((unsigned)NB, (unsigned)P), dim3(kScanThreads), 0, st, NB, W, ws.hist,
-                       ws.totals);
-    STIR_LAUNCH_CHECK();
+    if (scan_hist(ws, P, NB, W, st)) return -1;
     STIR_HIP(hipMemcpyAsync(nrows, ws.totals, sizeof(int64_t) * size_t(P) * NB, hipMemcpyDeviceToHost, st));
     STIR_HIP(hipStreamSynchronize(st));
   }
