@@ -426,10 +426,15 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   int dev = 0, cus = 256;
   STIR_HIP(hipGetDevice(&dev));
   STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  // units (one workgroup each) of about total steps / (8 per CU), at least 16 steps: tiles are
-  // cut only when the launch would otherwise leave most of the chip idle
+  // Units (one workgroup each) of at most `cap` steps.  A tile is cut only when it is long against
+  // the others -- more than about three average tiles -- or when the launch would otherwise
+  // leave most of the chip idle (few tiles): the longest unit is the critical path of the launch.
+  // CSFToELL3D pads every relation's rows by repeating its last row id, so the tiles that hold
+  // those rows carry thousands of zero-weight slots and are always cut.
   const int64_t steps_bound = slots / kStepEdges + tiles;
-  const int cap = (int)std::max<int64_t>(16, kUnitWaves * ceil_div(steps_bound, (int64_t)cus * 8));
+  const int64_t by_chip = kUnitWaves * ceil_div(steps_bound, (int64_t)cus * 8);
+  const int64_t by_tile = 2 * ceil_div(steps_bound, tiles);
+  const int cap = (int)std::max<int64_t>(16, std::min(by_chip, by_tile));
 
   size_t sort_bytes = 0, scan_bytes = 0;
   STIR_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, (const uint64_t*)nullptr, (uint64_t*)nullptr,

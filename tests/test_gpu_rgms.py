@@ -117,8 +117,10 @@ def test_rgms_tiled_repeat_calls_accumulate(dev):
     y2 = torch.zeros_like(y)
     f(w, x, y2, *triples, *mids)
     torch.cuda.synchronize()
-    # every tile is summed in a fixed order by one workgroup: repeatable bit for bit
-    assert torch.equal(y2, once)
+    # a tile is summed in a fixed order by one workgroup; only the few tiles cut into several
+    # units (those holding the repeated row ids of the ELL3D padding) meet in atomics
+    assert torch.allclose(y2, once, rtol=1e-6, atol=1e-6)
+    assert float((y2 != once).float().mean()) < 0.01
 
 
 def test_rgms_bf16(dev):
