@@ -305,7 +305,9 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
           acc1 = mfma32<BF16>(a, w[kk], acc1);
         }
       };
-      if (pos >= kStepEdges && (PW == 1 || r[PW - 1] < 0) && r[0] >= 0 && (PW == 1 || r[1] < 0)) {
+      bool single = pos >= kStepEdges;  // the requested runs cover the step ...
+      if constexpr (PW > 1) single = single && r[1] < 0;  // ... and the first one does so alone
+      if (single) {
         // one relation in the whole step: nothing to mask
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) acc1 = mfma32<BF16>(xa[kk], wf[0][kk], acc1);
