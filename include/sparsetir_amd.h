@@ -217,7 +217,9 @@ int stir_dbsr_spmm(int32_t dtype, int32_t out_dtype, int32_t nnz_rows, int32_t n
  * (operator :538-565).  A: nnzb*t*g (the 0/1 mask of ConDense as fp16, or edge weights),
  * B: dense features, at least max(indices)+1 rows of feat, C: mb*t*feat of out_dtype (STIR_F16
  * as in the reference, or STIR_F32), indptr: group_indptr (mb+1), indices: tile_indices
- * (nnzb*g).  The MFMA path needs tile_size t = 32 and group_size g = 16.
+ * (nnzb*g).  The MFMA path needs tile_size t = 32 and group_size g = 16.  C is written, not
+ * accumulated into; with fp32 output this takes two launches (row tiles with very many groups
+ * are cleared, then summed by several workgroups).
  */
 int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t group_size,
                      int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,

@@ -9,6 +9,12 @@
 // already in MFMA A-operand order (a lane's 8 k values are contiguous), the 32 gathered rows of
 // B go through LDS, interleaved into (k, k+1) pairs on the way, double-buffered, with the next
 // step's gathers in flight during the multiply.
+//
+// A row tile that touches thousands of distinct columns (a hub row of a power-law graph) would be
+// one long serial chain in one workgroup.  With fp32 output such tiles are cut into up to kSplit
+// units of at least kUnitSteps steps that add their results with atomics; a first launch clears the rows
+// of those tiles.  (fp16 output keeps one workgroup per tile: partial sums would be rounded to
+// fp16 once per unit.)
 #include "common.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -21,8 +27,31 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kTileF = 128;
 constexpr int kTile = 32;   // t
 constexpr int kGroup = 16;  // g
+constexpr int kUnitSteps = 16;  // steps (of two groups) per unit of a long tile
+constexpr int kSplit = 16;      // most units per tile (second grid dimension of the split launch)
 
-template <int OUT>  // 0: fp16 output, 1: fp32 output
+__device__ __forceinline__ int tile_steps(const int32_t* __restrict__ indptr, int64_t io) {
+  const int64_t rows_total = (int64_t)(indptr[io + 1] - indptr[io]) * kGroup;
+  return (int)((rows_total + 31) / 32);
+}
+
+// Clears the fp32 rows of the tiles that the split launch accumulates into.  grid (mb * f_tiles)
+__global__ __launch_bounds__(256) void tcspmm_clear_long_kernel(int feat, int64_t mb, int f_tiles,
+                                                                float* __restrict__ C,
+                                                                const int32_t* __restrict__ indptr) {
+  const int f_tile = (int)(blockIdx.x % f_tiles);
+  const int64_t io = blockIdx.x / f_tiles;
+  if (io >= mb || tile_steps(indptr, io) <= kUnitSteps) return;
+  const int f0 = f_tile * kTileF;
+  for (int e = threadIdx.x; e < kTile * kTileF; e += 256) {
+    const int row = e / kTileF, f = f0 + e % kTileF;
+    if (f < feat) C[(io * kTile + row) * feat + f] = 0.f;
+  }
+}
+
+// OUT: 0 = fp16 output, 1 = fp32 output.  SPLIT: grid is (mb * f_tiles, kSplit); the units of a
+// long tile take equal shares of its steps and add with atomics, unit 0 of a short tile stores.
+template <int OUT, bool SPLIT>
 __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f_tiles,
                                                      const uint16_t* __restrict__ A,
                                                      const uint16_t* __restrict__ B, void* __restrict__ C,
@@ -47,6 +76,20 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   const int64_t rows_total = (g_end - g_begin) * kGroup;  // gathered rows of B for this tile
   const int steps = (int)((rows_total + 31) / 32);
   const int32_t* rowlist = indices + g_begin * kGroup;
+  int it_begin = 0, it_end = steps;
+  bool add = false;
+  if constexpr (SPLIT) {
+    const int u = blockIdx.y;
+    if (steps > kUnitSteps) {
+      add = true;
+      const int len = max(kUnitSteps, (steps + kSplit - 1) / kSplit);  // even shares beyond kSplit units
+      it_begin = u * len;
+      it_end = min(steps, it_begin + len);
+      if (it_begin >= it_end) return;  // uniform over the workgroup
+    } else if (u > 0) {
+      return;
+    }
+  }
 
   u32x4 r0, r1, a_next[2];
   auto fetch = [&](int it) {
@@ -65,8 +108,8 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
     }
   };
 
-  if (steps > 0) fetch(0);
-  for (int it = 0; it < steps; ++it) {
+  if (it_begin < it_end) fetch(it_begin);
+  for (int it = it_begin; it < it_end; ++it) {
     const int buf = it & 1;
     const u32x4 a0 = a_next[0], a1 = a_next[1];
     u32x4 lo, hi;
@@ -79,7 +122,7 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
     }
     *reinterpret_cast<u32x4*>(&xs[buf][kp][fc * 8]) = lo;
     *reinterpret_cast<u32x4*>(&xs[buf][kp][fc * 8 + 4]) = hi;
-    if (it + 1 < steps) fetch(it + 1);
+    if (it + 1 < it_end) fetch(it + 1);
     __syncthreads();
     const int col = wave * 32 + n;
     u32x4 b0, b1;
@@ -100,7 +143,10 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
     const int row = (v & 3) + 4 * h + 8 * (v >> 2);
     const int64_t off = (io * kTile + row) * feat + fcol + n;
     if constexpr (OUT == 1) {
-      static_cast<float*>(C)[off] = acc[v];
+      if (add)
+        __hip_atomic_fetch_add(static_cast<float*>(C) + off, acc[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else
+        static_cast<float*>(C)[off] = acc[v];
     } else {
       const _Float16 hv = (_Float16)acc[v];
       static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
@@ -126,12 +172,16 @@ extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* B = static_cast<const uint16_t*>(d_B);
-  if (out_dtype == STIR_F32)
-    hipLaunchKernelGGL(tcspmm_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb, f_tiles, A,
-                       B, d_C, d_indptr, d_indices);
-  else
-    hipLaunchKernelGGL(tcspmm_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb, f_tiles, A,
-                       B, d_C, d_indptr, d_indices);
+  if (out_dtype == STIR_F32) {
+    hipLaunchKernelGGL(tcspmm_clear_long_kernel, dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
+                       f_tiles, static_cast<float*>(d_C), d_indptr);
+    STIR_LAUNCH_CHECK();
+    hipLaunchKernelGGL((tcspmm_kernel<1, true>), dim3((unsigned)blocks, kSplit), dim3(256), 0, st, feat,
+                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
+  } else {
+    hipLaunchKernelGGL((tcspmm_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
+                       f_tiles, A, B, d_C, d_indptr, d_indices);
+  }
   STIR_LAUNCH_CHECK();
   return 0;
 }

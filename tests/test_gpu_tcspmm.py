@@ -70,3 +70,19 @@ def test_tcspmm_empty_tiles_and_errors(dev):
     f = ops.build_tcspmm(1, 1, 32, 16, 16, 4)
     with pytest.raises(SparseTIRError, match="t=32"):
         f(z(256, torch.float16), z(128, torch.float16), z(512, torch.float16), z(2, torch.int32), z(16, torch.int32))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_tcspmm_hub_tile(dev, out_dtype):
+    """One row with 9000 distinct columns: its tile has 563 groups = 282 steps, which the fp32
+    path cuts into equal units that meet in atomics; C starts as NaN, so the rows of that tile
+    must be cleared first.  Another tile lies just above the length of one unit.  Two feature
+    tiles, the second one partial."""
+    m, n, feat = 200, 20000, 160
+    rng = np.random.default_rng(3)
+    deg = rng.integers(0, 12, m)
+    deg[77] = 9000
+    deg[150] = 530   # 34 groups = 17 steps: just above one unit
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    indices = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
+    _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=9)
