@@ -201,6 +201,131 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
   }
 }
 
+
+// Small launches (at most a couple of workgroups per CU): a workgroup's run time is the serial
+// chain of its block row's steps, each a memory round trip, and nothing else is resident to hide
+// it.  Here the four wavefronts of a workgroup split the steps of the block row instead of the
+// feature axis: wavefront w takes steps w, w + 4, ... for all 128 features (four accumulators),
+// stages its own X tile in its own piece of LDS (no workgroup barrier in the loop: the LDS
+// operations of one wavefront execute in order) and the four partial results are added through
+// LDS at the end.  Same tile and the same global traffic as bsr_spmm_kernel, a chain four times
+// shorter.
+constexpr int kSplitLdsWords = 4 * 4 * 16 * 64;  // reduction: [wavefront][feature tile][register][lane]
+
+template <bool BF16, int OUT>
+__global__ __launch_bounds__(256) void bsr_spmm_ksplit_kernel(int blk, int feat, int64_t slices, int f_tiles,
+                                                              const uint16_t* __restrict__ A,
+                                                              const uint16_t* __restrict__ X, void* __restrict__ Y,
+                                                              const int32_t* __restrict__ indptr,
+                                                              const int32_t* __restrict__ indices,
+                                                              const int32_t* __restrict__ row_ids) {
+  __shared__ __attribute__((aligned(16))) uint32_t lds[kSplitLdsWords];  // 64 KB
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int f_tile = (int)(blockIdx.x % f_tiles);
+  const int64_t slice = blockIdx.x / f_tiles;
+  const int sub = blk / 32;
+  const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * 32;
+  const int f0 = f_tile * kTileF;
+  // staging role of a lane: k pairs kp, kp + 4, kp + 8, kp + 12; 8-feature chunk fc
+  const int kp = lane >> 4, fc = lane & 15;
+  const bool stage_live = f0 + fc * 8 < feat;
+  uint32_t(*xs)[kTileF] = reinterpret_cast<uint32_t(*)[kTileF]>(lds + wave * (16 * kTileF));  // [k pair][feature]
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  const int i_out = row_ids ? row_ids[i] : i;
+  const int p_begin = indptr[i];
+  const int ksteps = blk / kTileK;
+  const int steps = (indptr[i + 1] - p_begin) * ksteps;
+
+  // The block columns of the row's first 64 blocks are fetched once, one per lane: looking them up
+  // step by step would put a second memory round trip in front of every step's loads of X.
+  const int nblk = indptr[i + 1] - p_begin;
+  const int j_lane = lane < nblk ? indices[p_begin + lane] : 0;
+  u32x4 r0[4], r1[4], areg[2];
+  auto fetch = [&](int it) {
+    const int b = it / ksteps, k0 = (it % ksteps) * kTileK;
+    const int p = p_begin + b;
+    const int64_t j = b < kWave ? __shfl(j_lane, b, kWave) : indices[p];
+    const uint16_t* ablk = A + (int64_t)p * blk * blk + (int64_t)(bi0 + n) * blk + k0;
+    areg[0] = *reinterpret_cast<const u32x4*>(ablk + 8 * h);
+    areg[1] = *reinterpret_cast<const u32x4*>(ablk + 16 + 8 * h);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      r0[q] = r1[q] = u32x4{0, 0, 0, 0};
+      if (stage_live) {
+        const uint16_t* xp = X + ((int64_t)j * blk + k0 + 2 * (kp + 4 * q)) * feat + f0 + fc * 8;
+        r0[q] = *reinterpret_cast<const u32x4*>(xp);
+        r1[q] = *reinterpret_cast<const u32x4*>(xp + feat);
+      }
+    }
+  };
+
+  if (wave < steps) fetch(wave);
+  for (int it = wave; it < steps; it += 4) {
+    const u32x4 a0 = areg[0], a1 = areg[1];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      u32x4 lo, hi;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        lo[2 * d] = __builtin_amdgcn_perm(r1[q][d], r0[q][d], 0x05040100);
+        lo[2 * d + 1] = __builtin_amdgcn_perm(r1[q][d], r0[q][d], 0x07060302);
+        hi[2 * d] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x05040100);
+        hi[2 * d + 1] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x07060302);
+      }
+      *reinterpret_cast<u32x4*>(&xs[kp + 4 * q][fc * 8]) = lo;
+      *reinterpret_cast<u32x4*>(&xs[kp + 4 * q][fc * 8 + 4]) = hi;
+    }
+    if (it + 4 < steps) fetch(it + 4);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int col = t * 32 + n;
+      u32x4 b0, b1;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        b0[d] = xs[4 * h + d][col];
+        b1[d] = xs[8 + 4 * h + d][col];
+      }
+      acc[t] = mfma32<BF16>(a0, b0, acc[t]);
+      acc[t] = mfma32<BF16>(a1, b1, acc[t]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // the next step's stores come after these reads
+  }
+
+  // ---- add the four partial results: wavefront w ends up with feature tile w
+  __syncthreads();  // every wavefront is done with its staging piece
+  float* red = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[((wave * 4 + t) * 16 + v) * 64 + lane] = acc[t][v];
+  __syncthreads();
+  const int fcol = f0 + wave * 32;
+  if (fcol >= feat) return;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sum += red[((w * 4 + wave) * 16 + v) * 64 + lane];
+    const int row = (v & 3) + 4 * h + 8 * (v >> 2);
+    const int64_t off = ((int64_t)i_out * blk + bi0 + row) * feat + fcol + n;
+    if constexpr (OUT == 1)
+      static_cast<float*>(Y)[off] = sum;
+    else
+      static_cast<uint16_t*>(Y)[off] = to16<BF16>(sum);
+  }
+}
+
 }  // namespace
 
 static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk, int32_t feat,
@@ -219,6 +344,30 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
+  // A launch of at most two workgroups per CU is bound by the chain of steps of its longest block
+  // row: the four wavefronts of a workgroup then split the steps instead of the features.
+  {
+    const int f_tiles_s = (int)stir::ceil_div(feat, kTileF);
+    const int64_t blocks_s = (int64_t)mb * (blk / 32) * f_tiles_s;
+    int dev = 0, cus = 256;
+    STIR_HIP(hipGetDevice(&dev));
+    STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (blocks_s <= 2 * (int64_t)cus) {
+      const int64_t slices_s = (int64_t)mb * (blk / 32);
+      dim3 grid_s((unsigned)blocks_s), block_s(256);
+#define STIR_BSR_S(BF, OUT)                                                                                  \
+  hipLaunchKernelGGL((bsr_spmm_ksplit_kernel<BF, OUT>), grid_s, block_s, 0, st, blk, feat, slices_s, f_tiles_s, \
+                     A, X, d_Y, d_indptr, d_indices, d_row_ids)
+      if (dtype == STIR_BF16) {
+        if (out_dtype == STIR_F32) STIR_BSR_S(true, 1); else STIR_BSR_S(true, 0);
+      } else {
+        if (out_dtype == STIR_F32) STIR_BSR_S(false, 1); else STIR_BSR_S(false, 0);
+      }
+#undef STIR_BSR_S
+      STIR_LAUNCH_CHECK();
+      return 0;
+    }
+  }
   // Two 32-wide accumulators per wavefront once the feature axis is wide enough to still yield
   // several workgroups per CU.  One prefetched step is enough: measured on MI355X, deeper
   // register rings (2-6 steps) change nothing, the kernel is bound by the traffic that misses

@@ -79,6 +79,20 @@ def test_bsr_tall_blocks(dev, blk, feat, dtype, out32):
     _check(got, cfg, a32, x32, not out32, f"blk={blk} feat={feat} {dtype}")
 
 
+@pytest.mark.parametrize("mb,nb,blk,feat,dtype", [
+    (160, 12, 32, 512, torch.float16),    # one accumulator per wavefront
+    (48, 20, 32, 1536, torch.bfloat16),   # two accumulators per wavefront
+    (24, 10, 64, 1536, torch.float16),    # two slices per workgroup as well
+])
+def test_bsr_many_workgroups(dev, mb, nb, blk, feat, dtype):
+    """More than two workgroups per CU: the kernel whose wavefronts split the feature axis (small
+    launches take the one whose wavefronts split the steps of a block row)."""
+    cfg = datasets.config4(seed=mb, mb=mb, nb=nb, blk=blk, density=0.3, feat=feat)
+    assert mb * (blk // 32) * ((feat + 127) // 128) > 512
+    got, a32, x32 = _run(dev, cfg, dtype)
+    _check(got, cfg, a32, x32, True, f"mb={mb} blk={blk} feat={feat} {dtype}")
+
+
 def test_bsr_rejects_unsupported(dev):
     z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
     f = ops.build_bsrmm(1, 1, 1, 16, 32)
