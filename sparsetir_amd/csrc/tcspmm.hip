@@ -91,6 +91,14 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
     }
   }
 
+  // The row ids of a step are requested one step before its rows of B, so that a step costs one
+  // memory round trip, not two in a row.
+  int row_a = 0, row_b = 0;
+  auto fetch_ids = [&](int it) {
+    const int64_t k = (int64_t)it * 32 + 2 * kp;
+    row_a = row_b = 0;
+    if (k < rows_total) row_a = rowlist[k], row_b = rowlist[k + 1];  // the same group: both exist
+  };
   u32x4 r0, r1, a_next[2];
   auto fetch = [&](int it) {
     // A[jo][n][8h .. 8h+7] for the step's two groups (zero when the tile has an odd group count)
@@ -101,14 +109,16 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
     r0 = r1 = u32x4{0, 0, 0, 0};
     const int64_t k = (int64_t)it * 32 + 2 * kp;
     if (stage_live && k < rows_total) {
-      // k and k+1 belong to the same group (groups hold 16 rows), so both exist
-      const int64_t row_a = rowlist[k], row_b = rowlist[k + 1];
-      r0 = *reinterpret_cast<const u32x4*>(B + row_a * feat + f0 + fc * 8);
-      r1 = *reinterpret_cast<const u32x4*>(B + row_b * feat + f0 + fc * 8);
+      r0 = *reinterpret_cast<const u32x4*>(B + (int64_t)row_a * feat + f0 + fc * 8);
+      r1 = *reinterpret_cast<const u32x4*>(B + (int64_t)row_b * feat + f0 + fc * 8);
     }
+    if (it + 1 < it_end) fetch_ids(it + 1);
   };
 
-  if (it_begin < it_end) fetch(it_begin);
+  if (it_begin < it_end) {
+    fetch_ids(it_begin);
+    fetch(it_begin);
+  }
   for (int it = it_begin; it < it_end; ++it) {
     const int buf = it & 1;
     const u32x4 a0 = a_next[0], a1 = a_next[1];
