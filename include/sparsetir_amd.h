@@ -158,9 +158,10 @@ int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const flo
  * part*num_buckets + bucket has width bucket_widths[bucket], nrows[k] ELL rows and the
  * device arrays d_A[k] (nrows*width f32), d_rows[k] (nrows), d_cols[k] (nrows*width), the
  * (A_k, rows_k, cols_k) triples of the reference's argument list (bench_spmm.py:208-222).
- * A bucket is accumulated with atomics when num_col_parts > 1 or it is the last bucket of
- * its partition, and stored otherwise (bench_spmm.py:170).  The plan keeps the pointers,
- * not copies: the arrays must outlive it.
+ * A bucket is added to C when num_col_parts > 1 or it is the last bucket of its partition,
+ * and stored otherwise (bench_spmm.py:170).  Adding is done with atomics, except that with 2 to
+ * 4 partitions the partitions run one after the other on the stream and only the last bucket of
+ * each needs atomics.  The plan keeps the pointers, not copies: the arrays must outlive it.
  */
 typedef struct stir_hyb_plan stir_hyb_plan;
 int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,

@@ -25,7 +25,7 @@ struct alignas(16) HybBucket {
   int64_t tile_begin;  // first wave tile of this bucket in the fused launch
   int32_t width;
   int32_t log2w;   // log2(width) when the bucket runs in slot-tile mode, else -1
-  int32_t atomic;  // accumulate with atomics instead of storing
+  int32_t atomic;  // 0: store the row, 1: add it with atomics, 2: add it with a plain read-modify-write
   int32_t chunks;  // row mode: wave tiles per ELL row (each covers kRowChunk slots)
 };
 
@@ -68,8 +68,20 @@ __device__ __forceinline__ void reduce_groups(float4 (&acc)[REP], int limit) {
 // no workgroup barrier is involved.
 template <int G, int REP>
 __device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int lane,
-                                          const float4 (&acc)[REP], bool atomic, float* stage) {
+                                          const float4 (&acc)[REP], int atomic, float* stage) {
   const int g = lane / G, gl = lane % G;
+  if (atomic == 2) {
+    // the only writer of this row in this launch: no atomics needed to add
+    float* base = C + row * feat + gl * 4;
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+      if (gl * 4 + r * G * 4 >= feat) continue;
+      float* q = base + r * G * 4;
+      const float o0 = q[0], o1 = q[1], o2 = q[2], o3 = q[3];
+      q[0] = o0 + acc[r].x, q[1] = o1 + acc[r].y, q[2] = o2 + acc[r].z, q[3] = o3 + acc[r].w;
+    }
+    return;
+  }
   if (!atomic) {
     float* base = C + row * feat + gl * 4;
 #pragma unroll
@@ -159,7 +171,7 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, int spli
   for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
   if (!(split_long && end - start > kLongRow)) csr_accumulate<G, REP>(acc, start, end, feat, A, B, indices, lane);
   reduce_groups<G, REP>(acc, kWave);
-  if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, false, nullptr);
+  if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, 0, nullptr);
 }
 
 // One wavefront per kLongPiece consecutive nonzeros: the parts of rows longer than kLongRow that
@@ -240,7 +252,7 @@ __device__ __forceinline__ void hyb_slot_tile(const HybBucket& bk, int64_t t, in
   const int64_t row0 = slot0 >> LOG2W;
   int my_row = -1;
   if (lane < ROWS && row0 + lane < bk.nrows) my_row = bk.rows[row0 + lane];
-  const bool atomic = bk.atomic != 0;
+  const int atomic = bk.atomic;
 
   float4 acc[REP];
 #pragma unroll
@@ -330,7 +342,7 @@ __device__ __forceinline__ void hyb_row_tile(const HybBucket& bk, int64_t t, int
     }
   }
   reduce_groups<G, REP>(acc, kWave);
-  if (g == 0) write_row<G, REP>(C, bk.rows[row], feat, lane, acc, bk.atomic != 0, stage);
+  if (g == 0) write_row<G, REP>(C, bk.rows[row], feat, lane, acc, bk.atomic, stage);
 }
 
 __device__ __forceinline__ int find_bucket(const HybBucket* __restrict__ table, int nb,
@@ -348,15 +360,15 @@ __device__ __forceinline__ int find_bucket(const HybBucket* __restrict__ table, 
 
 template <int G, int REP>
 __global__ __launch_bounds__(256) void hyb_spmm_kernel(const HybBucket* __restrict__ table, int nb,
-                                                       int64_t total_tiles, int feat,
+                                                       int64_t tile_base, int64_t tile_end, int feat,
                                                        const float* __restrict__ B,
                                                        float* __restrict__ C) {
   __shared__ float stage_all[4][kWave * 4 * REP];  // per-wavefront staging for atomic rows
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   float* stage = stage_all[wave];
-  const int64_t tile = (int64_t)blockIdx.x * 4 + wave;
-  if (tile >= total_tiles) return;
+  const int64_t tile = tile_base + (int64_t)blockIdx.x * 4 + wave;
+  if (tile >= tile_end) return;
   const int k = find_bucket(table, nb, tile);
   const HybBucket bk = table[k];
   const int64_t t = tile - bk.tile_begin;
@@ -413,6 +425,8 @@ int log2_exact(int64_t x) {
 
 }  // namespace
 
+constexpr int kMaxPhases = 4;
+
 struct stir_hyb_plan {
   int32_t m, n, num_col_parts, num_buckets;
   int device;
@@ -420,6 +434,13 @@ struct stir_hyb_plan {
   HybBucket* d_table_tiles;       // tile_begin counted in wave tiles (vectorised kernel)
   HybBucket* d_table_rows;        // tile_begin counted in ELL rows (generic kernel)
   int64_t total_tiles, total_rows;
+  // With 2..kMaxPhases column partitions the vectorised kernel is launched once per partition, one
+  // after the other on the stream: inside a partition an output row belongs to a single ELL row
+  // (or to several of the last bucket), so all but the last bucket add with a plain
+  // read-modify-write instead of atomics.  phase_bucket / phase_tile: first table entry / first
+  // wave tile of every phase, and the ends.
+  std::vector<int> phase_bucket;
+  std::vector<int64_t> phase_tile;
 };
 
 extern "C" {
@@ -480,13 +501,17 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
   std::vector<int> order;
   for (int k = 0; k < total; ++k)
     if (nrows[k] > 0) order.push_back(k);
+  const bool phased = num_col_parts > 1 && num_col_parts <= kMaxPhases;
   std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+    if (phased && a / num_buckets != b / num_buckets) return a / num_buckets < b / num_buckets;
     return bucket_widths[a % num_buckets] > bucket_widths[b % num_buckets];
   });
   const int nk = (int)order.size();
   std::vector<HybBucket> host(nk > 0 ? 2 * nk : 1);
   HybBucket* host_rows = host.data() + nk;
   int64_t tiles = 0, rows = 0;
+  std::vector<int> phase_bucket;
+  std::vector<int64_t> phase_tile;
   for (int q = 0; q < nk; ++q) {
     const int k = order[q];
     const int b = k % num_buckets;
@@ -497,18 +522,27 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
     e.cols = d_cols[k];
     e.nrows = nrows[k];
     e.width = w;
-    e.atomic = (num_col_parts > 1 || b == num_buckets - 1) ? 1 : 0;
+    const int fused_mode = (num_col_parts > 1 || b == num_buckets - 1) ? 1 : 0;
+    e.atomic = (phased && b != num_buckets - 1) ? 2 : fused_mode;
     const bool slot_mode = stir::is_pow2(w) && w <= kWave;
     e.log2w = slot_mode ? log2_exact(w) : -1;
-    e.chunks = (!slot_mode && e.atomic && w > kRowChunk) ? (int)stir::ceil_div(w, kRowChunk) : 1;
+    e.chunks = (!slot_mode && e.atomic == 1 && w > kRowChunk) ? (int)stir::ceil_div(w, kRowChunk) : 1;
     e.tile_begin = tiles;
     host[q] = e;
+    if (phased && (q == 0 || k / num_buckets != order[q - 1] / num_buckets)) {
+      phase_bucket.push_back(q);
+      phase_tile.push_back(tiles);
+    }
     tiles += slot_mode ? stir::ceil_div(nrows[k] * w, kWave) : nrows[k] * e.chunks;
     e.tile_begin = rows;
     e.chunks = 1;
+    e.atomic = fused_mode;  // the generic kernel runs all partitions in one launch
     host_rows[q] = e;
     rows += nrows[k];
   }
+  if (!phased) phase_bucket.push_back(0), phase_tile.push_back(0);
+  phase_bucket.push_back(nk);
+  phase_tile.push_back(tiles);
   stir_hyb_plan* p = new stir_hyb_plan();
   p->m = m;
   p->n = n;
@@ -517,6 +551,8 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
   p->nk = nk;
   p->total_tiles = tiles;
   p->total_rows = rows;
+  p->phase_bucket = phase_bucket;
+  p->phase_tile = phase_tile;
   p->d_table_tiles = nullptr;
   p->d_table_rows = nullptr;
   hipError_t e = hipGetDevice(&p->device);
@@ -546,12 +582,17 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
   STIR_REQUIRE(d_B && d_C, "hyb_spmm: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 block(256);
-  const int64_t nblocks = stir::ceil_div(plan->total_tiles, 4);
-  STIR_REQUIRE(nblocks < (int64_t(1) << 31), "hyb_spmm: %lld tiles exceed one launch", (long long)plan->total_tiles);
-  dim3 grid((unsigned)nblocks);
-#define STIR_HYB(G, REP)                                                                        \
-  hipLaunchKernelGGL((hyb_spmm_kernel<G, REP>), grid, block, 0, st, plan->d_table_tiles, plan->nk, \
-                     plan->total_tiles, feat, d_B, d_C)
+  STIR_REQUIRE(stir::ceil_div(plan->total_tiles, 4) < (int64_t(1) << 31), "hyb_spmm: %lld tiles exceed one launch",
+               (long long)plan->total_tiles);
+  // one launch per phase (a single one unless the plan runs its partitions one after the other)
+#define STIR_HYB(G, REP)                                                                                    \
+  for (size_t ph = 0; ph + 1 < plan->phase_bucket.size(); ++ph) {                                           \
+    const int64_t t0 = plan->phase_tile[ph], t1 = plan->phase_tile[ph + 1];                                  \
+    if (t1 == t0) continue;                                                                                 \
+    hipLaunchKernelGGL((hyb_spmm_kernel<G, REP>), dim3((unsigned)stir::ceil_div(t1 - t0, 4)), block, 0, st,  \
+                       plan->d_table_tiles + plan->phase_bucket[ph],                                        \
+                       plan->phase_bucket[ph + 1] - plan->phase_bucket[ph], t0, t1, feat, d_B, d_C);        \
+  }
   switch (vector_class(feat)) {
     case 0: STIR_HYB(4, 1); break;
     case 1: STIR_HYB(8, 1); break;
