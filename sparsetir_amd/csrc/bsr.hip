@@ -349,10 +349,7 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   {
     const int f_tiles_s = (int)stir::ceil_div(feat, kTileF);
     const int64_t blocks_s = (int64_t)mb * (blk / 32) * f_tiles_s;
-    int dev = 0, cus = 256;
-    STIR_HIP(hipGetDevice(&dev));
-    STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    if (blocks_s <= 2 * (int64_t)cus) {
+    if (blocks_s <= 2 * (int64_t)stir::compute_units()) {
       const int64_t slices_s = (int64_t)mb * (blk / 32);
       dim3 grid_s((unsigned)blocks_s), block_s(256);
 #define STIR_BSR_S(BF, OUT)                                                                                  \

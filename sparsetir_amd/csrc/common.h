@@ -45,4 +45,17 @@ namespace stir {
 constexpr int kWave = 64;
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+
+// Compute units of the current device (asked once per device and thread; 0 on failure).
+inline int compute_units() {
+  static thread_local int cached_dev = -1, cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev != cached_dev) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached_dev = dev, cached = cus;
+  }
+  return cached;
+}
 }  // namespace stir

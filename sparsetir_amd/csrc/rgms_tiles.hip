@@ -425,9 +425,7 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   const int nb = (int)host.size();
   const int64_t tiles = ceil_div(m, kTileRows);
   const int end_bit = bit_length((((uint64_t)tiles * num_rels) << 5) - 1);
-  int dev = 0, cus = 256;
-  STIR_HIP(hipGetDevice(&dev));
-  STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  const int cus = std::max(1, compute_units());
   // Units (one workgroup each) of at most `cap` steps.  A tile is cut only when it is long against
   // the others -- more than about three average tiles -- or when the launch would otherwise
   // leave most of the chip idle (few tiles): the longest unit is the critical path of the launch.
