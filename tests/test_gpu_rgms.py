@@ -314,3 +314,23 @@ def test_rgms_tiled_rejects_ids_out_of_range(dev):
         y = torch.zeros(m * 32, dtype=torch.float32, device=dev)
         with pytest.raises(Exception, match="outside"):
             f(w, x, y, *triples, *mids)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_rgms_tiled_random_shapes(dev, seed):
+    """Random relation counts, row/column ranges, bucket lists and feature sizes, all large enough
+    for the destination-tiled kernel."""
+    rng = np.random.default_rng(100 + seed)
+    R = int(rng.integers(1, 13))
+    m, n = int(rng.integers(33, 3000)), int(rng.integers(40, 3000))
+    per_rel = int(rng.integers(9000, 30000)) // R + 1
+    pairs = [(rng.integers(0, m, per_rel), rng.integers(0, n, per_rel)) for _ in range(R)]
+    group = int(rng.choice([16, 32, 64, 256]))
+    widths = sorted(set(int(w) for w in rng.choice([1, 2, 3, 4, 8, 16], size=int(rng.integers(1, 5)))))
+    widths = [w for w in widths if w <= group]
+    fin, fout = int(rng.choice([16, 32, 64])), int(rng.choice([32, 64]))
+    got, want, scale, info = _tiled_case(dev, pairs, m, n, R, fin, fout, group, widths, seed)
+    assert info[-1] >= 8192, "shape too small for the tiled kernel"
+    err = np.abs(got - want)
+    assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), (
+        f"R={R} m={m} n={n} group={group} widths={widths} fin={fin} fout={fout}: worst {err.max():.3e}")
