@@ -161,7 +161,13 @@ int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const flo
  * A bucket is added to C when num_col_parts > 1 or it is the last bucket of its partition,
  * and stored otherwise (bench_spmm.py:170).  Adding is done with atomics, except that with 2 to
  * 4 partitions the partitions run one after the other on the stream and only the last bucket of
- * each needs atomics.  The plan keeps the pointers, not copies: the arrays must outlive it.
+ * each needs atomics -- provided that inside every partition an output row is fed either by one
+ * ELL row of one bucket other than the last, or by ELL rows of the last bucket only, as in
+ * ColumnPartHyb output.  stir_hyb_plan_create tests this on the row arrays as they are when it is
+ * called (it synchronises the device and reads them once) and keeps atomics for every bucket when
+ * it does not hold; row ids outside [0, m) are an error.  A caller that rewrites the row arrays
+ * of a plan with 2 to 4 partitions must make a new plan.  The plan keeps the pointers, not
+ * copies: the arrays must outlive it.
  */
 typedef struct stir_hyb_plan stir_hyb_plan;
 int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,

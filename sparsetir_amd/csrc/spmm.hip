@@ -409,6 +409,24 @@ __global__ __launch_bounds__(256) void hyb_spmm_generic_kernel(const HybBucket* 
   }
 }
 
+// Marks (mark = 1) or looks up (mark = 0) the output rows of one bucket in a bitmap with one bit
+// per output row.  flags[0] is raised when a row is met that is already marked, flags[1] when a
+// row id lies outside [0, m).
+__global__ __launch_bounds__(256) void hyb_mark_rows_kernel(const int32_t* __restrict__ rows, int64_t nrows,
+                                                            int32_t m, uint32_t* __restrict__ bitmap, int mark,
+                                                            int32_t* __restrict__ flags) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nrows) return;
+  const int32_t r = rows[i];
+  if (r < 0 || r >= m) {
+    flags[1] = 1;
+    return;
+  }
+  const uint32_t bit = 1u << (r & 31);
+  const uint32_t seen = mark ? atomicOr(bitmap + (r >> 5), bit) : bitmap[r >> 5];
+  if (seen & bit) flags[0] = 1;
+}
+
 // 0..5: lane groups of 4, 8, 16, 32, 64 lanes and 64 lanes x 2 float4 cover feat; -1: generic kernel
 int vector_class(int feat) {
   if (feat % 4 != 0 || feat > 512) return -1;
@@ -423,24 +441,173 @@ int log2_exact(int64_t x) {
   return l;
 }
 
+// Whether the partitions may run one after the other with plain read-modify-write adds in all but
+// their last bucket: inside every partition an output row must belong to one ELL row of one
+// non-last bucket, or to ELL rows of the last bucket only.  ColumnPartHyb output always does;
+// arrays built by other means may not, and the reference adds those atomically
+// (examples/spmm/bench_spmm.py:170-177).  Reads the row arrays as they are now (after a device
+// synchronisation).  *ok = 0 when some row is shared; an error when a row id is out of range.
+int phases_have_single_writers(int32_t m, int num_col_parts, int num_buckets, const int64_t* nrows,
+                               const int32_t* const* d_rows, bool* ok) {
+  *ok = true;
+  if (m == 0) return 0;
+  const size_t words = ((size_t)m + 31) / 32;
+  uint32_t* d_bitmap = nullptr;
+  for (int k = 0; k < num_col_parts * num_buckets; ++k)
+    STIR_REQUIRE(stir::ceil_div(nrows[k], 256) < (int64_t(1) << 31), "hyb_plan_create: bucket %d too large", k);
+  STIR_HIP(hipDeviceSynchronize());
+  STIR_HIP(hipMalloc(reinterpret_cast<void**>(&d_bitmap), (words + 2) * sizeof(uint32_t)));
+  int32_t* d_flags = reinterpret_cast<int32_t*>(d_bitmap + words);
+  hipError_t e = hipMemset(d_bitmap, 0, (words + 2) * sizeof(uint32_t));
+  for (int p = 0; p < num_col_parts && e == hipSuccess; ++p) {
+    bool any = false;
+    for (int b = 0; b < num_buckets; ++b) {
+      const int k = p * num_buckets + b;
+      if (nrows[k] == 0) continue;
+      hipLaunchKernelGGL(hyb_mark_rows_kernel, dim3((unsigned)stir::ceil_div(nrows[k], 256)), dim3(256), 0, 0,
+                         d_rows[k], nrows[k], m, d_bitmap, b != num_buckets - 1 ? 1 : 0, d_flags);
+      any = true;
+    }
+    if (any && p + 1 < num_col_parts) e = hipMemsetAsync(d_bitmap, 0, words * sizeof(uint32_t), 0);
+  }
+  int32_t flags[2] = {0, 0};
+  if (e == hipSuccess) e = hipGetLastError();
+  if (e == hipSuccess) e = hipMemcpy(flags, d_flags, sizeof(flags), hipMemcpyDeviceToHost);
+  (void)hipFree(d_bitmap);
+  if (e != hipSuccess) return stir::fail("hyb_plan_create: %s", hipGetErrorString(e));
+  STIR_REQUIRE(flags[1] == 0, "hyb_plan_create: a row index lies outside [0, %d)", m);
+  *ok = flags[0] == 0;
+  return 0;
+}
+
 }  // namespace
 
 constexpr int kMaxPhases = 4;
 
+namespace {
+
+// Host image of a hyb operator: the bucket descriptors in launch order, once with tile_begin
+// counted in wave tiles (vectorised kernel) and once in ELL rows (generic kernel).
+struct HybTables {
+  std::vector<HybBucket> tiles, rows;
+  int64_t total_tiles = 0, total_rows = 0;
+  // first table entry / first wave tile of every launch of the vectorised kernel, and the ends
+  std::vector<int> phase_bucket;
+  std::vector<int64_t> phase_tile;
+};
+
+int check_hyb_arguments(const char* who, int32_t m, int32_t n, int32_t num_col_parts, int32_t num_buckets,
+                        const int32_t* bucket_widths, const int64_t* nrows, const float* const* d_A,
+                        const int32_t* const* d_rows, const int32_t* const* d_cols) {
+  STIR_REQUIRE(m >= 0 && n >= 0 && num_col_parts > 0 && num_buckets > 0, "%s: bad sizes", who);
+  STIR_REQUIRE(bucket_widths && nrows && d_A && d_rows && d_cols, "%s: null pointer argument", who);
+  for (int b = 0; b < num_buckets; ++b)
+    STIR_REQUIRE(bucket_widths[b] > 0, "%s: bucket width %d is not positive", who, bucket_widths[b]);
+  const int total = num_col_parts * num_buckets;
+  for (int k = 0; k < total; ++k) {
+    STIR_REQUIRE(nrows[k] >= 0, "%s: nrows[%d] is negative", who, k);
+    STIR_REQUIRE(nrows[k] == 0 || (d_A[k] && d_rows[k] && d_cols[k]), "%s: bucket %d has rows but a null array",
+                 who, k);
+  }
+  return 0;
+}
+
+// phased: the partitions run one after the other (one launch each) and all but the last bucket of
+// a partition add with a plain read-modify-write.
+void make_hyb_tables(int32_t num_col_parts, int32_t num_buckets, const int32_t* bucket_widths,
+                     const int64_t* nrows, const float* const* d_A, const int32_t* const* d_rows,
+                     const int32_t* const* d_cols, bool phased, HybTables* out) {
+  const int total = num_col_parts * num_buckets;
+  // Widest buckets first: their wavefronts run longest, so they are dispatched first and the
+  // launch does not end on a tail of hub rows.
+  std::vector<int> order;
+  for (int k = 0; k < total; ++k)
+    if (nrows[k] > 0) order.push_back(k);
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+    if (phased && a / num_buckets != b / num_buckets) return a / num_buckets < b / num_buckets;
+    return bucket_widths[a % num_buckets] > bucket_widths[b % num_buckets];
+  });
+  const int nk = (int)order.size();
+  out->tiles.resize(nk);
+  out->rows.resize(nk);
+  int64_t tiles = 0, rows = 0;
+  for (int q = 0; q < nk; ++q) {
+    const int k = order[q];
+    const int b = k % num_buckets;
+    const int w = bucket_widths[b];
+    HybBucket e;
+    e.A = d_A[k];
+    e.rows = d_rows[k];
+    e.cols = d_cols[k];
+    e.nrows = nrows[k];
+    e.width = w;
+    const int fused_mode = (num_col_parts > 1 || b == num_buckets - 1) ? 1 : 0;
+    e.atomic = (phased && b != num_buckets - 1) ? 2 : fused_mode;
+    const bool slot_mode = stir::is_pow2(w) && w <= kWave;
+    e.log2w = slot_mode ? log2_exact(w) : -1;
+    e.chunks = (!slot_mode && e.atomic == 1 && w > kRowChunk) ? (int)stir::ceil_div(w, kRowChunk) : 1;
+    e.tile_begin = tiles;
+    out->tiles[q] = e;
+    if (phased && (q == 0 || k / num_buckets != order[q - 1] / num_buckets)) {
+      out->phase_bucket.push_back(q);
+      out->phase_tile.push_back(tiles);
+    }
+    tiles += slot_mode ? stir::ceil_div(nrows[k] * w, kWave) : nrows[k] * e.chunks;
+    e.tile_begin = rows;
+    e.chunks = 1;
+    e.atomic = fused_mode;  // the generic kernel runs all partitions in one launch
+    out->rows[q] = e;
+    rows += nrows[k];
+  }
+  if (!phased) out->phase_bucket.push_back(0), out->phase_tile.push_back(0);
+  out->phase_bucket.push_back(nk);
+  out->phase_tile.push_back(tiles);
+  out->total_tiles = tiles;
+  out->total_rows = rows;
+}
+
+// Launches the kernels of a hyb operator whose descriptor tables are at d_tiles / d_rows.
+int launch_hyb(const HybTables& t, const HybBucket* d_tiles, const HybBucket* d_rows, int32_t feat,
+               const float* d_B, float* d_C, hipStream_t st) {
+  const int nk = (int)t.tiles.size();
+  dim3 block(256);
+  STIR_REQUIRE(stir::ceil_div(t.total_tiles, 4) < (int64_t(1) << 31), "hyb_spmm: %lld tiles exceed one launch",
+               (long long)t.total_tiles);
+  // one launch per phase (a single one unless the partitions run one after the other)
+#define STIR_HYB(G, REP)                                                                                    \
+  for (size_t ph = 0; ph + 1 < t.phase_bucket.size(); ++ph) {                                               \
+    const int64_t t0 = t.phase_tile[ph], t1 = t.phase_tile[ph + 1];                                          \
+    if (t1 == t0) continue;                                                                                 \
+    hipLaunchKernelGGL((hyb_spmm_kernel<G, REP>), dim3((unsigned)stir::ceil_div(t1 - t0, 4)), block, 0, st,  \
+                       d_tiles + t.phase_bucket[ph], t.phase_bucket[ph + 1] - t.phase_bucket[ph], t0, t1,   \
+                       feat, d_B, d_C);                                                                     \
+  }
+  switch (vector_class(feat)) {
+    case 0: STIR_HYB(4, 1); break;
+    case 1: STIR_HYB(8, 1); break;
+    case 2: STIR_HYB(16, 1); break;
+    case 3: STIR_HYB(32, 1); break;
+    case 4: STIR_HYB(64, 1); break;
+    case 5: STIR_HYB(64, 2); break;
+    default: {
+      const int64_t rb = stir::ceil_div(t.total_rows, 4);
+      STIR_REQUIRE(rb < (int64_t(1) << 31), "hyb_spmm: %lld rows exceed one launch", (long long)t.total_rows);
+      hipLaunchKernelGGL(hyb_spmm_generic_kernel, dim3((unsigned)rb), block, 0, st, d_rows, nk, t.total_rows,
+                         feat, d_B, d_C);
+    }
+  }
+#undef STIR_HYB
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace
+
 struct stir_hyb_plan {
   int32_t m, n, num_col_parts, num_buckets;
   int device;
-  int nk;                         // buckets with at least one ELL row
-  HybBucket* d_table_tiles;       // tile_begin counted in wave tiles (vectorised kernel)
-  HybBucket* d_table_rows;        // tile_begin counted in ELL rows (generic kernel)
-  int64_t total_tiles, total_rows;
-  // With 2..kMaxPhases column partitions the vectorised kernel is launched once per partition, one
-  // after the other on the stream: inside a partition an output row belongs to a single ELL row
-  // (or to several of the last bucket), so all but the last bucket add with a plain
-  // read-modify-write instead of atomics.  phase_bucket / phase_tile: first table entry / first
-  // wave tile of every phase, and the ends.
-  std::vector<int> phase_bucket;
-  std::vector<int64_t> phase_tile;
+  HybTables tables;
+  HybBucket* d_tables;  // tables.tiles followed by tables.rows
 };
 
 extern "C" {
@@ -487,86 +654,29 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
                          const float* const* d_A, const int32_t* const* d_rows,
                          const int32_t* const* d_cols) {
   STIR_REQUIRE(plan, "hyb_plan_create: plan is null");
-  STIR_REQUIRE(m >= 0 && n >= 0 && num_col_parts > 0 && num_buckets > 0, "hyb_plan_create: bad sizes");
-  for (int b = 0; b < num_buckets; ++b)
-    STIR_REQUIRE(bucket_widths[b] > 0, "hyb_plan_create: bucket width %d is not positive", bucket_widths[b]);
-  const int total = num_col_parts * num_buckets;
-  for (int k = 0; k < total; ++k) {
-    STIR_REQUIRE(nrows[k] >= 0, "hyb_plan_create: nrows[%d] is negative", k);
-    STIR_REQUIRE(nrows[k] == 0 || (d_A[k] && d_rows[k] && d_cols[k]),
-                 "hyb_plan_create: bucket %d has rows but a null array", k);
-  }
-  // Widest buckets first: their wavefronts run longest, so they are dispatched first and the
-  // launch does not end on a tail of hub rows.
-  std::vector<int> order;
-  for (int k = 0; k < total; ++k)
-    if (nrows[k] > 0) order.push_back(k);
-  const bool phased = num_col_parts > 1 && num_col_parts <= kMaxPhases;
-  std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
-    if (phased && a / num_buckets != b / num_buckets) return a / num_buckets < b / num_buckets;
-    return bucket_widths[a % num_buckets] > bucket_widths[b % num_buckets];
-  });
-  const int nk = (int)order.size();
-  std::vector<HybBucket> host(nk > 0 ? 2 * nk : 1);
-  HybBucket* host_rows = host.data() + nk;
-  int64_t tiles = 0, rows = 0;
-  std::vector<int> phase_bucket;
-  std::vector<int64_t> phase_tile;
-  for (int q = 0; q < nk; ++q) {
-    const int k = order[q];
-    const int b = k % num_buckets;
-    const int w = bucket_widths[b];
-    HybBucket e;
-    e.A = d_A[k];
-    e.rows = d_rows[k];
-    e.cols = d_cols[k];
-    e.nrows = nrows[k];
-    e.width = w;
-    const int fused_mode = (num_col_parts > 1 || b == num_buckets - 1) ? 1 : 0;
-    e.atomic = (phased && b != num_buckets - 1) ? 2 : fused_mode;
-    const bool slot_mode = stir::is_pow2(w) && w <= kWave;
-    e.log2w = slot_mode ? log2_exact(w) : -1;
-    e.chunks = (!slot_mode && e.atomic == 1 && w > kRowChunk) ? (int)stir::ceil_div(w, kRowChunk) : 1;
-    e.tile_begin = tiles;
-    host[q] = e;
-    if (phased && (q == 0 || k / num_buckets != order[q - 1] / num_buckets)) {
-      phase_bucket.push_back(q);
-      phase_tile.push_back(tiles);
-    }
-    tiles += slot_mode ? stir::ceil_div(nrows[k] * w, kWave) : nrows[k] * e.chunks;
-    e.tile_begin = rows;
-    e.chunks = 1;
-    e.atomic = fused_mode;  // the generic kernel runs all partitions in one launch
-    host_rows[q] = e;
-    rows += nrows[k];
-  }
-  if (!phased) phase_bucket.push_back(0), phase_tile.push_back(0);
-  phase_bucket.push_back(nk);
-  phase_tile.push_back(tiles);
+  if (check_hyb_arguments("hyb_plan_create", m, n, num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows,
+                          d_cols) != 0)
+    return -1;
+  bool phased = num_col_parts > 1 && num_col_parts <= kMaxPhases;
+  if (phased && phases_have_single_writers(m, num_col_parts, num_buckets, nrows, d_rows, &phased) != 0) return -1;
   stir_hyb_plan* p = new stir_hyb_plan();
   p->m = m;
   p->n = n;
   p->num_col_parts = num_col_parts;
   p->num_buckets = num_buckets;
-  p->nk = nk;
-  p->total_tiles = tiles;
-  p->total_rows = rows;
-  p->phase_bucket = phase_bucket;
-  p->phase_tile = phase_tile;
-  p->d_table_tiles = nullptr;
-  p->d_table_rows = nullptr;
+  p->d_tables = nullptr;
+  make_hyb_tables(num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols, phased, &p->tables);
+  const size_t nk = p->tables.tiles.size();
   hipError_t e = hipGetDevice(&p->device);
   if (e == hipSuccess && nk > 0) {
-    e = hipMalloc(reinterpret_cast<void**>(&p->d_table_tiles), sizeof(HybBucket) * 2 * nk);
-    if (e == hipSuccess) {
-      p->d_table_rows = p->d_table_tiles + nk;
-      e = hipMemcpy(p->d_table_tiles, host.data(), sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
-      if (e == hipSuccess)
-        e = hipMemcpy(p->d_table_rows, host_rows, sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
-    }
+    e = hipMalloc(reinterpret_cast<void**>(&p->d_tables), sizeof(HybBucket) * 2 * nk);
+    if (e == hipSuccess)
+      e = hipMemcpy(p->d_tables, p->tables.tiles.data(), sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+      e = hipMemcpy(p->d_tables + nk, p->tables.rows.data(), sizeof(HybBucket) * nk, hipMemcpyHostToDevice);
   }
   if (e != hipSuccess) {
-    if (p->d_table_tiles) (void)hipFree(p->d_table_tiles);
+    if (p->d_tables) (void)hipFree(p->d_tables);
     delete p;
     return stir::fail("hyb_plan_create: %s", hipGetErrorString(e));
   }
@@ -578,43 +688,16 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
                       void* stream) {
   STIR_REQUIRE(plan, "hyb_spmm: plan is null");
   STIR_REQUIRE(feat > 0, "hyb_spmm: feat=%d", feat);
-  if (plan->nk == 0) return 0;
+  const size_t nk = plan->tables.tiles.size();
+  if (nk == 0) return 0;
   STIR_REQUIRE(d_B && d_C, "hyb_spmm: null pointer argument");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  dim3 block(256);
-  STIR_REQUIRE(stir::ceil_div(plan->total_tiles, 4) < (int64_t(1) << 31), "hyb_spmm: %lld tiles exceed one launch",
-               (long long)plan->total_tiles);
-  // one launch per phase (a single one unless the plan runs its partitions one after the other)
-#define STIR_HYB(G, REP)                                                                                    \
-  for (size_t ph = 0; ph + 1 < plan->phase_bucket.size(); ++ph) {                                           \
-    const int64_t t0 = plan->phase_tile[ph], t1 = plan->phase_tile[ph + 1];                                  \
-    if (t1 == t0) continue;                                                                                 \
-    hipLaunchKernelGGL((hyb_spmm_kernel<G, REP>), dim3((unsigned)stir::ceil_div(t1 - t0, 4)), block, 0, st,  \
-                       plan->d_table_tiles + plan->phase_bucket[ph],                                        \
-                       plan->phase_bucket[ph + 1] - plan->phase_bucket[ph], t0, t1, feat, d_B, d_C);        \
-  }
-  switch (vector_class(feat)) {
-    case 0: STIR_HYB(4, 1); break;
-    case 1: STIR_HYB(8, 1); break;
-    case 2: STIR_HYB(16, 1); break;
-    case 3: STIR_HYB(32, 1); break;
-    case 4: STIR_HYB(64, 1); break;
-    case 5: STIR_HYB(64, 2); break;
-    default: {
-      const int64_t rb = stir::ceil_div(plan->total_rows, 4);
-      STIR_REQUIRE(rb < (int64_t(1) << 31), "hyb_spmm: %lld rows exceed one launch", (long long)plan->total_rows);
-      hipLaunchKernelGGL(hyb_spmm_generic_kernel, dim3((unsigned)rb), block, 0, st, plan->d_table_rows,
-                         plan->nk, plan->total_rows, feat, d_B, d_C);
-    }
-  }
-#undef STIR_HYB
-  STIR_LAUNCH_CHECK();
-  return 0;
+  return launch_hyb(plan->tables, plan->d_tables, plan->d_tables + nk, feat, d_B, d_C,
+                    static_cast<hipStream_t>(stream));
 }
 
 int stir_hyb_plan_destroy(stir_hyb_plan* plan) {
   if (!plan) return 0;
-  if (plan->d_table_tiles) (void)hipFree(plan->d_table_tiles);
+  if (plan->d_tables) (void)hipFree(plan->d_tables);
   delete plan;
   return 0;
 }

@@ -19,9 +19,14 @@ def cfg3():
     return datasets.config3()
 
 
-def test_config3_device_format_bit_exact(dev, cfg3):
+@pytest.mark.parametrize("parts,buckets", [
+    (2, [1, 2, 4, 8, 16, 32]),
+    (1, [1, 2, 4, 8, 16, 32, 64, 128, 256, 512]),   # the decomposition bench.py times
+    (16, [1, 2, 4, 8, 16, 32]),                     # examples/spmm/bench_spmm.py:233-253 for a graph of this size
+])
+def test_config3_device_format_bit_exact(dev, cfg3, parts, buckets):
     g = cfg3
-    m, n, parts, buckets = g["m"], g["n"], 2, [1, 2, 4, 8, 16, 32]
+    m, n = g["m"], g["n"]
     t = lambda a: torch.from_numpy(a).to(dev)
     rows, cols, mask = st.column_part_hyb(m, n, t(g["indptr"]), t(g["indices"]), parts, buckets)
     want = oracle.column_part_hyb(m, n, g["indptr"], g["indices"], parts, buckets)
@@ -35,10 +40,13 @@ def test_config3_device_format_bit_exact(dev, cfg3):
     assert total == len(g["indices"])  # every nonzero placed exactly once
 
 
-def test_config3_hyb_equals_csr_and_oracle_sample(dev, cfg3):
+@pytest.mark.parametrize("setting", ["bench", "reference"])
+def test_config3_hyb_equals_csr_and_oracle_sample(dev, cfg3, setting):
     g = cfg3
     m, n, feat = g["m"], g["n"], 128
-    parts, buckets = g["num_col_parts"], g["buckets"]
+    # "bench": the decomposition bench.py times; "reference": 16 partitions x widths 1..32, what
+    # examples/spmm/bench_spmm.py:233-253 picks for a graph of this size (every bucket adds with atomics)
+    parts, buckets = (g["num_col_parts"], g["buckets"]) if setting == "bench" else (16, [1, 2, 4, 8, 16, 32])
     indptr, indices = g["indptr"], g["indices"]
     nnz = len(indices)
     t = lambda a: torch.from_numpy(a).to(dev)
@@ -99,6 +107,15 @@ def test_config3_sddmm_edge_sample(dev, cfg3):
     want = np.einsum("ek,ek->e", ah, bh)
     scale = np.einsum("ek,ek->e", np.abs(ah), np.abs(bh))
     assert np.all(np.abs(out.cpu().numpy()[sel] - want) <= 1e-5 * scale)
+    # the edge-scaled form out_e = A_e <X[row], Y[col]> on the same inputs, A_e from U(0,1)
+    ev = torch.rand(nnz, device=dev, generator=torch.Generator(device=dev).manual_seed(9))
+    out2 = torch.full((nnz,), float("nan"), device=dev)
+    ops.build_sddmm_scaled(m, n, feat, nnz)(a, b, out2, args[3], args[4], mid, ev)
+    torch.cuda.synchronize()
+    evh = ev.cpu().numpy()[sel].astype(np.float64)
+    assert np.all(np.abs(out2.cpu().numpy()[sel] - want * evh) <= 2e-5 * scale * evh + 1e-30)
+    # and everywhere: scaled result == edge value * unscaled result up to one rounding
+    assert bool(((out2 - ev * out).abs() <= 1e-6 * (ev * out).abs() + 1e-30).all())
 
 
 def test_config5_rgms_full(dev):

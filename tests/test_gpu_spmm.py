@@ -167,7 +167,12 @@ def _hyb_as_coo(triples_np):
 
 @pytest.mark.parametrize("feat", [32, 64, 128, 256, 512, 96, 7, 4, 16, 40, 384])
 @pytest.mark.parametrize("parts,buckets", [(1, [1, 2, 4, 8, 16, 32]), (2, [1, 2, 4, 8, 16, 32, 64, 128, 256, 512]),
-                                           (4, [2, 3, 7]), (3, [1])])
+                                           (4, [2, 3, 7]), (3, [1]),
+                                           # more than four partitions: every bucket of the single launch adds
+                                           # with atomics; 16 x [1..32] is the reference's own setting for its
+                                           # largest graph (examples/spmm/bench_spmm.py:233-253)
+                                           (8, [1, 2, 4, 8, 16, 32, 64]), (16, [1, 2, 4, 8, 16, 32]),
+                                           (5, [2, 5, 300])])
 def test_hyb_spmm_matches_oracle(dev, feat, parts, buckets):
     m = n = 3001
     indptr, indices = random_csr(m, n, 60000, 17, skew=1.3)
@@ -208,7 +213,7 @@ def test_hyb_spmm_store_semantics_of_non_atomic_buckets(dev):
     assert np.allclose(twice[last_rows], 2 * once[last_rows], rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("feat", [32, 128])
+@pytest.mark.parametrize("feat", [32, 64, 128, 256])
 def test_hyb_spmm_config2_against_csr_kernel_and_oracle(dev, feat):
     g = datasets.config2()
     m, n, parts, buckets = g["m"], g["n"], g["num_col_parts"], g["buckets"]
@@ -223,6 +228,56 @@ def test_hyb_spmm_config2_against_csr_kernel_and_oracle(dev, feat):
     assert np.all(np.abs(got - csr) <= 2 * RTOL * scale + 1e-30)
     want = oracle.hyb_spmm(m, feat, x, triples, parts)
     assert np.all(np.abs(got - want) <= 2 * RTOL * scale + 1e-30)
+
+
+@pytest.mark.parametrize("where", ["same_bucket", "two_buckets", "with_last_bucket"])
+def test_hyb_spmm_caller_built_arrays_sharing_output_rows(dev, where):
+    """Arrays that ColumnPartHyb would not produce: inside one column partition an output row is
+    fed by several ELL rows of buckets other than the last.  The reference adds every bucket
+    atomically when there are several partitions (examples/spmm/bench_spmm.py:170-177), so the
+    sums must still be complete (with 2-4 partitions the library may only drop the atomics when
+    every such row has a single writer, which it checks when the plan is made)."""
+    m, n, feat, parts, buckets = 64, 512, 128, 2, [2, 4, 8]
+    rng = np.random.default_rng(3)
+    nrows = 4096  # many ELL rows onto few output rows: lost updates would be certain without atomics
+    def ell(width, count, row_ids):
+        cols = rng.integers(0, n // 2, (count, width)).astype(np.int32)
+        a = rng.random((count, width), dtype=np.float32) + 0.5
+        return a, np.asarray(row_ids, np.int32), cols
+    empty = lambda w: (np.zeros((0, w), np.float32), np.zeros(0, np.int32), np.zeros((0, w), np.int32))
+    part0 = [empty(2), empty(4), empty(8)]
+    if where == "same_bucket":
+        part0[0] = ell(2, nrows, rng.integers(0, 8, nrows))
+    elif where == "two_buckets":
+        part0[0] = ell(2, nrows, np.arange(nrows) % m)
+        part0[1] = ell(4, nrows, (np.arange(nrows) * 7) % m)
+    else:
+        part0[1] = ell(4, m, np.arange(m))
+        part0[2] = ell(8, nrows, np.sort(rng.integers(0, m, nrows)))
+    part1 = [ell(2, m, np.arange(m)), empty(4), ell(8, 10, np.arange(10))]
+    part1 = [(a, r, c + n // 2) for a, r, c in part1]
+    triples = part0 + part1
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    got, _ = _run_hyb(dev, m, n, feat, parts, buckets, triples, x)
+    import scipy.sparse as sp
+    r, c, v = _hyb_as_coo(triples)
+    exact = sp.coo_matrix((v.astype(np.float64), (r, c)), shape=(m, n)).tocsr() @ x.astype(np.float64)
+    scale = sp.coo_matrix((np.abs(v).astype(np.float64), (r, c)), shape=(m, n)).tocsr() @ np.abs(x).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= RTOL * scale + 1e-30)
+    want = oracle.hyb_spmm(m, feat, x, triples, parts)
+    assert np.all(np.abs(got - want) <= 2 * RTOL * scale + 1e-30)
+
+
+def test_hyb_plan_rejects_row_ids_out_of_range(dev):
+    m, n, feat, parts, buckets = 16, 32, 32, 2, [1, 2]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    f = ops.build_hyb_csrmm(m, n, feat, parts, buckets, [1, 0, 0, 0])
+    z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
+    args = [t(np.ones(1, np.float32)), t(np.asarray([m], np.int32)), z(1, torch.int32)]
+    for _ in range(3):
+        args += [z(0, torch.float32), z(0, torch.int32), z(0, torch.int32)]
+    with pytest.raises(SparseTIRError, match="row index"):
+        f(z(n * feat, torch.float32), z(m * feat, torch.float32), *args)
 
 
 def test_hyb_spmm_empty_and_degenerate(dev):
