@@ -179,6 +179,25 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
 int stir_hyb_plan_destroy(stir_hyb_plan* plan);
 
 /*
+ * hyb SpMM fp32 without a plan and without any allocation.  No counterpart in the reference: it
+ * is for callers that cannot allocate device memory -- code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  Takes the arguments of stir_hyb_plan_create
+ * followed by those of stir_hyb_spmm_f32 and computes what that pair computes; the bucket
+ * descriptors that a plan keeps in allocated device memory go, on every call, into a fixed
+ * 128 KiB array that the library holds on each GPU it runs on until the process ends.  Limit: at
+ * most 1024 buckets with rows (over all partitions); more is an error.  Always one launch of the
+ * SpMM kernel (plus one small launch per 32 buckets that writes the descriptors): with several
+ * partitions every bucket adds with atomics, as in the reference (examples/spmm/bench_spmm.py:170).
+ * Calls on one GPU share that array: calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream are ordered and safe.
+ */
+int stir_hyb_spmm_f32_noalloc(int32_t m, int32_t n, int32_t num_col_parts, int32_t num_buckets,
+                              const int32_t* bucket_widths, const int64_t* nrows,
+                              const float* const* d_A, const int32_t* const* d_rows,
+                              const int32_t* const* d_cols, int32_t feat, const float* d_B,
+                              float* d_C, void* stream);
+
+/*
  * SDDMM fp32.  _preproc is the reference's binary-search block: mid[e] = index of the row
  * that owns nonzero e (tests/python/sparsetir/sparse_tir_lowered_buffer_scripts.py:531-551);
  * stir_sddmm_f32 computes C[e] = <A[mid[e],:], B[indices[e],:]> with the reference's

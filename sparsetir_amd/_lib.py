@@ -36,6 +36,7 @@ SIGNATURES = {
     "stir_hyb_plan_create": (I32, [VP, I32, I32, I32, I32, VP, VP, VP, VP, VP]),
     "stir_hyb_spmm_f32": (I32, [VP, I32, VP, VP, VP]),
     "stir_hyb_plan_destroy": (I32, [VP]),
+    "stir_hyb_spmm_f32_noalloc": (I32, [I32, I32, I32, I32, VP, VP, VP, VP, VP, I32, VP, VP, VP]),
     "stir_sddmm_preproc": (I32, [I32, I64, VP, VP, VP]),
     "stir_sddmm_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP]),
     "stir_sddmm_scaled_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP, VP]),

@@ -7,11 +7,19 @@
 // wavefront with one coalesced load (lane l holds slot l of the 64-slot tile) and handed to
 // the lane groups through cross-lane reads, so no lane issues a redundant index load.
 #include <algorithm>
+#include <mutex>
 #include <vector>
 
 #include "common.h"
 #include "row_lookup.h"
 #include "../../include/sparsetir_amd.h"
+
+// Device memory of stir_hyb_spmm_f32_noalloc: room for the two descriptor tables of an operator
+// with up to kStaticBuckets non-empty buckets (64 bytes per descriptor and table).  One copy per
+// GPU, held until the process ends.  Host code reaches it through the per-device address that
+// static_scratch() returns, never through this name.
+constexpr int kStaticBuckets = 1024;
+static __device__ __align__(256) unsigned char scratch[2 * kStaticBuckets * 64];
 
 namespace {
 
@@ -427,6 +435,21 @@ __global__ __launch_bounds__(256) void hyb_mark_rows_kernel(const int32_t* __res
   if (seen & bit) flags[0] = 1;
 }
 
+// Copies `count` bucket descriptors, handed over as a kernel argument, to dst[first ...]: how the
+// entry point that allocates nothing gets its descriptor tables into device memory without a
+// host-to-device copy.
+constexpr int kTableChunk = 32;
+struct HybTableChunk {
+  HybBucket b[kTableChunk];
+};
+__global__ __launch_bounds__(256) void hyb_table_fill_kernel(HybTableChunk chunk, int count,
+                                                             HybBucket* __restrict__ dst) {
+  constexpr int kWords = sizeof(HybBucket) / 4;
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(&chunk);
+  uint32_t* out = reinterpret_cast<uint32_t*>(dst);
+  for (int i = threadIdx.x; i < count * kWords; i += 256) out[i] = src[i];
+}
+
 // 0..5: lane groups of 4, 8, 16, 32, 64 lanes and 64 lanes x 2 float4 cover feat; -1: generic kernel
 int vector_class(int feat) {
   if (feat % 4 != 0 || feat > 512) return -1;
@@ -601,6 +624,26 @@ int launch_hyb(const HybTables& t, const HybBucket* d_tiles, const HybBucket* d_
   return 0;
 }
 
+// Address of `scratch` on the current device, asked from the runtime once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(HybBucket** out) {
+  int dev = -1;
+  STIR_HIP(hipGetDevice(&dev));
+  STIR_REQUIRE(dev >= 0 && dev < kMaxDevices, "hyb_spmm_noalloc: device %d is not supported", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    STIR_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    STIR_REQUIRE(ptr, "hyb_spmm_noalloc: the scratch array has no address on device %d", dev);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = static_cast<HybBucket*>(g_scratch_ptr[dev]);
+  return 0;
+}
+
 }  // namespace
 
 struct stir_hyb_plan {
@@ -693,6 +736,41 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
   STIR_REQUIRE(d_B && d_C, "hyb_spmm: null pointer argument");
   return launch_hyb(plan->tables, plan->d_tables, plan->d_tables + nk, feat, d_B, d_C,
                     static_cast<hipStream_t>(stream));
+}
+
+int stir_hyb_spmm_f32_noalloc(int32_t m, int32_t n, int32_t num_col_parts, int32_t num_buckets,
+                              const int32_t* bucket_widths, const int64_t* nrows, const float* const* d_A,
+                              const int32_t* const* d_rows, const int32_t* const* d_cols, int32_t feat,
+                              const float* d_B, float* d_C, void* stream) {
+  static_assert(sizeof(HybBucket) == 64, "descriptor size the scratch array is laid out for");
+  if (check_hyb_arguments("hyb_spmm_noalloc", m, n, num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows,
+                          d_cols) != 0)
+    return -1;
+  STIR_REQUIRE(feat > 0, "hyb_spmm_noalloc: feat=%d", feat);
+  HybTables tables;
+  // one launch, every bucket adds with atomics when there are several partitions
+  // (examples/spmm/bench_spmm.py:170 of the reference): nothing is known about the row arrays here
+  make_hyb_tables(num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols, false, &tables);
+  const int nk = (int)tables.tiles.size();
+  if (nk == 0) return 0;
+  STIR_REQUIRE(nk <= kStaticBuckets, "hyb_spmm_noalloc: %d non-empty buckets, at most %d are supported", nk,
+               kStaticBuckets);
+  STIR_REQUIRE(d_B && d_C, "hyb_spmm_noalloc: null pointer argument");
+  HybBucket* d_tables = nullptr;
+  if (static_scratch(&d_tables) != 0) return -1;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // only the table the kernel for this feature width reads is written
+  const bool generic = vector_class(feat) < 0;
+  const std::vector<HybBucket>& src = generic ? tables.rows : tables.tiles;
+  HybBucket* dst = generic ? d_tables + kStaticBuckets : d_tables;
+  for (int first = 0; first < nk; first += kTableChunk) {
+    HybTableChunk chunk = {};
+    const int count = std::min(kTableChunk, nk - first);
+    std::copy(src.begin() + first, src.begin() + first + count, chunk.b);
+    hipLaunchKernelGGL(hyb_table_fill_kernel, dim3(1), dim3(256), 0, st, chunk, count, dst + first);
+  }
+  STIR_LAUNCH_CHECK();
+  return launch_hyb(tables, d_tables, d_tables + kStaticBuckets, feat, d_B, d_C, st);
 }
 
 int stir_hyb_plan_destroy(stir_hyb_plan* plan) {
