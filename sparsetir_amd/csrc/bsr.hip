@@ -1,16 +1,14 @@
 // BSR SpMM on the gfx950 matrix cores: Y[i-th block row] = sum over stored blocks p of
 // A_p (blk x blk) * X[indices[p]-th block of rows], 16-bit inputs, fp32 accumulation.
 //
-// A workgroup of four wavefronts owns one 32-row slice of a block row and a 128*NT-wide slice
-// of the feature axis; a wavefront owns NT 32-feature tiles, each a 32x32 fp32 accumulator fed
-// by v_mfma_f32_32x32x16_{f16,bf16}.  The A operand wants 8 consecutive k per lane, which is
-// exactly how a row of a stored block lies in memory, so it is loaded straight from global
-// memory (16 bytes per lane).  The X operand wants 8 consecutive k for one feature column, but
-// X is feature-contiguous, so the 32 x TF tile of X goes through LDS: every thread loads two
-// adjacent k rows (16 bytes each), interleaves them into (k, k+1) pairs and stores 32 bytes; a
-// lane's MFMA operand is then four 4-byte LDS reads.  Tiles are double-buffered in LDS and the
-// next step's global loads are in flight while the current one is multiplied.
+// A workgroup of four wavefronts owns 32 or 64 rows of a block row and a 128*NT-wide slice of the
+// feature axis; a wavefront owns NT 32-feature tiles per 32 rows, each a 32x32 fp32 accumulator
+// fed by v_mfma_f32_32x32x16_{f16,bf16}.  Both operands go through LDS: the MFMA B operand wants
+// 8 consecutive k for one feature per lane while X is feature-contiguous, and the A fragment is
+// shared by the four wavefronts (see bsr_tile).  Small launches use bsr_spmm_ksplit_kernel.
 #include <hip/hip_fp16.h>
+
+#include <numeric>
 
 #include "common.h"
 #include "../../include/sparsetir_amd.h"
@@ -23,6 +21,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __fp16 tr16x4 __attribute__((__vector_size__(4 * sizeof(__fp16))));  // result type of the transposing LDS read
+#define STIR_LDS __attribute__((address_space(3)))
 
 constexpr int kTileF = 128;  // features per workgroup
 constexpr int kTileK = 32;   // k rows staged per step
@@ -70,34 +71,64 @@ __device__ __forceinline__ bool decode_tile(int64_t L, int64_t slices, int f_til
   return slice < slices;
 }
 
-// 1-D grid (see decode_tile); block: 256 threads = 4 wavefronts; wavefront w owns features
-// [32*NT*w, 32*NT*(w+1)) of the TF = 128*NT wide tile and RS*NT 32x32 accumulators.  The X tile of
-// step it+1 is fetched into registers while step it is multiplied out of LDS (two LDS buffers,
-// one barrier per step).  RS = 2 (blocks of 64 rows and more): a workgroup takes two adjacent
-// 32-row slices of a block row, so every X fragment read from LDS feeds two MFMAs and the X tile
-// is fetched once for 64 rows.
-template <bool BF16, int OUT, int NT, int S, int RS>  // OUT: 0 = same 16-bit type as the inputs, 1 = fp32
-__global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles,
-                                                       const uint16_t* __restrict__ A,
-                                                       const uint16_t* __restrict__ X, void* __restrict__ Y,
-                                                       const int32_t* __restrict__ indptr,
-                                                       const int32_t* __restrict__ indices,
-                                                       const int32_t* __restrict__ row_ids) {
+// One tile of the output: the 32*RS rows [bi0, bi0 + 32*RS) of stored block row i times the
+// features [f0, f0 + 128*NT).  256 threads = 4 wavefronts; wavefront w owns features
+// [32*NT*w, 32*NT*(w+1)) of the tile and RS*NT 32x32 accumulators.  RS = 2 (blocks of 64 rows and
+// more): two adjacent 32-row slices of a block row, so every X fragment read from LDS feeds two
+// MFMAs and the X tile is fetched once for 64 rows.
+//
+// Per step (one stored block, 32 of its k columns) the workgroup brings a 32 x 128*NT tile of X
+// and the 32*RS x 32 piece of the block into LDS -- each thread loads 16-byte chunks, consecutive
+// lanes consecutive chunks of a row of X -- while the previous step is multiplied (two LDS
+// stages, one barrier per step).  LDS keeps X feature-contiguous, in 16-byte units of 8 features:
+// unit (k, c) sits at (k/4)*4*FCN + (k%4)*FCN + (c ^ 2*(k%4)), FCN = units per row.  The MFMA B
+// operand (8 consecutive k for one feature per lane) comes out of that image through the
+// transposing read ds_read_b64_tr_b16, which hands lane i of a block of 16 lanes four consecutive
+// k of column i when the lanes address rows k .. k+3, four features each; the XOR keeps both the
+// 16-byte stores of a row (8 lanes, one k) and those reads (4 rows x 2 units) on distinct banks.
+// The block piece is fetched once per workgroup (8*RS bytes per thread) and laid out by k chunk so
+// that a lane's A operand is one 16-byte read.
+// lds: 2 * (64*128*NT + 2048*RS) bytes.
+template <bool BF16, int OUT, int NT, int RS>  // OUT: 0 = same 16-bit type as the inputs, 1 = fp32
+__device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int feat, int i, int i_out, int bi0,
+                                         int f0, const uint16_t* __restrict__ A,
+                                         const uint16_t* __restrict__ X, void* __restrict__ Y,
+                                         const int32_t* __restrict__ indptr,
+                                         const int32_t* __restrict__ indices) {
   constexpr int TF = kTileF * NT;
-  constexpr int FC = TF / 8;      // 8-feature chunks per tile row
-  constexpr int KPT = 256 / FC;   // k pairs covered by one pass of the 256 threads
-  __shared__ uint32_t xs[2][kTileK / 2][TF];  // [buffer][k pair][feature] -> (X[2kp][f], X[2kp+1][f])
+  constexpr int FCN = TF / 8;            // 16-byte units per tile row
+  constexpr int XB = kTileK * TF * 2;    // bytes of X per stage
+  constexpr int SB = XB + 2048 * RS;     // bytes per stage
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
-  int64_t slice;
-  int f_tile;
-  if (!decode_tile(blockIdx.x, slices, f_tiles, slice, f_tile)) return;
-  const int sub = blk / (32 * RS);  // slices of 32*RS rows per block row
-  const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * (32 * RS);
-  const int f0 = f_tile * TF;
-  const int kp0 = tid / FC, fc = tid % FC;
-  const bool stage_live = f0 + fc * 8 < feat;  // feat is a multiple of 32, so chunks are whole
+
+  // staging role: 2*NT chunks of X per thread
+  uint32_t xoff[2 * NT], xdst[2 * NT];
+  bool xlive[2 * NT];
+#pragma unroll
+  for (int q = 0; q < 2 * NT; ++q) {
+    const int idx = 64 * (wave * 2 * NT + q) + lane, c = idx % FCN, k = idx / FCN;
+    xoff[q] = (uint32_t)(k * feat + 8 * c);  // in elements, from the tile's first element
+    xdst[q] = (uint32_t)(((k >> 2) * 4 * FCN + (k & 3) * FCN + (c ^ (2 * (k & 3)))) * 16);
+    xlive[q] = f0 + 8 * c < feat;  // feat is a multiple of 32, so chunks are whole
+  }
+  // ... and 8*RS bytes of the block: RS = 1: half of the unit (chunk tid/64, row (tid/2)%32);
+  // RS = 2: the unit (slice tid/128, chunk (tid/32)%4, row tid%32)
+  uint32_t aoff;
+  if constexpr (RS == 1)
+    aoff = (uint32_t)(((tid >> 1) & 31) * blk + (tid >> 6) * 8 + (tid & 1) * 4);
+  else
+    aoff = (uint32_t)((32 * (tid >> 7) + (tid & 31)) * blk + ((tid >> 5) & 3) * 8);
+  // operand reads, bytes inside a stage
+  const int sl = lane & 15, half16 = (lane >> 4) & 1;
+  uint32_t bread[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int kr = sl >> 2, c = (wave * NT + t) * 4 + 2 * half16 + ((sl & 3) >> 1);
+    bread[t] = (uint32_t)(((2 * h) * 4 * FCN + kr * FCN + (c ^ (2 * kr))) * 16 + (sl & 1) * 8);
+  }
+  const uint32_t aread = XB + (h * 32 + n) * 16;
 
   f32x16 acc[RS][NT];
 #pragma unroll
@@ -107,77 +138,55 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[rs][t][v] = 0.f;
 
-  // doubly-compressed form: stored block row i is block row row_ids[i] of the output
-  const int i_out = row_ids ? row_ids[i] : i;
   const int p_begin = indptr[i];
   const int ksteps = blk / kTileK;
   const int steps = (indptr[i + 1] - p_begin) * ksteps;
 
-  // Register ring of S prefetched steps: loads for step it+S are issued as soon as step it has
-  // been copied to LDS, so S tiles per wavefront are in flight while the matrix cores work.
-  u32x4 r0[S][NT], r1[S][NT], areg[S][RS][2];
-  auto fetch = [&](int it, int s) {
+  u32x4 xr[2 * NT];
+  u32x4 ar;  // RS = 1 uses the first two words
+  auto fetch = [&](int it) {
     const int p = p_begin + it / ksteps, k0 = (it % ksteps) * kTileK;
     const int64_t j = indices[p];
+    const uint16_t* xb = X + ((int64_t)j * blk + k0) * feat + f0;
+    const uint16_t* ab = A + (int64_t)p * blk * blk + (int64_t)bi0 * blk + k0;
 #pragma unroll
-    for (int rs = 0; rs < RS; ++rs) {
-      const uint16_t* ablk = A + (int64_t)p * blk * blk + (int64_t)(bi0 + 32 * rs + n) * blk + k0;
-      areg[s][rs][0] = *reinterpret_cast<const u32x4*>(ablk + 8 * h);       // k = k0 + 8h + (0..7)
-      areg[s][rs][1] = *reinterpret_cast<const u32x4*>(ablk + 16 + 8 * h);  // k = k0 + 16 + 8h + (0..7)
-    }
-#pragma unroll
-    for (int q = 0; q < NT; ++q) {
-      r0[s][q] = r1[s][q] = u32x4{0, 0, 0, 0};
-      if (stage_live) {
-        const uint16_t* xp = X + ((int64_t)j * blk + k0 + 2 * (kp0 + KPT * q)) * feat + f0 + fc * 8;
-        r0[s][q] = *reinterpret_cast<const u32x4*>(xp);
-        r1[s][q] = *reinterpret_cast<const u32x4*>(xp + feat);
-      }
+    for (int q = 0; q < 2 * NT; ++q)
+      xr[q] = xlive[q] ? *reinterpret_cast<const u32x4*>(xb + xoff[q]) : u32x4{0, 0, 0, 0};
+    if constexpr (RS == 1) {
+      const u32x2 v = *reinterpret_cast<const u32x2*>(ab + aoff);
+      ar[0] = v[0], ar[1] = v[1];
+    } else {
+      ar = *reinterpret_cast<const u32x4*>(ab + aoff);
     }
   };
 
+  if (steps > 0) fetch(0);
+  for (int it = 0; it < steps; ++it) {
+    char* stage = lds + (it & 1) * SB;
 #pragma unroll
-  for (int s = 0; s < S; ++s)
-    if (s < steps) fetch(s, s);
-  for (int it0 = 0; it0 < steps; it0 += S) {
+    for (int q = 0; q < 2 * NT; ++q) *reinterpret_cast<u32x4*>(stage + xdst[q]) = xr[q];
+    if constexpr (RS == 1)
+      *reinterpret_cast<u32x2*>(stage + XB + tid * 8) = u32x2{ar[0], ar[1]};
+    else
+      *reinterpret_cast<u32x4*>(stage + XB + tid * 16) = ar;
+    if (it + 1 < steps) fetch(it + 1);
+    __syncthreads();  // stage `it` is complete; the other stage's readers passed the previous barrier
+    u32x4 a[RS][2];
 #pragma unroll
-    for (int s = 0; s < S; ++s) {
-      const int it = it0 + s;
-      if (it < steps) {  // uniform over the workgroup
-        const int buf = it & 1;
-        u32x4 a0[RS], a1[RS];
+    for (int rs = 0; rs < RS; ++rs)
 #pragma unroll
-        for (int rs = 0; rs < RS; ++rs) a0[rs] = areg[s][rs][0], a1[rs] = areg[s][rs][1];
+      for (int m = 0; m < 2; ++m) a[rs][m] = *reinterpret_cast<const u32x4*>(stage + aread + rs * 2048 + m * 1024);
 #pragma unroll
-        for (int q = 0; q < NT; ++q) {
-          u32x4 lo, hi;  // (k, k+1) pairs for features fc*8 + 0..3 and 4..7
+    for (int m = 0; m < 2; ++m) {
 #pragma unroll
-          for (int d = 0; d < 2; ++d) {
-            lo[2 * d] = __builtin_amdgcn_perm(r1[s][q][d], r0[s][q][d], 0x05040100);      // low halves
-            lo[2 * d + 1] = __builtin_amdgcn_perm(r1[s][q][d], r0[s][q][d], 0x07060302);  // high halves
-            hi[2 * d] = __builtin_amdgcn_perm(r1[s][q][d + 2], r0[s][q][d + 2], 0x05040100);
-            hi[2 * d + 1] = __builtin_amdgcn_perm(r1[s][q][d + 2], r0[s][q][d + 2], 0x07060302);
-          }
-          *reinterpret_cast<u32x4*>(&xs[buf][kp0 + KPT * q][fc * 8]) = lo;
-          *reinterpret_cast<u32x4*>(&xs[buf][kp0 + KPT * q][fc * 8 + 4]) = hi;
-        }
-        if (it + S < steps) fetch(it + S, s);
-        __syncthreads();  // tile `it` is complete; the other buffer's readers passed the previous barrier
+      for (int t = 0; t < NT; ++t) {
+        const char* bp = stage + bread[t] + (4 * m) * FCN * 64;
+        const tr16x4 t0 = __builtin_amdgcn_ds_read_tr16_b64_v4f16((STIR_LDS tr16x4*)(bp));
+        const tr16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4f16((STIR_LDS tr16x4*)(bp + FCN * 64));
+        const u32x2 lo = __builtin_bit_cast(u32x2, t0), hi = __builtin_bit_cast(u32x2, t1);
+        const u32x4 b = {lo[0], lo[1], hi[0], hi[1]};
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const int col = (wave * NT + t) * 32 + n;
-          u32x4 b0, b1;
-#pragma unroll
-          for (int d = 0; d < 4; ++d) {
-            b0[d] = xs[buf][4 * h + d][col];
-            b1[d] = xs[buf][8 + 4 * h + d][col];
-          }
-#pragma unroll
-          for (int rs = 0; rs < RS; ++rs) {
-            acc[rs][t] = mfma32<BF16>(a0[rs], b0, acc[rs][t]);
-            acc[rs][t] = mfma32<BF16>(a1[rs], b1, acc[rs][t]);
-          }
-        }
+        for (int rs = 0; rs < RS; ++rs) acc[rs][t] = mfma32<BF16>(a[rs][m], b, acc[rs][t]);
       }
     }
   }
@@ -193,14 +202,172 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
         const int row = 32 * rs + (v & 3) + 4 * h + 8 * (v >> 2);
         const int64_t off = ((int64_t)i_out * blk + bi0 + row) * feat + fcol + n;
         if constexpr (OUT == 1)
-          static_cast<float*>(Y)[off] = acc[rs][t][v];
+          __builtin_nontemporal_store(acc[rs][t][v], static_cast<float*>(Y) + off);
         else
-          static_cast<uint16_t*>(Y)[off] = to16<BF16>(acc[rs][t][v]);
+          __builtin_nontemporal_store(to16<BF16>(acc[rs][t][v]), static_cast<uint16_t*>(Y) + off);
       }
     }
   }
 }
 
+// One workgroup per tile, 1-D grid (see decode_tile).
+template <bool BF16, int OUT, int NT, int RS>
+__global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles,
+                                                       const uint16_t* __restrict__ A,
+                                                       const uint16_t* __restrict__ X, void* __restrict__ Y,
+                                                       const int32_t* __restrict__ indptr,
+                                                       const int32_t* __restrict__ indices,
+                                                       const int32_t* __restrict__ row_ids) {
+  constexpr int TF = kTileF * NT;
+  __shared__ __attribute__((aligned(16))) char xs[2 * (kTileK * TF * 2 + 2048 * RS)];
+  int64_t slice;
+  int f_tile;
+  if (!decode_tile(blockIdx.x, slices, f_tiles, slice, f_tile)) return;
+  const int sub = blk / (32 * RS);  // slices of 32*RS rows per block row
+  const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * (32 * RS);
+  // doubly-compressed form: stored block row i is block row row_ids[i] of the output
+  const int i_out = row_ids ? row_ids[i] : i;
+  bsr_tile<BF16, OUT, NT, RS>(xs, blk, feat, i, i_out, bi0, f_tile * TF, A, X, Y, indptr, indices);
+}
+
+// ------------------------------------------------------------------ large launches, swept in step
+// When the X rows of one feature tile (nb*blk rows of 256*NT bytes) exceed a per-XCD L2 (4 MB),
+// workgroups that walk their block rows at unrelated times miss L2 on about half of their X
+// tiles.  Block columns are ascending inside a block row, so workgroups that start together on
+// block rows of equal length move through X together and share a narrow window of it.  This
+// kernel arranges that: exactly as many workgroups as are resident at once (gridDim.x = 8 * G,
+// workgroup b runs on XCD b % 8, the dispatch order of the hardware), each a loop over tiles; all
+// workgroups of an XCD work on the same feature tile, and in round r workgroup w of the XCD takes
+// the slice of rank r*G + w when slices are ordered by their number of blocks, longest first.  A
+// round's slices have (nearly) the same length, so no workgroup has to wait for another and the
+// workgroups still stay in step; nothing here synchronises workgroups, the order only decides
+// what L2 holds.  The ranking is computed by every workgroup from indptr before its first tile
+// (a stable counting sort in LDS: every workgroup gets the same permutation).
+constexpr int kSweepMaxSlices = 8192;  // permutation entries are 16 bits wide and live in LDS
+constexpr int kSweepBins = 1024;       // block rows with more blocks than this share the last bin
+constexpr int kSweepMaxItems = 128;    // tiles per workgroup and feature tile
+
+// Calls f(value, lanes holding it) once per distinct value among the lanes with valid = true.
+template <typename F>
+__device__ __forceinline__ void for_each_distinct(int value, bool valid, F f) {
+  uint64_t todo = __ballot(valid);
+  while (todo) {
+    const int src = __ffsll((long long)todo) - 1;
+    const int v = __shfl(value, src, kWave);
+    const uint64_t same = __ballot(valid && value == v);
+    f(v, same);
+    todo &= ~same;
+  }
+}
+
+// Fills items[0 .. count) with the slices this workgroup takes, one per round, for subset
+// `part` of `parts`: ranks (r*G + w)*parts + part.  lds: at least 4*kSweepBins + kSweepMaxSlices/2
+// words, free again when the call returns.
+__device__ __forceinline__ int sweep_my_slices(uint32_t* __restrict__ lds, uint16_t* __restrict__ items,
+                                               const int32_t* __restrict__ indptr, int slices, int sub,
+                                               int G, int w, int parts, int part) {
+  uint32_t* hist = lds;                                                       // [bin][wavefront]
+  uint16_t* perm = reinterpret_cast<uint16_t*>(lds + 4 * kSweepBins);         // [rank] -> slice
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  for (int b = tid; b < 4 * kSweepBins; b += 256) hist[b] = 0;
+  __syncthreads();
+  // wavefront `wave` ranks the contiguous quarter [s_begin, s_end) of the slices
+  const int quarter = ((slices + 3) / 4 + kWave - 1) / kWave * kWave;
+  const int s_begin = wave * quarter, s_end = min(slices, s_begin + quarter);
+  auto bin_of = [&](int s) {
+    const int i = s / sub;
+    const int len = indptr[i + 1] - indptr[i];
+    return kSweepBins - 1 - min(len, kSweepBins - 1);  // longest first
+  };
+  for (int s0 = s_begin; s0 < s_end; s0 += kWave) {
+    const int s = s0 + lane;
+    const bool valid = s < s_end;
+    const int bin = valid ? bin_of(s) : 0;
+    for_each_distinct(bin, valid, [&](int v, uint64_t same) {
+      if (lane == 0) hist[v * 4 + wave] += (uint32_t)__popcll(same);
+    });
+  }
+  __syncthreads();
+  // exclusive scan over hist in (bin, wavefront) order: 16 consecutive entries per thread
+  {
+    uint32_t local[16], sum = 0;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) local[q] = hist[tid * 16 + q], sum += local[q];
+    uint32_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const uint32_t up = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += up;
+    }
+    __shared__ uint32_t wave_total[4];
+    if (lane == kWave - 1) wave_total[wave] = incl;
+    __syncthreads();
+    uint32_t base = incl - sum;
+    for (int q = 0; q < wave; ++q) base += wave_total[q];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) hist[tid * 16 + q] = base, base += local[q];
+  }
+  __syncthreads();
+  // placement, in slice order inside every (bin, wavefront) run: stable
+  for (int s0 = s_begin; s0 < s_end; s0 += kWave) {
+    const int s = s0 + lane;
+    const bool valid = s < s_end;
+    const int bin = valid ? bin_of(s) : 0;
+    for_each_distinct(bin, valid, [&](int v, uint64_t same) {
+      const uint32_t first = hist[v * 4 + wave];
+      if (valid && bin == v) perm[first + __popcll(same & ((uint64_t(1) << lane) - 1))] = (uint16_t)s;
+      __builtin_amdgcn_wave_barrier();
+      if (lane == 0) hist[v * 4 + wave] = first + (uint32_t)__popcll(same);
+      __builtin_amdgcn_wave_barrier();
+    });
+  }
+  __syncthreads();
+  int count = 0;
+  for (int r = 0;; ++r) {
+    const int64_t rank = ((int64_t)r * G + w) * parts + part;
+    if (rank >= slices || r >= kSweepMaxItems) break;
+    if (tid == 0) items[r] = perm[rank];
+    ++count;
+  }
+  __syncthreads();
+  return count;
+}
+
+template <bool BF16, int OUT, int NT, int RS>
+__global__ __launch_bounds__(256) void bsr_spmm_sweep_kernel(int blk, int feat, int slices, int f_tiles, int parts,
+                                                             const uint16_t* __restrict__ A,
+                                                             const uint16_t* __restrict__ X, void* __restrict__ Y,
+                                                             const int32_t* __restrict__ indptr,
+                                                             const int32_t* __restrict__ indices,
+                                                             const int32_t* __restrict__ row_ids) {
+  constexpr int TF = kTileF * NT;
+  constexpr int kXsWords = 2 * (kTileK * TF * 2 + 2048 * RS) / 4;
+  constexpr int kSortWords = 4 * kSweepBins + kSweepMaxSlices / 2;
+  __shared__ __attribute__((aligned(16))) uint32_t lds[kXsWords > kSortWords ? kXsWords : kSortWords];
+  __shared__ uint16_t items[kSweepMaxItems];
+  const int xcd = blockIdx.x & 7, w = blockIdx.x >> 3, G = gridDim.x >> 3;
+  const int sub = blk / (32 * RS);
+  // unit u = f_tile + f_tiles * part (part: every parts-th slice by rank); XCD x takes units x, x + 8, ...
+  const int units = f_tiles * parts;
+  int part_of_items = -1, count = 0;
+  for (int u = xcd; u < units; u += 8) {
+    const int f_tile = u % f_tiles, part = u / f_tiles;
+    if (part != part_of_items) {
+      __syncthreads();  // the last tile's LDS reads are over
+      count = sweep_my_slices(lds, items, indptr, slices, sub, G, w, parts, part);
+      part_of_items = part;
+    }
+    for (int r = 0; r < count; ++r) {
+      const int slice = items[r];
+      const int i = slice / sub, bi0 = (slice % sub) * (32 * RS);
+      const int i_out = row_ids ? row_ids[i] : i;
+      __syncthreads();  // the previous tile's readers are done with both LDS buffers
+      bsr_tile<BF16, OUT, NT, RS>(reinterpret_cast<char*>(lds), blk, feat, i, i_out, bi0, f_tile * TF, A, X, Y,
+                                  indptr, indices);
+    }
+  }
+}
 
 // Small launches (at most a couple of workgroups per CU): a workgroup's run time is the serial
 // chain of its block row's steps, each a memory round trip, and nothing else is resident to hide
@@ -367,22 +534,51 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   }
   // Two 32-wide accumulators per wavefront once the feature axis is wide enough to still yield
   // several workgroups per CU.  One prefetched step is enough: measured on MI355X, deeper
-  // register rings (2-6 steps) change nothing, the kernel is bound by the traffic that misses
-  // the per-XCD L2, not by latency.
+  // register rings (2-6 steps) change nothing, the kernel is not bound by latency.
   const int nt = (feat >= 1024) ? 2 : 1;
   const int f_tiles = (int)stir::ceil_div(feat, kTileF * nt);
+  dim3 block(256);
+  // Launches whose X rows per feature tile do not fit a per-XCD L2 and that give every resident
+  // workgroup several tiles are swept in step (bsr_spmm_sweep_kernel).
+  const int cus = stir::compute_units();
+  const int64_t x_tile_bytes = (int64_t)nb * blk * kTileF * nt * 2;
+  const int parts = 8 / std::gcd(f_tiles, 8);
+#define STIR_BSR_SWEEP(BF, OUT, NTV, RSV)                                                                     \
+  {                                                                                                           \
+    static int occupancy = 0; /* workgroups of this kernel per CU; the same on every gfx950 device */        \
+    if (occupancy == 0) {                                                                                     \
+      int o = 0;                                                                                              \
+      STIR_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, bsr_spmm_sweep_kernel<BF, OUT, NTV, RSV>, 256, 0)); \
+      occupancy = o > 0 ? o : 1;                                                                              \
+    }                                                                                                         \
+    const int G = occupancy * (cus / 8);                                                                      \
+    const int64_t rounds = stir::ceil_div(stir::ceil_div(slices, parts), G);                                  \
+    if (rounds <= kSweepMaxItems && slices * f_tiles >= 4 * 8 * (int64_t)G) {                                 \
+      hipLaunchKernelGGL((bsr_spmm_sweep_kernel<BF, OUT, NTV, RSV>), dim3(8 * G), block, 0, st, blk, feat,    \
+                         (int)slices, f_tiles, parts, A, X, d_Y, d_indptr, d_indices, d_row_ids);             \
+      STIR_LAUNCH_CHECK();                                                                                    \
+      return 0;                                                                                               \
+    }                                                                                                         \
+  }
+  // (measured: 16384^2, 32x32 blocks, 10 %, 4096 features 650 -> 590 us, L2 hit rate 46 -> 57 %;
+  // with fewer than 8 feature tiles or two slices per workgroup the plain order is faster)
+  const bool sweep = cus >= 8 && cus % 8 == 0 && rs == 1 && f_tiles >= 8 && x_tile_bytes > (3 << 20) &&
+                     slices <= kSweepMaxSlices;
   const int64_t blocks = f_tiles >= 8 ? 8 * stir::ceil_div(f_tiles, 8) * slices : (int64_t)f_tiles * slices;
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "bsr_spmm: too many tiles for one launch");
-  dim3 grid((unsigned)blocks), block(256);
+  dim3 grid((unsigned)blocks);
 #define STIR_BSR_L(BF, OUT, NTV, RSV)                                                                      \
-  hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, 1, RSV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
-                     A, X, d_Y, d_indptr, d_indices, d_row_ids)
+  {                                                                                                        \
+    if (sweep) STIR_BSR_SWEEP(BF, OUT, NTV, RSV);                                                          \
+    hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, RSV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
+                       A, X, d_Y, d_indptr, d_indices, d_row_ids);                                         \
+  }
 #define STIR_BSR(BF, OUT)                                                          \
   do {                                                                             \
     if (nt == 2) {                                                                 \
-      if (rs == 2) STIR_BSR_L(BF, OUT, 2, 2); else STIR_BSR_L(BF, OUT, 2, 1);      \
+      if (rs == 2) STIR_BSR_L(BF, OUT, 2, 2) else STIR_BSR_L(BF, OUT, 2, 1)        \
     } else {                                                                       \
-      if (rs == 2) STIR_BSR_L(BF, OUT, 1, 2); else STIR_BSR_L(BF, OUT, 1, 1);      \
+      if (rs == 2) STIR_BSR_L(BF, OUT, 1, 2) else STIR_BSR_L(BF, OUT, 1, 1)        \
     }                                                                              \
   } while (0)
   if (dtype == STIR_BF16) {
@@ -392,6 +588,7 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   }
 #undef STIR_BSR
 #undef STIR_BSR_L
+#undef STIR_BSR_SWEEP
   STIR_LAUNCH_CHECK();
   return 0;
 }

@@ -93,6 +93,57 @@ def test_bsr_many_workgroups(dev, mb, nb, blk, feat, dtype):
     _check(got, cfg, a32, x32, True, f"mb={mb} blk={blk} feat={feat} {dtype}")
 
 
+@pytest.mark.parametrize("dtype,out32,varied", [(torch.float16, False, False), (torch.bfloat16, True, True)])
+def test_bsr_launch_swept_in_step(dev, dtype, out32, varied):
+    """A launch large enough for the kernel in which as many workgroups as are resident loop over
+    tiles, every workgroup ranking the block rows by length on its own (X rows of one feature tile
+    beyond 3 MB, at least 8 feature tiles, several tiles per resident workgroup).  Every block row
+    must be computed exactly once: compared on the GPU against the same sum formed block by block in
+    fp32 by torch, for all rows.  `varied`: block rows of very different lengths, empty ones and
+    one beyond the 1024 length classes of the ranking."""
+    mb, nb, blk, feat = 1100, 208, 32, 2048
+    rng = np.random.default_rng(17)
+    if varied:
+        nb = 1300
+        dens = rng.choice([0.0, 0.002, 0.01, 0.03], size=mb)
+        present = rng.random((mb, nb)) < dens[:, None]
+        present[7, :] = True         # 1300 blocks: the last length class
+        present[8, :1023] = True
+        present[9, :1024] = True
+    else:
+        present = rng.random((mb, nb)) < 0.05
+    indptr = np.zeros(mb + 1, np.int32)
+    np.cumsum(present.sum(axis=1), out=indptr[1:])
+    indices = np.nonzero(present)[1].astype(np.int32)
+    nnzb = len(indices)
+    assert nb * blk * 256 * 2 > 3 << 20 and feat // 256 >= 8
+    gen = torch.Generator(device=dev).manual_seed(3)
+    a = (torch.randn(nnzb * blk * blk, device=dev, generator=gen) * 0.02).to(dtype)
+    x = torch.randn(nb * blk * feat, device=dev, generator=gen).to(dtype)
+    od = torch.float32 if out32 else dtype
+    y = torch.full((mb * blk * feat,), float("nan"), dtype=od, device=dev)
+    d_ptr, d_idx = torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev)
+    ops.build_bsrmm(mb, nb, nnzb, blk, feat, dtype, od)(a, x, y, d_ptr, d_idx)
+    torch.cuda.synchronize()
+    # reference: per stored block one fp32 product, summed per block row (index_add), in chunks
+    rows_of = torch.repeat_interleave(torch.arange(mb, device=dev), torch.from_numpy(np.diff(indptr)).to(dev))
+    want = torch.zeros(mb, blk, feat, device=dev)
+    scale = torch.zeros(mb, blk, feat, device=dev)
+    a3, x3 = a.view(nnzb, blk, blk).float(), x.view(nb, blk, feat).float()
+    for lo in range(0, nnzb, 2048):
+        hi = min(nnzb, lo + 2048)
+        xb = x3[d_idx[lo:hi].long()]
+        want.index_add_(0, rows_of[lo:hi], torch.bmm(a3[lo:hi], xb))
+        scale.index_add_(0, rows_of[lo:hi], torch.bmm(a3[lo:hi].abs(), xb.abs()))
+    got = y.view(mb, blk, feat).float()
+    bound = 2e-5 * scale + (0.0 if out32 else RTOL * want.abs()) + 1e-30
+    bad = (got - want).abs() > bound
+    assert not bool(bad.any()), f"{int(bad.sum())} elements off, rows {torch.nonzero(bad.any(2).any(1))[:8].ravel().tolist()}"
+    # a block row without blocks is written as zeros
+    empty = torch.from_numpy(np.diff(indptr) == 0).to(dev)
+    assert bool((got[empty] == 0).all())
+
+
 def test_bsr_rejects_unsupported(dev):
     z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
     f = ops.build_bsrmm(1, 1, 1, 16, 32)
