@@ -15,24 +15,76 @@ prices the same kernel against HBM bandwidth with the algorithmic byte count
 8*nnz + 4*(m+1) + 4*n*feat + 4*m*feat (indices and values once, X once, Y once) and the
 per-launch duration measured with HIP events on the launch stream.  `cpu_baseline` times the
 C restatement of the reference's unscheduled CPU loop nest on one host core over a bounded
-row sample of the same graph.  `extra` carries the CSR row-split comparator and SDDMM.
+row sample of the same graph.  `extra` carries the same kernel on the graph with power-law
+columns (its own roofline block), the CSR row-split comparator, SDDMM, BSR, RGMS, TC-SpMM and the
+host format passes.  Small kernels are timed three ways: `us_per_call` (events around every call:
+what a Python caller sees, launch overhead included), `us_back_to_back` (one event pair around a
+run of calls) and `us_graph` (a captured HIP graph of 20 launches replayed: device time only,
+the figure a rocprofv3 kernel trace shows).
+
+Exit status 3 when a correctness check of the first call fails (the JSON line is still printed).
 """
 import argparse
+import ctypes
+import glob
+import hashlib
 import json
 import os
+import re
+import subprocess
 import sys
 import time
 
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; scaled by a
-# plain copy of known size), keyed by workload signature.  None when not measured.
-MEASURED_TRAFFIC = {
-    # profiles/hyb_spmm_config3_uniform.md: FETCH_SIZE 15,737,890 KiB x 2.0 + WRITE_SIZE 1,266,963 KiB x 1.0
-    "uniform/p1/b1-2-4-8-16-32-64-128-256-512/f128/s1.0": 33.53e9,
-}
+# ---- bandwidth probes: a small library of this benchmark's own (bench_probes.hip), not part of
+# the product library
+PROBES_SRC = os.path.join(ROOT, "bench_probes.hip")
+PROBES_LIB = os.path.join(ROOT, "libbench_probes.so")
+
+
+def build_probes():
+    cmd = [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "-O3", "-std=c++17", "-fPIC", "-shared",
+           "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-x", "hip", PROBES_SRC, "-o", PROBES_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on bench_probes.hip:\n" + r.stdout + r.stderr)
+    return PROBES_LIB
+
+
+def load_probes():
+    if not os.path.exists(PROBES_LIB):
+        build_probes()
+    L = ctypes.CDLL(PROBES_LIB)
+    VP, I64, I32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
+    L.bench_probe_copy.restype, L.bench_probe_copy.argtypes = I32, [VP, VP, I64, VP]
+    L.bench_probe_gather.restype, L.bench_probe_gather.argtypes = I32, [VP, I64, I32, I64, VP, VP]
+    return L
+
+
+def measured_traffic(workload):
+    """HBM-side bytes per launch of the headline kernel as measured with rocprofv3 --pmc
+    (FETCH_SIZE, WRITE_SIZE, scaled by a plain copy of known size).  The summaries under
+    profiles/ carry one line per measured workload,
+        traffic-bytes-per-launch: workload=<signature> bytes=<float> kernel-source-sha1=<sha1>
+    where the sha1 is that of sparsetir_amd/csrc/spmm.hip when the counters were taken.  Returns
+    (bytes, note); bytes is None when nothing was measured for this workload or the kernel source
+    has changed since."""
+    with open(os.path.join(ROOT, "sparsetir_amd", "csrc", "spmm.hip"), "rb") as f:
+        now = hashlib.sha1(f.read()).hexdigest()
+    pat = re.compile(r"traffic-bytes-per-launch:\s+workload=(\S+)\s+bytes=(\S+)\s+kernel-source-sha1=(\w+)")
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        for line in open(path):
+            mt = pat.search(line)
+            if mt and mt.group(1) == workload:
+                if mt.group(3) != now:
+                    return None, f"stale: spmm.hip changed since {os.path.basename(path)} was taken"
+                return float(mt.group(2)), os.path.basename(path)
+    return None, "not measured for this workload"
 
 
 def parse():
@@ -75,6 +127,40 @@ def time_steps(fn, steps, warmup, torch):
     return wall, float(np.mean(dev_ms)) / 1e3, float(np.min(dev_ms)) / 1e3
 
 
+def time_small(fn, calls, warmup, torch, graph=True):
+    """Three timings of a short kernel, in microseconds: events around every call, one event pair
+    around a run of calls, and a captured graph of 20 launches replayed (device time only)."""
+    _, per_call, _ = time_steps(fn, calls, warmup, torch)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(calls):
+        fn()
+    e1.record()
+    e1.synchronize()
+    out = {"us_per_call": per_call * 1e6, "us_back_to_back": e0.elapsed_time(e1) * 1e3 / calls}
+    if graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()  # plans are complete before capture begins
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(20):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            g.replay()
+        e1.record()
+        e1.synchronize()
+        out["us_graph"] = e0.elapsed_time(e1) * 1e3 / 100
+        del g
+    return out
+
+
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
@@ -107,11 +193,12 @@ def config2_sweep(torch, dev, ops, st, datasets, time_steps):
 
 
 def side_kernels(torch, dev, ops, st, datasets, time_steps):
-    """BSR SpMM (config 4 and a scaled-up shape) and RGMS (config 5): time, flop rate against the
-    dense fp16 MFMA peak, algorithmic bytes against the HBM peak."""
+    """BSR SpMM (config 4 and scaled-up shapes), RGMS (config 5), TC-SpMM and the host format
+    passes: time, flop rate against the dense fp16 MFMA peak, algorithmic bytes against the HBM
+    peak.  Rates use the back-to-back time; see time_small for the three timings."""
     out = {}
 
-    def bsr(tag, mb, nb, blk, density, feat, dtype):
+    def bsr(tag, mb, nb, blk, density, feat, dtype, calls=100):
         cfg = datasets.config4(seed=3, mb=mb, nb=nb, blk=blk, density=density, feat=32)
         nnzb = len(cfg["indices"])
         a = torch.from_numpy(cfg["data"]).to(dev).to(dtype).reshape(-1)
@@ -119,23 +206,35 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
         y = torch.zeros(mb * blk * feat, device=dev, dtype=dtype)
         ip, ix = torch.from_numpy(cfg["indptr"]).to(dev), torch.from_numpy(cfg["indices"]).to(dev)
         f = ops.build_bsrmm(mb, nb, nnzb, blk, feat, dtype)
-        _, d, _ = time_steps(lambda: f(a, x, y, ip, ix), 100, 5, torch)
+        tm = time_small(lambda: f(a, x, y, ip, ix), calls, 5, torch)
+        d = tm["us_back_to_back"] / 1e6
         flops = 2.0 * nnzb * blk * blk * feat
         byts = 2.0 * nnzb * blk * blk + 4 * nnzb + 4 * (mb + 1) + 2.0 * nb * blk * feat + 2.0 * mb * blk * feat
-        out[tag] = {"us": d * 1e6, "tflops": flops / d / 1e12, "frac_of_mfma_peak": flops / d / 1e12 / MFMA_F16_PEAK_TFLOPS,
-                    "alg_GBps": byts / d / 1e9, "frac_of_hbm_peak": byts / d / 1e9 / HBM_PEAK_GBS,
-                    "nnzb": nnzb, "shape": [mb * blk, nb * blk, feat], "blk": blk, "dtype": str(dtype).split(".")[-1]}
+        out[tag] = dict(tm, us=d * 1e6, tflops=flops / d / 1e12,
+                        frac_of_mfma_peak=flops / d / 1e12 / MFMA_F16_PEAK_TFLOPS, alg_GBps=byts / d / 1e9,
+                        frac_of_hbm_peak=byts / d / 1e9 / HBM_PEAK_GBS, nnzb=nnzb,
+                        shape=[mb * blk, nb * blk, feat], blk=blk, dtype=str(dtype).split(".")[-1])
 
     bsr("bsr_config4_f16", 128, 128, 32, 0.10, 512, torch.float16)
     bsr("bsr_config4_bf16", 128, 128, 32, 0.10, 512, torch.bfloat16)
-    bsr("bsr_16384x16384_f4096_f16", 512, 512, 32, 0.10, 4096, torch.float16)
+    bsr("bsr_16384x16384_f4096_f16", 512, 512, 32, 0.10, 4096, torch.float16, calls=20)
+    bsr("bsr_16384x16384_blk64_f4096_f16", 256, 256, 64, 0.10, 4096, torch.float16, calls=20)
+    bsr("bsr_16384x16384_blk128_f4096_f16", 128, 128, 128, 0.10, 4096, torch.float16, calls=20)
 
     cfg = datasets.config5()
     R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
     buckets, group = cfg["buckets"], 256
     rb = [group // b for b in buckets]
-    ptr, rows, cols, mask = st.csf_to_ell3d(cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"],
-                                            rb, buckets)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    E = len(cfg["indices1"])
+    st.csf_to_ell3d(*csf, rb, buckets)  # first call: page faults of the output arrays
+    t0 = time.perf_counter()
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    fmt_s = time.perf_counter() - t0
+    slots5 = int(sum(c.size for c in cols))
+    out["csf_to_ell3d_config5_host"] = {"ms": fmt_s * 1e3, "edges": E, "slots": slots5, "threads": 1,
+                                        "alg_GBps": (8.0 * E + 4.0 * sum(r.size for r in rows) + 8.0 * slots5)
+                                        / fmt_s / 1e9}
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     triples, mids = [], []
     for k in range(len(buckets)):
@@ -145,26 +244,37 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     w = t(cfg["w"].astype(np.float16).ravel())
     x = t(cfg["x"].astype(np.float16).ravel())
     y = torch.zeros(n * fout, device=dev)
-    _, d, _ = time_steps(lambda: f(w, x, y, *triples, *mids), 10, 1, torch)
-    E = len(cfg["indices1"])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    f(w, x, y, *triples, *mids)   # the first launch of a plan builds its edge index
+    torch.cuda.synchronize()
+    first_s = time.perf_counter() - t0
+    tm = time_small(lambda: f(w, x, y, *triples, *mids), 50, 3, torch)
+    d = tm["us_back_to_back"] / 1e6
     flops = 2.0 * E * fin * fout + 2.0 * E * fout
     byts = 8.0 * E + 2.0 * n * fin + 2.0 * R * fin * fout + 4.0 * n * fout
-    out["rgms_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts / d / 1e9,
-                           "frac_of_hbm_peak": byts / d / 1e9 / HBM_PEAK_GBS, "edges": E,
-                           "ell_rows": int(sum(r.size for r in rows)),
-                           "accumulation": "32-row output tiles, written once (no atomics)"}
+    out["rgms_config5"] = dict(tm, us=d * 1e6, first_call_ms=first_s * 1e3, tflops=flops / d / 1e12,
+                               alg_GBps=byts / d / 1e9, frac_of_hbm_peak=byts / d / 1e9 / HBM_PEAK_GBS, edges=E,
+                               ell_rows=int(sum(r.size for r in rows)),
+                               accumulation="32-row output tiles, written once (no atomics)")
 
     # SpMM over the condensed format (t = 32, g = 16) on the config-2 graph, fp16 in, fp32 out
     g2 = datasets.config2()
+    st.condense(g2["indptr"], g2["indices"], 32, 16)
+    t0 = time.perf_counter()
     gptr, tiles, cmask = st.condense(g2["indptr"], g2["indices"], 32, 16)
+    fmt_s = time.perf_counter() - t0
+    out["condense_config2_host"] = {"ms": fmt_s * 1e3, "edges": int(len(g2["indices"])), "groups": int(tiles.shape[0]),
+                                    "threads": 1}
     mb2, nnzb2, f2 = len(gptr) - 1, tiles.shape[0], 128
     tc = ops.build_tcspmm(mb2, nnzb2, f2, 32, 16, g2["n"], torch.float32)
     a2, b2 = t(cmask.astype(np.float16).ravel()), torch.randn(g2["n"] * f2, device=dev).half()
     c2 = torch.zeros(mb2 * 32 * f2, device=dev)
     gp, ti = t(gptr), t(tiles.ravel())
-    _, d, _ = time_steps(lambda: tc(a2, b2, c2, gp, ti), 50, 5, torch)
+    tm = time_small(lambda: tc(a2, b2, c2, gp, ti), 50, 5, torch)
+    d = tm["us_back_to_back"] / 1e6
     nnz2 = len(g2["indices"])
-    out["tcspmm_config2_feat128"] = {"us": d * 1e6, "useful_gflops": 2.0 * nnz2 * f2 / d / 1e9,
+    out["tcspmm_config2_feat128"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "useful_gflops": 2.0 * nnz2 * f2 / d / 1e9,
                                      "mfma_tflops": 2.0 * nnzb2 * 32 * 16 * f2 / d / 1e12, "groups": int(nnzb2),
                                      "mask_density": float(nnz2) / (nnzb2 * 32 * 16)}
 
@@ -181,46 +291,33 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
         triples += [t(mask[k].astype(np.float32).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
         mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
     f32 = ops.build_rgms_f32(n, n, R, fin, fout, rb32, buckets, [c.shape[0] for c in cols])
-    _, d, _ = time_steps(lambda: f32(w32, x32, y, *triples, *mids), 10, 1, torch)
-    out["rgms_f32_ell3d_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
+    tm = time_small(lambda: f32(w32, x32, y, *triples, *mids), 20, 2, torch)
+    d = tm["us_back_to_back"] / 1e6
+    out["rgms_f32_ell3d_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
                                      "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
                                      "ell_rows": int(sum(r.size for r in rows))}
     csf = [t(cfg[k]) for k in ("indptr0", "indices0", "indptr1", "indices1")]
     ones = torch.ones(E, device=dev)
     fc = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E)
-    _, d, _ = time_steps(lambda: fc(ones, w32, x32, y, *csf), 10, 1, torch)
-    out["rgms_f32_csf_config5"] = {"us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
+    tm = time_small(lambda: fc(ones, w32, x32, y, *csf), 20, 2, torch)
+    d = tm["us_back_to_back"] / 1e6
+    out["rgms_f32_csf_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
                                    "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
                                    "stored_rows": int(len(cfg["indices0"]))}
     return out
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported: this build has no "
-              "multi-GPU path (the kernel runs on one GPU's share at its real shape).", file=sys.stderr)
-        sys.exit(2)
-    import torch
-    import sparsetir_amd as st
-    from sparsetir_amd import datasets, ops
-
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(1)
-    dev = torch.device("cuda:0")
-    feat = args.feat
-
+def hyb_workload(args, columns, torch, dev, st, datasets, ops):
+    """Graph, device format pass and operators of config 3 with the given column distribution."""
     t0 = time.time()
-    g = datasets.config3(columns=args.columns, scale=args.scale)
+    g = datasets.config3(columns=columns, scale=args.scale)
     m, n = g["m"], g["n"]
     indptr, indices = g["indptr"], g["indices"]
     nnz = int(indices.shape[0])
     parts = args.parts if args.parts is not None else g["num_col_parts"]
     buckets = [int(b) for b in args.buckets.split(",")] if args.buckets else g["buckets"]
-    log(f"[bench] graph: {m} nodes, {nnz} edges, max degree {int(np.diff(indptr).max())} "
+    log(f"[bench] graph ({columns} columns): {m} nodes, {nnz} edges, max degree {int(np.diff(indptr).max())} "
         f"({time.time() - t0:.1f}s); hyb: {parts} column partitions, widths {buckets}")
-
     d_indptr = torch.from_numpy(indptr).to(dev)
     d_indices = torch.from_numpy(indices).to(dev)
     torch.cuda.synchronize()
@@ -242,29 +339,80 @@ def main():
     del mask
     log(f"[bench] device column_part_hyb: {fmt_s * 1e3:.1f} ms, {sum(nrows)} ELL rows, "
         f"{slots} slots ({slots / nnz:.3f} per edge)")
-
+    feat = args.feat
     gen = torch.Generator(device=dev)
     gen.manual_seed(2)
     x = torch.randn(n * feat, generator=gen, device=dev, dtype=torch.float32)
     c = torch.zeros(m * feat, device=dev, dtype=torch.float32)
     hyb = ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)
+    csr = ops.build_csrmm(m, n, feat, nnz)
+    sig = f"{columns}/p{parts}/b{'-'.join(map(str, buckets))}/f{feat}/s{args.scale}"
+    return dict(m=m, n=n, nnz=nnz, indptr=indptr, indices=indices, d_indptr=d_indptr, d_indices=d_indices,
+                parts=parts, buckets=buckets, triples=triples, nrows=nrows, slots=slots, fmt_s=fmt_s,
+                fmt_first_s=fmt_first_s, x=x, c=c, hyb=hyb, csr=csr, gen=gen, sig=sig, feat=feat)
+
+
+def check_first_call(wl, torch, dev):
+    """hyb against the CSR kernel on every element of the first call's output."""
+    m, feat, nnz = wl["m"], wl["feat"], wl["nnz"]
+    wl["c"].zero_()
+    wl["hyb"](wl["x"], wl["c"], *wl["triples"])
+    ones = torch.ones(nnz, device=dev, dtype=torch.float32)
+    c_csr = torch.empty(m * feat, device=dev, dtype=torch.float32)
+    wl["csr"](ones, wl["x"], c_csr, wl["d_indptr"], wl["d_indices"])
+    torch.cuda.synchronize()
+    deg = torch.from_numpy(np.diff(wl["indptr"]).astype(np.float32)).to(dev)
+    # |x| <~ 6 for N(0,1): bound the summed magnitude by deg * 6
+    tol = 1e-5 * (deg.clamp(min=1.0) * 6.0).repeat_interleave(feat)
+    diff = (wl["c"] - c_csr).abs()
+    ok = bool((diff <= tol).all().item())
+    worst = float(diff.max().item())
+    log(f"[bench] hyb vs csr kernel: max |diff| {worst:.3e}, within tolerance: {ok}")
+    return ok, worst, ones, c_csr
+
+
+def roofline_block(wl, dev_mean, dev_min, probes=None):
+    m, n, nnz, feat, slots = wl["m"], wl["n"], wl["nnz"], wl["feat"], wl["slots"]
+    alg_bytes = 8.0 * nnz + 4.0 * (m + 1) + 4.0 * n * feat + 4.0 * m * feat
+    achieved = alg_bytes / dev_mean / 1e9
+    traffic, note = measured_traffic(wl["sig"])
+    blk = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+           "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": note,
+           "kernel": "hyb_spmm_kernel<32,1>" if feat == 128 else "hyb_spmm_kernel",
+           "kernel_ms_mean": dev_mean * 1e3, "kernel_ms_min": dev_min * 1e3,
+           "algorithmic_bytes": alg_bytes,
+           "traffic_GBps": traffic / dev_mean / 1e9 if traffic else None,
+           "uncached_gather_bytes": 4.0 * slots * feat + 8.0 * slots + 4.0 * m * feat}
+    if probes is not None:
+        blk["probes"] = probes
+    return blk, alg_bytes
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported: this build has no "
+              "multi-GPU path (the kernel runs on one GPU's share at its real shape).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import sparsetir_amd as st
+    from sparsetir_amd import datasets, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    feat = args.feat
+
+    wl = hyb_workload(args, args.columns, torch, dev, st, datasets, ops)
+    m, n, nnz = wl["m"], wl["n"], wl["nnz"]
+    indptr, indices = wl["indptr"], wl["indices"]
+    x, c, hyb, csr, triples = wl["x"], wl["c"], wl["hyb"], wl["csr"], wl["triples"]
+    d_indptr, d_indices = wl["d_indptr"], wl["d_indices"]
 
     # ---- correctness of the first call: against the CSR kernel everywhere, and against the
     # CPU oracle on a row sample
-    hyb(x, c, *triples)
-    ones = torch.ones(nnz, device=dev, dtype=torch.float32)
-    c_csr = torch.empty(m * feat, device=dev, dtype=torch.float32)
-    csr = ops.build_csrmm(m, n, feat, nnz)
-    csr(ones, x, c_csr, d_indptr, d_indices)
-    torch.cuda.synchronize()
-    deg = torch.from_numpy(np.diff(indptr).astype(np.float32)).to(dev)
-    # |x| <~ 6 for N(0,1): bound the summed magnitude by deg * 6
-    tol = 1e-5 * (deg.clamp(min=1.0) * 6.0).repeat_interleave(feat)
-    diff = (c - c_csr).abs()
-    hyb_vs_csr_ok = bool((diff <= tol).all().item())
-    max_diff = float(diff.max().item())
-    log(f"[bench] hyb vs csr kernel: max |diff| {max_diff:.3e}, within tolerance: {hyb_vs_csr_ok}")
-
+    hyb_vs_csr_ok, max_diff, ones, c_csr = check_first_call(wl, torch, dev)
     check = {"hyb_vs_csr_max_abs_diff": max_diff, "hyb_vs_csr_ok": hyb_vs_csr_ok}
     cpu = None
     if not args.no_cpu:
@@ -294,16 +442,19 @@ def main():
     # Probes: a plain copy of known size (n*feat*4 bytes read and written; also the kernel the
     # FETCH_SIZE / WRITE_SIZE counters are scaled by under rocprofv3 --pmc) and nnz gathers of
     # feat*4-byte rows at pseudo-random indices (what the access pattern allows at best).
-    import ctypes
-    from sparsetir_amd import _lib
-    L = _lib.lib()
+    P = load_probes()
     vp = lambda t: ctypes.c_void_p(t.data_ptr())
     st0 = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     nbytes = (n * feat * 4) // 16 * 16
-    _, copy_s, _ = time_steps(lambda: _lib.check(L.stir_probe_copy(vp(x), vp(c_csr), nbytes, st0)), 3, 1, torch)
+
+    def probe(rc):
+        if rc != 0:
+            raise RuntimeError("bandwidth probe failed")
+
+    _, copy_s, _ = time_steps(lambda: probe(P.bench_probe_copy(vp(x), vp(c_csr), nbytes, st0)), 3, 1, torch)
     probes = {"copy_GBps": 2.0 * nbytes / copy_s / 1e9}
     if feat in (32, 64, 128, 256):
-        _, gat_s, _ = time_steps(lambda: _lib.check(L.stir_probe_gather(vp(x), n, feat, nnz, vp(c_csr), st0)),
+        _, gat_s, _ = time_steps(lambda: probe(P.bench_probe_gather(vp(x), n, feat, nnz, vp(c_csr), st0)),
                                  3, 1, torch)
         probes["random_row_gather_GBps"] = nnz * feat * 4.0 / gat_s / 1e9
     log(f"[bench] probes: {probes}")
@@ -311,9 +462,7 @@ def main():
     # ---- timed region
     wall, dev_mean, dev_min = time_steps(lambda: hyb(x, c, *triples), args.steps, args.warmup, torch)
     flops = 2.0 * nnz * feat
-    alg_bytes = 8.0 * nnz + 4.0 * (m + 1) + 4.0 * n * feat + 4.0 * m * feat
-    achieved = alg_bytes / dev_mean / 1e9
-    sig = f"{args.columns}/p{parts}/b{'-'.join(map(str, buckets))}/f{feat}/s{args.scale}"
+    roof, alg_bytes = roofline_block(wl, dev_mean, dev_min, probes)
     result = {
         "metric": "hyb SpMM GFLOP/s (fp32, feat %d, power-law graph %d nodes / %d edges)" % (feat, m, nnz),
         "value": flops / wall / 1e9,
@@ -329,16 +478,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": "config 3: hyb SpMM fp32, 2.45M-node / 61.9M-edge power-law graph, feat 128",
                    "nodes": m, "edges": nnz, "feat": feat, "columns": args.columns,
-                   "num_col_parts": parts, "buckets": buckets, "ell_slots": slots,
-                   "format_pass_ms": fmt_s * 1e3, "format_pass_first_call_ms": fmt_first_s * 1e3,
-                   "format_pass_alg_GBps": (4.0 * (m + 1) + 4.0 * nnz + 4.0 * (sum(nrows) + 2 * slots)) / fmt_s / 1e9},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(sig),
-                     "kernel": "hyb_spmm_kernel<32,1>" if feat == 128 else "hyb_spmm_kernel",
-                     "kernel_ms_mean": dev_mean * 1e3, "kernel_ms_min": dev_min * 1e3,
-                     "algorithmic_bytes": alg_bytes, "probes": probes,
-                     "traffic_GBps": (MEASURED_TRAFFIC.get(sig) or 0) / dev_mean / 1e9 or None,
-                     "uncached_gather_bytes": 4.0 * slots * feat + 8.0 * slots + 4.0 * m * feat},
+                   "num_col_parts": wl["parts"], "buckets": wl["buckets"], "ell_slots": wl["slots"],
+                   "format_pass_ms": wl["fmt_s"] * 1e3, "format_pass_first_call_ms": wl["fmt_first_s"] * 1e3,
+                   "format_pass_alg_GBps": (4.0 * (m + 1) + 4.0 * nnz + 4.0 * (sum(wl["nrows"]) + 2 * wl["slots"]))
+                   / wl["fmt_s"] / 1e9},
+        "roofline": roof,
         "cpu_baseline": cpu,
         "check": check,
     }
@@ -350,6 +494,7 @@ def main():
         extra["csr_spmm"] = {"gflops": flops / w2 / 1e9, "ms": d2 * 1e3, "alg_GBps": alg_bytes / d2 / 1e9}
         del c_csr, ones
         f2 = 64
+        gen = wl["gen"]
         a2 = torch.randn(m * f2, generator=gen, device=dev, dtype=torch.float32)
         b2 = torch.randn(n * f2, generator=gen, device=dev, dtype=torch.float32)
         out = torch.empty(nnz, device=dev, dtype=torch.float32)
@@ -366,13 +511,39 @@ def main():
                                         "alg_GBps": sd_bytes / d4 / 1e9,
                                         "frac_of_hbm_peak": sd_bytes / d4 / 1e9 / HBM_PEAK_GBS,
                                         "preproc_ms": d3 * 1e3}
-        del edge
-        del a2, b2, out, mid
+        del edge, a2, b2, out, mid, sargs
+        # the main workload's arrays are released before the next graph is built
+        del x, c, hyb, csr, triples, d_indptr, d_indices, indptr, indices
+        wl.clear()
+        torch.cuda.empty_cache()
+        if args.scale == 1.0 or args.columns == "uniform":
+            # the same kernel on the same-sized graph whose columns follow the power law as well
+            # (an undirected graph: hub rows are hub columns), where L2 and the memory-side cache
+            # hold the hot rows of X
+            other = "symmetric" if args.columns == "uniform" else "uniform"
+            w2l = hyb_workload(args, other, torch, dev, st, datasets, ops)
+            ok2, worst2, ones2, ccsr2 = check_first_call(w2l, torch, dev)
+            check[f"{other}_hyb_vs_csr_ok"] = ok2
+            ws, ds, dmin = time_steps(lambda: w2l["hyb"](w2l["x"], w2l["c"], *w2l["triples"]), steps, 2, torch)
+            wc, dc, _ = time_steps(lambda: w2l["csr"](ones2, w2l["x"], ccsr2, w2l["d_indptr"], w2l["d_indices"]),
+                                   steps, 1, torch)
+            roof2, _ = roofline_block(w2l, ds, dmin)
+            fl2 = 2.0 * w2l["nnz"] * feat
+            extra[f"hyb_spmm_{other}_columns"] = {"nodes": w2l["m"], "edges": w2l["nnz"], "gflops": fl2 / ws / 1e9,
+                                                  "ms_per_step": ws * 1e3, "csr_ms": dc * 1e3,
+                                                  "hyb_vs_csr_max_abs_diff": worst2, "roofline": roof2}
+            del ones2, ccsr2
+            w2l.clear()
+            torch.cuda.empty_cache()
         extra.update(side_kernels(torch, dev, ops, st, datasets, time_steps))
         extra["config2_hyb_vs_csr"] = config2_sweep(torch, dev, ops, st, datasets, time_steps)
         result["extra"] = extra
 
     print(json.dumps(result), flush=True)
+    failed = [k for k, v in check.items() if k.endswith("_ok") and not v]
+    if failed:
+        log(f"[bench] FAILED checks: {failed}")
+        sys.exit(3)
 
 
 if __name__ == "__main__":

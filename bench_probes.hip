@@ -1,8 +1,11 @@
-// Bandwidth probes used by the benchmark to state what this GPU sustains for the two access
-// patterns the SpMM/SDDMM kernels are made of: a plain streaming copy, and gathers of whole
-// feature rows at pseudo-random row indices (no sparse structure, no arithmetic to speak of).
-#include "common.h"
-#include "../../include/sparsetir_amd.h"
+// Bandwidth probes of bench.py, built into libbench_probes.so (not part of the product library):
+// what this GPU sustains for the two access patterns the SpMM/SDDMM kernels are made of -- a plain
+// streaming copy (also the kernel of known size that the FETCH_SIZE / WRITE_SIZE counters are
+// scaled by) and gathers of whole feature rows at pseudo-random row indices (no sparse structure,
+// no arithmetic to speak of).  Both return 0 on success and -1 on bad arguments or a failed launch.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
 
 namespace {
 
@@ -55,29 +58,30 @@ __global__ __launch_bounds__(256) void probe_gather_kernel(const float* __restri
 
 extern "C" {
 
-int stir_probe_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream) {
-  STIR_REQUIRE(d_src && d_dst && bytes >= 16 && bytes % 16 == 0, "probe_copy: need 16-byte multiples");
+// Copies `bytes` (a multiple of 16) from d_src to d_dst.
+int bench_probe_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream) {
+  if (!(d_src && d_dst && bytes >= 16 && bytes % 16 == 0)) return -1;
   hipLaunchKernelGGL(probe_copy_kernel, dim3(256 * 32), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const float4*>(d_src), static_cast<float4*>(d_dst), bytes / 16);
-  STIR_LAUNCH_CHECK();
-  return 0;
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-int stir_probe_gather(const float* d_table, int64_t rows, int32_t row_floats, int64_t num_gathers,
-                      float* d_sink, void* stream) {
-  STIR_REQUIRE(d_table && d_sink && rows > 0 && num_gathers > 0, "probe_gather: bad arguments");
-  STIR_REQUIRE(row_floats >= 32 && row_floats <= 256 && (row_floats & (row_floats - 1)) == 0,
-               "probe_gather: row_floats=%d must be a power of two in [32, 256]", row_floats);
+// num_gathers (rounded up to whole wavefronts) reads of row_floats*4 bytes each from a table of
+// `rows` rows; row_floats: a power of two in [32, 256].
+int bench_probe_gather(const float* d_table, int64_t rows, int32_t row_floats, int64_t num_gathers,
+                       float* d_sink, void* stream) {
+  if (!(d_table && d_sink && rows > 0 && num_gathers > 0)) return -1;
+  if (!(row_floats >= 32 && row_floats <= 256 && (row_floats & (row_floats - 1)) == 0)) return -1;
   const int lanes = row_floats / 4;
   const int groups_per_wave = 64 / lanes;
   const int per_group = 32;
-  const int64_t waves = stir::ceil_div(num_gathers, (int64_t)per_group * groups_per_wave);
-  const int64_t blocks = stir::ceil_div(waves, 4);
-  STIR_REQUIRE(blocks < (int64_t(1) << 31), "probe_gather: too many gathers for one launch");
+  const int64_t per_wave = (int64_t)per_group * groups_per_wave;
+  const int64_t waves = (num_gathers + per_wave - 1) / per_wave;
+  const int64_t blocks = (waves + 3) / 4;
+  if (blocks >= (int64_t(1) << 31)) return -1;
   hipLaunchKernelGGL(probe_gather_kernel, dim3((unsigned)blocks), dim3(256), 0,
                      static_cast<hipStream_t>(stream), d_table, rows, row_floats, lanes, per_group, d_sink);
-  STIR_LAUNCH_CHECK();
-  return 0;
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 }  // extern "C"

@@ -307,18 +307,6 @@ int stir_rgms_csf_f32(int32_t m, int32_t n, int32_t num_rels, int32_t feat_in, i
                       const int32_t* d_indices_i, const int32_t* d_indptr_j,
                       const int32_t* d_indices_j, void* stream);
 
-/* ----------------------------------------------------------------------- bandwidth probes */
-
-/*
- * Measurement aids with no counterpart in the reference: what the GPU sustains for a plain
- * copy (bytes read + bytes written) and for gathers of whole feature rows at pseudo-random
- * row indices -- the access pattern that bounds SpMM/SDDMM.  stir_probe_gather performs
- * num_gathers (rounded up to whole wavefronts) reads of row_floats*4 bytes each.
- */
-int stir_probe_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream);
-int stir_probe_gather(const float* d_table, int64_t rows, int32_t row_floats, int64_t num_gathers,
-                      float* d_sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -51,8 +51,6 @@ SIGNATURES = {
     "stir_rgms_f32": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
     "stir_rgms_f32_plan_destroy": (I32, [VP]),
     "stir_rgms_csf_f32": (I32, [I32, I32, I32, I32, I32, I64, I64, VP, VP, VP, VP, VP, VP, VP, VP, VP]),
-    "stir_probe_copy": (I32, [VP, VP, I64, VP]),
-    "stir_probe_gather": (I32, [VP, I64, I32, I64, VP, VP]),
 }
 
 _lib = None
