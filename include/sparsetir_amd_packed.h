@@ -105,6 +105,16 @@ enum {
  *      examples/rgms/rgcn/bench_rgcn_composable.py:208-221
  * "sparsetir.rgms_csf"       (A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j, feat_in, feat_out)
  *      examples/rgms/rgcn/bench_rgcn_non_composable.py:109         fp32, W [R, feat_out, feat_in]
+ * "sparsetir.invalidate_plans" ()
+ *      no counterpart in the reference, whose built operators read their index arrays on every
+ *      call.  Here "sparsetir.hyb_csrmm", "sparsetir.rgms" and "sparsetir.rgms_f32" keep one plan
+ *      each per process, reused while the array addresses and sizes of a call equal those of the
+ *      previous one.  A plan holds what was derived from the index arrays' contents (rgms: the
+ *      edge index built by the first launch over 8192 slots or more; hyb_csrmm with 2 to 4
+ *      partitions: whether its buckets need atomics).  A caller that rewrites rows / cols / mids
+ *      in place, or frees them and gets arrays of the same sizes at the same addresses, calls
+ *      this first; the next operator call then builds a fresh plan.  Edge weights (A_k), W, X, B
+ *      may change freely.
  *
  * Format pass (host tensors, kDLCPU; the reference returns nested Array<NDArray>, which needs
  * libtvm objects, so here a sizing call is followed by a fill call into caller-made tensors):
@@ -130,6 +140,7 @@ int stir_packed_tcspmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms_f32(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms_csf(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_invalidate_plans(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_csf_to_ell3d_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);

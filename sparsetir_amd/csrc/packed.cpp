@@ -485,6 +485,18 @@ int stir_packed_rgms_f32(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) 
   return packed_rgms_any("sparsetir.rgms_f32", true, v, tc, n);
 }
 
+int stir_packed_invalidate_plans(TVMValue*, int*, int n, TVMRetValueHandle, void*) {
+  if (n != 0) return packed_fail("sparsetir.invalidate_plans: num_args should be 0");
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  if (g_hyb_plan) stir_hyb_plan_destroy(g_hyb_plan);
+  if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
+  if (g_rgms_f32_plan) stir_rgms_f32_plan_destroy(g_rgms_f32_plan);
+  g_hyb_plan = nullptr;
+  g_rgms_plan = nullptr;
+  g_rgms_f32_plan = nullptr;
+  return 0;
+}
+
 int stir_packed_rgms_csf(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   Args a{"sparsetir.rgms_csf", v, tc, n};
   if (!a.count(10)) return -1;
@@ -678,6 +690,7 @@ static const PackedEntry kTable[] = {
     {"sparsetir.rgms", stir_packed_rgms},
     {"sparsetir.rgms_f32", stir_packed_rgms_f32},
     {"sparsetir.rgms_csf", stir_packed_rgms_csf},
+    {"sparsetir.invalidate_plans", stir_packed_invalidate_plans},
     {"tir.sparse.ColumnPartHyb.sizes", stir_packed_column_part_hyb_sizes},
     {"tir.sparse.ColumnPartHyb.fill", stir_packed_column_part_hyb_fill},
     {"tir.sparse.CSFToELL3D.sizes", stir_packed_csf_to_ell3d_sizes},

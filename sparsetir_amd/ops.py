@@ -151,6 +151,14 @@ class HybCsrMM(_Operator):
             self.L.stir_hyb_plan_destroy(self._plan)
             self._plan = None
 
+    def invalidate(self):
+        """Forget the plan made from the arrays of the last call.  The plan is reused while the
+        (A_k, rows_k, cols_k) arrays keep their addresses; with 2 to 4 column partitions it also
+        remembers whether the row arrays allowed dropping atomics.  Call this after rewriting row
+        arrays in place (the reference's operator reads them afresh on every call)."""
+        self._drop_plan()
+        self._key = None
+
     def __del__(self):
         try:
             self._drop_plan()
@@ -301,7 +309,14 @@ class TcSpMM(_Operator):
 
 class Rgms(_Operator):
     """RGMS on ELL3D buckets.  ``groups`` lists the group count of every bucket, ``rows_bkt`` /
-    ``cols_bkt`` the ELL rows per group and slots per ELL row."""
+    ``cols_bkt`` the ELL rows per group and slots per ELL row.
+
+    The operator keeps a plan made on the first call with a given set of bucket arrays (keyed by
+    their addresses).  From 8192 slots on, that plan holds an edge index derived from the contents
+    of the rows / cols / mids arrays: after changing those in place call :meth:`invalidate`, or the
+    old structure keeps being used (the reference's operator reads the arrays on every call).  The
+    edge weights ``A_k``, ``W`` and ``X`` are read on every call.  The first call of a plan
+    allocates and synchronises the stream, so it cannot be part of a captured graph."""
     name = "rgms"
 
     _in_dtype = torch.float16
@@ -339,6 +354,11 @@ class Rgms(_Operator):
         if self._plan is not None:
             getattr(self.L, self._fns[2])(self._plan)
             self._plan = None
+
+    def invalidate(self):
+        """Forget the plan (and the edge index) made from the arrays of the last call."""
+        self._drop_plan()
+        self._key = None
 
     def __del__(self):
         try:

@@ -168,3 +168,53 @@ def test_on_disk_cache_round_trip(tmp_path):
         _same(b, c)
     cached_column_part_hyb(str(tmp_path), 300, 200, indptr, indices, 2, [1, 2])  # other parameters: new entry
     assert len(list(tmp_path.iterdir())) == 2
+
+
+def test_on_disk_cache_ell3d_and_condense(tmp_path):
+    from sparsetir_amd.cache import cached_condense, cached_csf_to_ell3d
+
+    R, n = 5, 60
+    rng = np.random.default_rng(4)
+    ptr0, idx0, ptr1, idx1 = [0], [], [0], []
+    for r in range(R):
+        rows = np.sort(rng.choice(n, rng.integers(0, 20), replace=False))
+        for i in rows:
+            cols = np.sort(rng.choice(n, rng.integers(1, 9), replace=False))
+            idx0.append(i)
+            idx1.extend(cols)
+            ptr1.append(len(idx1))
+        ptr0.append(len(idx0))
+    csf = [np.asarray(a, np.int32) for a in (ptr0, idx0, ptr1, idx1)]
+    rb, cb = [8, 4, 2], [1, 2, 4]
+    want = oracle.csf_to_ell3d(*csf, rb, cb)
+    first = cached_csf_to_ell3d(str(tmp_path), *csf, rb, cb)
+    again = cached_csf_to_ell3d(str(tmp_path), *csf, rb, cb)
+    assert len(list(tmp_path.iterdir())) == 1
+    for q in range(4):
+        for b in range(len(cb)):
+            assert np.array_equal(first[q][b], want[q][b])
+            assert again[q][b].dtype == np.int32 and again[q][b].shape == want[q][b].shape
+            assert np.array_equal(again[q][b], want[q][b])
+    indptr, indices = random_csr(90, 70, 900, 3)
+    want = oracle.condense(indptr, indices, 8, 4)
+    first = cached_condense(str(tmp_path), indptr, indices, 8, 4)
+    again = cached_condense(str(tmp_path), indptr, indices, 8, 4)
+    assert len(list(tmp_path.iterdir())) == 2
+    for a, b, c in zip(first, again, want):
+        assert np.array_equal(a, c) and np.array_equal(b, c) and b.shape == c.shape
+
+
+def test_on_disk_cache_ignores_a_damaged_file(tmp_path):
+    from sparsetir_amd.cache import cached_column_part_hyb
+
+    indptr, indices = random_csr(50, 40, 300, 2)
+    cached_column_part_hyb(str(tmp_path), 50, 40, indptr, indices, 1, [1, 2])
+    (path,) = list(tmp_path.iterdir())
+    path.write_bytes(b"not an archive")
+    got = cached_column_part_hyb(str(tmp_path), 50, 40, indptr, indices, 1, [1, 2])
+    want = oracle.column_part_hyb(50, 40, indptr, indices, 1, [1, 2])
+    for a, c in zip(got, want):
+        _same(a, c)
+    again = cached_column_part_hyb(str(tmp_path), 50, 40, indptr, indices, 1, [1, 2])  # rewritten and readable
+    for a, c in zip(again, want):
+        _same(a, c)

@@ -238,3 +238,46 @@ def test_device_csr_to_bsr_errors(dev):
     with pytest.raises(SparseTIRError, match="outside"):
         st.csr_to_bsr(torch.tensor([0, 1] + [1] * 31, dtype=torch.int32, device=dev),
                       torch.tensor([99], dtype=torch.int32, device=dev), z(1, torch.float32), (32, 64), 32)
+
+
+def test_on_disk_cache_of_a_device_decomposition_feeds_the_hyb_operator(dev, tmp_path):
+    """A decomposition computed on the GPU is stored as host arrays; a later call (another
+    process in practice) gets device arrays back that equal the oracle's bit for bit and that the
+    hyb operator takes as they are."""
+    from sparsetir_amd import ops
+    from sparsetir_amd.cache import cached_column_part_hyb
+    from helpers import spmm_f64
+
+    m = n = 2500
+    parts, buckets, feat = 2, [1, 2, 4, 8], 64
+    indptr, indices = random_csr(m, n, 40000, 9, skew=1.1)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    first = cached_column_part_hyb(str(tmp_path), m, n, t(indptr), t(indices), parts, buckets)
+    assert len(list(tmp_path.iterdir())) == 1
+    again = cached_column_part_hyb(str(tmp_path), m, n, t(indptr), t(indices), parts, buckets)
+    assert len(list(tmp_path.iterdir())) == 1
+    want = oracle.column_part_hyb(m, n, indptr, indices, parts, buckets)
+    for q in range(3):
+        for p in range(parts):
+            for b in range(len(buckets)):
+                assert again[q][p][b].is_cuda and again[q][p][b].dtype == torch.int32
+                assert np.array_equal(first[q][p][b].cpu().numpy(), want[q][p][b])
+                assert np.array_equal(again[q][p][b].cpu().numpy(), want[q][p][b])
+    rows, cols, mask = again
+    triples, nrows = [], []
+    for p in range(parts):
+        for b in range(len(buckets)):
+            triples += [mask[p][b].reshape(-1).float(), rows[p][b], cols[p][b].reshape(-1)]
+            nrows.append(int(rows[p][b].shape[0]))
+    x = np.random.default_rng(1).standard_normal((n, feat), dtype=np.float32)
+    c = torch.zeros(m * feat, device=dev)
+    ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)(t(x.ravel()), c, *triples)
+    torch.cuda.synchronize()
+    ones = np.ones(len(indices), np.float32)
+    exact = spmm_f64(indptr, indices, ones, x)
+    scale = spmm_f64(indptr, indices, ones, np.abs(x))
+    assert np.all(np.abs(c.cpu().numpy().reshape(m, feat) - exact) <= 1e-5 * scale + 1e-30)
+    # a host-side call on the same matrix shares the entry
+    host = cached_column_part_hyb(str(tmp_path), m, n, indptr, indices, parts, buckets)
+    assert len(list(tmp_path.iterdir())) == 1
+    assert isinstance(host[0][0][0], np.ndarray) and np.array_equal(host[1][1][2], want[1][1][2])
