@@ -270,6 +270,18 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
 int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
                   int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
                   float* d_Y, void* stream);
+/*
+ * Optional promise, made before the first launch of a plan: the slot weights d_A[b] keep the
+ * values they have at that first launch for as long as the plan lives.  This is how the reference
+ * uses the operator -- its A_k is the 0/1 mask of CSFToELL3D, written once
+ * (examples/rgms/rgcn/bench_rgcn_tensorcore.py:840-851).  With the promise, plans over 8192 slots
+ * or more (and at most 2048 relations) leave slots of weight zero -- the ELL3D padding, 11 % of
+ * the slots at 100k nodes / 65 relations / 2M edges -- out of their edge index and keep the
+ * weights inside it (8 bytes per edge instead of 16, no weight loads at run time).  Without it
+ * (the default) weights are read at every launch and may change between launches.  Fails once the
+ * plan has been launched with the other setting.
+ */
+int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on);
 /* The same with bf16 W, X and slot weights (the reference has an fp16 example only). */
 int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
                    int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,

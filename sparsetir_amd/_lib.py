@@ -46,6 +46,7 @@ SIGNATURES = {
     "stir_rgms_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
     "stir_rgms_bf16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
+    "stir_rgms_plan_set_static_weights": (I32, [VP, I32]),
     "stir_rgms_plan_destroy": (I32, [VP]),
     "stir_rgms_f32_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f32": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),

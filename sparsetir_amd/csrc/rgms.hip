@@ -258,6 +258,7 @@ struct stir_rgms_plan {
   // num_rels) and kept
   std::vector<stir::TileBucket> tile_buckets;
   int64_t slots;
+  bool static_weights;  // promise of the caller, see stir_rgms_plan_set_static_weights
   stir::TileIndex tiles;
 };
 
@@ -311,6 +312,7 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   p->d_table = nullptr;
   p->tile_buckets = tile_buckets;
   p->slots = slots;
+  p->static_weights = false;
   hipError_t err = hipSuccess;
   if (nk > 0) {
     err = hipMalloc(reinterpret_cast<void**>(&p->d_table), sizeof(RgmsBucket) * nk);
@@ -346,7 +348,7 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
     // the plan's edge index and packed copy of W are filled in by the launches: a plan serves
     // one call at a time
     stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
-    if (stir::tile_index_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, st)) return -1;
+    if (stir::tile_index_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, mp->static_weights, st)) return -1;
     return stir::tile_rgms_launch(bf16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
   }
 #define STIR_RGMS(KK)                                                                              \
@@ -381,6 +383,14 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
 int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels, int32_t feat_in,
                    int32_t feat_out, const void* d_W, const void* d_X, float* d_Y, void* stream) {
   return rgms_launch(true, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
+}
+
+int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on) {
+  STIR_REQUIRE(plan, "rgms_plan_set_static_weights: plan is null");
+  STIR_REQUIRE(plan->tiles.m < 0 || plan->static_weights == (on != 0),
+               "rgms_plan_set_static_weights: the plan has been launched already");
+  plan->static_weights = on != 0;
+  return 0;
 }
 
 int stir_rgms_plan_destroy(stir_rgms_plan* plan) {

@@ -26,9 +26,10 @@ struct TileBucket {
 
 struct TileIndex {
   int32_t m = -1, n = -1, num_rels = -1;  // what the index was built for
+  bool packed_records = false;            // 8-byte records that carry the slot weights (see tile_index_prepare)
   int64_t edges = 0;                      // slots of all buckets
   int64_t units = 0;
-  void* d_edges = nullptr;  // edges x 16 bytes, sorted
+  void* d_edges = nullptr;  // edges x 16 (or 8) bytes, sorted
   void* d_units = nullptr;  // units x 16 bytes
   void* d_wpack = nullptr;  // W in MFMA operand order, rewritten by every launch
   size_t wpack_bytes = 0;
@@ -36,8 +37,13 @@ struct TileIndex {
 
 // Builds the index on `stream` (synchronises; allocates).  A no-op when it already exists for
 // the same m, n and num_rels.  Fails when a row id, column id or relation id is out of range.
+// static_weights: the caller promises that the slot weights keep the values they have now.  Slots
+// of weight zero (the padding of ELL3D) are then left out of the index and a record shrinks to
+// 8 bytes holding the weight itself (source row; weight << 16 | relation << 5 | row in tile), for
+// up to 2048 relations; otherwise records hold the weight's address and weights are read at
+// every launch.
 int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
-                       int32_t num_rels, hipStream_t stream);
+                       int32_t num_rels, bool static_weights, hipStream_t stream);
 // Y += RGMS(W, X) over the indexed edges.  W: [R, feat_in, feat_out], X: [n, feat_in], 16-bit.
 int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W,
                      const void* d_X, float* d_Y, hipStream_t stream);

@@ -38,6 +38,13 @@ struct alignas(16) Edge {
   uint32_t rel_dl;     // relation << 5 | destination row inside its tile
 };
 
+// Record of an index built for weights that do not change: no address, the weight itself.
+struct alignas(8) PackedEdge {
+  int32_t src;
+  uint32_t w_rel_dl;  // 16-bit weight << 16 | relation << 5 | destination row inside its tile
+};
+constexpr int kPackedMaxRels = 1 << 11;
+
 struct alignas(16) Unit {
   int64_t edge_begin;
   int32_t edge_count;
@@ -47,7 +54,10 @@ struct alignas(16) Unit {
 constexpr int kTileRows = 32;
 constexpr int kStepEdges = 32;
 constexpr int kMaxKK = 8;
-constexpr int kUnitWaves = 4;  // wavefronts that share a unit
+#ifndef STIR_UNIT_WAVES
+#define STIR_UNIT_WAVES 4
+#endif
+constexpr int kUnitWaves = STIR_UNIT_WAVES;  // wavefronts that share a unit
 
 __device__ __forceinline__ int bucket_of(const DevBucket* __restrict__ tab, int nb, int64_t q) {
   int lo = 0, hi = nb - 1;
@@ -59,8 +69,10 @@ __device__ __forceinline__ int bucket_of(const DevBucket* __restrict__ tab, int 
 }
 
 // key = (destination tile, relation, row inside the tile), value = slot
+// drop_zero: slots of weight zero get the key one past the last tile, so they sort behind every
+// tile and no unit covers them
 __global__ __launch_bounds__(256) void edge_keys_kernel(const DevBucket* __restrict__ tab, int nb, int64_t slots, int m,
-                                                        int num_rels, uint64_t* __restrict__ keys,
+                                                        int num_rels, int drop_zero, uint64_t* __restrict__ keys,
                                                         int32_t* __restrict__ vals, int32_t* __restrict__ bad) {
   const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (q >= slots) return;
@@ -75,13 +87,16 @@ __global__ __launch_bounds__(256) void edge_keys_kernel(const DevBucket* __restr
     *bad = 1;
     dest = rel = 0;
   }
-  keys[q] = ((((uint64_t)(dest >> 5)) * num_rels + rel) << 5) | (uint64_t)(dest & 31);
+  uint64_t key = ((((uint64_t)(dest >> 5)) * num_rels + rel) << 5) | (uint64_t)(dest & 31);
+  if (drop_zero && (bk.A[local] & 0x7fff) == 0) key = ((uint64_t)((m + kTileRows - 1) / kTileRows) * num_rels) << 5;
+  keys[q] = key;
   vals[q] = (int32_t)q;
 }
 
+template <typename Rec>
 __global__ __launch_bounds__(256) void edge_records_kernel(const DevBucket* __restrict__ tab, int nb, int64_t slots,
                                                            int n, int num_rels, const uint64_t* __restrict__ keys,
-                                                           const int32_t* __restrict__ vals, Edge* __restrict__ edges,
+                                                           const int32_t* __restrict__ vals, Rec* __restrict__ edges,
                                                            int32_t* __restrict__ bad) {
   const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (p >= slots) return;
@@ -94,12 +109,17 @@ __global__ __launch_bounds__(256) void edge_records_kernel(const DevBucket* __re
     src = 0;
   }
   const uint64_t key = keys[p];
-  const uint64_t addr = reinterpret_cast<uint64_t>(bk.A + local);
-  Edge e;
+  const uint32_t rel_dl = (uint32_t)(((key >> 5) % (uint64_t)num_rels) << 5) | (uint32_t)(key & 31);
+  Rec e;
   e.src = src;
-  e.w_lo = (uint32_t)addr;
-  e.w_hi = (uint32_t)(addr >> 32);
-  e.rel_dl = (uint32_t)(((key >> 5) % (uint64_t)num_rels) << 5) | (uint32_t)(key & 31);
+  if constexpr (sizeof(Rec) == sizeof(PackedEdge)) {
+    e.w_rel_dl = ((uint32_t)bk.A[local] << 16) | rel_dl;  // dropped slots (beyond the last tile) are never read
+  } else {
+    const uint64_t addr = reinterpret_cast<uint64_t>(bk.A + local);
+    e.w_lo = (uint32_t)addr;
+    e.w_hi = (uint32_t)(addr >> 32);
+    e.rel_dl = rel_dl;
+  }
   edges[p] = e;
 }
 
@@ -147,6 +167,20 @@ __global__ __launch_bounds__(256) void unit_fill_kernel(const int64_t* __restric
     un.tile_flag = (int32_t)(t << 1) | (nu > 1 ? 1 : 0);
     units[unit_begin[t] + u] = un;
   }
+}
+
+__global__ __launch_bounds__(256) void unit_sort_keys_kernel(const Unit* __restrict__ units, int64_t n,
+                                                             int32_t* __restrict__ keys, int32_t* __restrict__ vals) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  keys[i] = units[i].edge_count;
+  vals[i] = (int32_t)i;
+}
+
+__global__ __launch_bounds__(256) void unit_permute_kernel(const Unit* __restrict__ in, const int32_t* __restrict__ order,
+                                                           int64_t n, Unit* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = in[order[i]];
 }
 
 // W[rel][16kk + 8h + 2d (+1)][32nt + n] -> operand word d of lane (n, h), one wavefront per
@@ -220,13 +254,15 @@ constexpr int kSStride = 40;  // 16-bit elements per row of the S tile (32 used;
 // steps w, w + 4, ...: more wavefronts in flight per tile, since a step costs a full memory
 // round trip), each with its own accumulator tile; the four tiles are added through LDS and the
 // workgroup writes the 32 rows of Y once.  KK = feat_in / 16.
-template <int KK, bool BF16>
-__global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__ units,
-                                                        const Edge* __restrict__ edges, int m, int feat_out,
+template <int KK, bool BF16, typename Rec>
+__global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* __restrict__ units,
+                                                        const Rec* __restrict__ edges, int m, int feat_out,
                                                         const u32x4* __restrict__ Wp, const uint16_t* __restrict__ X,
                                                         float* __restrict__ Y) {
   constexpr int FIN = KK * 16;
+  constexpr bool kPacked = sizeof(Rec) == sizeof(PackedEdge);
   constexpr int PW = KK <= 4 ? 2 : 1;  // relations whose W fragments are requested together
+  constexpr int kThreads = 64 * kUnitWaves, kSumIters = kTileRows * 32 / kThreads;
   __shared__ __attribute__((aligned(16))) uint16_t s_all[kUnitWaves][kTileRows * kSStride];
   __shared__ float partial[kUnitWaves][16 * 64];  // [wavefront][accumulator register][lane]
   const int lane = threadIdx.x & 63;
@@ -254,15 +290,19 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
     for (int v = 0; v < 16; ++v) acc2[v] = 0.f;
     // lanes past the last edge repeat it with weight zero
     constexpr int64_t kStride = kUnitWaves * kStepEdges;  // edges between a wavefront's steps
-    Edge next = edges[min(u.edge_begin + wave * kStepEdges + mrow, e_end - 1)];
-    Edge after = edges[min(u.edge_begin + wave * kStepEdges + kStride + mrow, e_end - 1)];
+    Rec next = edges[min(u.edge_begin + wave * kStepEdges + mrow, e_end - 1)];
+    Rec after = edges[min(u.edge_begin + wave * kStepEdges + kStride + mrow, e_end - 1)];
 #pragma unroll 1
     for (int64_t e0 = u.edge_begin + wave * kStepEdges; e0 < e_end; e0 += kStride) {
-      const Edge cur = next;
+      const Rec cur = next;
       next = after;
       const int left = (int)min((int64_t)kStepEdges, e_end - e0);  // uniform
       const bool live = mrow < left;
-      const int rel = (int)(cur.rel_dl >> 5), dl = (int)(cur.rel_dl & 31);
+      int rel, dl;
+      if constexpr (kPacked)
+        rel = (int)((cur.w_rel_dl >> 5) & (kPackedMaxRels - 1)), dl = (int)(cur.w_rel_dl & 31);
+      else
+        rel = (int)(cur.rel_dl >> 5), dl = (int)(cur.rel_dl & 31);
       // the first PW runs of equal relation (the step is sorted by relation)
       int r[PW], pos = 0;
 #pragma unroll
@@ -280,7 +320,11 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
       const uint16_t* xp = X + (int64_t)cur.src * FIN + 8 * h;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) xa[kk] = *reinterpret_cast<const u32x4*>(xp + 16 * kk);
-      const uint16_t wbits = *reinterpret_cast<const GlobalU16*>(((uint64_t)cur.w_hi << 32) | cur.w_lo);
+      uint16_t wbits;
+      if constexpr (kPacked)
+        wbits = (uint16_t)(cur.w_rel_dl >> 16);
+      else
+        wbits = *reinterpret_cast<const GlobalU16*>(((uint64_t)cur.w_hi << 32) | cur.w_lo);
 #pragma unroll
       for (int q = 0; q < PW; ++q) {
         if (r[q] >= 0) {
@@ -348,17 +392,17 @@ __global__ __launch_bounds__(256) void rgms_tile_kernel(const Unit* __restrict__
 #pragma unroll
     for (int v = 0; v < 16; ++v) partial[wave][v * 64 + lane] = acc2[v];
     const bool atomic = u.tile_flag & 1;
-    float yold[4];  // requested before the barrier
+    float yold[kSumIters];  // requested before the barrier
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int elem = threadIdx.x + 256 * k;
+    for (int k = 0; k < kSumIters; ++k) {
+      const int elem = threadIdx.x + kThreads * k;
       const int64_t yrow = (int64_t)tile * kTileRows + (elem >> 5);
       yold[k] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + (elem & 31)] : 0.f;
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int elem = threadIdx.x + 256 * k, row = elem >> 5, col = elem & 31;
+    for (int k = 0; k < kSumIters; ++k) {
+      const int elem = threadIdx.x + kThreads * k, row = elem >> 5, col = elem & 31;
       const int at = ((row & 3) + 4 * (row >> 3)) * 64 + col + 32 * ((row >> 2) & 1);
       float sum = partial[0][at];
 #pragma unroll
@@ -402,8 +446,9 @@ void tile_index_free(TileIndex& ix) {
 }
 
 int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
-                       int32_t num_rels, hipStream_t stream) {
+                       int32_t num_rels, bool static_weights, hipStream_t stream) {
   if (ix.m == m && ix.n == n && ix.num_rels == num_rels) return 0;
+  const bool packed = static_weights && num_rels <= kPackedMaxRels;
   STIR_REQUIRE(num_rels > 0 && num_rels < (1 << 26), "rgms: num_rels=%d out of range", num_rels);
   if (ix.d_edges) STIR_HIP(hipFree(ix.d_edges));
   if (ix.d_units) STIR_HIP(hipFree(ix.d_units));
@@ -424,7 +469,8 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   }
   const int nb = (int)host.size();
   const int64_t tiles = ceil_div(m, kTileRows);
-  const int end_bit = bit_length((((uint64_t)tiles * num_rels) << 5) - 1);
+  // keys run up to (tiles * num_rels) << 5 inclusive: that value marks the dropped slots
+  const int end_bit = bit_length(((uint64_t)tiles * num_rels) << 5);
   const int cus = std::max(1, compute_units());
   // Units (one workgroup each) of at most `cap` steps.  A tile is cut only when it is long against
   // the others -- more than about three average tiles -- or when the launch would otherwise
@@ -454,20 +500,26 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   STIR_HIP(count.alloc(sizeof(int32_t) * size_t(tiles + 1)));
   STIR_HIP(ubegin.alloc(sizeof(int32_t) * size_t(tiles + 1)));
   DevBuf edges;
-  STIR_HIP(edges.alloc(sizeof(Edge) * size_t(slots)));
+  STIR_HIP(edges.alloc((packed ? sizeof(PackedEdge) : sizeof(Edge)) * size_t(slots)));
 
   STIR_HIP(hipMemcpyAsync(tab.p, host.data(), sizeof(DevBucket) * host.size(), hipMemcpyHostToDevice, stream));
   STIR_HIP(hipMemsetAsync(bad.p, 0, sizeof(int32_t), stream));
   const dim3 block(256);
   const dim3 slot_grid((unsigned)ceil_div(slots, 256)), tile_grid((unsigned)ceil_div(tiles + 1, 256));
   hipLaunchKernelGGL(edge_keys_kernel, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, m, num_rels,
-                     keys_in.as<uint64_t>(), vals_in.as<int32_t>(), bad.as<int32_t>());
+                     packed ? 1 : 0, keys_in.as<uint64_t>(), vals_in.as<int32_t>(), bad.as<int32_t>());
   STIR_LAUNCH_CHECK();
   STIR_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, sort_bytes, keys_in.as<const uint64_t>(), keys.as<uint64_t>(),
                                               vals_in.as<const int32_t>(), vals.as<int32_t>(), (int)slots, 0,
                                               end_bit, stream));
-  hipLaunchKernelGGL(edge_records_kernel, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, n, num_rels,
-                     keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<Edge>(), bad.as<int32_t>());
+  if (packed)
+    hipLaunchKernelGGL(edge_records_kernel<PackedEdge>, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, n,
+                       num_rels, keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<PackedEdge>(),
+                       bad.as<int32_t>());
+  else
+    hipLaunchKernelGGL(edge_records_kernel<Edge>, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, n,
+                       num_rels, keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<Edge>(),
+                       bad.as<int32_t>());
   STIR_LAUNCH_CHECK();
   hipLaunchKernelGGL(tile_bounds_kernel, tile_grid, block, 0, stream, keys.as<const uint64_t>(), slots, tiles,
                      num_rels, begin.as<int64_t>());
@@ -488,12 +540,40 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   hipLaunchKernelGGL(unit_fill_kernel, tile_grid, block, 0, stream, begin.as<const int64_t>(),
                      ubegin.as<const int32_t>(), tiles, cap, units.as<Unit>());
   STIR_LAUNCH_CHECK();
+  // Longest units first: workgroups are dispatched in unit order, and a long unit that starts in the
+  // last round of workgroups would be the tail of the launch.
+  if (h_units > 1) {
+    DevBuf ukeys_in, ukeys, uvals_in, uvals, utmp, sorted;
+    size_t usort_bytes = 0;
+    STIR_HIP(hipcub::DeviceRadixSort::SortPairsDescending(nullptr, usort_bytes, (const int32_t*)nullptr,
+                                                          (int32_t*)nullptr, (const int32_t*)nullptr,
+                                                          (int32_t*)nullptr, h_units, 0, 32, stream));
+    STIR_HIP(ukeys_in.alloc(sizeof(int32_t) * size_t(h_units)));
+    STIR_HIP(ukeys.alloc(sizeof(int32_t) * size_t(h_units)));
+    STIR_HIP(uvals_in.alloc(sizeof(int32_t) * size_t(h_units)));
+    STIR_HIP(uvals.alloc(sizeof(int32_t) * size_t(h_units)));
+    STIR_HIP(utmp.alloc(usort_bytes));
+    STIR_HIP(sorted.alloc(sizeof(Unit) * size_t(h_units)));
+    const dim3 unit_grid((unsigned)ceil_div(h_units, 256));
+    hipLaunchKernelGGL(unit_sort_keys_kernel, unit_grid, block, 0, stream, units.as<const Unit>(), (int64_t)h_units,
+                       ukeys_in.as<int32_t>(), uvals_in.as<int32_t>());
+    STIR_LAUNCH_CHECK();
+    STIR_HIP(hipcub::DeviceRadixSort::SortPairsDescending(utmp.p, usort_bytes, ukeys_in.as<const int32_t>(),
+                                                          ukeys.as<int32_t>(), uvals_in.as<const int32_t>(),
+                                                          uvals.as<int32_t>(), h_units, 0, 32, stream));
+    hipLaunchKernelGGL(unit_permute_kernel, unit_grid, block, 0, stream, units.as<const Unit>(),
+                       uvals.as<const int32_t>(), (int64_t)h_units, sorted.as<Unit>());
+    STIR_LAUNCH_CHECK();
+    STIR_HIP(hipStreamSynchronize(stream));
+    std::swap(units.p, sorted.p);
+  }
   STIR_HIP(hipStreamSynchronize(stream));
   ix.d_edges = edges.p, edges.p = nullptr;
   ix.d_units = units.p, units.p = nullptr;
   ix.edges = slots;
   ix.units = h_units;
   ix.m = m, ix.n = n, ix.num_rels = num_rels;
+  ix.packed_records = packed;
   return 0;
 }
 
@@ -520,15 +600,17 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   const dim3 grid((unsigned)ix.units), block(64 * kUnitWaves);
   const Unit* units = static_cast<const Unit*>(ix.d_units);
   const Edge* edges = static_cast<const Edge*>(ix.d_edges);
+  const PackedEdge* pedges = static_cast<const PackedEdge*>(ix.d_edges);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
-#define STIR_TILES(KKV)                                                                                          \
-  case KKV:                                                                                                      \
-    if (bf16)                                                                                                    \
-      hipLaunchKernelGGL((rgms_tile_kernel<KKV, true>), grid, block, 0, stream, units, edges, ix.m,    \
-                         feat_out, Wp, X, d_Y);                                                                  \
-    else                                                                                                         \
-      hipLaunchKernelGGL((rgms_tile_kernel<KKV, false>), grid, block, 0, stream, units, edges, ix.m,   \
-                         feat_out, Wp, X, d_Y);                                                                  \
+#define STIR_TILES_R(KKV, BF, REC, PTR) \
+  hipLaunchKernelGGL((rgms_tile_kernel<KKV, BF, REC>), grid, block, 0, stream, units, PTR, ix.m, feat_out, Wp, X, d_Y)
+#define STIR_TILES(KKV)                                                                          \
+  case KKV:                                                                                      \
+    if (ix.packed_records) {                                                                     \
+      if (bf16) STIR_TILES_R(KKV, true, PackedEdge, pedges); else STIR_TILES_R(KKV, false, PackedEdge, pedges); \
+    } else {                                                                                     \
+      if (bf16) STIR_TILES_R(KKV, true, Edge, edges); else STIR_TILES_R(KKV, false, Edge, edges); \
+    }                                                                                            \
     break
   switch (kk_count) {
     STIR_TILES(1);
@@ -541,6 +623,7 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
     STIR_TILES(8);
   }
 #undef STIR_TILES
+#undef STIR_TILES_R
   STIR_LAUNCH_CHECK();
   return 0;
 }

@@ -315,14 +315,19 @@ class Rgms(_Operator):
     their addresses).  From 8192 slots on, that plan holds an edge index derived from the contents
     of the rows / cols / mids arrays: after changing those in place call :meth:`invalidate`, or the
     old structure keeps being used (the reference's operator reads the arrays on every call).  The
-    edge weights ``A_k``, ``W`` and ``X`` are read on every call.  The first call of a plan
-    allocates and synchronises the stream, so it cannot be part of a captured graph."""
+    edge weights ``A_k``, ``W`` and ``X`` are read on every call -- unless the operator was built
+    with ``static_weights=True``, the promise that the ``A_k`` keep the values of the first call
+    (the reference's use: its ``A_k`` is the 0/1 mask); zero-weight padding slots are then left out
+    of the index and the weights live inside it.  The first call of a plan allocates and
+    synchronises the stream, so it cannot be part of a captured graph."""
     name = "rgms"
 
     _in_dtype = torch.float16
     _fns = ("stir_rgms_plan_create", "stir_rgms_f16", "stir_rgms_plan_destroy")
 
-    def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=None):
+    def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=None,
+                 static_weights=False):
+        self._static = bool(static_weights)
         if dtype is not None and self._in_dtype is torch.float16:
             if dtype not in (torch.float16, torch.bfloat16):
                 raise _lib.SparseTIRError("rgms: dtype must be torch.float16 or torch.bfloat16")
@@ -386,6 +391,8 @@ class Rgms(_Operator):
                                                          tab(triples[0::3]), tab(triples[1::3]),
                                                          tab(triples[2::3]), tab(mids)))
                 self._plan, self._key, self._keep = plan, key, rest
+                if self._static and self._in_dtype is not torch.float32:
+                    _lib.check(self.L.stir_rgms_plan_set_static_weights(plan, 1))
             _lib.check(getattr(self.L, self._fns[1])(self._plan, self.m, self.n, self.R, self.fin, self.fout,
                                                      _ptr(w), _ptr(x), _ptr(y), _stream()))
 
@@ -453,8 +460,9 @@ def build_tcspmm(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=to
     return TcSpMM(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype)
 
 
-def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=torch.float16):
-    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype)
+def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=torch.float16,
+               static_weights=False):
+    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype, static_weights)
 
 
 def build_rgms_f32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):

@@ -12,7 +12,7 @@ from helpers import random_csf, rgms_f64
 pytestmark = pytest.mark.gpu
 
 
-def _run(dev, csf, m, n, x, w, group, buckets, weighted, seed=0):
+def _run(dev, csf, m, n, x, w, group, buckets, weighted, seed=0, static=False, dtype=torch.float16):
     p0, i0, p1, i1 = csf
     R, fin, fout = w.shape
     rows_bkt = [max(1, group // b) for b in buckets]
@@ -28,11 +28,16 @@ def _run(dev, csf, m, n, x, w, group, buckets, weighted, seed=0):
         avals.append(a16)
         triples += [t(a16.ravel()), t(rows[b].ravel()), t(cols[b].ravel())]
         mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
-    f = ops.build_rgms(m, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols])
+    f = ops.build_rgms(m, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols], static_weights=static)
     y = torch.zeros(m * fout, dtype=torch.float32, device=dev)
     x16, w16 = x.astype(np.float16), w.astype(np.float16)
     f(t(w16.ravel()), t(x16.ravel()), y, *triples, *mids)
     torch.cuda.synchronize()
+    if static:  # a second call reuses the index that holds the weights
+        y2 = torch.zeros_like(y)
+        f(t(w16.ravel()), t(x16.ravel()), y2, *triples, *mids)
+        torch.cuda.synchronize()
+        assert torch.allclose(y, y2, rtol=1e-6, atol=1e-6)
     # edge weights in CSF order for the closed form: decode them from the ELL3D arrays
     coo = {}
     for b in range(len(buckets)):
@@ -92,6 +97,53 @@ def test_rgms_tiled_accumulation(dev, group, buckets):
     csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
     got, x32, w32, av = _run(dev, csf, cfg["m"], cfg["n"], cfg["x"], cfg["w"], group, buckets, True)
     _check(got, csf, av, x32, w32, cfg["m"], f"tiled group={group}")
+
+
+@pytest.mark.parametrize("group,buckets,weighted", [(256, [1, 2, 4, 8, 16], False), (32, [1, 2, 4, 8, 16, 32], True),
+                                                    (48, [1, 3, 4, 16], True)])
+def test_rgms_tiled_static_weights(dev, group, buckets, weighted):
+    """The plan that was promised unchanging slot weights: zero-weight (padding) slots are left out
+    of the edge index and the weights travel inside 8-byte records.  Same result as the oracle."""
+    cfg = datasets.config5(n=20000, num_rels=9, num_edges=200000, seed=11)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    got, x32, w32, av = _run(dev, csf, cfg["m"], cfg["n"], cfg["x"], cfg["w"], group, buckets, weighted, static=True)
+    _check(got, csf, av, x32, w32, cfg["m"], f"static group={group}")
+
+
+def test_rgms_static_weights_edge_cases(dev):
+    """Every slot weight zero: nothing is launched and Y keeps its content.  The promise cannot be
+    changed after the first launch.  bf16 weights take the same path."""
+    from sparsetir_amd._lib import SparseTIRError, lib, check
+    import ctypes
+    cfg = datasets.config5(n=6000, num_rels=4, num_edges=40000, seed=12)
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    R, fin, fout, buckets, group = 4, 32, 32, [1, 2, 4, 8], 64
+    rb = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    zero_triples, triples, mids = [], [], []
+    for b in range(len(buckets)):
+        zero_triples += [torch.zeros(mask[b].size, dtype=torch.bfloat16, device=dev), t(rows[b].ravel()), t(cols[b].ravel())]
+        triples += [t(mask[b].astype(np.float32).ravel()).bfloat16(), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    groups = [c.shape[0] for c in cols]
+    w = t(cfg["w"].ravel()).bfloat16()
+    x = t(cfg["x"].ravel()).bfloat16()
+    y = torch.full((cfg["m"] * fout,), 3.0, device=dev)
+    ops.build_rgms(cfg["m"], cfg["n"], R, fin, fout, rb, buckets, groups, torch.bfloat16, static_weights=True)(
+        w, x, y, *zero_triples, *mids)
+    torch.cuda.synchronize()
+    assert bool((y == 3.0).all())
+    # bf16 with the 0/1 mask: equals the plan without the promise
+    ya, yb = torch.zeros(cfg["m"] * fout, device=dev), torch.zeros(cfg["m"] * fout, device=dev)
+    fa = ops.build_rgms(cfg["m"], cfg["n"], R, fin, fout, rb, buckets, groups, torch.bfloat16, static_weights=True)
+    fb = ops.build_rgms(cfg["m"], cfg["n"], R, fin, fout, rb, buckets, groups, torch.bfloat16)
+    fa(w, x, ya, *triples, *mids)
+    fb(w, x, yb, *triples, *mids)
+    torch.cuda.synchronize()
+    assert ya.abs().sum() > 0 and torch.allclose(ya, yb, rtol=1e-5, atol=1e-5)
+    with pytest.raises(SparseTIRError, match="launched already"):
+        check(lib().stir_rgms_plan_set_static_weights(fa._plan, 0))
 
 
 def test_rgms_tiled_repeat_calls_accumulate(dev):
