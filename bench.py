@@ -99,6 +99,9 @@ def parse():
     ap.add_argument("--buckets", type=str, default=None, help="comma separated ELL widths")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip CSR / SDDMM side measurements")
+    ap.add_argument("--profile", action="store_true",
+                    help="few launches per kernel and no graph replays: for runs under rocprofv3 --pmc, "
+                         "which serialises and slows every launch")
     ap.add_argument("--cpu-rows", type=int, default=10**9,
                     help="rows in the cpu_baseline sample (default: every row, about 6 s on one core)")
     return ap.parse_args()
@@ -127,9 +130,14 @@ def time_steps(fn, steps, warmup, torch):
     return wall, float(np.mean(dev_ms)) / 1e3, float(np.min(dev_ms)) / 1e3
 
 
+PROFILE_RUN = False  # set by --profile
+
+
 def time_small(fn, calls, warmup, torch, graph=True):
     """Three timings of a short kernel, in microseconds: events around every call, one event pair
     around a run of calls, and a captured graph of 20 launches replayed (device time only)."""
+    if PROFILE_RUN:
+        calls, warmup, graph = 3, 1, False
     _, per_call, _ = time_steps(fn, calls, warmup, torch)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -158,6 +166,8 @@ def time_small(fn, calls, warmup, torch, graph=True):
         e1.synchronize()
         out["us_graph"] = e0.elapsed_time(e1) * 1e3 / 100
         del g
+    else:
+        out["us_graph"] = None
     return out
 
 
@@ -184,8 +194,9 @@ def config2_sweep(torch, dev, ops, st, datasets, time_steps):
         c = torch.zeros(m * feat, device=dev)
         hyb = ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)
         csr = ops.build_csrmm(m, n, feat, nnz)
-        _, dh, _ = time_steps(lambda: hyb(x, c, *triples), 50, 5, torch)
-        _, dc, _ = time_steps(lambda: csr(ones, x, c, d_ptr, d_idx), 50, 5, torch)
+        reps = 3 if PROFILE_RUN else 50
+        _, dh, _ = time_steps(lambda: hyb(x, c, *triples), reps, 2, torch)
+        _, dc, _ = time_steps(lambda: csr(ones, x, c, d_ptr, d_idx), reps, 2, torch)
         byts = 8.0 * nnz + 4.0 * (m + 1) + 4.0 * n * feat + 4.0 * m * feat
         out[f"feat{feat}"] = {"hyb_us": dh * 1e6, "csr_us": dc * 1e6, "hyb_gflops": 2.0 * nnz * feat / dh / 1e9,
                               "hyb_alg_GBps": byts / dh / 1e9}
@@ -393,7 +404,9 @@ def roofline_block(wl, dev_mean, dev_min, probes=None):
 
 
 def main():
+    global PROFILE_RUN
     args = parse()
+    PROFILE_RUN = args.profile
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported: this build has no "
               "multi-GPU path (the kernel runs on one GPU's share at its real shape).", file=sys.stderr)

@@ -139,16 +139,20 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
       for (int v = 0; v < 16; ++v) acc[rs][t][v] = 0.f;
 
   const int p_begin = indptr[i];
-  const int ksteps = blk / kTileK;
-  const int steps = (indptr[i + 1] - p_begin) * ksteps;
+  const int nblk = indptr[i + 1] - p_begin;
+  const int steps = nblk * (blk / kTileK);
 
+  // The step to fetch next: block pb of the row, k offset k0.  The block column of the block after
+  // the current one is requested a whole block ahead, so that no step waits for an index before
+  // it can ask for its rows of X.
+  int pb = 0, k0 = 0;
+  int j_cur = nblk > 0 ? indices[p_begin] : 0;
+  int j_nxt = nblk > 1 ? indices[p_begin + 1] : 0;
   u32x4 xr[2 * NT];
   u32x4 ar;  // RS = 1 uses the first two words
-  auto fetch = [&](int it) {
-    const int p = p_begin + it / ksteps, k0 = (it % ksteps) * kTileK;
-    const int64_t j = indices[p];
-    const uint16_t* xb = X + ((int64_t)j * blk + k0) * feat + f0;
-    const uint16_t* ab = A + (int64_t)p * blk * blk + (int64_t)bi0 * blk + k0;
+  auto fetch = [&]() {
+    const uint16_t* xb = X + ((int64_t)j_cur * blk + k0) * feat + f0;
+    const uint16_t* ab = A + (int64_t)(p_begin + pb) * blk * blk + (int64_t)bi0 * blk + k0;
 #pragma unroll
     for (int q = 0; q < 2 * NT; ++q)
       xr[q] = xlive[q] ? *reinterpret_cast<const u32x4*>(xb + xoff[q]) : u32x4{0, 0, 0, 0};
@@ -158,9 +162,16 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
     } else {
       ar = *reinterpret_cast<const u32x4*>(ab + aoff);
     }
+    k0 += kTileK;
+    if (k0 == blk) {
+      k0 = 0;
+      ++pb;
+      j_cur = j_nxt;
+      if (pb + 1 < nblk) j_nxt = indices[p_begin + pb + 1];
+    }
   };
 
-  if (steps > 0) fetch(0);
+  if (steps > 0) fetch();
   for (int it = 0; it < steps; ++it) {
     char* stage = lds + (it & 1) * SB;
 #pragma unroll
@@ -169,7 +180,7 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
       *reinterpret_cast<u32x2*>(stage + XB + tid * 8) = u32x2{ar[0], ar[1]};
     else
       *reinterpret_cast<u32x4*>(stage + XB + tid * 16) = ar;
-    if (it + 1 < steps) fetch(it + 1);
+    if (it + 1 < steps) fetch();
     __syncthreads();  // stage `it` is complete; the other stage's readers passed the previous barrier
     u32x4 a[RS][2];
 #pragma unroll
@@ -190,17 +201,22 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
       }
     }
   }
-  // acc[rs][t][v] is row 32 rs + (v%4) + 4h + 8(v/4), column n of the t-th 32x32 tile
+  // acc[rs][t][v] is row 32 rs + (v%4) + 4h + 8(v/4), column n of the t-th 32x32 tile.
+  // The row stride is made opaque here: when this function is inlined into a loop over tiles,
+  // the sixteen row offsets would otherwise be computed once before that loop and held in
+  // registers throughout it (60 registers, halving the resident workgroups).
+  int row_stride = feat;
+  asm volatile("" : "+s"(row_stride));
 #pragma unroll
   for (int rs = 0; rs < RS; ++rs) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int fcol = f0 + (wave * NT + t) * 32;
       if (fcol >= feat) continue;
+      const int64_t first = ((int64_t)i_out * blk + bi0 + 32 * rs + 4 * h) * row_stride + fcol + n;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int row = 32 * rs + (v & 3) + 4 * h + 8 * (v >> 2);
-        const int64_t off = ((int64_t)i_out * blk + bi0 + row) * feat + fcol + n;
+        const int64_t off = first + (int64_t)((v & 3) + 8 * (v >> 2)) * row_stride;
         if constexpr (OUT == 1)
           __builtin_nontemporal_store(acc[rs][t][v], static_cast<float*>(Y) + off);
         else
@@ -289,11 +305,12 @@ __device__ __forceinline__ int sweep_my_slices(uint32_t* __restrict__ lds, uint1
     });
   }
   __syncthreads();
-  // exclusive scan over hist in (bin, wavefront) order: 16 consecutive entries per thread
+  // exclusive scan over hist in (bin, wavefront) order: 16 consecutive entries per thread, read
+  // twice rather than held in registers (the tile loop decides the kernel's register count)
   {
-    uint32_t local[16], sum = 0;
-#pragma unroll
-    for (int q = 0; q < 16; ++q) local[q] = hist[tid * 16 + q], sum += local[q];
+    uint32_t sum = 0;
+#pragma unroll 1
+    for (int q = 0; q < 16; ++q) sum += hist[tid * 16 + q];
     uint32_t incl = sum;
 #pragma unroll
     for (int off = 1; off < kWave; off <<= 1) {
@@ -305,8 +322,12 @@ __device__ __forceinline__ int sweep_my_slices(uint32_t* __restrict__ lds, uint1
     __syncthreads();
     uint32_t base = incl - sum;
     for (int q = 0; q < wave; ++q) base += wave_total[q];
-#pragma unroll
-    for (int q = 0; q < 16; ++q) hist[tid * 16 + q] = base, base += local[q];
+#pragma unroll 1
+    for (int q = 0; q < 16; ++q) {
+      const uint32_t v = hist[tid * 16 + q];
+      hist[tid * 16 + q] = base;
+      base += v;
+    }
   }
   __syncthreads();
   // placement, in slice order inside every (bin, wavefront) run: stable
@@ -351,6 +372,7 @@ __global__ __launch_bounds__(256) void bsr_spmm_sweep_kernel(int blk, int feat, 
   // unit u = f_tile + f_tiles * part (part: every parts-th slice by rank); XCD x takes units x, x + 8, ...
   const int units = f_tiles * parts;
   int part_of_items = -1, count = 0;
+#pragma unroll 1
   for (int u = xcd; u < units; u += 8) {
     const int f_tile = u % f_tiles, part = u / f_tiles;
     if (part != part_of_items) {
@@ -358,6 +380,7 @@ __global__ __launch_bounds__(256) void bsr_spmm_sweep_kernel(int blk, int feat, 
       count = sweep_my_slices(lds, items, indptr, slices, sub, G, w, parts, part);
       part_of_items = part;
     }
+#pragma unroll 1
     for (int r = 0; r < count; ++r) {
       const int slice = items[r];
       const int i = slice / sub, bi0 = (slice % sub) * (32 * RS);
