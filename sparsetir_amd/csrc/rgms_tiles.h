@@ -33,6 +33,13 @@ struct TileIndex {
   void* d_units = nullptr;  // units x 16 bytes
   void* d_wpack = nullptr;  // W in MFMA operand order, rewritten by every launch
   size_t wpack_bytes = 0;
+  // For the launch whose workgroups stay resident (W in LDS): the sorted edges cut into equal
+  // shares of steps, one per team of wavefronts, each share a list of units.  Built at the first
+  // such launch and again when the number of teams changes.
+  std::vector<int64_t> tile_begin;  // host copy: first sorted edge of every tile, then the edge count
+  int64_t share_teams = 0;
+  void* d_share_ptr = nullptr;    // share_teams + 1 offsets into d_share_units
+  void* d_share_units = nullptr;  // units x 16 bytes, grouped by team
 };
 
 // Builds the index on `stream` (synchronises; allocates).  A no-op when it already exists for

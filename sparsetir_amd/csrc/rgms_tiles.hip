@@ -14,6 +14,10 @@
 
 #include <hipcub/hipcub.hpp>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 namespace stir {
 namespace {
 
@@ -238,8 +242,13 @@ __device__ __forceinline__ f32x16 stage2(u32x4 sa, const float* t, f32x16 acc) {
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       const h2 hi = __builtin_amdgcn_cvt_pkrtz(t[2 * d], t[2 * d + 1]);
-      const h2 lo = __builtin_amdgcn_cvt_pkrtz(t[2 * d] - (float)hi[0], t[2 * d + 1] - (float)hi[1]);
       bh[d] = __builtin_bit_cast(uint32_t, hi);
+      // residuals t - hi with the fp16 halves read in place (one instruction each instead of a
+      // conversion and a subtraction)
+      float r0, r1;
+      asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r0) : "v"(bh[d]), "v"(t[2 * d]));
+      asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r1) : "v"(bh[d]), "v"(t[2 * d + 1]));
+      const h2 lo = __builtin_amdgcn_cvt_pkrtz(r0, r1);
       bl[d] = __builtin_bit_cast(uint32_t, lo);
     }
     acc = mfma32<false>(sa, bh, acc);
@@ -420,6 +429,288 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
   }
 }
 
+// ---- the same computation by resident workgroups that keep all of W in LDS
+//
+// When W (num_rels x feat_in x feat_out 16-bit values) fits beside the S tiles in the 160 KB of LDS
+// of a compute unit, one workgroup per compute unit stays for the whole launch: it brings W into
+// LDS once, already in MFMA operand order (so no separate packing launch and no W traffic through
+// the vector memory path, which otherwise carries twice the bytes of the gathered X rows), and
+// its T teams of four wavefronts each work through one share of the launch.  The shares are cut
+// from the sorted edges by the host so that every team gets the same number of steps (build_shares).
+// The X rows of a step are requested one step ahead and the records three steps ahead; a team's
+// wavefronts synchronise among themselves only, through a counter in LDS.
+constexpr int kSBytes = kTileRows * kSStride * 2;  // S tile of one wavefront
+constexpr int kTeamLds = kUnitWaves * kSBytes;
+constexpr int kLdsMaxKK = 4;
+
+// lane -> 16-byte slot of its operand inside a fragment of W in LDS: consecutive lanes stay on
+// distinct banks, and so do the eight writers of one column phase (see the fill loop)
+__device__ __forceinline__ int w_slot(int lane) { return lane ^ ((lane >> 3) & 7); }
+
+template <int KK, bool BF16, typename Rec, int T>
+__global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
+    const int32_t* __restrict__ share_ptr, const Unit* __restrict__ share_units, const Rec* __restrict__ edges, int m,
+    int feat_out, int num_rels, const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
+    float* __restrict__ Y) {
+  constexpr int FIN = KK * 16;
+  constexpr bool kPacked = sizeof(Rec) == sizeof(PackedEdge);
+  constexpr int kThreads = 64 * kUnitWaves * T, kTeamThreads = 64 * kUnitWaves;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int ntiles = feat_out / 32;
+  const int frags = num_rels * ntiles * KK;
+  u32x4* Wl = reinterpret_cast<u32x4*>(lds);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int team = wave / kUnitWaves, tw = wave % kUnitWaves;
+  const int mrow = lane & 31, h = lane >> 5;
+  constexpr int kStride = kUnitWaves * kStepEdges;  // edges between a wavefront's steps
+
+  // lanes past the last edge of a unit repeat it (with weight zero, see `live`)
+  // (indexed from the unit's first edge, so that the lane's part of the address is 32 bits wide)
+  auto record = [&](const Unit& un, int e) {
+    return (edges + un.edge_begin)[min((uint32_t)(e + mrow), (uint32_t)(un.edge_count - 1))];
+  };
+  auto weight_of = [&](const Rec& rec) -> uint16_t {
+    if constexpr (kPacked)
+      return (uint16_t)(rec.w_rel_dl >> 16);
+    else
+      return *reinterpret_cast<const GlobalU16*>(((uint64_t)rec.w_hi << 32) | rec.w_lo);
+  };
+  auto fetch = [&](const Rec& rec, u32x4 (&x)[KK], uint16_t& wb) {
+    // byte offsets into X fit 32 bits (checked by the host)
+    const uint32_t at = (uint32_t)rec.src * (FIN * 2) + 16 * h;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+      x[kk] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(X) + at + 32 * kk);
+    wb = weight_of(rec);
+  };
+  // What a pass (one unit, one tile of 32 output features) starts from: the records of the
+  // wavefront's first three steps and the rows of X of the first.  The records are requested when
+  // the pass before begins and the rows when its last step is done, so that a pass does not open
+  // with two memory round trips; unit descriptors are read two units ahead for the same reason.
+  Rec cur, nx1, nx2;
+  u32x4 xa[KK], xb[KK];
+  uint16_t wa, wb;
+  auto first_records = [&](const Unit& un, Rec& r0, Rec& r1, Rec& r2) {
+    const int e = tw * kStepEdges;
+    r0 = record(un, e), r1 = record(un, e + kStride), r2 = record(un, e + 2 * kStride);
+  };
+
+  // the team's share of the launch: units share_ptr[team] .. share_ptr[team + 1].  Its first
+  // descriptors and records are requested before W is brought in, which takes as long.
+  const int u_first = share_ptr[blockIdx.x * T + team], u_last = share_ptr[blockIdx.x * T + team + 1];
+  Unit u, u1;
+  u.edge_begin = 0, u.edge_count = 1, u.tile_flag = 0;
+  if (u_first < u_last) u = share_units[u_first];
+  u1 = u;
+  if (u_first + 1 < u_last) u1 = share_units[u_first + 1];
+  first_records(u, cur, nx1, nx2);
+
+  // W[rel][16kk + 8h + i][32nt + 8c + j], i, j < 8, is one thread's block: eight 16-byte loads,
+  // transposed in registers into the operands of lanes (8c + j, h).  Eight consecutive threads
+  // take the eight (c, h) of a fragment, so their stores of equal j go to distinct banks.  Two
+  // blocks per thread are in flight.
+  {
+    auto block_rows = [&](int blk, u32x4 (&in)[8]) {
+      const int g = blk & 7, f = blk >> 3;
+      const int kk = f % KK, nt = (f / KK) % ntiles, rel = f / (KK * ntiles);
+      const uint16_t* w = W + ((int64_t)rel * FIN + 16 * kk + 8 * (g >> 2)) * feat_out + 32 * nt + 8 * (g & 3);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) in[i] = *reinterpret_cast<const u32x4*>(w + (int64_t)i * feat_out);
+    };
+    auto block_store = [&](int blk, const u32x4 (&in)[8]) {
+      const int g = blk & 7, f = blk >> 3;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          o[d] = __builtin_amdgcn_perm(in[2 * d + 1][j / 2], in[2 * d][j / 2], (j & 1) ? 0x07060302u : 0x05040100u);
+        Wl[f * 64 + w_slot(8 * g + j)] = o;
+      }
+    };
+    const int blocks = frags * 8;
+    for (int blk = threadIdx.x; blk < blocks; blk += 2 * kThreads) {
+      u32x4 in0[8], in1[8];
+      const bool second = blk + kThreads < blocks;
+      block_rows(blk, in0);
+      if (second) block_rows(blk + kThreads, in1);
+      block_store(blk, in0);
+      if (second) block_store(blk + kThreads, in1);
+    }
+  }
+  unsigned char* team_lds = lds + (size_t)frags * 1024 + team * kTeamLds;
+  uint16_t* S = reinterpret_cast<uint16_t*>(team_lds + tw * kSBytes);
+  float* my_partial = reinterpret_cast<float*>(team_lds + tw * kSBytes);  // 8 registers x 64 lanes, over S
+  // The team's wavefronts meet at a counter in LDS (a workgroup barrier would tie the teams of the
+  // workgroup together; every wavefront of a team runs the same sequence of meetings, so each
+  // wait ends).  The counter sits in the unused tail of row 26 of the first S tile, which neither
+  // the S accesses nor the partial sums (the first 2 KB of each tile) touch.
+  uint32_t* meet = reinterpret_cast<uint32_t*>(team_lds + 26 * kSStride * 2 + 64);
+  uint32_t met = 0;
+  auto team_barrier = [&]() {
+    met += kUnitWaves;
+    if (lane == 0) __hip_atomic_fetch_add(meet, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    while (__hip_atomic_load(meet, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < met) __builtin_amdgcn_s_sleep(1);
+  };
+  {
+    uint32_t* s32 = reinterpret_cast<uint32_t*>(S);
+#pragma unroll
+    for (int k = 0; k < kSBytes / 4 / 64; ++k) s32[lane + 64 * k] = 0;  // the meeting counter too
+  }
+  __syncthreads();
+  if (u_first >= u_last) return;  // no workgroup barrier below this line
+  const int slot = w_slot(lane);
+  const int jcol = 16 * (mrow >> 4) + 8 * ((mrow >> 2) & 1) + 4 * ((mrow >> 3) & 1) + (mrow & 3);
+  const int team_tid = threadIdx.x & (kTeamThreads - 1);
+  constexpr int kSumIters = 16 * 32 / kTeamThreads;
+  fetch(cur, xa, wa);
+  for (int ui = u_first;; ++ui) {
+    const bool more_units = ui + 1 < u_last;
+    Unit u2 = u1;
+    if (ui + 2 < u_last) u2 = share_units[ui + 2];
+    const int e_end = u.edge_count, e_first = tw * kStepEdges;  // counted from the unit's first edge
+    const int tile = u.tile_flag >> 1;
+    const bool atomic = u.tile_flag & 1;
+
+    for (int nti = 0; nti < ntiles; ++nti) {
+      // The next pass: the same unit at the next feature tile, or the next unit.
+      const bool next_pass = nti + 1 < ntiles || more_units;
+      Rec p0 = cur, p1 = cur, p2 = cur;
+      if (next_pass) first_records(nti + 1 < ntiles ? u : u1, p0, p1, p2);
+      float yold[2][kSumIters];  // what the tile's rows hold now: needed at the end only
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int k = 0; k < kSumIters; ++k) {
+          const int elem = team_tid + kTeamThreads * k;
+          const int64_t yrow = (int64_t)tile * kTileRows + 16 * half + (elem >> 5);
+          yold[half][k] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + (elem & 31)] : 0.f;
+        }
+      f32x16 acc2;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc2[v] = 0.f;
+      auto step = [&](const Rec& rec, const u32x4 (&x)[KK], uint16_t wbits, int e0) {
+        const int left = min(kStepEdges, e_end - e0);  // uniform
+        const bool live = mrow < left;
+        int rel, dl;
+        if constexpr (kPacked)
+          rel = (int)((rec.w_rel_dl >> 5) & (kPackedMaxRels - 1)), dl = (int)(rec.w_rel_dl & 31);
+        else
+          rel = (int)(rec.rel_dl >> 5), dl = (int)(rec.rel_dl & 31);
+
+        // ---- stage 1: one MFMA chain per run of equal relation (the step is sorted by relation)
+        f32x16 acc1;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc1[v] = 0.f;  // a constant operand of the first MFMA, not 16 moves
+        int rq = __builtin_amdgcn_readlane(rel, 0);
+        int pos_e = __popcll(__ballot(rel == rq) & 0xffffffffull);
+        if (pos_e >= kStepEdges) {
+          // one relation in the whole step: nothing to mask
+          const u32x4* w = Wl + (rq * ntiles + nti) * (KK * 64) + slot;
+#pragma unroll
+          for (int kk = 0; kk < KK; ++kk) acc1 = mfma32<BF16>(x[kk], w[kk * 64], acc1);
+        } else {
+          auto add_run = [&](int r_, f32x16 c) {
+            const u32x4* w = Wl + (r_ * ntiles + nti) * (KK * 64) + slot;
+            const bool sel = rel == r_;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+              u32x4 a_;
+#pragma unroll
+              for (int d = 0; d < 4; ++d) a_[d] = sel ? x[kk][d] : 0u;
+              c = mfma32<BF16>(a_, w[kk * 64], c);
+            }
+            return c;
+          };
+          acc1 = add_run(rq, acc1);
+          do {
+            rq = __builtin_amdgcn_readlane(rel, pos_e);
+            pos_e += __popcll(__ballot(rel == rq) & 0xffffffffull);
+            acc1 = add_run(rq, acc1);
+          } while (pos_e < kStepEdges);
+        }
+
+        // ---- stage 2
+        if (h == 0) S[dl * kSStride + jcol] = live ? wbits : (uint16_t)0;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const u32x4 sa0 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 8 * h);
+        u32x4 sa1 = {0u, 0u, 0u, 0u};
+        if (left > 16) sa1 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 16 + 8 * h);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (h == 0) S[dl * kSStride + jcol] = 0;
+        float t[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) t[v] = acc1[v];
+        acc2 = stage2<BF16>(sa0, t, acc2);
+        if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
+      };
+      // Two steps per turn of the loop, so that the two sets of X registers swap roles without
+      // copies: while a step is computed, the rows of X of the step after it are on their way,
+      // and so are the records three steps ahead.
+#pragma unroll 1
+      for (int e0 = e_first; e0 < e_end; e0 += 2 * kStride) {
+        fetch(nx1, xb, wb);
+        const Rec nx3 = record(u, e0 + 3 * kStride);
+        step(cur, xa, wa, e0);
+        if (e0 + kStride >= e_end) break;
+        fetch(nx2, xa, wa);
+        const Rec nx4 = record(u, e0 + 4 * kStride);
+        step(nx1, xb, wb, e0 + kStride);
+        cur = nx2, nx1 = nx3, nx2 = nx4;
+      }
+
+      // Everything requested so far has had the whole pass to arrive.  Naming the old values of
+      // Y here settles them, so that the stores below do not wait for the loads that follow.
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int k = 0; k < kSumIters; ++k) asm volatile("" : "+v"(yold[half][k]));
+      if (next_pass) {
+        cur = p0, nx1 = p1, nx2 = p2;
+        fetch(cur, xa, wa);
+      }
+
+      // ---- add the team's four tiles, 16 rows at a time (the partial sums lie over the S tiles),
+      // and write back.  acc2[v] of lane (n, h) is row (v%4) + 4h + 8(v/4), output feature 32 nti + n.
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if (half == 1) team_barrier();  // the sums of the first half have been read
+#pragma unroll
+        for (int v = 0; v < 8; ++v) my_partial[v * 64 + lane] = acc2[8 * half + v];
+        team_barrier();
+#pragma unroll
+        for (int k = 0; k < kSumIters; ++k) {
+          const int elem = team_tid + kTeamThreads * k, row = elem >> 5, col = elem & 31;
+          const int at = ((row & 3) + 4 * (row >> 3)) * 64 + col + 32 * ((row >> 2) & 1);
+          float sum = 0.f;
+#pragma unroll
+          for (int w = 0; w < kUnitWaves; ++w) sum += reinterpret_cast<const float*>(team_lds + w * kSBytes)[at];
+          const int64_t yrow = (int64_t)tile * kTileRows + 16 * half + row;
+          if (yrow < m) {
+            float* y = Y + yrow * feat_out + 32 * nti + col;
+            if (atomic)
+              __hip_atomic_fetch_add(y, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else
+              *y = yold[half][k] + sum;
+          }
+        }
+      }
+      team_barrier();
+      {
+        // the partial sums lay over the first 2 KB of the S tile
+        uint32_t* s32 = reinterpret_cast<uint32_t*>(S);
+#pragma unroll
+        for (int k = 0; k < 2048 / 4 / 64; ++k) s32[lane + 64 * k] = 0;
+      }
+    }
+    if (!more_units) break;
+    u = u1, u1 = u2;
+  }
+}
+
 struct DevBuf {
   void* p = nullptr;
   ~DevBuf() {
@@ -436,12 +727,108 @@ int bit_length(uint64_t x) {
   return b;
 }
 
+// LDS a workgroup may ask for on the current device (0 on failure)
+size_t lds_bytes_per_workgroup() {
+  static thread_local int cached_dev = -1;
+  static thread_local size_t cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev != cached_dev) {
+    int bytes = 0;
+    if (hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
+    cached_dev = dev, cached = (size_t)bytes;
+  }
+  return cached;
+}
+
+// Kernels that use more than 64 KB of dynamic LDS have to be told so once per device.
+int allow_lds(const void* fn) {
+  static std::mutex mu;
+  static std::set<std::pair<int, const void*>> done;
+  int dev = 0;
+  STIR_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({dev, fn})) return 0;
+  STIR_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_per_workgroup()));
+  done.insert({dev, fn});
+  return 0;
+}
+
+// Four teams (16 wavefronts of 128 registers) only for the variants that fit those registers.
+constexpr bool resident_four_teams(bool packed, int kk) { return packed && kk <= 2; }
+int resident_max_teams(bool packed, int kk) { return resident_four_teams(packed, kk) ? 4 : 3; }
+
+template <int KK, bool BF16, typename Rec>
+int launch_resident(int teams, dim3 grid, size_t lds, hipStream_t stream, const int32_t* share_ptr,
+                    const Unit* share_units, const Rec* edges, int m, int feat_out, int num_rels, const uint16_t* W,
+                    const uint16_t* X, float* Y) {
+  auto go = [&](auto* fn) -> int {
+    if (int rc = allow_lds(reinterpret_cast<const void*>(fn))) return rc;
+    hipLaunchKernelGGL(fn, grid, dim3(64 * kUnitWaves * teams), lds, stream, share_ptr, share_units, edges, m, feat_out,
+                       num_rels, W, X, Y);
+    return 0;
+  };
+  if (teams == 2) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 2>);
+  if (teams == 3) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 3>);
+  if constexpr (resident_four_teams(sizeof(Rec) == sizeof(PackedEdge), KK)) {
+    if (teams == 4) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 4>);
+  }
+  return fail("rgms: no kernel for %d teams", teams);
+}
+
+// Cuts the sorted edges into `teams` shares of (nearly) equal numbers of steps, in tile order.  A
+// tile that lies inside one share is a unit that writes its rows of Y alone; the pieces of a
+// tile that is cut by a share boundary all add with atomics.
+int build_shares(TileIndex& ix, int64_t teams, hipStream_t stream) {
+  const int64_t tiles = (int64_t)ix.tile_begin.size() - 1;
+  std::vector<int64_t> first_step(size_t(tiles + 1), 0);
+  for (int64_t t = 0; t < tiles; ++t)
+    first_step[t + 1] = first_step[t] + ceil_div(ix.tile_begin[t + 1] - ix.tile_begin[t], (int64_t)kStepEdges);
+  const int64_t total = first_step[tiles];
+  std::vector<int32_t> ptr(size_t(teams + 1), 0);
+  std::vector<Unit> units;
+  units.reserve(size_t(tiles + 2 * teams));
+  int64_t t = 0;
+  for (int64_t g = 0; g < teams; ++g) {
+    // steps [s0, s1) of the numbering over all tiles
+    const int64_t s0 = total * g / teams, s1 = total * (g + 1) / teams;
+    ptr[g] = (int32_t)units.size();
+    while (t < tiles && first_step[t + 1] <= s0) ++t;
+    for (int64_t k = t; k < tiles && first_step[k] < s1; ++k) {
+      const int64_t a = std::max(s0, first_step[k]), b = std::min(s1, first_step[k + 1]);
+      if (a >= b) continue;
+      const bool whole = a == first_step[k] && b == first_step[k + 1];
+      Unit un;
+      un.edge_begin = ix.tile_begin[k] + (a - first_step[k]) * kStepEdges;
+      un.edge_count = (int32_t)(std::min(ix.tile_begin[k + 1], ix.tile_begin[k] + (b - first_step[k]) * kStepEdges) -
+                                un.edge_begin);
+      un.tile_flag = (int32_t)(k << 1) | (whole ? 0 : 1);
+      units.push_back(un);
+    }
+  }
+  ptr[teams] = (int32_t)units.size();
+  STIR_REQUIRE(units.size() < (size_t(1) << 31), "rgms: too many units");
+  if (ix.d_share_ptr) STIR_HIP(hipFree(ix.d_share_ptr));
+  if (ix.d_share_units) STIR_HIP(hipFree(ix.d_share_units));
+  ix.d_share_ptr = ix.d_share_units = nullptr;
+  ix.share_teams = 0;
+  STIR_HIP(hipMalloc(&ix.d_share_ptr, sizeof(int32_t) * ptr.size()));
+  STIR_HIP(hipMalloc(&ix.d_share_units, sizeof(Unit) * std::max<size_t>(units.size(), 1)));
+  STIR_HIP(hipMemcpyAsync(ix.d_share_ptr, ptr.data(), sizeof(int32_t) * ptr.size(), hipMemcpyHostToDevice, stream));
+  STIR_HIP(hipMemcpyAsync(ix.d_share_units, units.data(), sizeof(Unit) * units.size(), hipMemcpyHostToDevice, stream));
+  STIR_HIP(hipStreamSynchronize(stream));  // the host vectors go away
+  ix.share_teams = teams;
+  return 0;
+}
+
 }  // namespace
 
 void tile_index_free(TileIndex& ix) {
   if (ix.d_edges) (void)hipFree(ix.d_edges);
   if (ix.d_units) (void)hipFree(ix.d_units);
   if (ix.d_wpack) (void)hipFree(ix.d_wpack);
+  if (ix.d_share_ptr) (void)hipFree(ix.d_share_ptr);
+  if (ix.d_share_units) (void)hipFree(ix.d_share_units);
   ix = TileIndex();
 }
 
@@ -452,7 +839,11 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   STIR_REQUIRE(num_rels > 0 && num_rels < (1 << 26), "rgms: num_rels=%d out of range", num_rels);
   if (ix.d_edges) STIR_HIP(hipFree(ix.d_edges));
   if (ix.d_units) STIR_HIP(hipFree(ix.d_units));
-  ix.d_edges = ix.d_units = nullptr;
+  if (ix.d_share_ptr) STIR_HIP(hipFree(ix.d_share_ptr));
+  if (ix.d_share_units) STIR_HIP(hipFree(ix.d_share_units));
+  ix.d_edges = ix.d_units = ix.d_share_ptr = ix.d_share_units = nullptr;
+  ix.share_teams = 0;
+  ix.tile_begin.clear();
   ix.m = -1;
   ix.edges = ix.units = 0;
   std::vector<DevBucket> host;
@@ -530,6 +921,9 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   STIR_HIP(hipcub::DeviceScan::ExclusiveSum(tmp.p, scan_bytes, count.as<const int32_t>(), ubegin.as<int32_t>(),
                                             (int)(tiles + 1), stream));
   int32_t h_bad = 0, h_units = 0;
+  ix.tile_begin.resize(size_t(tiles + 1));
+  STIR_HIP(hipMemcpyAsync(ix.tile_begin.data(), begin.p, sizeof(int64_t) * size_t(tiles + 1), hipMemcpyDeviceToHost,
+                          stream));
   STIR_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
   STIR_HIP(hipMemcpyAsync(&h_units, ubegin.as<int32_t>() + tiles, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
   STIR_HIP(hipStreamSynchronize(stream));
@@ -585,7 +979,58 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   const int kk_count = feat_in / 16;
   const int64_t frags = (int64_t)ix.num_rels * (feat_out / 32) * kk_count;
   STIR_REQUIRE(frags < (int64_t(1) << 25), "rgms: W of %lld operand fragments exceeds the 32-bit fragment offsets", (long long)frags);
-  const size_t need = size_t(frags) * 64 * sizeof(u32x4);
+  const Unit* units = static_cast<const Unit*>(ix.d_units);
+  const Edge* edges = static_cast<const Edge*>(ix.d_edges);
+  const PackedEdge* pedges = static_cast<const PackedEdge*>(ix.d_edges);
+  const uint16_t* X = static_cast<const uint16_t*>(d_X);
+  const uint16_t* W = static_cast<const uint16_t*>(d_W);
+
+  // W resident in LDS when it fits beside the S tiles of at least two teams
+  const size_t w_bytes = size_t(frags) * 64 * sizeof(u32x4);
+  int teams = 0;
+  if (kk_count <= kLdsMaxKK && reinterpret_cast<uintptr_t>(d_W) % 16 == 0 &&
+      (int64_t)ix.n * feat_in * 2 < (int64_t(1) << 32)) {
+    const size_t lds_limit = lds_bytes_per_workgroup();
+    // four teams (16 wavefronts, 128 registers each) only where the kernel fits those registers
+    const int tmax = resident_max_teams(ix.packed_records, kk_count);
+    for (int t = tmax; t >= 2 && teams == 0; --t)
+      if (w_bytes + size_t(t) * kTeamLds <= lds_limit) teams = t;
+  }
+  if (teams) {
+    const size_t lds = w_bytes + size_t(teams) * kTeamLds;
+    // one workgroup per compute unit, fewer when a team would get less than a handful of steps
+    const int64_t steps_bound = ix.edges / kStepEdges + (int64_t)ix.tile_begin.size();
+    const int64_t wgs = std::min<int64_t>(std::max(1, compute_units()), ceil_div(steps_bound, (int64_t)teams * 8));
+    if (ix.share_teams != wgs * teams)
+      if (int rc = build_shares(ix, wgs * teams, stream)) return rc;
+    const dim3 grid((unsigned)wgs);
+    const int32_t* share_ptr = static_cast<const int32_t*>(ix.d_share_ptr);
+    const Unit* share_units = static_cast<const Unit*>(ix.d_share_units);
+#define STIR_LDS_R(KKV, BF, REC, PTR)                                                                   \
+  if (int rc = launch_resident<KKV, BF, REC>(teams, grid, lds, stream, share_ptr, share_units, PTR, ix.m, feat_out, \
+                                             ix.num_rels, W, X, d_Y))                                  \
+    return rc
+#define STIR_LDS(KKV)                                                                          \
+  case KKV:                                                                                    \
+    if (ix.packed_records) {                                                                   \
+      if (bf16) { STIR_LDS_R(KKV, true, PackedEdge, pedges); } else { STIR_LDS_R(KKV, false, PackedEdge, pedges); } \
+    } else {                                                                                   \
+      if (bf16) { STIR_LDS_R(KKV, true, Edge, edges); } else { STIR_LDS_R(KKV, false, Edge, edges); } \
+    }                                                                                          \
+    break
+    switch (kk_count) {
+      STIR_LDS(1);
+      STIR_LDS(2);
+      STIR_LDS(3);
+      STIR_LDS(4);
+    }
+#undef STIR_LDS
+#undef STIR_LDS_R
+    STIR_LAUNCH_CHECK();
+    return 0;
+  }
+
+  const size_t need = w_bytes;
   if (need > ix.wpack_bytes) {
     if (ix.d_wpack) STIR_HIP(hipFree(ix.d_wpack));
     ix.d_wpack = nullptr;
@@ -595,13 +1040,9 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   }
   u32x4* Wp = static_cast<u32x4*>(ix.d_wpack);
   hipLaunchKernelGGL(pack_w_kernel, dim3((unsigned)ceil_div(frags, 4)), dim3(256), 0, stream,
-                     static_cast<const uint16_t*>(d_W), Wp, frags, kk_count, feat_out);
+                     W, Wp, frags, kk_count, feat_out);
   STIR_LAUNCH_CHECK();
   const dim3 grid((unsigned)ix.units), block(64 * kUnitWaves);
-  const Unit* units = static_cast<const Unit*>(ix.d_units);
-  const Edge* edges = static_cast<const Edge*>(ix.d_edges);
-  const PackedEdge* pedges = static_cast<const PackedEdge*>(ix.d_edges);
-  const uint16_t* X = static_cast<const uint16_t*>(d_X);
 #define STIR_TILES_R(KKV, BF, REC, PTR) \
   hipLaunchKernelGGL((rgms_tile_kernel<KKV, BF, REC>), grid, block, 0, stream, units, PTR, ix.m, feat_out, Wp, X, d_Y)
 #define STIR_TILES(KKV)                                                                          \
@@ -629,3 +1070,4 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
 }
 
 }  // namespace stir
+

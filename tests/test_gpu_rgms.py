@@ -386,3 +386,49 @@ def test_rgms_tiled_random_shapes(dev, seed):
     err = np.abs(got - want)
     assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), (
         f"R={R} m={m} n={n} group={group} widths={widths} fin={fin} fout={fout}: worst {err.max():.3e}")
+
+
+@pytest.mark.parametrize("R,fin,fout,static", [
+    (60, 32, 32, True),    # W of 120 KB: resident kernel, four teams of wavefronts per compute unit
+    (65, 32, 32, False),   # 130 KB: three teams
+    (68, 32, 32, True),    # 136 KB: two teams
+    (80, 32, 32, False),   # 160 KB: W does not fit the LDS, the kernel that reads W from memory
+    (20, 64, 64, True),    # two feature tiles out, four operand blocks in
+    (33, 48, 32, False),   # feat_in that is not a power of two
+])
+def test_rgms_tiled_sizes_of_w(dev, R, fin, fout, static):
+    """The destination-tiled operator picks its kernel by the size of W (num_rels x feat_in x
+    feat_out): all regimes against the float64 closed form, and W at an address that is not a
+    multiple of 16 bytes (served by the kernel that reads W from memory)."""
+    rng = np.random.default_rng(1000 + R)
+    m, n = 3001, 2500
+    per_rel = 60000 // R
+    pairs = [(rng.integers(0, m, per_rel), rng.integers(0, n, per_rel)) for _ in range(R)]
+    csf = _csf_from_pairs(pairs, n)
+    group, buckets = 64, [1, 2, 4, 8]
+    rows_bkt = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    assert slots_of(mask) >= 8192
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    x = t(rng.standard_normal((n, fin), dtype=np.float32)).half()
+    w_store = torch.zeros(R * fin * fout + 8, dtype=torch.float16, device=dev)
+    w_vals = t(rng.standard_normal((R, fin, fout), dtype=np.float32) * 0.1).half()
+    triples, mids = [], []
+    for b in range(len(buckets)):
+        triples += [t(mask[b].astype(np.float16).ravel()), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    ones = np.ones(len(csf[3]), np.float32)
+    x32, w32 = x.float().cpu().numpy(), w_vals.float().cpu().numpy()
+    want = rgms_f64(*csf, ones, x32, w32, m)
+    scale = rgms_f64(*csf, ones, np.abs(x32), np.abs(w32), m)
+    for shift in (0, 1):  # 0: aligned, 1: two bytes off
+        w = w_store[shift:shift + R * fin * fout]
+        w.copy_(w_vals.reshape(-1))
+        f = ops.build_rgms(m, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols], static_weights=static)
+        y = torch.zeros(m * fout, dtype=torch.float32, device=dev)
+        f(w, x.reshape(-1), y, *triples, *mids)
+        f(w, x.reshape(-1), y, *triples, *mids)  # the operator accumulates: twice the sum
+        torch.cuda.synchronize()
+        got = y.cpu().numpy().reshape(m, fout) / 2
+        err = np.abs(got - want)
+        assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), f"shift={shift}: worst {err.max():.3e}"
