@@ -347,16 +347,17 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
       // ---- stage 1
       f32x16 acc1;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc1[v] = 0.f;
-      auto add_run = [&](int rq, const u32x4* w) {
+      for (int v = 0; v < 16; ++v) acc1[v] = 0.f;  // a constant operand of the first MFMA, not 16 moves
+      auto add_run = [&](int rq, const u32x4* w, f32x16 c) {
         const bool sel = rel == rq;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
           u32x4 a;
 #pragma unroll
           for (int d = 0; d < 4; ++d) a[d] = sel ? xa[kk][d] : 0u;
-          acc1 = mfma32<BF16>(a, w[kk], acc1);
+          c = mfma32<BF16>(a, w[kk], c);
         }
+        return c;
       };
       bool single = pos >= kStepEdges;  // the requested runs cover the step ...
       if constexpr (PW > 1) single = single && r[1] < 0;  // ... and the first one does so alone
@@ -365,9 +366,10 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) acc1 = mfma32<BF16>(xa[kk], wf[0][kk], acc1);
       } else {
+        acc1 = add_run(r[0], wf[0], acc1);
 #pragma unroll
-        for (int q = 0; q < PW; ++q)
-          if (r[q] >= 0) add_run(r[q], wf[q]);
+        for (int q = 1; q < PW; ++q)
+          if (r[q] >= 0) acc1 = add_run(r[q], wf[q], acc1);
       }
       while (pos < kStepEdges) {  // steps with more than PW relations: one at a time
         const int rq = __builtin_amdgcn_readlane(rel, pos);
@@ -376,7 +378,7 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
         u32x4 wl[KK];
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) wl[kk] = w[kk * 64];
-        add_run(rq, wl);
+        acc1 = add_run(rq, wl, acc1);
       }
 
       // ---- stage 2
@@ -548,10 +550,16 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
   // the S accesses nor the partial sums (the first 2 KB of each tile) touch.
   uint32_t* meet = reinterpret_cast<uint32_t*>(team_lds + 26 * kSStride * 2 + 64);
   uint32_t met = 0;
-  auto team_barrier = [&]() {
+  auto team_arrive = [&]() {
     met += kUnitWaves;
     if (lane == 0) __hip_atomic_fetch_add(meet, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  auto team_wait = [&]() {
     while (__hip_atomic_load(meet, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < met) __builtin_amdgcn_s_sleep(1);
+  };
+  auto team_barrier = [&]() {
+    team_arrive();
+    team_wait();
   };
   {
     uint32_t* s32 = reinterpret_cast<uint32_t*>(S);
@@ -632,6 +640,7 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
         }
 
         // ---- stage 2
+        if (e0 == e_first) team_wait();  // the sums of the pass before have been read out of the S tiles
         if (h == 0) S[dl * kSStride + jcol] = live ? wbits : (uint16_t)0;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -673,6 +682,7 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
         fetch(cur, xa, wa);
       }
 
+      if (e_first >= e_end) team_wait();  // (a wavefront without steps has not met the others yet)
       // ---- add the team's four tiles, 16 rows at a time (the partial sums lie over the S tiles),
       // and write back.  acc2[v] of lane (n, h) is row (v%4) + 4h + 8(v/4), output feature 32 nti + n.
 #pragma unroll
@@ -687,7 +697,11 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
           const int at = ((row & 3) + 4 * (row >> 3)) * 64 + col + 32 * ((row >> 2) & 1);
           float sum = 0.f;
 #pragma unroll
-          for (int w = 0; w < kUnitWaves; ++w) sum += reinterpret_cast<const float*>(team_lds + w * kSBytes)[at];
+          for (int w = 0; w < kUnitWaves; ++w) {
+            float* part = reinterpret_cast<float*>(team_lds + w * kSBytes) + at;
+            sum += *part;
+            if (half == 1) *part = 0.f;  // the S tiles are all zeros again after the second half
+          }
           const int64_t yrow = (int64_t)tile * kTileRows + 16 * half + row;
           if (yrow < m) {
             float* y = Y + yrow * feat_out + 32 * nti + col;
@@ -698,13 +712,7 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
           }
         }
       }
-      team_barrier();
-      {
-        // the partial sums lay over the first 2 KB of the S tile
-        uint32_t* s32 = reinterpret_cast<uint32_t*>(S);
-#pragma unroll
-        for (int k = 0; k < 2048 / 4 / 64; ++k) s32[lane + 64 * k] = 0;
-      }
+      team_arrive();  // waited for where the next pass first writes to its S tile
     }
     if (!more_units) break;
     u = u1, u1 = u2;
@@ -776,35 +784,50 @@ int launch_resident(int teams, dim3 grid, size_t lds, hipStream_t stream, const 
   return fail("rgms: no kernel for %d teams", teams);
 }
 
-// Cuts the sorted edges into `teams` shares of (nearly) equal numbers of steps, in tile order.  A
-// tile that lies inside one share is a unit that writes its rows of Y alone; the pieces of a
-// tile that is cut by a share boundary all add with atomics.
+// What a unit costs a team beyond its steps (summing the four partial tiles, writing Y back, the
+// start of the next pass), in steps.  Measured: about 3300 cycles against 1650 per step of each of
+// the four wavefronts, i.e. the time of 8 steps of the unit.
+constexpr int64_t kUnitOverheadSteps = 8;
+
+// Cuts the sorted edges into `teams` shares of (nearly) equal cost, in tile order; the cost of a
+// tile is its steps plus the overhead above.  A tile that lies inside one share is a unit that
+// writes its rows of Y alone; the pieces of a tile that is cut by a share boundary all add with
+// atomics.  A boundary that falls into the overhead part of a tile moves to the tile's start.
 int build_shares(TileIndex& ix, int64_t teams, hipStream_t stream) {
   const int64_t tiles = (int64_t)ix.tile_begin.size() - 1;
-  std::vector<int64_t> first_step(size_t(tiles + 1), 0);
-  for (int64_t t = 0; t < tiles; ++t)
-    first_step[t + 1] = first_step[t] + ceil_div(ix.tile_begin[t + 1] - ix.tile_begin[t], (int64_t)kStepEdges);
-  const int64_t total = first_step[tiles];
+  // cost coordinate: tile t occupies [at[t], at[t + 1]), its overhead first, then its steps
+  std::vector<int64_t> at(size_t(tiles + 1), 0);
+  auto steps_of = [&](int64_t t) { return ceil_div(ix.tile_begin[t + 1] - ix.tile_begin[t], (int64_t)kStepEdges); };
+  for (int64_t t = 0; t < tiles; ++t) at[t + 1] = at[t] + (steps_of(t) ? steps_of(t) + kUnitOverheadSteps : 0);
+  const int64_t total = at[tiles];
+  // boundary g as (tile, step inside the tile)
+  auto boundary = [&](int64_t g, int64_t& t) -> int64_t {
+    const int64_t c = total * g / teams;
+    while (t < tiles && at[t + 1] <= c) ++t;
+    if (t >= tiles) return 0;
+    return std::max<int64_t>(0, c - at[t] - kUnitOverheadSteps);
+  };
   std::vector<int32_t> ptr(size_t(teams + 1), 0);
   std::vector<Unit> units;
   units.reserve(size_t(tiles + 2 * teams));
-  int64_t t = 0;
+  int64_t t0 = 0, s0 = boundary(0, t0);
   for (int64_t g = 0; g < teams; ++g) {
-    // steps [s0, s1) of the numbering over all tiles
-    const int64_t s0 = total * g / teams, s1 = total * (g + 1) / teams;
+    int64_t t1 = t0;
+    const int64_t s1 = g + 1 < teams ? boundary(g + 1, t1) : 0;
+    if (g + 1 == teams) t1 = tiles;
     ptr[g] = (int32_t)units.size();
-    while (t < tiles && first_step[t + 1] <= s0) ++t;
-    for (int64_t k = t; k < tiles && first_step[k] < s1; ++k) {
-      const int64_t a = std::max(s0, first_step[k]), b = std::min(s1, first_step[k + 1]);
+    // steps [s0, end) of tile t0, whole tiles between, steps [0, s1) of tile t1
+    for (int64_t k = t0; k <= t1 && k < tiles; ++k) {
+      const int64_t n = steps_of(k);
+      const int64_t a = k == t0 ? s0 : 0, b = k == t1 ? s1 : n;
       if (a >= b) continue;
-      const bool whole = a == first_step[k] && b == first_step[k + 1];
       Unit un;
-      un.edge_begin = ix.tile_begin[k] + (a - first_step[k]) * kStepEdges;
-      un.edge_count = (int32_t)(std::min(ix.tile_begin[k + 1], ix.tile_begin[k] + (b - first_step[k]) * kStepEdges) -
-                                un.edge_begin);
-      un.tile_flag = (int32_t)(k << 1) | (whole ? 0 : 1);
+      un.edge_begin = ix.tile_begin[k] + a * kStepEdges;
+      un.edge_count = (int32_t)(std::min(ix.tile_begin[k + 1], ix.tile_begin[k] + b * kStepEdges) - un.edge_begin);
+      un.tile_flag = (int32_t)(k << 1) | ((a == 0 && b == n) ? 0 : 1);
       units.push_back(un);
     }
+    t0 = t1, s0 = s1;
   }
   ptr[teams] = (int32_t)units.size();
   STIR_REQUIRE(units.size() < (size_t(1) << 31), "rgms: too many units");
