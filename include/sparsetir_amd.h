@@ -259,8 +259,12 @@ int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t g
  * arrays d_A[b] (groups*rb*cb fp16 edge weights, the 0/1 mask in the reference), d_rows[b]
  * (groups*rb), d_cols[b] (groups*rb*cb) and d_mids[b] (groups: relation of each group).
  * The plan keeps the array pointers.  From 8192 slots on, the first launch builds an edge index
- * from the three index arrays (they must not change afterwards; the weights may) and every launch
- * rewrites a packed copy of W held by the plan, so a plan serves one call at a time.
+ * from the three index arrays (they must not change afterwards; the weights may), and the first
+ * launch with given feature sizes a work list for them (both allocate and synchronise the
+ * stream; later launches do neither).  W is read anew at every launch.  When W does not fit the
+ * LDS of a compute unit beside the kernel's tiles (about 130 KB: 65 relations of 32 x 32), when
+ * feat_in exceeds 64 or d_W is not 16-byte aligned, every launch rewrites a packed copy of W held
+ * by the plan; a plan therefore serves one call at a time.
  */
 typedef struct stir_rgms_plan stir_rgms_plan;
 int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int32_t* rows_bkt,
