@@ -271,7 +271,7 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
         out[tag] = dict(tm, us=d * 1e6, first_call_ms=first_s * 1e3, tflops=flops / d / 1e12,
                         alg_GBps=byts / d / 1e9, frac_of_hbm_peak=byts / d / 1e9 / HBM_PEAK_GBS, edges=E,
                         ell_rows=int(sum(r.size for r in rows)), static_weights=static,
-                        accumulation="32-row output tiles, written once (no atomics)")
+                        accumulation="32-row output tiles written once; tiles cut by a share boundary add with atomics")
 
     # SpMM over the condensed format (t = 32, g = 16) on the config-2 graph, fp16 in, fp32 out
     g2 = datasets.config2()
