@@ -437,35 +437,40 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
 // of a compute unit, one workgroup per compute unit stays for the whole launch: it brings W into
 // LDS once, already in MFMA operand order (so no separate packing launch and no W traffic through
 // the vector memory path, which otherwise carries twice the bytes of the gathered X rows), and
-// its T teams of four wavefronts each work through one share of the launch.  The shares are cut
-// from the sorted edges by the host so that every team gets the same number of steps (build_shares).
+// its T teams of two wavefronts each work through one share of the launch.  The shares are cut
+// from the sorted edges by the host so that every team gets the same amount of work (build_shares).
+// The two wavefronts of a team take the steps of a unit in turn, each with a full 32 x 32 tile of
+// partial sums; at the end each keeps 16 rows, receives the partner's part of them through LDS and
+// writes them back (teams of four spent a quarter of the launch meeting and summing: 41 against
+// 36 us; single wavefronts cut nearly every tile in two and pay for it in atomics: 38 us).
 // The X rows of a step are requested one step ahead and the records three steps ahead; a team's
 // wavefronts synchronise among themselves only, through a counter in LDS.
 constexpr int kSBytes = kTileRows * kSStride * 2;  // S tile of one wavefront
-constexpr int kTeamLds = kUnitWaves * kSBytes;
 constexpr int kLdsMaxKK = 4;
+constexpr int kTeamWaves = 2;  // wavefronts that share a unit in the resident kernel
 
 // lane -> 16-byte slot of its operand inside a fragment of W in LDS: consecutive lanes stay on
 // distinct banks, and so do the eight writers of one column phase (see the fill loop)
 __device__ __forceinline__ int w_slot(int lane) { return lane ^ ((lane >> 3) & 7); }
 
 template <int KK, bool BF16, typename Rec, int T>
-__global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
+__global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
     const int32_t* __restrict__ share_ptr, const Unit* __restrict__ share_units, const Rec* __restrict__ edges, int m,
     int feat_out, int num_rels, const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
     float* __restrict__ Y) {
   constexpr int FIN = KK * 16;
   constexpr bool kPacked = sizeof(Rec) == sizeof(PackedEdge);
-  constexpr int kThreads = 64 * kUnitWaves * T, kTeamThreads = 64 * kUnitWaves;
+  constexpr int UW = kTeamWaves;
+  constexpr int kThreads = 64 * UW * T;  // T teams of two wavefronts
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int ntiles = feat_out / 32;
   const int frags = num_rels * ntiles * KK;
   u32x4* Wl = reinterpret_cast<u32x4*>(lds);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int team = wave / kUnitWaves, tw = wave % kUnitWaves;
+  const int team = wave / UW, tw = wave % UW;
   const int mrow = lane & 31, h = lane >> 5;
-  constexpr int kStride = kUnitWaves * kStepEdges;  // edges between a wavefront's steps
+  constexpr int kStride = UW * kStepEdges;  // edges between a wavefront's steps
 
   // lanes past the last edge of a unit repeat it (with weight zero, see `live`)
   // (indexed from the unit's first edge, so that the lane's part of the address is 32 bits wide)
@@ -541,7 +546,7 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
       if (second) block_store(blk + kThreads, in1);
     }
   }
-  unsigned char* team_lds = lds + (size_t)frags * 1024 + team * kTeamLds;
+  unsigned char* team_lds = lds + (size_t)frags * 1024 + team * (UW * kSBytes);
   uint16_t* S = reinterpret_cast<uint16_t*>(team_lds + tw * kSBytes);
   float* my_partial = reinterpret_cast<float*>(team_lds + tw * kSBytes);  // 8 registers x 64 lanes, over S
   // The team's wavefronts meet at a counter in LDS (a workgroup barrier would tie the teams of the
@@ -551,7 +556,7 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
   uint32_t* meet = reinterpret_cast<uint32_t*>(team_lds + 26 * kSStride * 2 + 64);
   uint32_t met = 0;
   auto team_arrive = [&]() {
-    met += kUnitWaves;
+    met += UW;
     if (lane == 0) __hip_atomic_fetch_add(meet, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   auto team_wait = [&]() {
@@ -570,8 +575,6 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
   if (u_first >= u_last) return;  // no workgroup barrier below this line
   const int slot = w_slot(lane);
   const int jcol = 16 * (mrow >> 4) + 8 * ((mrow >> 2) & 1) + 4 * ((mrow >> 3) & 1) + (mrow & 3);
-  const int team_tid = threadIdx.x & (kTeamThreads - 1);
-  constexpr int kSumIters = 16 * 32 / kTeamThreads;
   fetch(cur, xa, wa);
   for (int ui = u_first;; ++ui) {
     const bool more_units = ui + 1 < u_last;
@@ -586,15 +589,14 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
       const bool next_pass = nti + 1 < ntiles || more_units;
       Rec p0 = cur, p1 = cur, p2 = cur;
       if (next_pass) first_records(nti + 1 < ntiles ? u : u1, p0, p1, p2);
-      float yold[2][kSumIters];  // what the tile's rows hold now: needed at the end only
+      // What the wavefront's 16 rows of the tile hold now, in accumulator layout (register v of lane
+      // (n, h) is row 16 tw + (v%4) + 4h + 8(v/4), feature n); needed at the end only.
+      float yold[8];
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
-#pragma unroll
-        for (int k = 0; k < kSumIters; ++k) {
-          const int elem = team_tid + kTeamThreads * k;
-          const int64_t yrow = (int64_t)tile * kTileRows + 16 * half + (elem >> 5);
-          yold[half][k] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + (elem & 31)] : 0.f;
-        }
+      for (int v = 0; v < 8; ++v) {
+        const int64_t yrow = (int64_t)tile * kTileRows + 16 * tw + (v & 3) + 4 * h + 8 * (v >> 2);
+        yold[v] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + mrow] : 0.f;
+      }
       f32x16 acc2;
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc2[v] = 0.f;
@@ -674,42 +676,43 @@ __global__ __launch_bounds__(64 * kUnitWaves * T) void rgms_tile_lds_kernel(
       // Everything requested so far has had the whole pass to arrive.  Naming the old values of
       // Y here settles them, so that the stores below do not wait for the loads that follow.
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
-#pragma unroll
-        for (int k = 0; k < kSumIters; ++k) asm volatile("" : "+v"(yold[half][k]));
+      for (int v = 0; v < 8; ++v) asm volatile("" : "+v"(yold[v]));
       if (next_pass) {
         cur = p0, nx1 = p1, nx2 = p2;
         fetch(cur, xa, wa);
       }
 
       if (e_first >= e_end) team_wait();  // (a wavefront without steps has not met the others yet)
-      // ---- add the team's four tiles, 16 rows at a time (the partial sums lie over the S tiles),
-      // and write back.  acc2[v] of lane (n, h) is row (v%4) + 4h + 8(v/4), output feature 32 nti + n.
+      // ---- teams of two: each wavefront owns 16 rows of the tile (eight accumulator registers),
+      // hands the other eight to its partner through LDS and writes its rows back from registers.
+      float* theirs = reinterpret_cast<float*>(team_lds + (1 - tw) * kSBytes);
+      if (tw == 0) {
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        if (half == 1) team_barrier();  // the sums of the first half have been read
+        for (int v = 0; v < 8; ++v) my_partial[v * 64 + lane] = acc2[8 + v];
+      } else {
 #pragma unroll
-        for (int v = 0; v < 8; ++v) my_partial[v * 64 + lane] = acc2[8 * half + v];
-        team_barrier();
+        for (int v = 0; v < 8; ++v) my_partial[v * 64 + lane] = acc2[v];
+      }
+      team_barrier();
+      float own[8];
+      if (tw == 0) {
 #pragma unroll
-        for (int k = 0; k < kSumIters; ++k) {
-          const int elem = team_tid + kTeamThreads * k, row = elem >> 5, col = elem & 31;
-          const int at = ((row & 3) + 4 * (row >> 3)) * 64 + col + 32 * ((row >> 2) & 1);
-          float sum = 0.f;
+        for (int v = 0; v < 8; ++v) own[v] = acc2[v] + theirs[v * 64 + lane];
+      } else {
 #pragma unroll
-          for (int w = 0; w < kUnitWaves; ++w) {
-            float* part = reinterpret_cast<float*>(team_lds + w * kSBytes) + at;
-            sum += *part;
-            if (half == 1) *part = 0.f;  // the S tiles are all zeros again after the second half
-          }
-          const int64_t yrow = (int64_t)tile * kTileRows + 16 * half + row;
-          if (yrow < m) {
-            float* y = Y + yrow * feat_out + 32 * nti + col;
-            if (atomic)
-              __hip_atomic_fetch_add(y, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            else
-              *y = yold[half][k] + sum;
-          }
+        for (int v = 0; v < 8; ++v) own[v] = acc2[8 + v] + theirs[v * 64 + lane];
+      }
+#pragma unroll
+      for (int v = 0; v < 8; ++v) theirs[v * 64 + lane] = 0.f;  // the partner's S tile is all zeros again
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        const int64_t yrow = (int64_t)tile * kTileRows + 16 * tw + (v & 3) + 4 * h + 8 * (v >> 2);
+        if (yrow < m) {
+          float* y = Y + yrow * feat_out + 32 * nti + mrow;
+          if (atomic)
+            __hip_atomic_fetch_add(y, own[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else
+            *y = yold[v] + own[v];
         }
       }
       team_arrive();  // waited for where the next pass first writes to its S tile
@@ -762,32 +765,34 @@ int allow_lds(const void* fn) {
   return 0;
 }
 
-// Four teams (16 wavefronts of 128 registers) only for the variants that fit those registers.
-constexpr bool resident_four_teams(bool packed, int kk) { return packed && kk <= 2; }
-int resident_max_teams(bool packed, int kk) { return resident_four_teams(packed, kk) ? 4 : 3; }
+// A resident workgroup has 8, 12 or 16 wavefronts ("quads" of four: each wavefront needs an S tile
+// in LDS beside W); 16 only for the variants that fit 128 registers.
+constexpr bool resident_four_quads(bool packed, int kk) { return packed && kk <= 2; }
+int resident_max_quads(bool packed, int kk) { return resident_four_quads(packed, kk) ? 4 : 3; }
 
+// Launches the resident kernel with `quads` x 4 wavefronts per workgroup.
 template <int KK, bool BF16, typename Rec>
-int launch_resident(int teams, dim3 grid, size_t lds, hipStream_t stream, const int32_t* share_ptr,
+int launch_resident(int quads, dim3 grid, size_t lds, hipStream_t stream, const int32_t* share_ptr,
                     const Unit* share_units, const Rec* edges, int m, int feat_out, int num_rels, const uint16_t* W,
                     const uint16_t* X, float* Y) {
   auto go = [&](auto* fn) -> int {
     if (int rc = allow_lds(reinterpret_cast<const void*>(fn))) return rc;
-    hipLaunchKernelGGL(fn, grid, dim3(64 * kUnitWaves * teams), lds, stream, share_ptr, share_units, edges, m, feat_out,
-                       num_rels, W, X, Y);
+    hipLaunchKernelGGL(fn, grid, dim3(256 * quads), lds, stream, share_ptr, share_units, edges, m, feat_out, num_rels, W,
+                       X, Y);
     return 0;
   };
-  if (teams == 2) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 2>);
-  if (teams == 3) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 3>);
-  if constexpr (resident_four_teams(sizeof(Rec) == sizeof(PackedEdge), KK)) {
-    if (teams == 4) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 4>);
+  constexpr int kTeamsPerQuad = 4 / kTeamWaves;
+  if (quads == 2) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 2 * kTeamsPerQuad>);
+  if (quads == 3) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 3 * kTeamsPerQuad>);
+  if constexpr (resident_four_quads(sizeof(Rec) == sizeof(PackedEdge), KK)) {
+    if (quads == 4) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 4 * kTeamsPerQuad>);
   }
-  return fail("rgms: no kernel for %d teams", teams);
+  return fail("rgms: no kernel for %d wavefronts per workgroup", 4 * quads);
 }
 
-// What a unit costs a team beyond its steps (summing the four partial tiles, writing Y back, the
-// start of the next pass), in steps.  Measured: about 3300 cycles against 1650 per step of each of
-// the four wavefronts, i.e. the time of 8 steps of the unit.
-constexpr int64_t kUnitOverheadSteps = 8;
+// What a unit costs a team beyond its steps (exchanging half of the tile with the partner, writing
+// Y back, the start of the next pass), in steps of the unit.  Measured optimum, flat between 2 and 6.
+constexpr int64_t kUnitOverheadSteps = 3;
 
 // Cuts the sorted edges into `teams` shares of (nearly) equal cost, in tile order; the cost of a
 // tile is its steps plus the overhead above.  A tile that lies inside one share is a unit that
@@ -1010,17 +1015,16 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
 
   // W resident in LDS when it fits beside the S tiles of at least two teams
   const size_t w_bytes = size_t(frags) * 64 * sizeof(u32x4);
-  int teams = 0;
+  int quads = 0;
   if (kk_count <= kLdsMaxKK && reinterpret_cast<uintptr_t>(d_W) % 16 == 0 &&
       (int64_t)ix.n * feat_in * 2 < (int64_t(1) << 32)) {
     const size_t lds_limit = lds_bytes_per_workgroup();
-    // four teams (16 wavefronts, 128 registers each) only where the kernel fits those registers
-    const int tmax = resident_max_teams(ix.packed_records, kk_count);
-    for (int t = tmax; t >= 2 && teams == 0; --t)
-      if (w_bytes + size_t(t) * kTeamLds <= lds_limit) teams = t;
+    for (int q = resident_max_quads(ix.packed_records, kk_count); q >= 2 && quads == 0; --q)
+      if (w_bytes + size_t(q) * 4 * kSBytes <= lds_limit) quads = q;
   }
-  if (teams) {
-    const size_t lds = w_bytes + size_t(teams) * kTeamLds;
+  if (quads) {
+    const int teams = quads * 4 / kTeamWaves;  // per workgroup
+    const size_t lds = w_bytes + size_t(quads) * 4 * kSBytes;
     // one workgroup per compute unit, fewer when a team would get less than a handful of steps
     const int64_t steps_bound = ix.edges / kStepEdges + (int64_t)ix.tile_begin.size();
     const int64_t wgs = std::min<int64_t>(std::max(1, compute_units()), ceil_div(steps_bound, (int64_t)teams * 8));
@@ -1030,7 +1034,7 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
     const int32_t* share_ptr = static_cast<const int32_t*>(ix.d_share_ptr);
     const Unit* share_units = static_cast<const Unit*>(ix.d_share_units);
 #define STIR_LDS_R(KKV, BF, REC, PTR)                                                                   \
-  if (int rc = launch_resident<KKV, BF, REC>(teams, grid, lds, stream, share_ptr, share_units, PTR, ix.m, feat_out, \
+  if (int rc = launch_resident<KKV, BF, REC>(quads, grid, lds, stream, share_ptr, share_units, PTR, ix.m, feat_out, \
                                              ix.num_rels, W, X, d_Y))                                  \
     return rc
 #define STIR_LDS(KKV)                                                                          \
