@@ -83,6 +83,8 @@ def test_bsr_tall_blocks(dev, blk, feat, dtype, out32):
     (160, 12, 32, 512, torch.float16),    # one accumulator per wavefront
     (48, 20, 32, 1536, torch.bfloat16),   # two accumulators per wavefront
     (24, 10, 64, 1536, torch.float16),    # two slices per workgroup as well
+    (9, 6, 128, 2080, torch.float16),     # 128-row blocks, last feature tile partial
+    (10, 4, 256, 1024, torch.bfloat16),   # 256-row blocks
 ])
 def test_bsr_many_workgroups(dev, mb, nb, blk, feat, dtype):
     """More than two workgroups per CU: the kernel whose wavefronts split the feature axis (small
