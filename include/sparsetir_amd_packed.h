@@ -115,6 +115,12 @@ enum {
  *      in place, or frees them and gets arrays of the same sizes at the same addresses, calls
  *      this first; the next operator call then builds a fresh plan.  Edge weights (A_k), W, X, B
  *      may change freely.
+ * "sparsetir.rgms_static_weights" (on)
+ *      no counterpart in the reference.  on != 0: the plans "sparsetir.rgms" makes from now on carry
+ *      the promise of stir_rgms_plan_set_static_weights -- the A_k keep the values they have at the
+ *      plan's first call (the reference's A_k is the 0/1 mask of CSFToELL3D, written once) -- and
+ *      leave the zero-weight padding slots out of their edge index.  Drops the cached plan when the
+ *      setting changes.  Default off.
  *
  * Format pass (host tensors, kDLCPU; the reference returns nested Array<NDArray>, which needs
  * libtvm objects, so here a sizing call is followed by a fill call into caller-made tensors):
@@ -141,6 +147,7 @@ int stir_packed_rgms(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms_f32(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms_csf(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_invalidate_plans(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_rgms_static_weights(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_csf_to_ell3d_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);

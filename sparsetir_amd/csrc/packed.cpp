@@ -178,6 +178,7 @@ HybKey g_hyb_key;
 stir_hyb_plan* g_hyb_plan = nullptr;
 HybKey g_rgms_key;
 stir_rgms_plan* g_rgms_plan = nullptr;
+bool g_rgms_static_weights = false;  // promise for the plans "sparsetir.rgms" makes from now on
 HybKey g_rgms_f32_key;
 stir_rgms_f32_plan* g_rgms_f32_plan = nullptr;
 
@@ -471,6 +472,11 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
     if (stir_rgms_plan_create(&g_rgms_plan, nb, rb.data(), cb.data(), groups.data(), Ak.data(), Rk.data(),
                               Ck.data(), Mk.data()))
       return forward(-1);
+    if (g_rgms_static_weights && stir_rgms_plan_set_static_weights(g_rgms_plan, 1)) {
+      stir_rgms_plan_destroy(g_rgms_plan);
+      g_rgms_plan = nullptr;
+      return forward(-1);
+    }
     g_rgms_key = key;
   }
   return forward((bf ? stir_rgms_bf16 : stir_rgms_f16)(g_rgms_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data,
@@ -494,6 +500,21 @@ int stir_packed_invalidate_plans(TVMValue*, int*, int n, TVMRetValueHandle, void
   g_hyb_plan = nullptr;
   g_rgms_plan = nullptr;
   g_rgms_f32_plan = nullptr;
+  return 0;
+}
+
+int stir_packed_rgms_static_weights(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.rgms_static_weights", v, tc, n};
+  if (!a.count(1)) return -1;
+  const int64_t on = a.integer(0, "on");
+  if (!a.ok) return -1;
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  if (g_rgms_static_weights != (on != 0)) {
+    // the cached plan was made under the other setting
+    if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
+    g_rgms_plan = nullptr;
+  }
+  g_rgms_static_weights = on != 0;
   return 0;
 }
 
@@ -691,6 +712,7 @@ static const PackedEntry kTable[] = {
     {"sparsetir.rgms_f32", stir_packed_rgms_f32},
     {"sparsetir.rgms_csf", stir_packed_rgms_csf},
     {"sparsetir.invalidate_plans", stir_packed_invalidate_plans},
+    {"sparsetir.rgms_static_weights", stir_packed_rgms_static_weights},
     {"tir.sparse.ColumnPartHyb.sizes", stir_packed_column_part_hyb_sizes},
     {"tir.sparse.ColumnPartHyb.fill", stir_packed_column_part_hyb_fill},
     {"tir.sparse.CSFToELL3D.sizes", stir_packed_csf_to_ell3d_sizes},

@@ -210,3 +210,41 @@ def test_index_arrays_rewritten_in_place_need_invalidate(dev):
     torch.cuda.synchronize()
     assert torch.allclose(y1, after, rtol=1e-5, atol=1e-5)
     assert torch.allclose(y1p, after, rtol=1e-5, atol=1e-5)
+
+
+def test_packed_rgms_static_weights(dev):
+    """"sparsetir.rgms_static_weights"(1) makes the packed RGMS operator build its plans with the
+    promise that the slot weights stay as they are: same result as without it, for weights that
+    include zeros on real edges, and the setting can be switched back."""
+    R, n, fin, fout, group, buckets = 5, 2500, 32, 32, 32, [1, 2, 4, 8]
+    csf = random_csf(R, n, 30000, seed=21)
+    rb = [group // b for b in buckets]
+    iptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    assert sum(c.size for c in cols) >= 8192
+    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    rng = np.random.default_rng(21)
+    w = t(rng.standard_normal(R * fin * fout).astype(np.float16) * 0.1)
+    xx = t(rng.standard_normal(n * fin).astype(np.float16))
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        a = mask[k].astype(np.float16) * (rng.random(mask[k].shape) < 0.8)  # some real edges weigh zero
+        triples += [t(a.ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(iptr[k]))))
+    g = packed.get_global_func("sparsetir.rgms")
+    promise = packed.get_global_func("sparsetir.rgms_static_weights")
+    results = []
+    try:
+        for on in (0, 1, 0):
+            promise(on)
+            y = torch.zeros(n * fout, device=dev)
+            g(w, xx, y, *triples, *mids, fin, fout)
+            g(w, xx, y, *triples, *mids, fin, fout)  # second call of the same plan: accumulates
+            torch.cuda.synchronize()
+            results.append(y)
+    finally:
+        promise(0)
+    assert results[0].abs().sum() > 0
+    assert torch.allclose(results[0], results[1], rtol=1e-5, atol=1e-5)
+    assert torch.allclose(results[0], results[2], rtol=1e-5, atol=1e-5)
+    with pytest.raises(SparseTIRError, match="num_args"):
+        promise()
