@@ -292,6 +292,12 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     out["tcspmm_config2_feat128"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "useful_gflops": 2.0 * nnz2 * f2 / d / 1e9,
                                      "mfma_tflops": 2.0 * nnzb2 * 32 * 16 * f2 / d / 1e12, "groups": int(nnzb2),
                                      "mask_density": float(nnz2) / (nnzb2 * 32 * 16)}
+    # the reference's own form of this operator writes fp16 (bench_tc_spmm.py: fp16 accumulator fragments)
+    tc16 = ops.build_tcspmm(mb2, nnzb2, f2, 32, 16, g2["n"], torch.float16)
+    c16 = torch.zeros(mb2 * 32 * f2, device=dev, dtype=torch.float16)
+    tm = time_small(lambda: tc16(a2, b2, c16, gp, ti), 50, 5, torch)
+    out["tcspmm_config2_feat128_f16_out"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"],
+                                             "us": tm["us_back_to_back"]}
 
     # fp32 forms: ELL3D buckets with 32-slot groups (the reference's composable fp32 setting) and the
     # CSF traversal; W is [R, fout, fin]

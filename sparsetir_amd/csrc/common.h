@@ -4,6 +4,9 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
+#include <set>
+#include <utility>
 
 namespace stir {
 
@@ -57,5 +60,32 @@ inline int compute_units() {
     cached_dev = dev, cached = cus;
   }
   return cached;
+}
+
+// LDS a workgroup may ask for on the current device (0 on failure)
+inline size_t lds_bytes_per_workgroup() {
+  static thread_local int cached_dev = -1;
+  static thread_local size_t cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev != cached_dev) {
+    int bytes = 0;
+    if (hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
+    cached_dev = dev, cached = (size_t)bytes;
+  }
+  return cached;
+}
+
+// Kernels that use more than 64 KB of dynamic LDS have to be told so once per device.
+inline int allow_lds(const void* fn) {
+  static std::mutex mu;
+  static std::set<std::pair<int, const void*>> done;
+  int dev = 0;
+  STIR_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({dev, fn})) return 0;
+  STIR_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_per_workgroup()));
+  done.insert({dev, fn});
+  return 0;
 }
 }  // namespace stir

@@ -14,9 +14,6 @@
 
 #include <hipcub/hipcub.hpp>
 
-#include <mutex>
-#include <set>
-#include <utility>
 
 namespace stir {
 namespace {
@@ -736,33 +733,6 @@ int bit_length(uint64_t x) {
   int b = 0;
   while (x) ++b, x >>= 1;
   return b;
-}
-
-// LDS a workgroup may ask for on the current device (0 on failure)
-size_t lds_bytes_per_workgroup() {
-  static thread_local int cached_dev = -1;
-  static thread_local size_t cached = 0;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 0;
-  if (dev != cached_dev) {
-    int bytes = 0;
-    if (hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
-    cached_dev = dev, cached = (size_t)bytes;
-  }
-  return cached;
-}
-
-// Kernels that use more than 64 KB of dynamic LDS have to be told so once per device.
-int allow_lds(const void* fn) {
-  static std::mutex mu;
-  static std::set<std::pair<int, const void*>> done;
-  int dev = 0;
-  STIR_HIP(hipGetDevice(&dev));
-  std::lock_guard<std::mutex> lock(mu);
-  if (done.count({dev, fn})) return 0;
-  STIR_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_per_workgroup()));
-  done.insert({dev, fn});
-  return 0;
 }
 
 // A resident workgroup has 8, 12 or 16 wavefronts ("quads" of four: each wavefront needs an S tile

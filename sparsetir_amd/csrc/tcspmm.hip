@@ -13,8 +13,11 @@
 // A row tile that touches thousands of distinct columns (a hub row of a power-law graph) would be
 // one long serial chain in one workgroup.  With fp32 output such tiles are cut into up to kSplit
 // units of at least kUnitSteps steps that add their results with atomics; a first launch clears the rows
-// of those tiles.  (fp16 output keeps one workgroup per tile: partial sums would be rounded to
-// fp16 once per unit.)
+// of those tiles.  With fp16 output partial sums would be rounded once per unit; there, tiles of
+// more than kLongSteps steps are left to a second launch (tcspmm_long_kernel) whose workgroups
+// have 8 wavefronts that split the steps of the tile among them and add their fp32 partial sums
+// through LDS before the one write of the tile.  (For fp32 output that launch is the slower of the
+// two ways: a hub tile is a chain of steps/8 instead of steps/16, and the launches run in turn.)
 #include "common.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -29,6 +32,8 @@ constexpr int kTile = 32;   // t
 constexpr int kGroup = 16;  // g
 constexpr int kUnitSteps = 16;  // steps (of two groups) per unit of a long tile
 constexpr int kSplit = 16;      // most units per tile (second grid dimension of the split launch)
+constexpr int kLongSteps = 16;  // fp16 output: tiles with more steps go to the second launch
+constexpr int kLongWaves = 8;   // wavefronts per workgroup there (16 would leave 128 registers each: spills)
 
 __device__ __forceinline__ int tile_steps(const int32_t* __restrict__ indptr, int64_t io) {
   const int64_t rows_total = (int64_t)(indptr[io + 1] - indptr[io]) * kGroup;
@@ -76,6 +81,9 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   const int64_t rows_total = (g_end - g_begin) * kGroup;  // gathered rows of B for this tile
   const int steps = (int)((rows_total + 31) / 32);
   const int32_t* rowlist = indices + g_begin * kGroup;
+  if constexpr (OUT == 0) {
+    if (steps > kLongSteps) return;  // left to tcspmm_long_kernel; uniform over the workgroup
+  }
   int it_begin = 0, it_end = steps;
   bool add = false;
   if constexpr (SPLIT) {
@@ -164,6 +172,134 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   }
 }
 
+// fp16 output: the tiles the kernel above skips.  512 threads; wavefront w takes steps w, w + 8, ... of the
+// tile for all 128 features (four accumulators), gathers the step's 32 rows of B itself (lane:
+// k pairs kp, kp + 4, kp + 8, kp + 12 and 8-feature chunk fc) into its own 8 KB piece of LDS -- no
+// workgroup barrier in the loop, the LDS operations of one wavefront execute in order -- and the
+// partial results are added through LDS, one 32-feature tile at a time.
+// Dynamic LDS: kLongWaves * 16 * kTileF words (64 KB).
+__global__ __launch_bounds__(64 * kLongWaves) void tcspmm_long_kernel(int feat, int64_t mb, int f_tiles,
+                                                                      const uint16_t* __restrict__ A,
+                                                                      const uint16_t* __restrict__ B,
+                                                                      void* __restrict__ C,
+                                                                      const int32_t* __restrict__ indptr,
+                                                                      const int32_t* __restrict__ indices) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int f_tile = (int)(blockIdx.x % f_tiles);
+  const int64_t io = blockIdx.x / f_tiles;
+  if (io >= mb) return;
+  const int64_t g_begin = indptr[io], g_end = indptr[io + 1];
+  const int64_t rows_total = (g_end - g_begin) * kGroup;
+  const int steps = (int)((rows_total + 31) / 32);
+  if (steps <= kLongSteps) return;  // uniform over the workgroup
+  const int f0 = f_tile * kTileF;
+  const int kp = lane >> 4, fc = lane & 15;
+  const bool stage_live = f0 + fc * 8 < feat;
+  const int32_t* rowlist = indices + g_begin * kGroup;
+  uint32_t(*xs)[kTileF] = reinterpret_cast<uint32_t(*)[kTileF]>(lds + wave * (16 * kTileF));  // [k pair][feature]
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  // row ids one step (of this wavefront) before the rows of B, as in the kernel above
+  int row_a[4], row_b[4];
+  auto fetch_ids = [&](int it) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t k = (int64_t)it * 32 + 2 * (kp + 4 * q);
+      row_a[q] = row_b[q] = 0;
+      if (k < rows_total) row_a[q] = rowlist[k], row_b[q] = rowlist[k + 1];
+    }
+  };
+  u32x4 r0[4], r1[4], a_next[2];
+  auto fetch = [&](int it) {
+    const int64_t jo = g_begin + 2 * it;
+    a_next[0] = *reinterpret_cast<const u32x4*>(A + (jo * kTile + n) * kGroup + 8 * h);
+    a_next[1] = u32x4{0, 0, 0, 0};
+    if (jo + 1 < g_end) a_next[1] = *reinterpret_cast<const u32x4*>(A + ((jo + 1) * kTile + n) * kGroup + 8 * h);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      r0[q] = r1[q] = u32x4{0, 0, 0, 0};
+      const int64_t k = (int64_t)it * 32 + 2 * (kp + 4 * q);
+      if (stage_live && k < rows_total) {
+        r0[q] = *reinterpret_cast<const u32x4*>(B + (int64_t)row_a[q] * feat + f0 + fc * 8);
+        r1[q] = *reinterpret_cast<const u32x4*>(B + (int64_t)row_b[q] * feat + f0 + fc * 8);
+      }
+    }
+    if (it + kLongWaves < steps) fetch_ids(it + kLongWaves);
+  };
+
+  // steps > kLongSteps >= kLongWaves: every wavefront has a step
+  fetch_ids(wave);
+  fetch(wave);
+  for (int it = wave; it < steps; it += kLongWaves) {
+    const u32x4 a0 = a_next[0], a1 = a_next[1];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      u32x4 lo, hi;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        lo[2 * d] = __builtin_amdgcn_perm(r1[q][d], r0[q][d], 0x05040100);
+        lo[2 * d + 1] = __builtin_amdgcn_perm(r1[q][d], r0[q][d], 0x07060302);
+        hi[2 * d] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x05040100);
+        hi[2 * d + 1] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x07060302);
+      }
+      *reinterpret_cast<u32x4*>(&xs[kp + 4 * q][fc * 8]) = lo;
+      *reinterpret_cast<u32x4*>(&xs[kp + 4 * q][fc * 8 + 4]) = hi;
+    }
+    if (it + kLongWaves < steps) fetch(it + kLongWaves);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int col = t * 32 + n;
+      u32x4 b0, b1;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        b0[d] = xs[4 * h + d][col];
+        b1[d] = xs[8 + 4 * h + d][col];
+      }
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a0), __builtin_bit_cast(f16x8, b0),
+                                                     acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a1), __builtin_bit_cast(f16x8, b1),
+                                                     acc[t], 0, 0, 0);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // the next step's stores come after these reads
+  }
+
+  // ---- the partial tiles, one 32-feature tile at a time: a thread sums register v of lane l
+  // over the wavefronts; that is row (v%4) + 4(l/32) + 8(v/4), feature l%32 of the tile.
+  float* red = reinterpret_cast<float*>(lds);  // [wavefront][register][lane], 32 KB
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    __syncthreads();  // staging pieces (t = 0) or the sums of the tile before are done with
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[t][v];
+    __syncthreads();
+#pragma unroll
+    for (int e = tid; e < 16 * 64; e += 64 * kLongWaves) {
+      const int v = e >> 6, l = e & 63;
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kLongWaves; ++w) sum += red[(w * 16 + v) * 64 + l];
+      const int fcol = f0 + t * 32 + (l & 31);
+      if (fcol < feat) {
+        const int row = (v & 3) + 4 * (l >> 5) + 8 * (v >> 2);
+        const int64_t off = (io * kTile + row) * feat + fcol;
+        const _Float16 hv = (_Float16)sum;
+        static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
+      }
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t group_size,
@@ -191,6 +327,10 @@ extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size
   } else {
     hipLaunchKernelGGL((tcspmm_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
                        f_tiles, A, B, d_C, d_indptr, d_indices);
+    STIR_LAUNCH_CHECK();
+    constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kTileF * sizeof(uint32_t);
+    hipLaunchKernelGGL(tcspmm_long_kernel, dim3((unsigned)blocks), dim3(64 * kLongWaves), kLongLds, st, feat,
+                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
   }
   STIR_LAUNCH_CHECK();
   return 0;
