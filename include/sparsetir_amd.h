@@ -166,8 +166,12 @@ int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const flo
  * ColumnPartHyb output.  stir_hyb_plan_create tests this on the row arrays as they are when it is
  * called (it synchronises the device and reads them once) and keeps atomics for every bucket when
  * it does not hold; row ids outside [0, m) are an error.  A caller that rewrites the row arrays
- * of a plan with 2 to 4 partitions must make a new plan.  The plan keeps the pointers, not
- * copies: the arrays must outlive it.
+ * of a plan with 2 to 4 partitions must make a new plan.  With more than 4 partitions the plan
+ * lists the slots of every output row once (column ids copied, values read through their
+ * addresses at every call; 12 bytes of device memory per slot, skipped when that is more than a
+ * quarter of the free memory) and its launches write every output row once instead of once per
+ * partition; a caller that rewrites the row or column arrays of such a plan must make a new one.
+ * The plan keeps the pointers of the value arrays, not copies: the arrays must outlive it.
  */
 typedef struct stir_hyb_plan stir_hyb_plan;
 int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,

@@ -6,6 +6,8 @@
 // step with fully coalesced 16-byte loads.  Column indices and values are fetched once per
 // wavefront with one coalesced load (lane l holds slot l of the 64-slot tile) and handed to
 // the lane groups through cross-lane reads, so no lane issues a redundant index load.
+#include <hipcub/hipcub.hpp>
+
 #include <algorithm>
 #include <mutex>
 #include <vector>
@@ -122,7 +124,9 @@ __device__ __forceinline__ void write_row(float* C, int64_t row, int feat, int l
 // ----------------------------------------------------------------------------- CSR SpMM
 // Partial sum of A[p] * B[indices[p], :] over p in [start, end) for one wavefront: the 64/G lane
 // groups take the nonzeros round-robin; the caller combines the groups.
-template <int G, int REP>
+// INDIRECT: A is an array of addresses of the values (the merged rows of a hyb plan, whose values
+// stay in the caller's bucket arrays), and nonzeros whose value is 0 -- ELL padding -- fetch no row.
+template <int G, int REP, bool INDIRECT = false>
 __device__ __forceinline__ void csr_accumulate(float4 (&acc)[REP], int start, int end, int feat,
                                                const float* __restrict__ A, const float* __restrict__ B,
                                                const int32_t* __restrict__ indices, int lane) {
@@ -132,7 +136,13 @@ __device__ __forceinline__ void csr_accumulate(float4 (&acc)[REP], int start, in
   for (int base = start; base < end; base += kWave) {
     const int p = base + lane;
     const int my_col = p < end ? __builtin_nontemporal_load(indices + p) : 0;
-    const float my_val = p < end ? __builtin_nontemporal_load(A + p) : 0.f;
+    float my_val = 0.f;
+    if (p < end) {
+      if constexpr (INDIRECT)
+        my_val = *__builtin_nontemporal_load(reinterpret_cast<const float* const*>(A) + p);
+      else
+        my_val = __builtin_nontemporal_load(A + p);
+    }
     const int cnt = min(kWave, end - base);
     for (int j0 = 0; j0 < cnt; j0 += NG * UNROLL) {
       float4 x[UNROLL][REP];
@@ -145,7 +155,8 @@ __device__ __forceinline__ void csr_accumulate(float4 (&acc)[REP], int start, in
         const float* bp = B + (int64_t)col * feat + gl * 4;
 #pragma unroll
         for (int r = 0; r < REP; ++r)
-          x[u][r] = (j < cnt && gl * 4 + r * G * 4 < feat) ? ld4(bp + r * G * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+          x[u][r] = (j < cnt && gl * 4 + r * G * 4 < feat && (!INDIRECT || v[u] != 0.f)) ? ld4(bp + r * G * 4)
+                                                                                          : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u)
@@ -162,7 +173,7 @@ constexpr int kLongRow = 256;
 constexpr int kLongPiece = 256;
 
 // One wavefront per row.  With split_long the rows above kLongRow are zero-filled here.
-template <int G, int REP>
+template <int G, int REP, bool INDIRECT = false>
 __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, int split_long,
                                                        const float* __restrict__ A,
                                                        const float* __restrict__ B,
@@ -177,15 +188,23 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, int spli
   float4 acc[REP];
 #pragma unroll
   for (int r = 0; r < REP; ++r) acc[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (!(split_long && end - start > kLongRow)) csr_accumulate<G, REP>(acc, start, end, feat, A, B, indices, lane);
+  if (!(split_long && end - start > kLongRow))
+    csr_accumulate<G, REP, INDIRECT>(acc, start, end, feat, A, B, indices, lane);
   reduce_groups<G, REP>(acc, kWave);
-  if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, 0, nullptr);
+  if constexpr (INDIRECT) {
+    // merged rows of a hyb plan: the operator adds to C, as its buckets do; this wavefront is the
+    // row's only writer in this launch, long rows are left to csr_long_rows_kernel altogether
+    if (end - start > kLongRow) return;
+    if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, 2, nullptr);
+  } else {
+    if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, 0, nullptr);
+  }
 }
 
 // One wavefront per kLongPiece consecutive nonzeros: the parts of rows longer than kLongRow that
 // fall into the piece are summed and added to C (cleared by csr_spmm_kernel) with atomics.
 // Pieces that touch no long row -- nearly all of them -- end after looking at their rows.
-template <int G, int REP>
+template <int G, int REP, bool INDIRECT = false>
 __global__ __launch_bounds__(256) void csr_long_rows_kernel(int m, int feat, int64_t first, int64_t nnz,
                                                             const float* __restrict__ A,
                                                             const float* __restrict__ B,
@@ -216,7 +235,7 @@ __global__ __launch_bounds__(256) void csr_long_rows_kernel(int m, int feat, int
       float4 acc[REP];
 #pragma unroll
       for (int q = 0; q < REP; ++q) acc[q] = make_float4(0.f, 0.f, 0.f, 0.f);
-      csr_accumulate<G, REP>(acc, (int)s, (int)e, feat, A, B, indices, lane);
+      csr_accumulate<G, REP, INDIRECT>(acc, (int)s, (int)e, feat, A, B, indices, lane);
       reduce_groups<G, REP>(acc, kWave);
       if (g == 0) write_row<G, REP>(C, row, feat, lane, acc, true, stage_all[wave]);
     }
@@ -435,6 +454,49 @@ __global__ __launch_bounds__(256) void hyb_mark_rows_kernel(const int32_t* __res
   if (seen & bit) flags[0] = 1;
 }
 
+// ---- merged rows (plans with more column partitions than run as phases)
+// With p column partitions an output row is the sum of up to p ELL rows, each in another bucket:
+// added with atomics that is p read-modify-writes of the row through the L2 atomic units
+// (config 3 with the reference's 16 partitions: 39 M ELL rows of mostly one or two slots, 20 GB of
+// atomic traffic).  Such a plan lists, once, the slots of every output row one after the other --
+// their column ids and the addresses of their values, which stay in the caller's arrays -- and
+// its launches run the CSR row kernels over that list: every row is read and written once (the
+// operator adds to C, like its buckets would).
+
+// count[r] += width for the output row r of every ELL row of one bucket; flags[1] when a row id
+// lies outside [0, m)
+__global__ __launch_bounds__(256) void hyb_count_slots_kernel(const int32_t* __restrict__ rows, int64_t nrows,
+                                                              int32_t width, int32_t m, int32_t* __restrict__ count,
+                                                              int32_t* __restrict__ flags) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nrows) return;
+  const int32_t r = rows[i];
+  if (r < 0 || r >= m) {
+    flags[1] = 1;
+    return;
+  }
+  atomicAdd(count + r, width);
+}
+
+// The slots of ELL row i of one bucket go to the next `width` places of its output row's list
+// (cursor[r] starts at the row's first place).
+__global__ __launch_bounds__(256) void hyb_place_slots_kernel(const int32_t* __restrict__ rows,
+                                                              const int32_t* __restrict__ cols,
+                                                              const float* __restrict__ A, int64_t nrows,
+                                                              int32_t width, int32_t* __restrict__ cursor,
+                                                              int32_t* __restrict__ merged_cols,
+                                                              const float** __restrict__ merged_vals) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nrows) return;
+  const int32_t r = rows[i];  // in range: hyb_count_slots_kernel has looked at it
+  const int32_t at = atomicAdd(cursor + r, width);
+  const int64_t first = i * width;
+  for (int32_t j = 0; j < width; ++j) {
+    merged_cols[at + j] = cols[first + j];
+    merged_vals[at + j] = A + first + j;
+  }
+}
+
 // Copies `count` bucket descriptors, handed over as a kernel argument, to dst[first ...]: how the
 // entry point that allocates nothing gets its descriptor tables into device memory without a
 // host-to-device copy.
@@ -589,6 +651,120 @@ void make_hyb_tables(int32_t num_col_parts, int32_t num_buckets, const int32_t* 
   out->total_rows = rows;
 }
 
+// The merged rows of a plan (see hyb_count_slots_kernel): CSR over all slots of the operator.
+struct MergedRows {
+  int32_t* slot_ptr = nullptr;       // m + 1
+  int32_t* cols = nullptr;           // slots
+  const float** vals = nullptr;      // slots: addresses inside the caller's value arrays
+  int64_t slots = 0;
+  void release() {
+    if (slot_ptr) (void)hipFree(slot_ptr);
+    if (cols) (void)hipFree(cols);
+    if (vals) (void)hipFree(vals);
+    slot_ptr = cols = nullptr;
+    vals = nullptr;
+    slots = 0;
+  }
+};
+
+// Builds the merged rows from the bucket arrays as they are now (synchronises the device).
+// *built = false, and nothing allocated, when the list would not fit 31-bit offsets or a quarter
+// of the free device memory.
+int build_merged_rows(int32_t m, int total_buckets, int num_buckets, const int32_t* bucket_widths,
+                      const int64_t* nrows, const float* const* d_A, const int32_t* const* d_rows,
+                      const int32_t* const* d_cols, MergedRows* out, bool* built) {
+  *built = false;
+  int64_t slots = 0;
+  for (int k = 0; k < total_buckets; ++k) {
+    STIR_REQUIRE(stir::ceil_div(nrows[k], 256) < (int64_t(1) << 31), "hyb_plan_create: bucket %d too large", k);
+    slots += nrows[k] * bucket_widths[k % num_buckets];
+  }
+  if (m == 0 || slots == 0 || slots >= (int64_t(1) << 31)) return 0;
+  size_t free_bytes = 0, total_bytes = 0;
+  STIR_HIP(hipMemGetInfo(&free_bytes, &total_bytes));
+  const size_t need = size_t(slots) * 12 + size_t(m + 1) * 12;
+  if (need > free_bytes / 4) return 0;
+  STIR_HIP(hipDeviceSynchronize());
+  MergedRows mr;
+  int32_t *count = nullptr, *flags = nullptr;
+  void* tmp = nullptr;
+  size_t tmp_bytes = 0;
+  auto cleanup = [&]() {
+    if (count) (void)hipFree(count);
+    if (tmp) (void)hipFree(tmp);
+  };
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&count), sizeof(int32_t) * (size_t(m) + 3));
+  if (e == hipSuccess) e = hipMemset(count, 0, sizeof(int32_t) * (size_t(m) + 3));
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&mr.slot_ptr), sizeof(int32_t) * (size_t(m) + 1));
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&mr.cols), sizeof(int32_t) * size_t(slots));
+  if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&mr.vals), sizeof(float*) * size_t(slots));
+  if (e == hipSuccess)
+    e = hipcub::DeviceScan::ExclusiveSum(nullptr, tmp_bytes, (const int32_t*)nullptr, (int32_t*)nullptr, m + 1, 0);
+  if (e == hipSuccess) e = hipMalloc(&tmp, tmp_bytes ? tmp_bytes : 16);
+  if (e != hipSuccess) {
+    cleanup();
+    mr.release();
+    return stir::fail("hyb_plan_create: %s", hipGetErrorString(e));
+  }
+  flags = count + m + 1;  // count[m] stays 0: the scan turns it into the number of slots
+  for (int k = 0; k < total_buckets; ++k)
+    if (nrows[k] > 0)
+      hipLaunchKernelGGL(hyb_count_slots_kernel, dim3((unsigned)stir::ceil_div(nrows[k], 256)), dim3(256), 0, 0,
+                         d_rows[k], nrows[k], bucket_widths[k % num_buckets], m, count, flags);
+  int32_t h_flags[2] = {0, 0};
+  e = hipGetLastError();
+  if (e == hipSuccess) e = hipMemcpy(h_flags, flags, sizeof(h_flags), hipMemcpyDeviceToHost);
+  if (e == hipSuccess && h_flags[1] == 0) {
+    e = hipcub::DeviceScan::ExclusiveSum(tmp, tmp_bytes, (const int32_t*)count, mr.slot_ptr, m + 1, 0);
+    // the counts become the cursors of the placement
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(count, mr.slot_ptr, sizeof(int32_t) * size_t(m), hipMemcpyDeviceToDevice, 0);
+    for (int k = 0; k < total_buckets && e == hipSuccess; ++k)
+      if (nrows[k] > 0)
+        hipLaunchKernelGGL(hyb_place_slots_kernel, dim3((unsigned)stir::ceil_div(nrows[k], 256)), dim3(256), 0, 0,
+                           d_rows[k], d_cols[k], d_A[k], nrows[k], bucket_widths[k % num_buckets], count, mr.cols,
+                           mr.vals);
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+  }
+  cleanup();
+  if (e != hipSuccess || h_flags[1] != 0) {
+    mr.release();
+    if (e != hipSuccess) return stir::fail("hyb_plan_create: %s", hipGetErrorString(e));
+    return stir::fail("hyb_plan_create: a row index lies outside [0, %d)", m);
+  }
+  mr.slots = slots;
+  *out = mr;
+  *built = true;
+  return 0;
+}
+
+// Launches the CSR row kernels over the merged rows.  feat must have a vector class.
+int launch_merged(const MergedRows& mr, int32_t m, int32_t feat, const float* d_B, float* d_C, hipStream_t st) {
+  dim3 grid((unsigned)stir::ceil_div(m, 4)), block(256);
+  dim3 pieces((unsigned)stir::ceil_div(stir::ceil_div(mr.slots, kLongPiece), 4));
+  const float* vals = reinterpret_cast<const float*>(mr.vals);
+#define STIR_MERGED(G, REP)                                                                                   \
+  {                                                                                                           \
+    hipLaunchKernelGGL((csr_spmm_kernel<G, REP, true>), grid, block, 0, st, m, feat, 1, vals, d_B, d_C,       \
+                       mr.slot_ptr, mr.cols);                                                                 \
+    hipLaunchKernelGGL((csr_long_rows_kernel<G, REP, true>), pieces, block, 0, st, m, feat, (int64_t)0, mr.slots, \
+                       vals, d_B, d_C, mr.slot_ptr, mr.cols);                                                 \
+  }
+  switch (vector_class(feat)) {
+    case 0: STIR_MERGED(4, 1); break;
+    case 1: STIR_MERGED(8, 1); break;
+    case 2: STIR_MERGED(16, 1); break;
+    case 3: STIR_MERGED(32, 1); break;
+    case 4: STIR_MERGED(64, 1); break;
+    case 5: STIR_MERGED(64, 2); break;
+    default: return stir::fail("hyb_spmm: feat=%d has no vectorised kernel", feat);
+  }
+#undef STIR_MERGED
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
 // Launches the kernels of a hyb operator whose descriptor tables are at d_tiles / d_rows.
 int launch_hyb(const HybTables& t, const HybBucket* d_tiles, const HybBucket* d_rows, int32_t feat,
                const float* d_B, float* d_C, hipStream_t st) {
@@ -651,6 +827,8 @@ struct stir_hyb_plan {
   int device;
   HybTables tables;
   HybBucket* d_tables;  // tables.tiles followed by tables.rows
+  bool merged;          // more partitions than run as phases: launches go over `rows`
+  MergedRows rows;
 };
 
 extern "C" {
@@ -708,6 +886,13 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
   p->num_col_parts = num_col_parts;
   p->num_buckets = num_buckets;
   p->d_tables = nullptr;
+  p->merged = false;
+  if (num_col_parts > kMaxPhases &&
+      build_merged_rows(m, num_col_parts * num_buckets, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols,
+                        &p->rows, &p->merged) != 0) {
+    delete p;
+    return -1;
+  }
   make_hyb_tables(num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols, phased, &p->tables);
   const size_t nk = p->tables.tiles.size();
   hipError_t e = hipGetDevice(&p->device);
@@ -720,6 +905,7 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
   }
   if (e != hipSuccess) {
     if (p->d_tables) (void)hipFree(p->d_tables);
+    p->rows.release();
     delete p;
     return stir::fail("hyb_plan_create: %s", hipGetErrorString(e));
   }
@@ -734,6 +920,8 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
   const size_t nk = plan->tables.tiles.size();
   if (nk == 0) return 0;
   STIR_REQUIRE(d_B && d_C, "hyb_spmm: null pointer argument");
+  if (plan->merged && vector_class(feat) >= 0)
+    return launch_merged(plan->rows, plan->m, feat, d_B, d_C, static_cast<hipStream_t>(stream));
   return launch_hyb(plan->tables, plan->d_tables, plan->d_tables + nk, feat, d_B, d_C,
                     static_cast<hipStream_t>(stream));
 }
@@ -776,6 +964,7 @@ int stir_hyb_spmm_f32_noalloc(int32_t m, int32_t n, int32_t num_col_parts, int32
 int stir_hyb_plan_destroy(stir_hyb_plan* plan) {
   if (!plan) return 0;
   if (plan->d_tables) (void)hipFree(plan->d_tables);
+  plan->rows.release();
   delete plan;
   return 0;
 }

@@ -303,3 +303,42 @@ def test_time_evaluator_protocol(dev):
     assert 0 < secs < 1e-2
     assert f.entry_name == "main"
     _check(c.cpu().numpy().reshape(m, feat), g["indptr"], g["indices"], g["values"], g["x"], "after timing")
+
+
+@pytest.mark.parametrize("parts,buckets", [(8, [1, 2, 4, 8]), (16, [1, 2, 4, 8, 16, 32]), (6, [3, 300])])
+def test_hyb_spmm_many_partitions_add_and_follow_the_weights(dev, parts, buckets):
+    """More than four column partitions: the plan lists the slots of every output row once and its
+    launches go over that list.  The operator still adds to C (the reference's buckets add with
+    atomics when there are several partitions, examples/spmm/bench_spmm.py:170-177), also for a
+    row of thousands of entries, and still reads the weights at every call."""
+    m, n, feat = 2000, 2500, 64
+    indptr, indices = random_csr(m, n, 50000, parts, skew=1.2)
+    # one row with entries in every partition, far beyond one wavefront's share
+    hub = np.sort(np.random.default_rng(parts).choice(n, 2200, replace=False)).astype(np.int32)
+    deg = np.diff(indptr)
+    indices = np.concatenate([indices[:indptr[7]], hub, indices[indptr[8]:]]).astype(np.int32)
+    deg[7] = len(hub)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    triples = _hyb_setup(dev, indptr, indices, m, n, parts, buckets, weighted=True, seed=parts)
+    x = np.random.default_rng(1).standard_normal((n, feat), dtype=np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    f = ops.build_hyb_csrmm(m, n, feat, parts, buckets, [len(r) for _, r, _ in triples])
+    args = []
+    for a, r, c in triples:
+        args += [t(a.ravel()), t(r), t(c.ravel())]
+    import scipy.sparse as sp
+    r, c, v = _hyb_as_coo(triples)
+    exact = sp.csr_matrix((v.astype(np.float64), (r, c)), shape=(m, n)) @ x.astype(np.float64)
+    scale = sp.csr_matrix((np.abs(v).astype(np.float64), (r, c)), shape=(m, n)) @ np.abs(x).astype(np.float64)
+    start = np.random.default_rng(2).standard_normal((m, feat), dtype=np.float32)
+    cdev = t(start.ravel().copy())
+    f(t(x.ravel()), cdev, *args)
+    got = cdev.cpu().numpy().reshape(m, feat)
+    assert np.all(np.abs(got - (start + exact)) <= RTOL * (scale + np.abs(start)) + 1e-30)
+    # the weights doubled in place: the same plan gives twice the product
+    for k in range(0, len(args), 3):
+        args[k].mul_(2)
+    cdev.zero_()
+    f(t(x.ravel()), cdev, *args)
+    got2 = cdev.cpu().numpy().reshape(m, feat)
+    assert np.all(np.abs(got2 - 2 * exact) <= 2 * RTOL * scale + 1e-30)
