@@ -535,6 +535,41 @@ def main():
                                         "frac_of_hbm_peak": sd_bytes / d4 / 1e9 / HBM_PEAK_GBS,
                                         "preproc_ms": d3 * 1e3}
         del edge, a2, b2, out, mid, sargs
+        if args.parts is None and args.buckets is None and not getattr(args, "profile", False):
+            # the reference's own decomposition for a graph of this size: 16 column partitions, widths
+            # 1..32 (examples/spmm/bench_spmm.py:233-253); the bench line above uses 1 x 1..512
+            rparts, rbuckets = 16, [1, 2, 4, 8, 16, 32]
+            rr, rc, rm = st.column_part_hyb(m, n, d_indptr, d_indices, rparts, rbuckets)
+            rtriples, rnrows = [], []
+            for p in range(rparts):
+                for b in range(len(rbuckets)):
+                    rtriples += [rm[p][b].reshape(-1).float(), rr[p][b], rc[p][b].reshape(-1)]
+                    rnrows.append(int(rr[p][b].shape[0]))
+            del rr, rc, rm
+            rhyb = ops.build_hyb_csrmm(m, n, feat, rparts, rbuckets, rnrows)
+            c.zero_()
+            hyb(x, c, *triples)
+            c_ref = torch.zeros_like(c)
+            rhyb(x, c_ref, *rtriples)
+            torch.cuda.synchronize()
+            rdiff = float((c_ref - c).abs().max().item())
+            deg_max = float(np.diff(indptr).max())
+            check["reference_decomposition_vs_bench_decomposition_ok"] = bool(rdiff <= 1e-5 * 6.0 * max(deg_max, 1.0))
+
+            def rstep():
+                c_ref.zero_()  # the operator adds to C
+                rhyb(x, c_ref, *rtriples)
+
+            wr, dr, _ = time_steps(rstep, steps, 1, torch)
+            wz, dz, _ = time_steps(lambda: c_ref.zero_(), steps, 1, torch)
+            extra["hyb_spmm_reference_decomposition"] = {"num_col_parts": rparts, "buckets": rbuckets,
+                                                         "ell_rows": int(sum(rnrows)),
+                                                         "ms_per_step_with_clearing_C": wr * 1e3,
+                                                         "clearing_C_ms": wz * 1e3, "ms": (wr - wz) * 1e3,
+                                                         "gflops": flops / (wr - wz) / 1e9,
+                                                         "max_abs_diff_to_bench_decomposition": rdiff}
+            del rtriples, rhyb, c_ref
+            torch.cuda.empty_cache()
         # the main workload's arrays are released before the next graph is built
         del x, c, hyb, csr, triples, d_indptr, d_indices, indptr, indices
         wl.clear()
