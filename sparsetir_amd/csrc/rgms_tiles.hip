@@ -256,6 +256,31 @@ __device__ __forceinline__ f32x16 stage2(u32x4 sa, const float* t, f32x16 acc) {
 
 constexpr int kSStride = 40;  // 16-bit elements per row of the S tile (32 used; 80-byte rows)
 
+// Stage 2 of a step: acc2 += S @ T, with T = acc1 as it left stage 1 and S[i, e] = weight of edge e
+// if it ends in row i of the tile.  The lane of edge e (lanes 0..31) puts its weight at
+// (dl, jcol) of the wavefront's all-zero S tile, every lane reads its operand row, and the entry
+// is cleared again; LDS operations of one wavefront execute in order, so no barrier is needed.
+// Steps of at most 16 edges skip the second half of k.
+template <bool BF16>
+__device__ __forceinline__ f32x16 scatter_step(uint16_t* S, int dl, int jcol, int mrow, int h, uint16_t weight,
+                                               int left, const f32x16& acc1, f32x16 acc2) {
+  if (h == 0) S[dl * kSStride + jcol] = weight;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  const u32x4 sa0 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 8 * h);
+  u32x4 sa1 = {0u, 0u, 0u, 0u};
+  if (left > 16) sa1 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 16 + 8 * h);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  if (h == 0) S[dl * kSStride + jcol] = 0;
+  float t[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) t[v] = acc1[v];
+  acc2 = stage2<BF16>(sa0, t, acc2);
+  if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
+  return acc2;
+}
+
 // One workgroup per unit.  Its four wavefronts take the unit's steps in turn (wavefront w the
 // steps w, w + 4, ...: more wavefronts in flight per tile, since a step costs a full memory
 // round trip), each with its own accumulator tile; the four tiles are added through LDS and the
@@ -379,20 +404,7 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
       }
 
       // ---- stage 2
-      if (h == 0) S[dl * kSStride + jcol] = live ? wbits : (uint16_t)0;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      const u32x4 sa0 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 8 * h);
-      u32x4 sa1 = {0u, 0u, 0u, 0u};
-      if (left > 16) sa1 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 16 + 8 * h);
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      if (h == 0) S[dl * kSStride + jcol] = 0;
-      float t[16];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) t[v] = acc1[v];
-      acc2 = stage2<BF16>(sa0, t, acc2);
-      if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
+      acc2 = scatter_step<BF16>(S, dl, jcol, mrow, h, live ? wbits : (uint16_t)0, left, acc1, acc2);
     }
 
     // ---- add the four tiles and write back.  acc2[v] of lane (n, h) is row (v%4) + 4h + 8(v/4)
@@ -640,20 +652,7 @@ __global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
 
         // ---- stage 2
         if (e0 == e_first) team_wait();  // the sums of the pass before have been read out of the S tiles
-        if (h == 0) S[dl * kSStride + jcol] = live ? wbits : (uint16_t)0;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        const u32x4 sa0 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 8 * h);
-        u32x4 sa1 = {0u, 0u, 0u, 0u};
-        if (left > 16) sa1 = *reinterpret_cast<const u32x4*>(S + mrow * kSStride + 16 + 8 * h);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        if (h == 0) S[dl * kSStride + jcol] = 0;
-        float t[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) t[v] = acc1[v];
-        acc2 = stage2<BF16>(sa0, t, acc2);
-        if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
+        acc2 = scatter_step<BF16>(S, dl, jcol, mrow, h, live ? wbits : (uint16_t)0, left, acc1, acc2);
       };
       // Two steps per turn of the loop, so that the two sets of X registers swap roles without
       // copies: while a step is computed, the rows of X of the step after it are on their way,
@@ -735,10 +734,10 @@ int bit_length(uint64_t x) {
   return b;
 }
 
-// A resident workgroup has 8, 12 or 16 wavefronts ("quads" of four: each wavefront needs an S tile
-// in LDS beside W); 16 only for the variants that fit 128 registers.
-constexpr bool resident_four_quads(bool packed, int kk) { return packed && kk <= 2; }
-int resident_max_quads(bool packed, int kk) { return resident_four_quads(packed, kk) ? 4 : 3; }
+// A resident workgroup has 8 or 12 wavefronts ("quads" of four: each wavefront needs an S tile in
+// LDS beside W).  16 would leave 128 registers per wavefront, which the kernel only just fits or
+// spills, and measured no faster where W left the room (60 relations of 32 x 32).
+constexpr int kResidentMaxQuads = 3;
 
 // Launches the resident kernel with `quads` x 4 wavefronts per workgroup.
 template <int KK, bool BF16, typename Rec>
@@ -754,9 +753,6 @@ int launch_resident(int quads, dim3 grid, size_t lds, hipStream_t stream, const 
   constexpr int kTeamsPerQuad = 4 / kTeamWaves;
   if (quads == 2) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 2 * kTeamsPerQuad>);
   if (quads == 3) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 3 * kTeamsPerQuad>);
-  if constexpr (resident_four_quads(sizeof(Rec) == sizeof(PackedEdge), KK)) {
-    if (quads == 4) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 4 * kTeamsPerQuad>);
-  }
   return fail("rgms: no kernel for %d wavefronts per workgroup", 4 * quads);
 }
 
@@ -989,7 +985,7 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   if (kk_count <= kLdsMaxKK && reinterpret_cast<uintptr_t>(d_W) % 16 == 0 &&
       (int64_t)ix.n * feat_in * 2 < (int64_t(1) << 32)) {
     const size_t lds_limit = lds_bytes_per_workgroup();
-    for (int q = resident_max_quads(ix.packed_records, kk_count); q >= 2 && quads == 0; --q)
+    for (int q = kResidentMaxQuads; q >= 2 && quads == 0; --q)
       if (w_bytes + size_t(q) * 4 * kSBytes <= lds_limit) quads = q;
   }
   if (quads) {
