@@ -154,8 +154,10 @@ class HybCsrMM(_Operator):
     def invalidate(self):
         """Forget the plan made from the arrays of the last call.  The plan is reused while the
         (A_k, rows_k, cols_k) arrays keep their addresses; with 2 to 4 column partitions it also
-        remembers whether the row arrays allowed dropping atomics.  Call this after rewriting row
-        arrays in place (the reference's operator reads them afresh on every call)."""
+        remembers whether the row arrays allowed dropping atomics, and with more than 4 it holds a
+        list of every output row's slots made from the row and column arrays (the weights A_k are
+        read at every call).  Call this after rewriting row or column arrays in place (the
+        reference's operator reads them afresh on every call)."""
         self._drop_plan()
         self._key = None
 
