@@ -342,3 +342,34 @@ def test_hyb_spmm_many_partitions_add_and_follow_the_weights(dev, parts, buckets
     f(t(x.ravel()), cdev, *args)
     got2 = cdev.cpu().numpy().reshape(m, feat)
     assert np.all(np.abs(got2 - 2 * exact) <= 2 * RTOL * scale + 1e-30)
+
+
+def test_hyb_spmm_many_partitions_invalidate_after_rewriting_columns(dev):
+    """A plan with more than four partitions holds a copy of the column ids: a caller that rewrites
+    the column arrays in place tells the operator (invalidate) and then gets the result for the
+    new columns, the one a fresh operator computes."""
+    m, n, feat, parts, buckets = 1500, 1800, 32, 6, [1, 2, 4, 8]
+    indptr, indices = random_csr(m, n, 30000, 5, skew=1.1)
+    triples = _hyb_setup(dev, indptr, indices, m, n, parts, buckets, weighted=True, seed=3)
+    x = np.random.default_rng(3).standard_normal((n, feat), dtype=np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    args = []
+    for a, r, c in triples:
+        args += [t(a.ravel()), t(r), t(c.ravel())]
+    nrows = [len(r) for _, r, _ in triples]
+    xd = t(x.ravel())
+
+    def run(op):
+        cdev = torch.zeros(m * feat, dtype=torch.float32, device=dev)
+        op(xd, cdev, *args)
+        torch.cuda.synchronize()
+        return cdev
+
+    f = ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)
+    before = run(f)
+    for k in range(2, len(args), 3):
+        args[k].copy_((args[k] + 7) % n)   # other columns at the same addresses
+    fresh = run(ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows))
+    assert not torch.allclose(fresh, before, rtol=1e-3, atol=1e-3)
+    f.invalidate()
+    assert torch.allclose(run(f), fresh, rtol=1e-5, atol=1e-5)
