@@ -265,10 +265,12 @@ int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t g
  * The plan keeps the array pointers.  From 8192 slots on, the first launch builds an edge index
  * from the three index arrays (they must not change afterwards; the weights may), and the first
  * launch with given feature sizes a work list for them (both allocate and synchronise the
- * stream; later launches do neither).  W is read anew at every launch.  When W does not fit the
- * LDS of a compute unit beside the kernel's tiles (about 130 KB: 65 relations of 32 x 32), when
- * feat_in exceeds 64 or d_W is not 16-byte aligned, every launch rewrites a packed copy of W held
- * by the plan; a plan therefore serves one call at a time.
+ * stream; later launches do neither).  W is read anew at every launch.  W that does not fit the
+ * LDS of a compute unit beside the kernel's tiles (about 130 KB: 65 relations of 32 x 32) is
+ * served as up to three ranges of relations, each with an index and a launch of its own.  With
+ * more relations than that, with feat_in above 64 or a d_W that is not 16-byte aligned, every
+ * launch rewrites a packed copy of W held by the plan; a plan therefore serves one call at a
+ * time.
  */
 typedef struct stir_rgms_plan stir_rgms_plan;
 int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int32_t* rows_bkt,

@@ -259,7 +259,7 @@ struct stir_rgms_plan {
   std::vector<stir::TileBucket> tile_buckets;
   int64_t slots;
   bool static_weights;  // promise of the caller, see stir_rgms_plan_set_static_weights
-  stir::TileIndex tiles;
+  stir::TileIndexSet tiles;
 };
 
 extern "C" {
@@ -348,8 +348,9 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
     // the plan's edge index and packed copy of W are filled in by the launches: a plan serves
     // one call at a time
     stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
-    if (stir::tile_index_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, mp->static_weights, st)) return -1;
-    return stir::tile_rgms_launch(bf16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
+    if (stir::tile_set_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, feat_in, feat_out, mp->static_weights, st))
+      return -1;
+    return stir::tile_set_launch(bf16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
   }
 #define STIR_RGMS(KK)                                                                              \
   case KK:                                                                                         \
@@ -396,7 +397,7 @@ int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on) {
 int stir_rgms_plan_destroy(stir_rgms_plan* plan) {
   if (!plan) return 0;
   if (plan->d_table) (void)hipFree(plan->d_table);
-  stir::tile_index_free(plan->tiles);
+  stir::tile_set_free(plan->tiles);
   delete plan;
   return 0;
 }

@@ -25,8 +25,9 @@ struct TileBucket {
 };
 
 struct TileIndex {
-  int32_t m = -1, n = -1, num_rels = -1;  // what the index was built for
-  bool packed_records = false;            // 8-byte records that carry the slot weights (see tile_index_prepare)
+  int32_t m = -1, n = -1, num_rels = -1;  // what the index was built for; num_rels counts from rel_lo
+  int32_t rel_lo = 0;                     // first relation of the index
+  bool packed_records = false;            // 8-byte records that carry the slot weights (see tile_set_prepare)
   int64_t edges = 0;                      // slots of all buckets
   int64_t units = 0;
   void* d_edges = nullptr;  // edges x 16 (or 8) bytes, sorted
@@ -42,18 +43,26 @@ struct TileIndex {
   void* d_share_units = nullptr;  // units x 16 bytes, grouped by team
 };
 
-// Builds the index on `stream` (synchronises; allocates).  A no-op when it already exists for
-// the same m, n and num_rels.  Fails when a row id, column id or relation id is out of range.
+// The indices of a plan: one for all relations, or -- when W does not fit the LDS of a compute unit
+// and a few ranges of relations do -- one per range, launched one after the other.
+struct TileIndexSet {
+  int32_t m = -1, n = -1, num_rels = -1, rels_per_part = 0;  // what the set was built for
+  std::vector<TileIndex> parts;                               // part p: relations from p * rels_per_part
+};
+
+// Builds the indices on `stream` (synchronises; allocates).  A no-op when they already exist for
+// the same m, n and num_rels and the feature sizes lead to the same ranges of relations.  Fails
+// when a row id, column id or relation id is out of range.
 // static_weights: the caller promises that the slot weights keep the values they have now.  Slots
 // of weight zero (the padding of ELL3D) are then left out of the index and a record shrinks to
 // 8 bytes holding the weight itself (source row; weight << 16 | relation << 5 | row in tile), for
-// up to 2048 relations; otherwise records hold the weight's address and weights are read at
-// every launch.
-int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
-                       int32_t num_rels, bool static_weights, hipStream_t stream);
+// up to 2048 relations per index; otherwise records hold the weight's address and weights are
+// read at every launch.
+int tile_set_prepare(TileIndexSet& set, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
+                     int32_t num_rels, int32_t feat_in, int32_t feat_out, bool static_weights, hipStream_t stream);
 // Y += RGMS(W, X) over the indexed edges.  W: [R, feat_in, feat_out], X: [n, feat_in], 16-bit.
-int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W,
-                     const void* d_X, float* d_Y, hipStream_t stream);
-void tile_index_free(TileIndex& ix);
+int tile_set_launch(bool bf16, TileIndexSet& set, int32_t feat_in, int32_t feat_out, const void* d_W,
+                    const void* d_X, float* d_Y, hipStream_t stream);
+void tile_set_free(TileIndexSet& set);
 
 }  // namespace stir

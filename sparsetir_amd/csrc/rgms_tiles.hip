@@ -69,12 +69,13 @@ __device__ __forceinline__ int bucket_of(const DevBucket* __restrict__ tab, int 
   return lo;
 }
 
-// key = (destination tile, relation, row inside the tile), value = slot
-// drop_zero: slots of weight zero get the key one past the last tile, so they sort behind every
-// tile and no unit covers them
+// key = (destination tile, relation - rel_lo, row inside the tile), value = slot
+// Slots of a relation outside [rel_lo, rel_lo + rel_count) and, with drop_zero, slots of weight
+// zero get the key one past the last tile, so they sort behind every tile and no unit covers them.
 __global__ __launch_bounds__(256) void edge_keys_kernel(const DevBucket* __restrict__ tab, int nb, int64_t slots, int m,
-                                                        int num_rels, int drop_zero, uint64_t* __restrict__ keys,
-                                                        int32_t* __restrict__ vals, int32_t* __restrict__ bad) {
+                                                        int num_rels, int rel_lo, int rel_count, int drop_zero,
+                                                        uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
+                                                        int32_t* __restrict__ bad) {
   const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (q >= slots) return;
   const DevBucket bk = tab[bucket_of(tab, nb, q)];
@@ -88,15 +89,18 @@ __global__ __launch_bounds__(256) void edge_keys_kernel(const DevBucket* __restr
     *bad = 1;
     dest = rel = 0;
   }
-  uint64_t key = ((((uint64_t)(dest >> 5)) * num_rels + rel) << 5) | (uint64_t)(dest & 31);
-  if (drop_zero && (bk.A[local] & 0x7fff) == 0) key = ((uint64_t)((m + kTileRows - 1) / kTileRows) * num_rels) << 5;
+  rel -= rel_lo;
+  uint64_t key = ((((uint64_t)(dest >> 5)) * rel_count + rel) << 5) | (uint64_t)(dest & 31);
+  if ((unsigned)rel >= (unsigned)rel_count || (drop_zero && (bk.A[local] & 0x7fff) == 0))
+    key = ((uint64_t)((m + kTileRows - 1) / kTileRows) * rel_count) << 5;
   keys[q] = key;
   vals[q] = (int32_t)q;
 }
 
 template <typename Rec>
 __global__ __launch_bounds__(256) void edge_records_kernel(const DevBucket* __restrict__ tab, int nb, int64_t slots,
-                                                           int n, int num_rels, const uint64_t* __restrict__ keys,
+                                                           int64_t kept, int n, int num_rels,
+                                                           const uint64_t* __restrict__ keys,
                                                            const int32_t* __restrict__ vals, Rec* __restrict__ edges,
                                                            int32_t* __restrict__ bad) {
   const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -114,14 +118,14 @@ __global__ __launch_bounds__(256) void edge_records_kernel(const DevBucket* __re
   Rec e;
   e.src = src;
   if constexpr (sizeof(Rec) == sizeof(PackedEdge)) {
-    e.w_rel_dl = ((uint32_t)bk.A[local] << 16) | rel_dl;  // dropped slots (beyond the last tile) are never read
+    e.w_rel_dl = ((uint32_t)bk.A[local] << 16) | rel_dl;
   } else {
     const uint64_t addr = reinterpret_cast<uint64_t>(bk.A + local);
     e.w_lo = (uint32_t)addr;
     e.w_hi = (uint32_t)(addr >> 32);
     e.rel_dl = rel_dl;
   }
-  edges[p] = e;
+  if (p < kept) edges[p] = e;  // the slots behind the last tile are checked, not recorded
 }
 
 // begin[t] = first sorted edge of tile t (t = tiles gives the edge count)
@@ -738,6 +742,9 @@ int bit_length(uint64_t x) {
 // LDS beside W).  16 would leave 128 registers per wavefront, which the kernel only just fits or
 // spills, and measured no faster where W left the room (60 relations of 32 x 32).
 constexpr int kResidentMaxQuads = 3;
+// W beyond the LDS: at most this many ranges of relations, each with a launch of its own; more
+// relations than that read W from memory in one launch
+constexpr int kMaxRelationParts = 3;
 
 // Launches the resident kernel with `quads` x 4 wavefronts per workgroup.
 template <int KK, bool BF16, typename Rec>
@@ -815,22 +822,11 @@ int build_shares(TileIndex& ix, int64_t teams, hipStream_t stream) {
   return 0;
 }
 
-}  // namespace
-
-void tile_index_free(TileIndex& ix) {
-  if (ix.d_edges) (void)hipFree(ix.d_edges);
-  if (ix.d_units) (void)hipFree(ix.d_units);
-  if (ix.d_wpack) (void)hipFree(ix.d_wpack);
-  if (ix.d_share_ptr) (void)hipFree(ix.d_share_ptr);
-  if (ix.d_share_units) (void)hipFree(ix.d_share_units);
-  ix = TileIndex();
-}
-
-int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
-                       int32_t num_rels, bool static_weights, hipStream_t stream) {
-  if (ix.m == m && ix.n == n && ix.num_rels == num_rels) return 0;
+// The index of the relations [rel_lo, rel_lo + rel_count) of all_rels; ix.num_rels becomes rel_count.
+int tile_index_build(TileIndex& ix, const std::vector<TileBucket>& buckets, int32_t m, int32_t n, int32_t all_rels,
+                     int32_t rel_lo, int32_t rel_count, bool static_weights, hipStream_t stream) {
+  const int32_t num_rels = rel_count;
   const bool packed = static_weights && num_rels <= kPackedMaxRels;
-  STIR_REQUIRE(num_rels > 0 && num_rels < (1 << 26), "rgms: num_rels=%d out of range", num_rels);
   if (ix.d_edges) STIR_HIP(hipFree(ix.d_edges));
   if (ix.d_units) STIR_HIP(hipFree(ix.d_units));
   if (ix.d_share_ptr) STIR_HIP(hipFree(ix.d_share_ptr));
@@ -848,6 +844,7 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
     slots += b.groups * b.rb * b.cb;
   }
   STIR_REQUIRE(slots < (int64_t(1) << 31), "rgms: %lld slots exceed the edge index", (long long)slots);
+  ix.rel_lo = rel_lo;
   if (slots == 0 || m == 0) {
     ix.m = m, ix.n = n, ix.num_rels = num_rels;
     return 0;
@@ -884,28 +881,16 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   STIR_HIP(begin.alloc(sizeof(int64_t) * size_t(tiles + 1)));
   STIR_HIP(count.alloc(sizeof(int32_t) * size_t(tiles + 1)));
   STIR_HIP(ubegin.alloc(sizeof(int32_t) * size_t(tiles + 1)));
-  DevBuf edges;
-  STIR_HIP(edges.alloc((packed ? sizeof(PackedEdge) : sizeof(Edge)) * size_t(slots)));
-
   STIR_HIP(hipMemcpyAsync(tab.p, host.data(), sizeof(DevBucket) * host.size(), hipMemcpyHostToDevice, stream));
   STIR_HIP(hipMemsetAsync(bad.p, 0, sizeof(int32_t), stream));
   const dim3 block(256);
   const dim3 slot_grid((unsigned)ceil_div(slots, 256)), tile_grid((unsigned)ceil_div(tiles + 1, 256));
-  hipLaunchKernelGGL(edge_keys_kernel, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, m, num_rels,
-                     packed ? 1 : 0, keys_in.as<uint64_t>(), vals_in.as<int32_t>(), bad.as<int32_t>());
+  hipLaunchKernelGGL(edge_keys_kernel, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, m, all_rels,
+                     rel_lo, rel_count, packed ? 1 : 0, keys_in.as<uint64_t>(), vals_in.as<int32_t>(), bad.as<int32_t>());
   STIR_LAUNCH_CHECK();
   STIR_HIP(hipcub::DeviceRadixSort::SortPairs(tmp.p, sort_bytes, keys_in.as<const uint64_t>(), keys.as<uint64_t>(),
                                               vals_in.as<const int32_t>(), vals.as<int32_t>(), (int)slots, 0,
                                               end_bit, stream));
-  if (packed)
-    hipLaunchKernelGGL(edge_records_kernel<PackedEdge>, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, n,
-                       num_rels, keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<PackedEdge>(),
-                       bad.as<int32_t>());
-  else
-    hipLaunchKernelGGL(edge_records_kernel<Edge>, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, n,
-                       num_rels, keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<Edge>(),
-                       bad.as<int32_t>());
-  STIR_LAUNCH_CHECK();
   hipLaunchKernelGGL(tile_bounds_kernel, tile_grid, block, 0, stream, keys.as<const uint64_t>(), slots, tiles,
                      num_rels, begin.as<int64_t>());
   STIR_LAUNCH_CHECK();
@@ -921,7 +906,22 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   STIR_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
   STIR_HIP(hipMemcpyAsync(&h_units, ubegin.as<int32_t>() + tiles, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
   STIR_HIP(hipStreamSynchronize(stream));
-  if (h_bad == 1) return fail("rgms: a row id lies outside [0, %d) or a relation id outside [0, %d)", m, num_rels);
+  if (h_bad == 1) return fail("rgms: a row id lies outside [0, %d) or a relation id outside [0, %d)", m, all_rels);
+  // records of the slots that lie in a tile (the others belong to other relations or are padding)
+  const int64_t kept = ix.tile_begin[size_t(tiles)];
+  DevBuf edges;
+  STIR_HIP(edges.alloc((packed ? sizeof(PackedEdge) : sizeof(Edge)) * size_t(std::max<int64_t>(kept, 1))));
+  if (packed)
+    hipLaunchKernelGGL(edge_records_kernel<PackedEdge>, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots,
+                       kept, n, num_rels, keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<PackedEdge>(),
+                       bad.as<int32_t>());
+  else
+    hipLaunchKernelGGL(edge_records_kernel<Edge>, slot_grid, block, 0, stream, tab.as<DevBucket>(), nb, slots, kept, n,
+                       num_rels, keys.as<const uint64_t>(), vals.as<const int32_t>(), edges.as<Edge>(),
+                       bad.as<int32_t>());
+  STIR_LAUNCH_CHECK();
+  STIR_HIP(hipMemcpyAsync(&h_bad, bad.p, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+  STIR_HIP(hipStreamSynchronize(stream));
   if (h_bad == 2) return fail("rgms: a column id lies outside [0, %d)", n);
   DevBuf units;
   STIR_HIP(units.alloc(sizeof(Unit) * size_t(h_units)));
@@ -958,13 +958,14 @@ int tile_index_prepare(TileIndex& ix, const std::vector<TileBucket>& buckets, in
   STIR_HIP(hipStreamSynchronize(stream));
   ix.d_edges = edges.p, edges.p = nullptr;
   ix.d_units = units.p, units.p = nullptr;
-  ix.edges = slots;
+  ix.edges = kept;
   ix.units = h_units;
   ix.m = m, ix.n = n, ix.num_rels = num_rels;
   ix.packed_records = packed;
   return 0;
 }
 
+// Y += RGMS(W, X) over the edges of one index; W starts at the index's first relation.
 int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
                      float* d_Y, hipStream_t stream) {
   STIR_REQUIRE(ix.m >= 0, "rgms: the edge index has not been built");
@@ -1059,6 +1060,64 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
 #undef STIR_TILES
 #undef STIR_TILES_R
   STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace
+
+void tile_index_free(TileIndex& ix) {
+  if (ix.d_edges) (void)hipFree(ix.d_edges);
+  if (ix.d_units) (void)hipFree(ix.d_units);
+  if (ix.d_wpack) (void)hipFree(ix.d_wpack);
+  if (ix.d_share_ptr) (void)hipFree(ix.d_share_ptr);
+  if (ix.d_share_units) (void)hipFree(ix.d_share_units);
+  ix = TileIndex();
+}
+
+void tile_set_free(TileIndexSet& set) {
+  for (TileIndex& ix : set.parts) tile_index_free(ix);
+  set = TileIndexSet();
+}
+
+int tile_set_prepare(TileIndexSet& set, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
+                     int32_t num_rels, int32_t feat_in, int32_t feat_out, bool static_weights, hipStream_t stream) {
+  STIR_REQUIRE(num_rels > 0 && num_rels < (1 << 26), "rgms: num_rels=%d out of range", num_rels);
+  // Relations per part: all of them, unless W is too large for the LDS of a compute unit and a few
+  // ranges of relations are not -- then every range gets an index and a launch of its own.
+  int32_t per_part = num_rels;
+  if (feat_in % 16 == 0 && feat_in / 16 <= kLdsMaxKK && feat_out % 32 == 0 &&
+      (int64_t)n * feat_in * 2 < (int64_t(1) << 32)) {
+    const size_t rel_bytes = size_t(feat_out / 32) * (feat_in / 16) * 64 * sizeof(u32x4);
+    const size_t lds_limit = lds_bytes_per_workgroup();
+    auto fit = [&](int quads) { return (int64_t)((lds_limit - size_t(quads) * 4 * kSBytes) / rel_bytes); };
+    if (num_rels > fit(2) && fit(kResidentMaxQuads) > 0) {
+      const int64_t parts = ceil_div((int64_t)num_rels, fit(kResidentMaxQuads));
+      if (parts <= kMaxRelationParts) per_part = (int32_t)ceil_div((int64_t)num_rels, parts);
+    }
+  }
+  if (set.m == m && set.n == n && set.num_rels == num_rels && set.rels_per_part == per_part) return 0;
+  tile_set_free(set);
+  const int parts = (int)ceil_div(num_rels, per_part);
+  set.parts.resize(size_t(parts));
+  for (int p = 0; p < parts; ++p) {
+    const int32_t lo = p * per_part;
+    if (int rc = tile_index_build(set.parts[size_t(p)], buckets, m, n, num_rels, lo, std::min(per_part, num_rels - lo),
+                                  static_weights, stream)) {
+      tile_set_free(set);
+      return rc;
+    }
+  }
+  set.m = m, set.n = n, set.num_rels = num_rels, set.rels_per_part = per_part;
+  return 0;
+}
+
+int tile_set_launch(bool bf16, TileIndexSet& set, int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
+                    float* d_Y, hipStream_t stream) {
+  STIR_REQUIRE(set.m >= 0, "rgms: the edge index has not been built");
+  for (TileIndex& ix : set.parts) {
+    const uint16_t* W = static_cast<const uint16_t*>(d_W) + (int64_t)ix.rel_lo * feat_in * feat_out;
+    if (int rc = tile_rgms_launch(bf16, ix, feat_in, feat_out, W, d_X, d_Y, stream)) return rc;
+  }
   return 0;
 }
 

@@ -388,11 +388,54 @@ def test_rgms_tiled_random_shapes(dev, seed):
         f"R={R} m={m} n={n} group={group} widths={widths} fin={fin} fout={fout}: worst {err.max():.3e}")
 
 
+@pytest.mark.parametrize("R,skew", [
+    (100, 1.0),   # two ranges of 50 relations, each with W in the LDS
+    (150, 1.2),   # three ranges, a long tail of small relations
+    (200, 0.0),   # too many ranges: one launch that reads W from memory
+    (1000, 1.5),  # relations without edges among them
+])
+def test_rgms_tiled_more_relations_than_fit_the_lds(dev, R, skew):
+    """More relations than the LDS of a compute unit holds (the reference's AIFB, BGS and AM
+    graphs, examples/rgms/rgcn/bench_rgcn_tensorcore.py:917, have about 90 to 270 with their
+    inverses): the plan indexes a few ranges of relations apart and launches them in turn, or reads
+    W from memory.  Relation sizes follow a power law and are shuffled, so a range mixes large
+    and small relations; against the float64 closed form, added to a Y that is not zero."""
+    rng = np.random.default_rng(77 + R)
+    m, n, fin, fout = 2100, 1900, 32, 32
+    size = 1.0 / np.arange(1, R + 1) ** skew
+    size = rng.permutation(np.floor(size / size.sum() * 50000).astype(np.int64))
+    assert (size == 0).any() == (R == 1000)
+    pairs = [(rng.integers(0, m, k), rng.integers(0, n, k)) for k in size]
+    csf = _csf_from_pairs(pairs, n)
+    group, buckets = 64, [1, 2, 4, 8]
+    rows_bkt = [group // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
+    assert slots_of(mask) >= 8192
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    x = t(rng.standard_normal((n, fin), dtype=np.float32)).half()
+    w = t(rng.standard_normal((R, fin, fout), dtype=np.float32) * 0.1).half()
+    triples, mids = [], []
+    for b in range(len(buckets)):
+        triples += [t(mask[b].astype(np.float16).ravel()), t(rows[b].ravel()), t(cols[b].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[b]))))
+    ones = np.ones(len(csf[3]), np.float32)
+    x32, w32 = x.float().cpu().numpy(), w.float().cpu().numpy()
+    want = rgms_f64(*csf, ones, x32, w32, m)
+    scale = rgms_f64(*csf, ones, np.abs(x32), np.abs(w32), m)
+    for static in (False, True):
+        f = ops.build_rgms(m, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols], static_weights=static)
+        y = torch.full((m * fout,), 0.5, dtype=torch.float32, device=dev)
+        f(w.reshape(-1), x.reshape(-1), y, *triples, *mids)
+        torch.cuda.synchronize()
+        err = np.abs(y.cpu().numpy().reshape(m, fout) - 0.5 - want)
+        assert np.all(err <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-6), f"static={static}: worst {err.max():.3e}"
+
+
 @pytest.mark.parametrize("R,fin,fout,static", [
-    (60, 32, 32, True),    # W of 120 KB: resident kernel, four teams of wavefronts per compute unit
-    (65, 32, 32, False),   # 130 KB: three teams
-    (68, 32, 32, True),    # 136 KB: two teams
-    (80, 32, 32, False),   # 160 KB: W does not fit the LDS, the kernel that reads W from memory
+    (60, 32, 32, True),    # W of 120 KB: resident kernel, 12 wavefronts per compute unit
+    (65, 32, 32, False),   # 130 KB: the most that leaves room for 12
+    (68, 32, 32, True),    # 136 KB: 8 wavefronts
+    (80, 32, 32, False),   # 160 KB: two ranges of 40 relations, a launch each
     (20, 64, 64, True),    # two feature tiles out, four operand blocks in
     (33, 48, 32, False),   # feat_in that is not a power of two
 ])
