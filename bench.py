@@ -228,6 +228,8 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
 
     bsr("bsr_config4_f16", 128, 128, 32, 0.10, 512, torch.float16)
     bsr("bsr_config4_bf16", 128, 128, 32, 0.10, 512, torch.bfloat16)
+    # config 4's weight against 16 times the activation columns: X stays in L2, the launch is long
+    bsr("bsr_config4_weight_f8192_f16", 128, 128, 32, 0.10, 8192, torch.float16, calls=50)
     bsr("bsr_16384x16384_f4096_f16", 512, 512, 32, 0.10, 4096, torch.float16, calls=20)
     bsr("bsr_16384x16384_blk64_f4096_f16", 256, 256, 64, 0.10, 4096, torch.float16, calls=20)
     bsr("bsr_16384x16384_blk128_f4096_f16", 128, 128, 128, 0.10, 4096, torch.float16, calls=20)
