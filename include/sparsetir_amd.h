@@ -120,6 +120,33 @@ int stir_column_part_hyb_device_values(int32_t num_rows, int32_t num_cols, const
                                        float* const* d_A, void* stream);
 
 /*
+ * CSFToELL3D on the GPU, bit-exact with stir_csf_to_ell3d_sizes / _fill above (the reference runs
+ * this on the CPU only, src/sparse/format.cc:195-202).  num_stored_rows is the length of
+ * csf_indices_0, nnz that of csf_indices_1.  The row ids of every relation must ascend strictly
+ * (the sequential routine lets two stored rows with one id share an ELL row; the device pass
+ * rejects such input, the host routine takes it).  At most 32 buckets.  d_workspace must hold
+ * stir_csf_to_ell3d_device_workspace_bytes(num_rels, num_stored_rows, num_buckets) bytes and stay
+ * untouched between _sizes and _fill; _sizes synchronises the stream and returns groups on the
+ * host, _fill takes them back and writes device arrays through host tables of device pointers.
+ */
+size_t stir_csf_to_ell3d_device_workspace_bytes(int32_t num_rels, int64_t num_stored_rows,
+                                                int32_t num_buckets);
+int stir_csf_to_ell3d_device_sizes(int32_t num_rels, int64_t num_stored_rows, int64_t nnz,
+                                   const int32_t* d_indptr0, const int32_t* d_indices0,
+                                   const int32_t* d_indptr1, const int32_t* d_indices1,
+                                   const int32_t* rows_bkt, const int32_t* cols_bkt,
+                                   int32_t num_buckets, void* d_workspace, int64_t* groups,
+                                   void* stream);
+int stir_csf_to_ell3d_device_fill(int32_t num_rels, int64_t num_stored_rows, int64_t nnz,
+                                  const int32_t* d_indptr0, const int32_t* d_indices0,
+                                  const int32_t* d_indptr1, const int32_t* d_indices1,
+                                  const int32_t* rows_bkt, const int32_t* cols_bkt,
+                                  int32_t num_buckets, void* d_workspace, const int64_t* groups,
+                                  int32_t* const* d_indptr, int32_t* const* d_row_indices,
+                                  int32_t* const* d_col_indices, int32_t* const* d_mask,
+                                  void* stream);
+
+/*
  * CSR -> BSR packing on the GPU (blk x blk blocks; m and n multiples of blk): the canonical BSR
  * arrays that scipy's csr_matrix.tobsr hands the reference's example
  * (examples/blocksparse/bsr_spmm.py:441-445) -- block columns ascending in each block row,

@@ -133,6 +133,8 @@ enum {
  * "tir.sparse.CSFToELL3D.sizes"    (indptr0, indices0, indptr1, indices1, rows_bkt, cols_bkt, groups_out)
  * "tir.sparse.CSFToELL3D.fill"     (indptr0, indices0, indptr1, indices1, rows_bkt, cols_bkt,
  *                                   indptr_0, rows_0, cols_0, mask_0, indptr_1, ...) src/sparse/format.cc:180-343
+ *      With kDLROCM/kDLCUDA CSF arrays the conversion runs on the GPU and the outputs are device
+ *      tensors (row ids must ascend strictly inside a relation; .sizes first, on the same thread).
  * "tir.sparse.ConDense.sizes"      (indptr, indices, t, g, group_indptr_out, num_groups_out)
  * "tir.sparse.ConDense.fill"       (indptr, indices, t, g, tile_indices_out, mask_out)  src/sparse/format.cc:353-429
  */

@@ -622,8 +622,11 @@ int stir_packed_column_part_hyb_fill(TVMValue* v, int* tc, int n, TVMRetValueHan
 static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
   Args a{fn, v, tc, n};
   if (n < 7) return packed_fail("%s: num_args should be at least 7", fn);
-  Arr P0 = a.arr(0, "csf_indptr_0", kDLInt, 32, kHost), I0 = a.arr(1, "csf_indices_0", kDLInt, 32, kHost),
-      P1 = a.arr(2, "csf_indptr_1", kDLInt, 32, kHost), I1 = a.arr(3, "csf_indices_1", kDLInt, 32, kHost),
+  // CSF arrays on the GPU take the device pass and its outputs are device arrays too
+  const bool dev = a.on_device(0);
+  const Where w = dev ? kDevice : kHost;
+  Arr P0 = a.arr(0, "csf_indptr_0", kDLInt, 32, w), I0 = a.arr(1, "csf_indices_0", kDLInt, 32, w),
+      P1 = a.arr(2, "csf_indptr_1", kDLInt, 32, w), I1 = a.arr(3, "csf_indices_1", kDLInt, 32, w),
       RB = a.arr(4, "nnz_rows_bkt", kDLInt, 32, kHost), CB = a.arr(5, "nnz_cols_bkt", kDLInt, 32, kHost);
   if (!a.ok) return -1;
   if (RB.len != CB.len) return packed_fail("%s: Input nnz_rows and nnz_cols should have same length.", fn);
@@ -632,29 +635,53 @@ static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
   if (rels < 0 || !fits_i32(rels)) return packed_fail("%s: csf_indptr_0 must have at least one entry", fn);
   const int32_t *p0 = (const int32_t*)P0.data, *i0 = (const int32_t*)I0.data, *p1 = (const int32_t*)P1.data,
                 *i1 = (const int32_t*)I1.data, *rb = (const int32_t*)RB.data, *cb = (const int32_t*)CB.data;
+  if (dev && P1.len != I0.len + 1)
+    return packed_fail("%s: csf_indptr_1 must have one entry more than csf_indices_0", fn);
+  DeviceGuard g;
+  if (dev && g.enter(a.dev_id)) return forward(-1);
+  // the device path keeps its scratch between the sizing and the fill call
+  static thread_local void* ws = nullptr;
+  static thread_local size_t ws_bytes = 0;
   if (!fill) {
     if (!a.count(7)) return -1;
     Arr G = a.arr(6, "groups_out", kDLInt, 64, kHost);
     if (!a.ok || !a.len(G, "groups_out", nb)) return -1;
-    return forward(stir_csf_to_ell3d_sizes((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, (int64_t*)G.data));
+    if (!dev) return forward(stir_csf_to_ell3d_sizes((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, (int64_t*)G.data));
+    const size_t need = stir_csf_to_ell3d_device_workspace_bytes((int32_t)rels, I0.len, nb);
+    if (need > ws_bytes) {
+      if (ws) (void)hipFree(ws);
+      ws = nullptr;
+      ws_bytes = 0;
+      if (hipMalloc(&ws, need) != hipSuccess) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
+      ws_bytes = need;
+    }
+    return forward(stir_csf_to_ell3d_device_sizes((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
+                                                  (int64_t*)G.data, g_stream));
   }
   if (!a.count(6 + 4 * nb)) return -1;
   std::vector<int32_t*> OP(nb), R(nb), C(nb), M(nb);
+  std::vector<int64_t> groups(nb);
   for (int b = 0; b < nb; ++b) {
-    Arr op = a.arr(6 + 4 * b, "indptr_k", kDLInt, 32, kHost), r = a.arr(7 + 4 * b, "rows_k", kDLInt, 32, kHost),
-        c = a.arr(8 + 4 * b, "cols_k", kDLInt, 32, kHost), mk = a.arr(9 + 4 * b, "mask_k", kDLInt, 32, kHost);
+    Arr op = a.arr(6 + 4 * b, "indptr_k", kDLInt, 32, w), r = a.arr(7 + 4 * b, "rows_k", kDLInt, 32, w),
+        c = a.arr(8 + 4 * b, "cols_k", kDLInt, 32, w), mk = a.arr(9 + 4 * b, "mask_k", kDLInt, 32, w);
     if (!a.ok) return -1;
     a.len(op, "indptr_k", rels + 1);
     a.len(c, "cols_k", r.len * cb[b]);
     a.len(mk, "mask_k", r.len * cb[b]);
     if (!a.ok) return -1;
+    if (rb[b] <= 0 || r.len % rb[b] != 0) return packed_fail("%s: rows_k does not hold whole groups", fn);
+    groups[b] = r.len / rb[b];
     OP[b] = (int32_t*)op.data;
     R[b] = (int32_t*)r.data;
     C[b] = (int32_t*)c.data;
     M[b] = (int32_t*)mk.data;
   }
-  return forward(stir_csf_to_ell3d_fill((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, OP.data(), R.data(), C.data(),
-                                        M.data()));
+  if (!dev)
+    return forward(stir_csf_to_ell3d_fill((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, OP.data(), R.data(), C.data(),
+                                          M.data()));
+  if (!ws) return packed_fail("%s: call tir.sparse.CSFToELL3D.sizes first on this thread", fn);
+  return forward(stir_csf_to_ell3d_device_fill((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
+                                               groups.data(), OP.data(), R.data(), C.data(), M.data(), g_stream));
 }
 
 int stir_packed_csf_to_ell3d_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {

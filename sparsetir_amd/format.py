@@ -219,7 +219,14 @@ def csf_to_ell3d(csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1, nnz_r
 
     Returns ``(indptr, row_indices, col_indices, mask)``, each a list over buckets, shaped
     ``(R+1,)``, ``(G, rb)``, ``(G, rb, cb)``, ``(G, rb, cb)``.
+
+    Extension: CUDA tensors are converted on the GPU and CUDA tensors come back (the reference
+    accepts CPU arrays only, src/sparse/format.cc:195-202); the row ids of every relation must
+    then ascend strictly.
     """
+    if any(_is_cuda_tensor(a) for a in (csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1)):
+        return _csf_to_ell3d_device(csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1,
+                                    nnz_rows_bkt, nnz_cols_bkt)
     L = _lib.lib()
     p0 = _host_i32(csf_indptr_0, "csf_indptr_0")
     i0 = _host_i32(csf_indices_0, "csf_indices_0")
@@ -244,4 +251,49 @@ def csf_to_ell3d(csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1, nnz_r
         _lib.ptr_table([a.ctypes.data for a in rows]),
         _lib.ptr_table([a.ctypes.data for a in cols]),
         _lib.ptr_table([a.ctypes.data for a in mask])))
+    return out_ptr, rows, cols, mask
+
+
+def _csf_to_ell3d_device(p0, i0, p1, i1, nnz_rows_bkt, nnz_cols_bkt):
+    import torch
+
+    L = _lib.lib()
+    names = ("csf_indptr_0", "csf_indices_0", "csf_indptr_1", "csf_indices_1")
+    for t, name in zip((p0, i0, p1, i1), names):
+        if not _is_cuda_tensor(t):
+            raise _lib.SparseTIRError("CSFToELL3D(device): the four CSF arrays must all be CUDA tensors")
+        if t.dtype != torch.int32:
+            raise _lib.SparseTIRError(
+                f"Only support int32 index data type, got {t.element_size() * 8} bits for {name}.")
+    p0, i0, p1, i1 = (t.contiguous().reshape(-1) for t in (p0, i0, p1, i1))
+    rb = np.ascontiguousarray(np.asarray(list(nnz_rows_bkt), dtype=np.int32))
+    cb = np.ascontiguousarray(np.asarray(list(nnz_cols_bkt), dtype=np.int32))
+    if len(rb) != len(cb):
+        raise _lib.SparseTIRError("Input nnz_rows and nnz_cols should have same length.")
+    nb = len(cb)
+    num_rels = p0.numel() - 1
+    stored, nnz = i0.numel(), i1.numel()
+    if num_rels < 0 or p1.numel() != stored + 1:
+        raise _lib.SparseTIRError("CSFToELL3D: csf_indptr_1 must have one entry more than csf_indices_0")
+    dev = p0.device
+    dp = lambda t: ctypes.c_void_p(t.data_ptr())
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        ws_bytes = L.stir_csf_to_ell3d_device_workspace_bytes(num_rels, stored, max(nb, 1))
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+        groups = np.zeros(max(nb, 1), np.int64)
+        _lib.check(L.stir_csf_to_ell3d_device_sizes(num_rels, stored, nnz, dp(p0), dp(i0), dp(p1), dp(i1),
+                                                    _vp(rb), _vp(cb), nb, dp(ws), _vp(groups), stream))
+        out_ptr = [torch.empty(num_rels + 1, dtype=torch.int32, device=dev) for _ in range(nb)]
+        rows = [torch.empty((int(groups[b]), int(rb[b])), dtype=torch.int32, device=dev) for b in range(nb)]
+        cols = [torch.empty((int(groups[b]), int(rb[b]), int(cb[b])), dtype=torch.int32, device=dev)
+                for b in range(nb)]
+        mask = [torch.empty((int(groups[b]), int(rb[b]), int(cb[b])), dtype=torch.int32, device=dev)
+                for b in range(nb)]
+        table = lambda xs: _lib.ptr_table([a.data_ptr() if a.numel() else 0 for a in xs])
+        _lib.check(L.stir_csf_to_ell3d_device_fill(num_rels, stored, nnz, dp(p0), dp(i0), dp(p1), dp(i1),
+                                                   _vp(rb), _vp(cb), nb, dp(ws), _vp(groups), table(out_ptr),
+                                                   table(rows), table(cols), table(mask), stream))
+        # the workspace is read by the fill kernels: keep it alive until they are done
+        torch.cuda.current_stream().synchronize()
     return out_ptr, rows, cols, mask

@@ -1,4 +1,5 @@
-"""Device-side ColumnPartHyb: index arrays bit-exact with the oracle."""
+"""Device-side format passes (ColumnPartHyb, CSFToELL3D, CSR to BSR): index arrays bit-exact with
+the oracle."""
 import numpy as np
 import pytest
 import torch
@@ -7,7 +8,7 @@ import oracle
 import sparsetir_amd as st
 from sparsetir_amd import datasets
 from sparsetir_amd._lib import SparseTIRError
-from helpers import coo_pairs, decode_hyb, random_csr
+from helpers import coo_pairs, decode_hyb, random_csf, random_csr
 
 pytestmark = pytest.mark.gpu
 
@@ -281,3 +282,88 @@ def test_on_disk_cache_of_a_device_decomposition_feeds_the_hyb_operator(dev, tmp
     host = cached_column_part_hyb(str(tmp_path), m, n, indptr, indices, parts, buckets)
     assert len(list(tmp_path.iterdir())) == 1
     assert isinstance(host[0][0][0], np.ndarray) and np.array_equal(host[1][1][2], want[1][1][2])
+
+
+# ------------------------------------------------------------------------------- CSFToELL3D
+
+def _device_ell3d(dev, csf, rows_bkt, cols_bkt):
+    got = st.csf_to_ell3d(*[torch.from_numpy(a).to(dev) for a in csf], rows_bkt, cols_bkt)
+    assert all(a.is_cuda for kind in got for a in kind)
+    return [[a.cpu().numpy() for a in kind] for kind in got]
+
+
+def _assert_same_ell3d(got, want):
+    for name, g, w in zip(["indptr", "rows", "cols", "mask"], got, want):
+        assert len(g) == len(w)
+        for b, (a, c) in enumerate(zip(g, w)):
+            assert a.shape == c.shape, (name, b, a.shape, c.shape)
+            assert np.array_equal(a, c), (name, b)
+
+
+@pytest.mark.parametrize("rels,n,edges,rows_bkt,cols_bkt,seed", [
+    (3, 30, 200, [4, 2, 1], [1, 2, 4], 0),
+    (65, 2000, 40000, [256, 128, 64, 32, 16], [1, 2, 4, 8, 16], 1),
+    (7, 100, 3000, [32, 16, 8, 4, 2], [1, 2, 4, 8, 16], 2),   # rows longer than the widest bucket
+    (4, 20, 100, [3, 5], [2, 3], 3),                          # widths that are not powers of two
+    (2, 10, 0, [2, 1], [1, 2], 4),                            # no edges
+    (0, 10, 0, [2, 1], [1, 2], 5),                            # no relations
+    (300, 5000, 100000, [64, 8, 1], [1, 8, 64], 6),           # more relations than a workgroup scans at once
+    (5, 40000, 300000, [128], [3], 7),                        # one bucket, every row split or padded
+    (1, 3, 9, [7, 7], [1, 2], 8),
+])
+def test_device_csf_to_ell3d_bit_exact(dev, rels, n, edges, rows_bkt, cols_bkt, seed):
+    csf = random_csf(rels, n, edges, seed)
+    got = _device_ell3d(dev, csf, rows_bkt, cols_bkt)
+    _assert_same_ell3d(got, oracle.csf_to_ell3d(*csf, rows_bkt, cols_bkt))
+
+
+def test_device_csf_to_ell3d_empty_relations_and_hub_rows(dev):
+    """Relations without rows at the start, in the middle and at the end, a stored row with
+    thousands of columns (one thread of the row pass, many of the entry pass) and stored rows
+    without columns."""
+    rng = np.random.default_rng(3)
+    n = 6000
+    indptr0, indices0, indptr1, indices1 = [0], [], [0], []
+    for r in range(9):
+        rows = [] if r in (0, 4, 8) else sorted(rng.choice(n, size=int(rng.integers(1, 40)), replace=False).tolist())
+        for q, row in enumerate(rows):
+            cnt = 5000 if (r == 2 and q == 0) else (0 if q % 7 == 3 else int(rng.integers(1, 30)))
+            indices1 += sorted(rng.choice(n, size=cnt, replace=False).tolist())
+            indptr1.append(len(indices1))
+        indices0 += rows
+        indptr0.append(len(indices0))
+    csf = tuple(np.asarray(a, np.int32) for a in (indptr0, indices0, indptr1, indices1))
+    for rows_bkt, cols_bkt in (([16, 8, 4], [1, 4, 16]), ([5], [7]), ([1, 1, 1, 1], [1, 2, 3, 4])):
+        got = _device_ell3d(dev, csf, rows_bkt, cols_bkt)
+        _assert_same_ell3d(got, oracle.csf_to_ell3d(*csf, rows_bkt, cols_bkt))
+
+
+def test_device_csf_to_ell3d_config5(dev):
+    cfg = datasets.config5()
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    rows_bkt = [256 // b for b in cfg["buckets"]]
+    got = _device_ell3d(dev, csf, rows_bkt, cfg["buckets"])
+    _assert_same_ell3d(got, oracle.csf_to_ell3d(*csf, rows_bkt, cfg["buckets"]))
+
+
+def test_device_csf_to_ell3d_errors(dev):
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    good = (i32([0, 2]), i32([1, 4]), i32([0, 1, 3]), i32([0, 2, 3]))
+    st.csf_to_ell3d(*good, [1, 1], [1, 2])
+    with pytest.raises(SparseTIRError, match="ascending"):
+        st.csf_to_ell3d(*good, [1, 1], [2, 2])
+    with pytest.raises(SparseTIRError, match="same length"):
+        st.csf_to_ell3d(*good, [1], [1, 2])
+    with pytest.raises(SparseTIRError, match="int32"):
+        st.csf_to_ell3d(good[0].long(), *good[1:], [1], [1])
+    with pytest.raises(SparseTIRError, match="CUDA"):
+        st.csf_to_ell3d(good[0].cpu(), *good[1:], [1], [1])
+    # the same row id twice in a relation: the sequential rule would let the two share an ELL row
+    with pytest.raises(SparseTIRError, match="ascend strictly"):
+        st.csf_to_ell3d(i32([0, 2]), i32([4, 4]), good[2], good[3], [1, 1], [1, 2])
+    with pytest.raises(SparseTIRError, match="indptr1 decreases"):
+        st.csf_to_ell3d(good[0], good[1], i32([0, 4, 3]), good[3], [1, 1], [1, 2])
+    with pytest.raises(SparseTIRError, match="do not fit"):
+        st.csf_to_ell3d(i32([0, 1]), good[1], good[2], good[3], [1, 1], [1, 2])
+    with pytest.raises(SparseTIRError, match="indptr0 decreases"):
+        st.csf_to_ell3d(i32([0, 3, 2]), good[1], good[2], good[3], [1, 1], [1, 2])

@@ -38,6 +38,29 @@ def test_packed_csrmm_and_sddmm(dev):
     assert np.allclose(out.cpu().numpy(), sddmm_f64(indptr, indices, a2, x), rtol=1e-4, atol=1e-4)
 
 
+def test_packed_device_csf_to_ell3d(dev):
+    """tir.sparse.CSFToELL3D.sizes / .fill with the CSF arrays on the GPU: device outputs equal
+    to the oracle's arrays."""
+    csf = random_csf(9, 300, 6000, 4)
+    d_csf = [torch.from_numpy(a).to(dev) for a in csf]
+    rb, cb = np.asarray([8, 4, 2, 1], np.int32), np.asarray([1, 2, 4, 8], np.int32)
+    groups = np.zeros(4, np.int64)
+    packed.get_global_func("tir.sparse.CSFToELL3D.sizes")(*d_csf, rb, cb, groups)
+    outs = []
+    for b in range(4):
+        g = int(groups[b])
+        outs += [torch.empty(10, dtype=torch.int32, device=dev),
+                 torch.empty(g * int(rb[b]), dtype=torch.int32, device=dev),
+                 torch.empty(g * int(rb[b]) * int(cb[b]), dtype=torch.int32, device=dev),
+                 torch.empty(g * int(rb[b]) * int(cb[b]), dtype=torch.int32, device=dev)]
+    packed.get_global_func("tir.sparse.CSFToELL3D.fill")(*d_csf, rb, cb, *outs)
+    torch.cuda.synchronize()
+    want = oracle.csf_to_ell3d(*csf, rb, cb)
+    for b in range(4):
+        for q in range(4):
+            assert np.array_equal(outs[4 * b + q].cpu().numpy(), want[q][b].ravel()), (b, q)
+
+
 def test_packed_device_column_part_hyb_and_hyb_csrmm(dev):
     m = n = 900
     feat, parts, buckets = 128, 2, [1, 2, 4, 8, 16]
