@@ -298,6 +298,20 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     fmt_s = time.perf_counter() - t0
     out["condense_config2_host"] = {"ms": fmt_s * 1e3, "edges": int(len(g2["indices"])), "groups": int(tiles.shape[0]),
                                     "threads": 1}
+    # the same pass on the GPU (CSR arrays resident): per call, allocations and the sizing round trip included
+    d_ptr2, d_idx2 = t(g2["indptr"]), t(g2["indices"])
+    dev_out = st.condense(d_ptr2, d_idx2, 32, 16)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        dev_out = st.condense(d_ptr2, d_idx2, 32, 16)
+    torch.cuda.synchronize()
+    dev_s = (time.perf_counter() - t0) / 5
+    out["condense_config2_device"] = {
+        "ms": dev_s * 1e3,
+        "equals_host_arrays": all(bool((a.cpu() == torch.from_numpy(b)).all())
+                                  for a, b in zip(dev_out, (gptr, tiles, cmask)))}
+    del dev_out, d_ptr2, d_idx2
     mb2, nnzb2, f2 = len(gptr) - 1, tiles.shape[0], 128
     tc = ops.build_tcspmm(mb2, nnzb2, f2, 32, 16, g2["n"], torch.float32)
     a2, b2 = t(cmask.astype(np.float16).ravel()), torch.randn(g2["n"] * f2, device=dev).half()

@@ -147,6 +147,24 @@ int stir_csf_to_ell3d_device_fill(int32_t num_rels, int64_t num_stored_rows, int
                                   void* stream);
 
 /*
+ * ConDense on the GPU, bit-exact with stir_condense_sizes / _fill above (the reference runs this
+ * on the CPU only, src/sparse/format.cc:360-361).  nnz is the length of indices; column indices
+ * must not be negative.  d_workspace must hold stir_condense_device_workspace_bytes(n, nnz, t)
+ * bytes (32 bytes per nonzero plus sort scratch) and stay untouched between _sizes and _fill.
+ * _sizes writes d_group_indptr (ceil(n/t) + 1 entries, a device array), synchronises the stream
+ * and returns the number of groups on the host; _fill writes d_tile_indices (num_groups * g) and
+ * d_mask (num_groups * t * g).
+ */
+size_t stir_condense_device_workspace_bytes(int32_t n, int64_t nnz, int32_t t);
+int stir_condense_device_sizes(int32_t n, int64_t nnz, const int32_t* d_indptr,
+                               const int32_t* d_indices, int32_t t, int32_t g, void* d_workspace,
+                               int32_t* d_group_indptr, int64_t* num_groups, void* stream);
+int stir_condense_device_fill(int32_t n, int64_t nnz, const int32_t* d_indptr,
+                              const int32_t* d_indices, int32_t t, int32_t g, void* d_workspace,
+                              const int32_t* d_group_indptr, int64_t num_groups,
+                              int32_t* d_tile_indices, int32_t* d_mask, void* stream);
+
+/*
  * CSR -> BSR packing on the GPU (blk x blk blocks; m and n multiples of blk): the canonical BSR
  * arrays that scipy's csr_matrix.tobsr hands the reference's example
  * (examples/blocksparse/bsr_spmm.py:441-445) -- block columns ascending in each block row,

@@ -137,6 +137,9 @@ enum {
  *      tensors (row ids must ascend strictly inside a relation; .sizes first, on the same thread).
  * "tir.sparse.ConDense.sizes"      (indptr, indices, t, g, group_indptr_out, num_groups_out)
  * "tir.sparse.ConDense.fill"       (indptr, indices, t, g, tile_indices_out, mask_out)  src/sparse/format.cc:353-429
+ *      With kDLROCM/kDLCUDA indptr and indices the condensing runs on the GPU: group_indptr_out and
+ *      the outputs of .fill are device tensors, and .fill takes the filled group_indptr as a seventh
+ *      argument (.sizes first, on the same thread).
  */
 int stir_packed_csrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_hyb_csrmm(TVMValue*, int*, int, TVMRetValueHandle, void*);

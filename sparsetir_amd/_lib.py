@@ -32,6 +32,9 @@ SIGNATURES = {
     "stir_csf_to_ell3d_device_workspace_bytes": (SZ, [I32, I64, I32]),
     "stir_csf_to_ell3d_device_sizes": (I32, [I32, I64, I64, VP, VP, VP, VP, VP, VP, I32, VP, VP, VP]),
     "stir_csf_to_ell3d_device_fill": (I32, [I32, I64, I64, VP, VP, VP, VP, VP, VP, I32, VP, VP, VP, VP, VP, VP, VP]),
+    "stir_condense_device_workspace_bytes": (SZ, [I32, I64, I32]),
+    "stir_condense_device_sizes": (I32, [I32, I64, VP, VP, I32, I32, VP, VP, VP, VP]),
+    "stir_condense_device_fill": (I32, [I32, I64, VP, VP, I32, I32, VP, VP, I64, VP, VP, VP]),
     "stir_csr_to_bsr_workspace_bytes": (SZ, [I32, I32, I32]),
     "stir_csr_to_bsr_sizes": (I32, [I32, I32, I32, VP, VP, VP, VP, VP, VP]),
     "stir_csr_to_bsr_fill": (I32, [I32, I32, I32, VP, VP, VP, VP, VP, VP, VP, I32, I64, VP]),

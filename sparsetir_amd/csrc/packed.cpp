@@ -691,34 +691,70 @@ int stir_packed_csf_to_ell3d_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle
   return csf_format("tir.sparse.CSFToELL3D.fill", true, v, tc, n);
 }
 
+// the device path keeps its scratch between the sizing and the fill call
+static thread_local void* g_condense_ws = nullptr;
+static thread_local size_t g_condense_ws_bytes = 0;
+
 int stir_packed_condense_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   Args a{"tir.sparse.ConDense.sizes", v, tc, n};
   if (!a.count(6)) return -1;
-  Arr P = a.arr(0, "indptr", kDLInt, 32, kHost), I = a.arr(1, "indices", kDLInt, 32, kHost);
+  // CSR arrays on the GPU take the device pass; group_indptr_out is then a device tensor too
+  const bool dev = a.on_device(0);
+  const Where w = dev ? kDevice : kHost;
+  Arr P = a.arr(0, "indptr", kDLInt, 32, w), I = a.arr(1, "indices", kDLInt, 32, w);
   const int64_t t = a.integer(2, "t"), g = a.integer(3, "g");
-  Arr GP = a.arr(4, "group_indptr_out", kDLInt, 32, kHost), NG = a.arr(5, "num_groups_out", kDLInt, 64, kHost);
+  Arr GP = a.arr(4, "group_indptr_out", kDLInt, 32, w), NG = a.arr(5, "num_groups_out", kDLInt, 64, kHost);
   if (!a.ok) return -1;
   const int64_t rows = P.len - 1;
   if (rows < 0 || t <= 0 || g <= 0 || !fits_i32(t) || !fits_i32(g)) return packed_fail("%s: bad sizes", a.fn);
   a.len(GP, "group_indptr_out", (rows + t - 1) / t + 1);
   a.len(NG, "num_groups_out", 1);
   if (!a.ok) return -1;
-  return forward(stir_condense_sizes((int32_t)rows, (const int32_t*)P.data, (const int32_t*)I.data, (int32_t)t,
-                                     (int32_t)g, (int32_t*)GP.data, (int64_t*)NG.data));
+  if (!dev)
+    return forward(stir_condense_sizes((int32_t)rows, (const int32_t*)P.data, (const int32_t*)I.data, (int32_t)t,
+                                       (int32_t)g, (int32_t*)GP.data, (int64_t*)NG.data));
+  DeviceGuard guard;
+  if (guard.enter(a.dev_id)) return forward(-1);
+  const size_t need = stir_condense_device_workspace_bytes((int32_t)rows, I.len, (int32_t)t);
+  if (need > g_condense_ws_bytes) {
+    if (g_condense_ws) (void)hipFree(g_condense_ws);
+    g_condense_ws = nullptr;
+    g_condense_ws_bytes = 0;
+    if (hipMalloc(&g_condense_ws, need) != hipSuccess)
+      return packed_fail("%s: cannot allocate %zu bytes of scratch", a.fn, need);
+    g_condense_ws_bytes = need;
+  }
+  return forward(stir_condense_device_sizes((int32_t)rows, I.len, (const int32_t*)P.data, (const int32_t*)I.data,
+                                            (int32_t)t, (int32_t)g, g_condense_ws, (int32_t*)GP.data,
+                                            (int64_t*)NG.data, g_stream));
 }
 
+// Device form: (indptr, indices, t, g, tile_indices_out, mask_out, group_indptr) -- the seventh
+// argument is the array the sizing call filled.
 int stir_packed_condense_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   Args a{"tir.sparse.ConDense.fill", v, tc, n};
-  if (!a.count(6)) return -1;
-  Arr P = a.arr(0, "indptr", kDLInt, 32, kHost), I = a.arr(1, "indices", kDLInt, 32, kHost);
+  if (n < 6) return packed_fail("%s: num_args should be at least 6", a.fn);
+  const bool dev = a.on_device(0);
+  if (!a.count(dev ? 7 : 6)) return -1;
+  const Where w = dev ? kDevice : kHost;
+  Arr P = a.arr(0, "indptr", kDLInt, 32, w), I = a.arr(1, "indices", kDLInt, 32, w);
   const int64_t t = a.integer(2, "t"), g = a.integer(3, "g");
-  Arr TI = a.arr(4, "tile_indices_out", kDLInt, 32, kHost), MK = a.arr(5, "mask_out", kDLInt, 32, kHost);
+  Arr TI = a.arr(4, "tile_indices_out", kDLInt, 32, w), MK = a.arr(5, "mask_out", kDLInt, 32, w);
   if (!a.ok) return -1;
   const int64_t rows = P.len - 1;
   if (rows < 0 || t <= 0 || g <= 0 || !fits_i32(t) || !fits_i32(g)) return packed_fail("%s: bad sizes", a.fn);
   if (TI.len % g != 0 || MK.len != TI.len * t) return packed_fail("%s: output lengths do not fit t and g", a.fn);
-  return forward(stir_condense_fill((int32_t)rows, (const int32_t*)P.data, (const int32_t*)I.data, (int32_t)t,
-                                    (int32_t)g, (int32_t*)TI.data, (int32_t*)MK.data));
+  if (!dev)
+    return forward(stir_condense_fill((int32_t)rows, (const int32_t*)P.data, (const int32_t*)I.data, (int32_t)t,
+                                      (int32_t)g, (int32_t*)TI.data, (int32_t*)MK.data));
+  Arr GP = a.arr(6, "group_indptr", kDLInt, 32, kDevice);
+  if (!a.ok || !a.len(GP, "group_indptr", (rows + t - 1) / t + 1)) return -1;
+  if (!g_condense_ws) return packed_fail("%s: call tir.sparse.ConDense.sizes first on this thread", a.fn);
+  DeviceGuard guard;
+  if (guard.enter(a.dev_id)) return forward(-1);
+  return forward(stir_condense_device_fill((int32_t)rows, I.len, (const int32_t*)P.data, (const int32_t*)I.data,
+                                           (int32_t)t, (int32_t)g, g_condense_ws, (const int32_t*)GP.data,
+                                           TI.len / g, (int32_t*)TI.data, (int32_t*)MK.data, g_stream));
 }
 
 // ------------------------------------------------------------------------------ registry

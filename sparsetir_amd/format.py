@@ -194,7 +194,12 @@ def condense(indptr_nd, indices_nd, t, g):
 
     Returns ``(group_indptr, tile_indices, mask)`` shaped ``(ceil(n/t)+1,)``, ``(G, g)``,
     ``(G, t, g)``.
+
+    Extension: CUDA tensors are condensed on the GPU and CUDA tensors come back (the reference
+    accepts CPU arrays only, src/sparse/format.cc:360-361).
     """
+    if _is_cuda_tensor(indptr_nd) or _is_cuda_tensor(indices_nd):
+        return _condense_device(indptr_nd, indices_nd, t, g)
     L = _lib.lib()
     indptr = _host_i32(indptr_nd, "indptr")
     indices = _host_i32(indices_nd, "indices")
@@ -297,3 +302,39 @@ def _csf_to_ell3d_device(p0, i0, p1, i1, nnz_rows_bkt, nnz_cols_bkt):
         # the workspace is read by the fill kernels: keep it alive until they are done
         torch.cuda.current_stream().synchronize()
     return out_ptr, rows, cols, mask
+
+
+def _condense_device(indptr, indices, t, g):
+    import torch
+
+    L = _lib.lib()
+    for a, name in ((indptr, "indptr"), (indices, "indices")):
+        if not _is_cuda_tensor(a):
+            raise _lib.SparseTIRError("ConDense(device): indptr and indices must both be CUDA tensors")
+        if a.dtype != torch.int32:
+            raise _lib.SparseTIRError(
+                f"Only support int32 index data type, got {a.element_size() * 8} bits for {name}.")
+    t, g = int(t), int(g)
+    if t <= 0 or g <= 0:
+        raise _lib.SparseTIRError(f"ConDense: t={t} g={g} must be positive")
+    indptr, indices = indptr.contiguous().reshape(-1), indices.contiguous().reshape(-1)
+    n, nnz = indptr.numel() - 1, indices.numel()
+    if n < 0:
+        raise _lib.SparseTIRError("ConDense: indptr must have at least one entry")
+    dev = indptr.device
+    dp = lambda a: ctypes.c_void_p(a.data_ptr() if a.numel() else 0)
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        ws = torch.empty(max(L.stir_condense_device_workspace_bytes(n, nnz, t), 256), dtype=torch.uint8, device=dev)
+        gptr = torch.empty((n + t - 1) // t + 1, dtype=torch.int32, device=dev)
+        ng = ctypes.c_int64(0)
+        _lib.check(L.stir_condense_device_sizes(n, nnz, dp(indptr), dp(indices), t, g, dp(ws), dp(gptr),
+                                                ctypes.byref(ng), stream))
+        G = ng.value
+        tile_indices = torch.empty((G, g), dtype=torch.int32, device=dev)
+        mask = torch.empty((G, t, g), dtype=torch.int32, device=dev)
+        _lib.check(L.stir_condense_device_fill(n, nnz, dp(indptr), dp(indices), t, g, dp(ws), dp(gptr), G,
+                                               dp(tile_indices), dp(mask), stream))
+        # the workspace is read by the fill kernels: keep it alive until they are done
+        torch.cuda.current_stream().synchronize()
+    return gptr, tile_indices, mask

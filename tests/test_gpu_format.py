@@ -367,3 +367,44 @@ def test_device_csf_to_ell3d_errors(dev):
         st.csf_to_ell3d(i32([0, 1]), good[1], good[2], good[3], [1, 1], [1, 2])
     with pytest.raises(SparseTIRError, match="indptr0 decreases"):
         st.csf_to_ell3d(i32([0, 3, 2]), good[1], good[2], good[3], [1, 1], [1, 2])
+
+
+# ------------------------------------------------------------------------------- ConDense
+
+@pytest.mark.parametrize("m,n,nnz,t,g,seed,skew", [
+    (130, 90, 2000, 8, 4, 0, 0.0),
+    (1000, 1000, 30000, 32, 16, 1, 1.2),     # the setting of the tensor-core SpMM
+    (77, 5000, 9000, 1, 1, 2, 1.0),          # tiles of one row, groups of one column
+    (513, 40, 12000, 64, 3, 3, 0.0),         # nearly every column in every tile
+    (100, 100, 0, 4, 4, 4, 0.0),             # no nonzeros
+    (5, 7, 20, 32, 16, 5, 0.0),              # one partial tile
+    (20000, 3000, 200000, 32, 16, 6, 1.5),   # a tile with thousands of distinct columns
+])
+def test_device_condense_bit_exact(dev, m, n, nnz, t, g, seed, skew):
+    indptr, indices = random_csr(m, n, nnz, seed, skew=skew, sort=seed % 2 == 0)
+    got = st.condense(torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev), t, g)
+    assert all(a.is_cuda for a in got)
+    want = oracle.condense(indptr, indices, t, g)
+    for name, a, b in zip(["group_indptr", "tile_indices", "mask"], got, want):
+        a = a.cpu().numpy()
+        assert a.shape == b.shape, (name, a.shape, b.shape)
+        assert np.array_equal(a, b), name
+
+
+def test_device_condense_config2_graph_and_errors(dev):
+    g2 = datasets.config2()
+    got = st.condense(torch.from_numpy(g2["indptr"]).to(dev), torch.from_numpy(g2["indices"]).to(dev), 32, 16)
+    want = oracle.condense(g2["indptr"], g2["indices"], 32, 16)
+    for a, b in zip(got, want):
+        assert np.array_equal(a.cpu().numpy(), b)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    with pytest.raises(SparseTIRError, match="positive"):
+        st.condense(i32([0, 1]), i32([0]), 0, 4)
+    with pytest.raises(SparseTIRError, match="int32"):
+        st.condense(i32([0, 1]).long(), i32([0]), 4, 4)
+    with pytest.raises(SparseTIRError, match="indptr decreases"):
+        st.condense(i32([0, 2, 1, 3]), i32([0, 1, 2]), 4, 4)
+    with pytest.raises(SparseTIRError, match="from 0 to the number of nonzeros"):
+        st.condense(i32([0, 1, 2]), i32([0, 1, 2]), 4, 4)
+    with pytest.raises(SparseTIRError, match="negative"):
+        st.condense(i32([0, 1, 2]), i32([3, -1]), 4, 4)

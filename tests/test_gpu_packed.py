@@ -61,6 +61,23 @@ def test_packed_device_csf_to_ell3d(dev):
             assert np.array_equal(outs[4 * b + q].cpu().numpy(), want[q][b].ravel()), (b, q)
 
 
+def test_packed_device_condense(dev):
+    """tir.sparse.ConDense.sizes / .fill with the CSR arrays on the GPU."""
+    indptr, indices = random_csr(700, 400, 9000, 5, skew=1.1)
+    d_ptr, d_idx = torch.from_numpy(indptr).to(dev), torch.from_numpy(indices).to(dev)
+    t, g = 32, 16
+    gptr = torch.empty((700 + t - 1) // t + 1, dtype=torch.int32, device=dev)
+    ng = np.zeros(1, np.int64)
+    packed.get_global_func("tir.sparse.ConDense.sizes")(d_ptr, d_idx, t, g, gptr, ng)
+    tiles = torch.empty(int(ng[0]) * g, dtype=torch.int32, device=dev)
+    mask = torch.empty(int(ng[0]) * t * g, dtype=torch.int32, device=dev)
+    packed.get_global_func("tir.sparse.ConDense.fill")(d_ptr, d_idx, t, g, tiles, mask, gptr)
+    torch.cuda.synchronize()
+    want = oracle.condense(indptr, indices, t, g)
+    for a, b in zip((gptr, tiles, mask), want):
+        assert np.array_equal(a.cpu().numpy(), b.ravel())
+
+
 def test_packed_device_column_part_hyb_and_hyb_csrmm(dev):
     m = n = 900
     feat, parts, buckets = 128, 2, [1, 2, 4, 8, 16]
