@@ -122,8 +122,9 @@ enum {
  *      leave the zero-weight padding slots out of their edge index.  Drops the cached plan when the
  *      setting changes.  Default off.
  *
- * Format pass (host tensors, kDLCPU; the reference returns nested Array<NDArray>, which needs
- * libtvm objects, so here a sizing call is followed by a fill call into caller-made tensors):
+ * Format pass (host tensors, kDLCPU, as in the reference, or device tensors; the reference returns
+ * nested Array<NDArray>, which needs libtvm objects, so here a sizing call is followed by a fill
+ * call into caller-made tensors):
  *
  * "tir.sparse.ColumnPartHyb.sizes" (num_rows, num_cols, indptr, indices, num_col_parts, buckets, nrows_out)
  * "tir.sparse.ColumnPartHyb.fill"  (num_rows, num_cols, indptr, indices, num_col_parts, buckets,
