@@ -6,9 +6,9 @@ rebuild theirs on every run).  This keeps the results across processes: the inde
 decomposition are stored as one ``.npz`` per (input arrays, parameters), keyed by a hash of both.
 
 All three routines are covered -- ``column_part_hyb``, ``csf_to_ell3d`` and ``condense`` -- with the
-return nesting of :mod:`sparsetir_amd.format`.  ``cached_column_part_hyb`` also takes CUDA tensors:
-the decomposition then runs on the GPU, host copies go to disk, and a later hit is uploaded to the
-device the inputs live on, so the result can be handed to the hyb operator either way.
+return nesting of :mod:`sparsetir_amd.format`.  All three also take CUDA tensors: the routine then
+runs on the GPU, host copies go to disk, and a later hit is uploaded to the device the inputs live
+on, so the result can be handed to the operators either way.
 
 A file is written under a temporary name and renamed, so a reader never sees half a file; a file
 that cannot be read (truncated, foreign) is ignored and rewritten.
@@ -94,30 +94,60 @@ def cached_column_part_hyb(cache_dir, num_rows, num_cols, indptr, indices, num_c
     return get("rows"), get("cols"), get("mask")
 
 
+def _device_of(arrays):
+    for a in arrays:
+        if _is_cuda(a):
+            return a.device
+    return None
+
+
+def _uploader(dev):
+    """Identity for host callers; for CUDA callers a function that puts a cached array on `dev`."""
+    if dev is None:
+        return lambda a: a
+    import torch
+
+    return lambda a: torch.from_numpy(a).to(dev)
+
+
+def _on_host(a):
+    return a.cpu().numpy() if hasattr(a, "detach") else a
+
+
 def cached_csf_to_ell3d(cache_dir, csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1, nnz_rows_bkt,
                         nnz_cols_bkt):
     """``csf_to_ell3d`` memoised under ``cache_dir``: ``(indptr, row_indices, col_indices, mask)``,
-    each a list over buckets of int32 numpy arrays."""
-    csf = [_host(a) for a in (csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1)]
+    each a list over buckets of int32 numpy arrays -- or, when the CSF arrays are CUDA tensors, of
+    CUDA tensors on their device (converted on the GPU on a miss; host copies go to disk)."""
+    given = (csf_indptr_0, csf_indices_0, csf_indptr_1, csf_indices_1)
+    dev = _device_of(given)
+    csf = [_host(a) for a in given]
     rb, cb = [int(v) for v in nnz_rows_bkt], [int(v) for v in nnz_cols_bkt]
     nb = len(cb)
     path = os.path.join(cache_dir, _key(csf, ("csf_to_ell3d", tuple(rb), tuple(cb))) + ".npz")
     kinds = ("indptr", "rows", "cols", "mask")
     z = _load(path, [f"{kind}_{b}" for kind in kinds for b in range(nb)])
     if z is None:
-        out = _format.csf_to_ell3d(*csf, rb, cb)
-        _store(cache_dir, path, {f"{kind}_{b}": out[q][b] for q, kind in enumerate(kinds) for b in range(nb)})
+        out = _format.csf_to_ell3d(*(given if dev is not None else csf), rb, cb)
+        _store(cache_dir, path, {f"{kind}_{b}": _on_host(out[q][b]) for q, kind in enumerate(kinds) for b in range(nb)})
         return out
-    return tuple([z[f"{kind}_{b}"] for b in range(nb)] for kind in kinds)
+    put = _uploader(dev)
+    return tuple([put(z[f"{kind}_{b}"]) for b in range(nb)] for kind in kinds)
 
 
 def cached_condense(cache_dir, indptr, indices, t, g):
-    """``condense`` memoised under ``cache_dir``: ``(group_indptr, tile_indices, mask)``."""
+    """``condense`` memoised under ``cache_dir``: ``(group_indptr, tile_indices, mask)``, numpy arrays
+    for host inputs and CUDA tensors for CUDA inputs (condensed on the GPU on a miss)."""
+    dev = _device_of((indptr, indices))
     h_ptr, h_idx = _host(indptr), _host(indices)
     path = os.path.join(cache_dir, _key((h_ptr, h_idx), ("condense", int(t), int(g))) + ".npz")
     z = _load(path, ["group_indptr", "tile_indices", "mask"])
     if z is None:
-        gptr, tiles, mask = _format.condense(h_ptr, h_idx, t, g)
-        _store(cache_dir, path, {"group_indptr": gptr, "tile_indices": tiles, "mask": mask})
+        if dev is not None:
+            gptr, tiles, mask = _format.condense(indptr, indices, t, g)
+        else:
+            gptr, tiles, mask = _format.condense(h_ptr, h_idx, t, g)
+        _store(cache_dir, path, {"group_indptr": _on_host(gptr), "tile_indices": _on_host(tiles), "mask": _on_host(mask)})
         return gptr, tiles, mask
-    return z["group_indptr"], z["tile_indices"], z["mask"]
+    put = _uploader(dev)
+    return put(z["group_indptr"]), put(z["tile_indices"]), put(z["mask"])

@@ -408,3 +408,27 @@ def test_device_condense_config2_graph_and_errors(dev):
         st.condense(i32([0, 1, 2]), i32([0, 1, 2]), 4, 4)
     with pytest.raises(SparseTIRError, match="negative"):
         st.condense(i32([0, 1, 2]), i32([3, -1]), 4, 4)
+
+
+def test_on_disk_cache_of_device_ell3d_and_condensed_formats(dev, tmp_path):
+    """CUDA inputs: computed on the GPU on a miss, uploaded from disk on a hit, the same arrays
+    (the oracle's) both times, and one file per decomposition whoever asked first."""
+    from sparsetir_amd.cache import cached_condense, cached_csf_to_ell3d
+    t = lambda a: torch.from_numpy(a).to(dev)
+    csf = random_csf(6, 300, 5000, 2)
+    rb, cb = [8, 4, 2], [1, 2, 4]
+    want = oracle.csf_to_ell3d(*csf, rb, cb)
+    for turn in range(2):
+        got = cached_csf_to_ell3d(str(tmp_path), *[t(a) for a in csf], rb, cb)
+        assert all(a.is_cuda for kind in got for a in kind)
+        _assert_same_ell3d([[a.cpu().numpy() for a in kind] for kind in got], want)
+    host = cached_csf_to_ell3d(str(tmp_path), *csf, rb, cb)  # a host caller hits the file the GPU wrote
+    _assert_same_ell3d(host, want)
+    assert len(list(tmp_path.iterdir())) == 1
+    indptr, indices = random_csr(400, 300, 6000, 3, skew=1.0)
+    want = oracle.condense(indptr, indices, 32, 16)
+    for turn in range(2):
+        got = cached_condense(str(tmp_path), t(indptr), t(indices), 32, 16)
+        for a, b in zip(got, want):
+            assert a.is_cuda and np.array_equal(a.cpu().numpy(), b)
+    assert len(list(tmp_path.iterdir())) == 2
