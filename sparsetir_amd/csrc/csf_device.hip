@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void csf_pad_kernel(int rels, int64_t rows, co
   if (id >= (int64_t)B.nb * rels) return;
   const int b = (int)(id / rels), r = (int)(id % rels);
   const int32_t* pb = pre + (int64_t)b * (rows + 1);
-  const int64_t ell = pb[p0[r + 1]] - pb[p0[r]];
+  const int64_t ell = pb[clamp_row(p0[r + 1], rows)] - pb[clamp_row(p0[r], rows)];
   if (ell <= 0) return;
   const int32_t* gb = gptr + (int64_t)b * (rels + 1);
   const int64_t first = (int64_t)gb[r] * B.rb[b], end = (int64_t)gb[r + 1] * B.rb[b];
