@@ -1,5 +1,6 @@
 // TVM PackedFunc adapters: unpack TVMValue/DLTensor arguments, validate them the way the
 // reference's generated host stubs do, and call the plain C ABI.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <mutex>
@@ -546,6 +547,34 @@ int stir_packed_rgms_csf(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) 
 
 // ----------------------------------------------------------------------------- format pass
 
+// Scratch of a device format pass, kept per thread between its sizing and its fill call.  It
+// belongs to the device it was allocated on: a call for another device starts over.
+struct FormatScratch {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  int dev = -1;
+  // at least `need` bytes on device `dev_id` (which must be current), nullptr when that fails
+  void* reserve(int dev_id, size_t need) {
+    if (ptr && (dev != dev_id || need > bytes)) {
+      (void)hipFree(ptr);
+      ptr = nullptr;
+      bytes = 0;
+    }
+    if (!ptr) {
+      if (hipMalloc(&ptr, std::max<size_t>(need, 256)) != hipSuccess) {
+        ptr = nullptr;
+        return nullptr;
+      }
+      bytes = std::max<size_t>(need, 256);
+      dev = dev_id;
+    }
+    return ptr;
+  }
+  // what the sizing call left for device `dev_id`, or nullptr
+  void* get(int dev_id) const { return dev == dev_id ? ptr : nullptr; }
+};
+static thread_local FormatScratch g_hyb_scratch, g_csf_scratch, g_condense_scratch;
+
 static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
   Args a{fn, v, tc, n};
   if (n < 7) return packed_fail("%s: num_args should be at least 7", fn);
@@ -564,9 +593,6 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
   const int64_t nk = parts * nb;
   DeviceGuard g;
   if (dev && g.enter(a.dev_id)) return forward(-1);
-  // the device path keeps its scratch between the sizing and the fill call
-  static thread_local void* ws = nullptr;
-  static thread_local size_t ws_bytes = 0;
   if (!fill) {
     if (!a.count(7)) return -1;
     Arr N = a.arr(6, "nrows_out", kDLInt, 64, kHost);
@@ -576,13 +602,8 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
                                                 (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data,
                                                 nb, (int64_t*)N.data));
     const size_t need = stir_column_part_hyb_device_workspace_bytes((int32_t)num_rows, (int32_t)parts, nb, I.len);
-    if (need > ws_bytes) {
-      if (ws) (void)hipFree(ws);
-      ws = nullptr;
-      ws_bytes = 0;
-      if (hipMalloc(&ws, need) != hipSuccess) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
-      ws_bytes = need;
-    }
+    void* ws = g_hyb_scratch.reserve(a.dev_id, need);
+    if (!ws) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
     return forward(stir_column_part_hyb_device_sizes((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
                                                      (const int32_t*)I.data, (int32_t)parts,
                                                      (const int32_t*)Bk.data, nb, ws, (int64_t*)N.data, g_stream));
@@ -605,6 +626,7 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
     return forward(stir_column_part_hyb_fill((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
                                              (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data, nb,
                                              R.data(), C.data(), M.data()));
+  void* ws = g_hyb_scratch.get(a.dev_id);
   if (!ws) return packed_fail("%s: call tir.sparse.ColumnPartHyb.sizes first on this thread", fn);
   int rc = stir_column_part_hyb_device_fill((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
                                             (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data, nb,
@@ -639,22 +661,14 @@ static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
     return packed_fail("%s: csf_indptr_1 must have one entry more than csf_indices_0", fn);
   DeviceGuard g;
   if (dev && g.enter(a.dev_id)) return forward(-1);
-  // the device path keeps its scratch between the sizing and the fill call
-  static thread_local void* ws = nullptr;
-  static thread_local size_t ws_bytes = 0;
   if (!fill) {
     if (!a.count(7)) return -1;
     Arr G = a.arr(6, "groups_out", kDLInt, 64, kHost);
     if (!a.ok || !a.len(G, "groups_out", nb)) return -1;
     if (!dev) return forward(stir_csf_to_ell3d_sizes((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, (int64_t*)G.data));
     const size_t need = stir_csf_to_ell3d_device_workspace_bytes((int32_t)rels, I0.len, nb);
-    if (need > ws_bytes) {
-      if (ws) (void)hipFree(ws);
-      ws = nullptr;
-      ws_bytes = 0;
-      if (hipMalloc(&ws, need) != hipSuccess) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
-      ws_bytes = need;
-    }
+    void* ws = g_csf_scratch.reserve(a.dev_id, need);
+    if (!ws) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
     return forward(stir_csf_to_ell3d_device_sizes((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
                                                   (int64_t*)G.data, g_stream));
   }
@@ -679,6 +693,7 @@ static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
   if (!dev)
     return forward(stir_csf_to_ell3d_fill((int32_t)rels, p0, i0, p1, i1, rb, cb, nb, OP.data(), R.data(), C.data(),
                                           M.data()));
+  void* ws = g_csf_scratch.get(a.dev_id);
   if (!ws) return packed_fail("%s: call tir.sparse.CSFToELL3D.sizes first on this thread", fn);
   return forward(stir_csf_to_ell3d_device_fill((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
                                                groups.data(), OP.data(), R.data(), C.data(), M.data(), g_stream));
@@ -690,10 +705,6 @@ int stir_packed_csf_to_ell3d_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandl
 int stir_packed_csf_to_ell3d_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   return csf_format("tir.sparse.CSFToELL3D.fill", true, v, tc, n);
 }
-
-// the device path keeps its scratch between the sizing and the fill call
-static thread_local void* g_condense_ws = nullptr;
-static thread_local size_t g_condense_ws_bytes = 0;
 
 int stir_packed_condense_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
   Args a{"tir.sparse.ConDense.sizes", v, tc, n};
@@ -716,14 +727,8 @@ int stir_packed_condense_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, v
   DeviceGuard guard;
   if (guard.enter(a.dev_id)) return forward(-1);
   const size_t need = stir_condense_device_workspace_bytes((int32_t)rows, I.len, (int32_t)t);
-  if (need > g_condense_ws_bytes) {
-    if (g_condense_ws) (void)hipFree(g_condense_ws);
-    g_condense_ws = nullptr;
-    g_condense_ws_bytes = 0;
-    if (hipMalloc(&g_condense_ws, need) != hipSuccess)
-      return packed_fail("%s: cannot allocate %zu bytes of scratch", a.fn, need);
-    g_condense_ws_bytes = need;
-  }
+  void* g_condense_ws = g_condense_scratch.reserve(a.dev_id, need);
+  if (!g_condense_ws) return packed_fail("%s: cannot allocate %zu bytes of scratch", a.fn, need);
   return forward(stir_condense_device_sizes((int32_t)rows, I.len, (const int32_t*)P.data, (const int32_t*)I.data,
                                             (int32_t)t, (int32_t)g, g_condense_ws, (int32_t*)GP.data,
                                             (int64_t*)NG.data, g_stream));
@@ -749,6 +754,7 @@ int stir_packed_condense_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, vo
                                       (int32_t)g, (int32_t*)TI.data, (int32_t*)MK.data));
   Arr GP = a.arr(6, "group_indptr", kDLInt, 32, kDevice);
   if (!a.ok || !a.len(GP, "group_indptr", (rows + t - 1) / t + 1)) return -1;
+  void* g_condense_ws = g_condense_scratch.get(a.dev_id);
   if (!g_condense_ws) return packed_fail("%s: call tir.sparse.ConDense.sizes first on this thread", a.fn);
   DeviceGuard guard;
   if (guard.enter(a.dev_id)) return forward(-1);
