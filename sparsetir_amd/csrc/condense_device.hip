@@ -19,11 +19,11 @@ namespace {
 using stir::ceil_div;
 using stir::kWave;
 
-enum Flag { kBadEnds = 1, kBadIndptr = 2, kBadColumn = 4, kTooLarge = 8 };
+enum Flag { kBadEnds = 1, kBadIndptr = 2, kBadColumn = 4 };
 
 struct Workspace {
   int32_t* flags;     // [16]
-  int64_t* total;     // [1] groups
+  int32_t* counts;    // [tiles + 1] groups per tile
   uint64_t* keys_in;  // [nnz]
   uint64_t* keys;     // [nnz] sorted
   int32_t* rows_in;   // [nnz] row of every nonzero
@@ -47,14 +47,16 @@ int bit_length(uint64_t x) {
   return b;
 }
 
-size_t scratch_bytes(int64_t nnz) {
-  size_t sort_bytes = 0, scan_bytes = 0;
+size_t scratch_bytes(int64_t nnz, int64_t tiles) {
+  size_t sort_bytes = 0, scan_bytes = 0, tile_scan_bytes = 0;
   (void)hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, (const uint64_t*)nullptr, (uint64_t*)nullptr,
                                            (const int32_t*)nullptr, (int32_t*)nullptr, (int)nnz, 0, 64,
                                            (hipStream_t) nullptr);
   HeadIter it(hipcub::CountingInputIterator<int64_t>(0), HeadFlag{nullptr});
   (void)hipcub::DeviceScan::InclusiveSum(nullptr, scan_bytes, it, (int32_t*)nullptr, (int)nnz, (hipStream_t) nullptr);
-  return std::max(sort_bytes, scan_bytes);
+  (void)hipcub::DeviceScan::ExclusiveSum(nullptr, tile_scan_bytes, (const int32_t*)nullptr, (int32_t*)nullptr,
+                                         (int)(tiles + 1), (hipStream_t) nullptr);
+  return std::max(std::max(sort_bytes, scan_bytes), tile_scan_bytes);
 }
 
 Workspace layout(void* d_ws, int64_t tiles, int64_t nnz) {
@@ -67,14 +69,14 @@ Workspace layout(void* d_ws, int64_t tiles, int64_t nnz) {
   };
   const size_t e = size_t(std::max<int64_t>(nnz, 1));
   w.flags = reinterpret_cast<int32_t*>(take(16 * sizeof(int32_t)));
-  w.total = reinterpret_cast<int64_t*>(take(sizeof(int64_t)));
+  w.counts = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * size_t(tiles + 1)));
   w.keys_in = reinterpret_cast<uint64_t*>(take(sizeof(uint64_t) * e));
   w.keys = reinterpret_cast<uint64_t*>(take(sizeof(uint64_t) * e));
   w.rows_in = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * e));
   w.rows = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * e));
   w.rank = reinterpret_cast<int32_t*>(take(sizeof(int32_t) * e));
   w.begin = reinterpret_cast<int64_t*>(take(sizeof(int64_t) * size_t(tiles + 1)));
-  w.tmp_bytes = scratch_bytes(nnz);
+  w.tmp_bytes = scratch_bytes(nnz, tiles);
   w.tmp = take(w.tmp_bytes);
   w.total_bytes = off;
   return w;
@@ -131,32 +133,18 @@ __device__ __forceinline__ int64_t distinct_before(const int32_t* __restrict__ r
   return pos > 0 ? rank[pos - 1] : 0;
 }
 
-// One workgroup: groups per tile -> offsets.
-__global__ __launch_bounds__(256) void condense_groups_kernel(int64_t tiles, int g, const int64_t* __restrict__ begin,
-                                                              const int32_t* __restrict__ rank,
-                                                              int32_t* __restrict__ group_indptr,
-                                                              int64_t* __restrict__ total, int32_t* __restrict__ flags) {
-  using Scan = hipcub::BlockScan<int64_t, 256>;
-  __shared__ typename Scan::TempStorage tmp;
-  int64_t carry = 0;
-  for (int64_t t0 = 0; t0 < tiles; t0 += 256) {
-    const int64_t tile = t0 + threadIdx.x;
-    int64_t grp = 0;
-    if (tile < tiles) {
-      const int64_t distinct = distinct_before(rank, begin[tile + 1]) - distinct_before(rank, begin[tile]);
-      grp = (distinct + g - 1) / g;
-    }
-    int64_t before, sum;
-    Scan(tmp).ExclusiveSum(grp, before, sum);
-    __syncthreads();
-    if (tile < tiles) group_indptr[tile] = (int32_t)(carry + before);
-    carry += sum;
+// groups per tile (one more entry, zero, so that the scan's last output is the total)
+__global__ __launch_bounds__(256) void condense_count_kernel(int64_t tiles, int g, const int64_t* __restrict__ begin,
+                                                             const int32_t* __restrict__ rank,
+                                                             int32_t* __restrict__ counts) {
+  const int64_t tile = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (tile > tiles) return;
+  int64_t grp = 0;
+  if (tile < tiles) {
+    const int64_t distinct = distinct_before(rank, begin[tile + 1]) - distinct_before(rank, begin[tile]);
+    grp = (distinct + g - 1) / g;
   }
-  if (threadIdx.x == 0) {
-    group_indptr[tiles] = (int32_t)carry;
-    *total = carry;
-    if (carry >= (int64_t(1) << 31)) atomicOr(flags, (int)kTooLarge);
-  }
+  counts[tile] = (int32_t)grp;  // at most the tile's nonzeros
 }
 
 __global__ __launch_bounds__(256) void condense_zero_kernel(int32_t* __restrict__ a, int64_t na,
@@ -238,14 +226,20 @@ int stir_condense_device_sizes(int32_t n, int64_t nnz, const int32_t* d_indptr, 
   hipLaunchKernelGGL(condense_bounds_kernel, dim3((unsigned)ceil_div(tiles + 1, 256)), dim3(256), 0, st, tiles, nnz,
                      w.keys, w.begin);
   STIR_LAUNCH_CHECK();
-  hipLaunchKernelGGL(condense_groups_kernel, dim3(1), dim3(256), 0, st, tiles, g, w.begin, w.rank, d_group_indptr,
-                     w.total, w.flags);
+  hipLaunchKernelGGL(condense_count_kernel, dim3((unsigned)ceil_div(tiles + 1, 256)), dim3(256), 0, st, tiles, g,
+                     w.begin, w.rank, w.counts);
   STIR_LAUNCH_CHECK();
+  {
+    size_t bytes = w.tmp_bytes;
+    STIR_HIP(hipcub::DeviceScan::ExclusiveSum(w.tmp, bytes, (const int32_t*)w.counts, d_group_indptr, (int)(tiles + 1),
+                                              st));
+  }
+  int32_t h_total = 0;  // the groups cannot outnumber the nonzeros, which fit 31 bits
   STIR_HIP(hipMemcpyAsync(&h_flags, w.flags, sizeof(int32_t), hipMemcpyDeviceToHost, st));
-  STIR_HIP(hipMemcpyAsync(num_groups, w.total, sizeof(int64_t), hipMemcpyDeviceToHost, st));
+  STIR_HIP(hipMemcpyAsync(&h_total, d_group_indptr + tiles, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   STIR_HIP(hipStreamSynchronize(st));
+  *num_groups = h_total;
   STIR_REQUIRE(!(h_flags & kBadColumn), "%s: a column index is negative", who);
-  STIR_REQUIRE(!(h_flags & kTooLarge), "%s: 2^31 groups or more", who);
   return 0;
 }
 
