@@ -15,9 +15,11 @@
 // units of at least kUnitSteps steps that add their results with atomics; a first launch clears the rows
 // of those tiles.  With fp16 output partial sums would be rounded once per unit; there, tiles of
 // more than kLongSteps steps are left to a second launch (tcspmm_long_kernel) whose workgroups
-// have 8 wavefronts that split the steps of the tile among them and add their fp32 partial sums
+// have 16 wavefronts that split the steps of the tile among them and add their fp32 partial sums
 // through LDS before the one write of the tile.  (For fp32 output that launch is the slower of the
-// two ways: a hub tile is a chain of steps/8 instead of steps/16, and the launches run in turn.)
+// two ways: the launches run in turn.  Running them side by side on two streams was tried for
+// fp16 output and lost: workgroups of 16 wavefronts wait for room beside the other launch, and
+// the hub tile's chain runs slower on a shared compute unit than the overlap gains.)
 #include "common.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -33,7 +35,8 @@ constexpr int kGroup = 16;  // g
 constexpr int kUnitSteps = 16;  // steps (of two groups) per unit of a long tile
 constexpr int kSplit = 16;      // most units per tile (second grid dimension of the split launch)
 constexpr int kLongSteps = 16;  // fp16 output: tiles with more steps go to the second launch
-constexpr int kLongWaves = 8;   // wavefronts per workgroup there (16 would leave 128 registers each: spills)
+constexpr int kLongScan = 8;    // ... each workgroup of which looks at this many row tiles
+constexpr int kLongNT = 2;      // ... whose workgroups own 32 * kLongNT features and have 32 / kLongNT * 4 wavefronts
 
 __device__ __forceinline__ int tile_steps(const int32_t* __restrict__ indptr, int64_t io) {
   const int64_t rows_total = (int64_t)(indptr[io + 1] - indptr[io]) * kGroup;
@@ -172,76 +175,106 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   }
 }
 
-// fp16 output: the tiles the kernel above skips.  512 threads; wavefront w takes steps w, w + 8, ... of the
-// tile for all 128 features (four accumulators), gathers the step's 32 rows of B itself (lane:
-// k pairs kp, kp + 4, kp + 8, kp + 12 and 8-feature chunk fc) into its own 8 KB piece of LDS -- no
-// workgroup barrier in the loop, the LDS operations of one wavefront execute in order -- and the
-// partial results are added through LDS, one 32-feature tile at a time.
-// Dynamic LDS: kLongWaves * 16 * kTileF words (64 KB).
-__global__ __launch_bounds__(64 * kLongWaves) void tcspmm_long_kernel(int feat, int64_t mb, int f_tiles,
+// fp16 output: the tiles the kernel above skips.  A workgroup owns (row tile, 32 * NTL features)
+// and has 32 / NTL wavefronts: 8 with all four 32-feature accumulators of a 128-feature slice, or
+// (what is launched) 16 with two -- 64 features; half the accumulators and half the staged bytes
+// per wavefront, so that 16 fit the register file.  Wavefront w takes steps w, w + WAVES, ... of the
+// tile, gathers the step's 32 rows of B itself (lane: k pairs kp, kp + KP, ... and 8-feature chunk
+// fc) into its own piece of LDS -- no workgroup barrier in the loop, the LDS operations of one
+// wavefront execute in order -- and the partial results are added through LDS, one 32-feature
+// tile at a time.  The steps of a tile are a chain per wavefront (a step is a round trip to
+// memory): more wavefronts per tile shorten the launch, whose length is that of its longest tile.
+// Dynamic LDS: WAVES * 16 * 32 * NTL words (64 KB either way).
+template <int NTL>
+__global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, int64_t mb, int f_tiles,
                                                                       const uint16_t* __restrict__ A,
                                                                       const uint16_t* __restrict__ B,
                                                                       void* __restrict__ C,
                                                                       const int32_t* __restrict__ indptr,
                                                                       const int32_t* __restrict__ indices) {
+  constexpr int WAVES = 32 / NTL;  // wavefronts per workgroup
+  constexpr int TF = 32 * NTL;     // features per workgroup
+  constexpr int CH = TF / 8;       // 8-feature chunks of a staged row
+  constexpr int KP = 64 / CH;      // k pairs a wavefront stages at once
+  constexpr int Q = 16 / KP;       // ... times Q = the 16 k pairs of a step
   extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int f_tile = (int)(blockIdx.x % f_tiles);
-  const int64_t io = blockIdx.x / f_tiles;
-  if (io >= mb) return;
+  const int f0 = f_tile * TF;
+  const int kp = lane / CH, fc = lane % CH;
+  const bool stage_live = f0 + fc * 8 < feat;
+  uint32_t(*xs)[TF] = reinterpret_cast<uint32_t(*)[TF]>(lds + wave * (16 * TF));  // [k pair][feature]
+  // A workgroup looks at kLongScan row tiles and works on the long ones among them (most have
+  // none): a workgroup per tile would start tens of thousands that only find out that their tile
+  // is short, each holding 64 KB of LDS while it does.  Its tiles lie a whole grid apart -- long
+  // tiles come in runs (the hub rows of a graph sorted by degree) and would otherwise queue up in
+  // one workgroup.
+  const int64_t io_stride = gridDim.x / f_tiles;
+  // which of them are long: lane k asks for the group range of the k-th tile, all at once
+  uint64_t todo;
+  {
+    const int64_t io = blockIdx.x / f_tiles + (int64_t)lane * io_stride;
+    int64_t groups = 0;
+    if (lane < kLongScan && io < mb) groups = indptr[io + 1] - indptr[io];
+    todo = __ballot((groups * kGroup + 31) / 32 > kLongSteps);
+  }
+  bool used_lds = false;
+  while (todo) {
+  const int k_tile = __ffsll((long long)todo) - 1;
+  todo &= todo - 1;
+  const int64_t io = blockIdx.x / f_tiles + (int64_t)k_tile * io_stride;
   const int64_t g_begin = indptr[io], g_end = indptr[io + 1];
   const int64_t rows_total = (g_end - g_begin) * kGroup;
   const int steps = (int)((rows_total + 31) / 32);
-  if (steps <= kLongSteps) return;  // uniform over the workgroup
-  const int f0 = f_tile * kTileF;
-  const int kp = lane >> 4, fc = lane & 15;
-  const bool stage_live = f0 + fc * 8 < feat;
+  if (used_lds) __syncthreads();       // the sums of the tile before have been read
+  used_lds = true;
   const int32_t* rowlist = indices + g_begin * kGroup;
-  uint32_t(*xs)[kTileF] = reinterpret_cast<uint32_t(*)[kTileF]>(lds + wave * (16 * kTileF));  // [k pair][feature]
 
-  f32x16 acc[4];
+  f32x16 acc[NTL];
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < NTL; ++t)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
 
   // row ids one step (of this wavefront) before the rows of B, as in the kernel above
-  int row_a[4], row_b[4];
+  int row_a[Q], row_b[Q];
   auto fetch_ids = [&](int it) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int64_t k = (int64_t)it * 32 + 2 * (kp + 4 * q);
+    for (int q = 0; q < Q; ++q) {
+      const int64_t k = (int64_t)it * 32 + 2 * (kp + KP * q);
       row_a[q] = row_b[q] = 0;
       if (k < rows_total) row_a[q] = rowlist[k], row_b[q] = rowlist[k + 1];
     }
   };
-  u32x4 r0[4], r1[4], a_next[2];
+  u32x4 r0[Q], r1[Q], a_next[2];
   auto fetch = [&](int it) {
     const int64_t jo = g_begin + 2 * it;
     a_next[0] = *reinterpret_cast<const u32x4*>(A + (jo * kTile + n) * kGroup + 8 * h);
     a_next[1] = u32x4{0, 0, 0, 0};
     if (jo + 1 < g_end) a_next[1] = *reinterpret_cast<const u32x4*>(A + ((jo + 1) * kTile + n) * kGroup + 8 * h);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < Q; ++q) {
       r0[q] = r1[q] = u32x4{0, 0, 0, 0};
-      const int64_t k = (int64_t)it * 32 + 2 * (kp + 4 * q);
+      const int64_t k = (int64_t)it * 32 + 2 * (kp + KP * q);
       if (stage_live && k < rows_total) {
         r0[q] = *reinterpret_cast<const u32x4*>(B + (int64_t)row_a[q] * feat + f0 + fc * 8);
         r1[q] = *reinterpret_cast<const u32x4*>(B + (int64_t)row_b[q] * feat + f0 + fc * 8);
       }
     }
-    if (it + kLongWaves < steps) fetch_ids(it + kLongWaves);
+    if (it + WAVES < steps) fetch_ids(it + WAVES);
   };
 
-  // steps > kLongSteps >= kLongWaves: every wavefront has a step
-  fetch_ids(wave);
-  fetch(wave);
-  for (int it = wave; it < steps; it += kLongWaves) {
+  // a wavefront without a step (steps < WAVES) only takes part in the sums
+  if (wave < steps) {
+    fetch_ids(wave);
+    fetch(wave);
+  }
+  for (int it = wave; it < steps; it += WAVES) {
     const u32x4 a0 = a_next[0], a1 = a_next[1];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < Q; ++q) {
       u32x4 lo, hi;
 #pragma unroll
       for (int d = 0; d < 2; ++d) {
@@ -250,14 +283,14 @@ __global__ __launch_bounds__(64 * kLongWaves) void tcspmm_long_kernel(int feat, 
         hi[2 * d] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x05040100);
         hi[2 * d + 1] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x07060302);
       }
-      *reinterpret_cast<u32x4*>(&xs[kp + 4 * q][fc * 8]) = lo;
-      *reinterpret_cast<u32x4*>(&xs[kp + 4 * q][fc * 8 + 4]) = hi;
+      *reinterpret_cast<u32x4*>(&xs[kp + KP * q][fc * 8]) = lo;
+      *reinterpret_cast<u32x4*>(&xs[kp + KP * q][fc * 8 + 4]) = hi;
     }
-    if (it + kLongWaves < steps) fetch(it + kLongWaves);
+    if (it + WAVES < steps) fetch(it + WAVES);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < NTL; ++t) {
       const int col = t * 32 + n;
       u32x4 b0, b1;
 #pragma unroll
@@ -276,19 +309,19 @@ __global__ __launch_bounds__(64 * kLongWaves) void tcspmm_long_kernel(int feat, 
 
   // ---- the partial tiles, one 32-feature tile at a time: a thread sums register v of lane l
   // over the wavefronts; that is row (v%4) + 4(l/32) + 8(v/4), feature l%32 of the tile.
-  float* red = reinterpret_cast<float*>(lds);  // [wavefront][register][lane], 32 KB
+  float* red = reinterpret_cast<float*>(lds);  // [wavefront][register][lane], 4 KB per wavefront
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < NTL; ++t) {
     __syncthreads();  // staging pieces (t = 0) or the sums of the tile before are done with
 #pragma unroll
     for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[t][v];
     __syncthreads();
 #pragma unroll
-    for (int e = tid; e < 16 * 64; e += 64 * kLongWaves) {
+    for (int e = tid; e < 16 * 64; e += 64 * WAVES) {
       const int v = e >> 6, l = e & 63;
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < kLongWaves; ++w) sum += red[(w * 16 + v) * 64 + l];
+      for (int w = 0; w < WAVES; ++w) sum += red[(w * 16 + v) * 64 + l];
       const int fcol = f0 + t * 32 + (l & 31);
       if (fcol < feat) {
         const int row = (v & 3) + 4 * (l >> 5) + 8 * (v >> 2);
@@ -298,6 +331,7 @@ __global__ __launch_bounds__(64 * kLongWaves) void tcspmm_long_kernel(int feat, 
       }
     }
   }
+  }  // row tiles of this workgroup
 }
 
 }  // namespace
@@ -325,12 +359,17 @@ extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size
     hipLaunchKernelGGL((tcspmm_kernel<1, true>), dim3((unsigned)blocks, kSplit), dim3(256), 0, st, feat,
                        (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
   } else {
+    // the two launches write different row tiles
+    constexpr int kLongTF = 32 * kLongNT, kLongWaves = 32 / kLongNT;
+    constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kLongTF * sizeof(uint32_t);
+    const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
+    const int64_t long_blocks = stir::ceil_div((int64_t)mb, kLongScan) * long_f_tiles;
+    STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
     hipLaunchKernelGGL((tcspmm_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
                        f_tiles, A, B, d_C, d_indptr, d_indices);
     STIR_LAUNCH_CHECK();
-    constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kTileF * sizeof(uint32_t);
-    hipLaunchKernelGGL(tcspmm_long_kernel, dim3((unsigned)blocks), dim3(64 * kLongWaves), kLongLds, st, feat,
-                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
+    hipLaunchKernelGGL(tcspmm_long_kernel<kLongNT>, dim3((unsigned)long_blocks), dim3(64 * kLongWaves), kLongLds, st,
+                       feat, (int64_t)mb, long_f_tiles, A, B, d_C, d_indptr, d_indices);
   }
   STIR_LAUNCH_CHECK();
   return 0;
