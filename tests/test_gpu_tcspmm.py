@@ -86,3 +86,15 @@ def test_tcspmm_hub_tile(dev, out_dtype):
     indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
     indices = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
     _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=9)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("tiles,feat", [(40, 96), (9, 64), (67, 32)])
+def test_tcspmm_every_tile_long(dev, tiles, feat, out_dtype):
+    """Rows of about 40 entries over 3000 columns: every row tile has more than a thousand
+    distinct columns, i.e. 35 to 40 steps.  With fp16 output a workgroup of the launch for long
+    tiles then works on several tiles in turn (it looks at eight, a whole grid apart); tile counts
+    that are and are not multiples of eight, and a last tile with fewer than 32 rows."""
+    m, n = tiles * 32 - 5, 3000
+    indptr, indices = random_csr(m, n, 40 * m, tiles, skew=0.0)
+    _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=tiles)
