@@ -290,6 +290,29 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
                         ell_rows=int(sum(r.size for r in rows)), static_weights=static,
                         accumulation="32-row output tiles written once; tiles cut by a share boundary add with atomics")
 
+    # The same layer with 130 relations (the reference's BGS and AM graphs have 200 to 270 with their
+    # inverses): W is twice what the LDS of a compute unit holds, so the plan runs two ranges of
+    # relations one after the other.  The ELL3D arrays come from the device format pass.
+    cfg_r = datasets.config5(seed=5, num_rels=130)
+    Rr = cfg_r["num_rels"]
+    d_csf = [t(cfg_r[k]) for k in ("indptr0", "indices0", "indptr1", "indices1")]
+    ptr_r, rows_r, cols_r, mask_r = st.csf_to_ell3d(*d_csf, rb, buckets)
+    triples_r, mids_r = [], []
+    rel_ids = torch.arange(Rr, dtype=torch.int32, device=dev)
+    for k in range(len(buckets)):
+        triples_r += [mask_r[k].reshape(-1).half(), rows_r[k].reshape(-1), cols_r[k].reshape(-1)]
+        mids_r.append(torch.repeat_interleave(rel_ids, (ptr_r[k][1:] - ptr_r[k][:-1]).long()))
+    w_r = t(cfg_r["w"].astype(np.float16).ravel())
+    x_r = t(cfg_r["x"].astype(np.float16).ravel())
+    f = ops.build_rgms(n, n, Rr, fin, fout, rb, buckets, [c.shape[0] for c in cols_r], static_weights=True)
+    f(w_r, x_r, y, *triples_r, *mids_r)
+    tm = time_small(lambda: f(w_r, x_r, y, *triples_r, *mids_r), 50, 3, torch)
+    Er = int(cfg_r["indices1"].shape[0])
+    out["rgms_130_relations"] = dict(tm, us=tm["us_back_to_back"], edges=Er, num_rels=Rr, static_weights=True,
+                                     tflops=(2.0 * Er * fin * fout + 2.0 * Er * fout) / tm["us_back_to_back"] / 1e6,
+                                     launches_per_call=2)
+    del d_csf, triples_r, mids_r, w_r, x_r, f
+
     # SpMM over the condensed format (t = 32, g = 16) on the config-2 graph, fp16 in, fp32 out
     g2 = datasets.config2()
     st.condense(g2["indptr"], g2["indices"], 32, 16)
