@@ -135,17 +135,21 @@ PROFILE_RUN = False  # set by --profile
 
 def time_small(fn, calls, warmup, torch, graph=True):
     """Three timings of a short kernel, in microseconds: events around every call, one event pair
-    around a run of calls, and a captured graph of 20 launches replayed (device time only)."""
+    around a run of calls (the median of three such runs), and a captured graph of 20 launches
+    replayed (device time only)."""
     if PROFILE_RUN:
         calls, warmup, graph = 3, 1, False
     _, per_call, _ = time_steps(fn, calls, warmup, torch)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(calls):
-        fn()
-    e1.record()
-    e1.synchronize()
-    out = {"us_per_call": per_call * 1e6, "us_back_to_back": e0.elapsed_time(e1) * 1e3 / calls}
+    batches = []
+    for _ in range(1 if PROFILE_RUN else 3):  # the median of three runs: clocks drift between neighbours
+        e0.record()
+        for _ in range(calls):
+            fn()
+        e1.record()
+        e1.synchronize()
+        batches.append(e0.elapsed_time(e1) * 1e3 / calls)
+    out = {"us_per_call": per_call * 1e6, "us_back_to_back": sorted(batches)[len(batches) // 2]}
     if graph:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
