@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void csf_classify_kernel(int rels, int64_t row
       if (p0[mid] <= i) lo = mid; else hi = mid - 1;
     }
     rel_of[i] = lo;
-    if (i > p0[lo] && i0[i - 1] >= i0[i]) bad |= kRowOrder;
+    if (i > 0 && i > p0[lo] && i0[i - 1] >= i0[i]) bad |= kRowOrder;  // i > 0: indptr0 may hold anything yet
   }
   if (bad) atomicOr(flags, bad);
 }
