@@ -195,3 +195,153 @@ def test_offsets_beyond_2_to_31_elements(dev):
     ref = (a.view(m, feat)[rowid].double() * x.view(n, feat)[d_idx.long()].double()).sum(1)
     mag = (a.view(m, feat)[rowid].double() * x.view(n, feat)[d_idx.long()].double()).abs().sum(1)
     assert torch.all((out.double() - ref).abs() <= 1e-5 * mag + 1e-30)
+
+
+def _far_ids(rng, count, total, replace=False):
+    """Ids out of [0, total): most of them near the end, a few near the start."""
+    tail = min(200_000, total // 2)
+    pool = np.concatenate([np.arange(total - tail, total), np.arange(0, min(1000, total - tail))])
+    return np.sort(rng.choice(pool, count, replace=replace))
+
+
+@pytest.mark.parametrize("out32", [False, True])
+def test_bsr_offsets_beyond_2_to_31_elements(dev, out32):
+    """X and Y with 2.6e9 elements each: the blocks of X and the block rows of Y that start beyond
+    the 2^31-th element (and the 2^32-th byte) must be reached with 64-bit offsets.  Non-empty
+    block rows against fp32 products by torch, every other block row must be zero."""
+    mb = nb = 40_000
+    blk, feat = 32, 2048
+    assert nb * blk * feat > 2**31 and mb * blk * feat > 2**31
+    rng = np.random.default_rng(21)
+    live = _far_ids(rng, 160, mb)
+    counts = np.zeros(mb, np.int64)
+    counts[live] = rng.integers(1, 7, len(live))
+    indptr = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    indices = np.concatenate([_far_ids(rng, counts[i], nb) for i in live]).astype(np.int32)
+    nnzb = len(indices)
+    gen = torch.Generator(device=dev).manual_seed(21)
+    a = (torch.randn(nnzb * blk * blk, device=dev, generator=gen) * 0.05).half()
+    x = torch.randn(nb * blk * feat, device=dev, generator=gen, dtype=torch.float16)
+    odt = torch.float32 if out32 else torch.float16
+    y = torch.ones(mb * blk * feat, device=dev, dtype=odt)
+    t = lambda v: torch.from_numpy(v).to(dev)
+    ops.build_bsrmm(mb, nb, nnzb, blk, feat, torch.float16, odt)(a, x, y, t(indptr), t(indices))
+    torch.cuda.synchronize()
+    yv, xv = y.view(mb, blk, feat), x.view(nb, blk, feat)
+    for i in live:
+        want = torch.zeros(blk, feat, device=dev)
+        scale = torch.zeros(blk, feat, device=dev)
+        for p in range(indptr[i], indptr[i + 1]):
+            blk_a = a[p * blk * blk:(p + 1) * blk * blk].view(blk, blk).float()
+            want += blk_a @ xv[indices[p]].float()
+            scale += blk_a.abs() @ xv[indices[p]].float().abs()
+        tol = (1e-5 if out32 else 2e-2) * want.abs() + 1e-5 * scale + 1e-30
+        assert bool(((yv[i].float() - want).abs() <= tol).all()), int(i)
+    # all the rest is zero: the non-zero entries of Y are those of the live block rows
+    assert int(torch.count_nonzero(y)) == int(torch.count_nonzero(yv[t(live)]))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_tcspmm_offsets_beyond_2_to_31_elements(dev, out_dtype):
+    """B and C with 2.3e9 / 2.5e9 elements: tiles at the far end of C, among them one long enough
+    for the launch of the long tiles, gather rows at the far end of B."""
+    n, feat, mb = 18_000_000, 128, 600_000
+    m = mb * 32
+    assert n * feat > 2**31 and m * feat > 2**31
+    rng = np.random.default_rng(22)
+    deg = np.zeros(m, np.int64)
+    live_tiles = _far_ids(rng, 24, mb)
+    for k, tile in enumerate(live_tiles):
+        rows = np.arange(tile * 32, tile * 32 + 32)
+        deg[rows] = rng.integers(0, 6, 32) if k != len(live_tiles) - 2 else 40  # one tile of 1280 columns
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    live_rows = np.nonzero(deg)[0]
+    indices = np.concatenate([_far_ids(rng, deg[r], n) for r in live_rows]).astype(np.int32)
+    gptr, tiles, mask = st.condense(indptr, indices, 32, 16)
+    nnzb = tiles.shape[0]
+    assert int(np.diff(gptr).max()) * 16 > 16 * 32  # more than 16 steps of 32 columns in one tile
+    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    gen = torch.Generator(device=dev).manual_seed(22)
+    b = torch.randn(n * feat, device=dev, generator=gen, dtype=torch.float16)
+    c = torch.ones(m * feat, device=dev, dtype=out_dtype)
+    ops.build_tcspmm(mb, nnzb, feat, 32, 16, n, out_dtype)(
+        t(mask.astype(np.float16).ravel()), b, c, t(gptr), t(tiles.ravel()))
+    torch.cuda.synchronize()
+    d_rows, d_idx = t(live_rows), t(indices)
+    rowid = torch.repeat_interleave(torch.arange(len(live_rows), device=dev), t(deg[live_rows]))
+    gathered = b.view(n, feat)[d_idx.long()].double()
+    want = torch.zeros(len(live_rows), feat, device=dev, dtype=torch.float64).index_add_(0, rowid, gathered)
+    scale = torch.zeros(len(live_rows), feat, device=dev, dtype=torch.float64).index_add_(0, rowid, gathered.abs())
+    got = c.view(m, feat)[d_rows].double()
+    rtol = 2e-2 if out_dtype == torch.float16 else 1e-5
+    assert bool(((got - want).abs() <= rtol * want.abs() + 1e-5 * scale + 1e-30).all())
+    assert int(torch.count_nonzero(c)) == int(torch.count_nonzero(c.view(m, feat)[d_rows]))
+
+
+def test_rgms_x_beyond_2_to_32_bytes(dev):
+    """70 M nodes: X has 4.5 GB and Y 9 GB, so source rows beyond the 2^32-th byte and destination
+    tiles beyond the 2^31-th float are used.  Expected values from per-edge fp64 products by
+    torch; everything outside the destination rows stays zero."""
+    n = m = 70_000_000
+    R, fin, fout = 8, 32, 32
+    assert n * fin * 2 > 2**32 and m * fout > 2**31
+    rng = np.random.default_rng(23)
+    p0, i0, p1, i1 = [0], [], [0], []
+    for r in range(R):
+        rows = np.unique(_far_ids(rng, 800, m))
+        for i in rows:
+            cols = np.unique(_far_ids(rng, rng.integers(1, 17), n, replace=True))
+            i1.append(cols)
+            p1.append(p1[-1] + len(cols))
+        i0.append(rows)
+        p0.append(p0[-1] + len(rows))
+    csf = (np.array(p0, np.int32), np.concatenate(i0).astype(np.int32), np.array(p1, np.int32),
+           np.concatenate(i1).astype(np.int32))
+    buckets = [1, 2, 4, 8, 16]
+    rb = [32 // b for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    assert sum(c.size for c in cols) >= 8192  # the destination-tile path
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float16).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
+    gen = torch.Generator(device=dev).manual_seed(23)
+    x = torch.randn(n * fin, device=dev, generator=gen, dtype=torch.float16)
+    w = (torch.randn(R * fin * fout, device=dev, generator=gen) * 0.1).half()
+    y = torch.zeros(m * fout, device=dev)
+    ops.build_rgms(m, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols])(w, x, y, *triples, *mids)
+    torch.cuda.synchronize()
+    # per edge: X[col] @ W[rel], summed per destination row
+    rel = np.repeat(np.arange(R), np.diff(csf[0]))           # relation of every stored row
+    e_rel = t(np.repeat(rel, np.diff(csf[2])).astype(np.int64))
+    e_row = np.repeat(csf[1], np.diff(csf[2]))
+    dst, inv = np.unique(e_row, return_inverse=True)
+    xe = x.view(n, fin)[t(csf[3]).long()].double()
+    we = w.view(R, fin, fout).double()[e_rel]
+    prod = torch.bmm(xe[:, None, :], we)[:, 0, :]
+    mag = torch.bmm(xe.abs()[:, None, :], we.abs())[:, 0, :]
+    want = torch.zeros(len(dst), fout, device=dev, dtype=torch.float64).index_add_(0, t(inv.astype(np.int64)), prod)
+    scale = torch.zeros(len(dst), fout, device=dev, dtype=torch.float64).index_add_(0, t(inv.astype(np.int64)), mag)
+    d_dst = t(dst.astype(np.int64))
+    got = y.view(m, fout)[d_dst].double()
+    assert bool(((got - want).abs() <= 2e-2 * want.abs() + 1e-5 * scale + 1e-30).all())
+    assert int(torch.count_nonzero(y)) == int(torch.count_nonzero(y.view(m, fout)[d_dst]))
+
+    # the fp32 forms on the same graph (X has 9 GB there): W is laid out [relation, out, in]
+    x32 = x.float()
+    w32 = w.view(R, fin, fout).float().transpose(1, 2).contiguous().view(-1)
+    triples32 = [a.float() if a.dtype == torch.float16 else a for a in triples]
+    for form in ("ell3d", "csf"):
+        y.zero_()
+        if form == "ell3d":
+            ops.build_rgms_f32(m, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols])(
+                w32, x32, y, *triples32, *mids)
+        else:
+            ones = torch.ones(len(csf[3]), device=dev)
+            ops.build_rgms_csf(m, n, R, fin, fout, len(csf[1]), len(csf[3]))(
+                ones, w32, x32, y, t(csf[0]), t(csf[1]), t(csf[2]), t(csf[3]))
+        torch.cuda.synchronize()
+        got = y.view(m, fout)[d_dst].double()
+        assert bool(((got - want).abs() <= 1e-5 * scale + 1e-30).all()), form
+        assert int(torch.count_nonzero(y)) == int(torch.count_nonzero(y.view(m, fout)[d_dst])), form
