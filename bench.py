@@ -63,6 +63,8 @@ def load_probes():
     VP, I64, I32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
     L.bench_probe_copy.restype, L.bench_probe_copy.argtypes = I32, [VP, VP, I64, VP]
     L.bench_probe_gather.restype, L.bench_probe_gather.argtypes = I32, [VP, I64, I32, I64, VP, VP]
+    L.bench_probe_mfma_f16.restype = I32
+    L.bench_probe_mfma_f16.argtypes = [I32, I32, I32, VP, ctypes.POINTER(ctypes.c_double), VP]
     return L
 
 
@@ -538,6 +540,14 @@ def main():
         _, gat_s, _ = time_steps(lambda: probe(P.bench_probe_gather(vp(x), n, feat, nnz, vp(c_csr), st0)),
                                  3, 1, torch)
         probes["random_row_gather_GBps"] = nnz * feat * 4.0 / gat_s / 1e9
+    # ... and the rate at which the matrix cores take v_mfma_f32_32x32x16_f16 from registers (four
+    # wavefronts per SIMD, four independent accumulators each, 2.4 ms): what the 2.5 PFLOP/s that
+    # the BSR / TC-SpMM / RGMS lines are priced against amounts to at the clock this GPU sustains
+    mfma_flop = ctypes.c_double(0.0)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    _, mfma_s, _ = time_steps(lambda: probe(P.bench_probe_mfma_f16(cus, 4, 8192, vp(c_csr), ctypes.byref(mfma_flop),
+                                                                   st0)), 3, 1, torch)
+    probes["mfma_f16_32x32x16_TFLOPs"] = mfma_flop.value / mfma_s / 1e12
     log(f"[bench] probes: {probes}")
 
     # ---- timed region

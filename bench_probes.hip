@@ -1,8 +1,10 @@
-// Bandwidth probes of bench.py, built into libbench_probes.so (not part of the product library):
-// what this GPU sustains for the two access patterns the SpMM/SDDMM kernels are made of -- a plain
-// streaming copy (also the kernel of known size that the FETCH_SIZE / WRITE_SIZE counters are
-// scaled by) and gathers of whole feature rows at pseudo-random row indices (no sparse structure,
-// no arithmetic to speak of).  Both return 0 on success and -1 on bad arguments or a failed launch.
+// Probes of bench.py, built into libbench_probes.so (not part of the product library): what this
+// GPU sustains for the two access patterns the SpMM/SDDMM kernels are made of -- a plain streaming
+// copy (also the kernel of known size that the FETCH_SIZE / WRITE_SIZE counters are scaled by) and
+// gathers of whole feature rows at pseudo-random row indices (no sparse structure, no arithmetic
+// to speak of) -- and the rate at which its matrix cores take v_mfma_f32_32x32x16_f16 from
+// registers, the instruction the BSR, TC-SpMM and RGMS kernels are built on.  All return 0 on
+// success and -1 on bad arguments or a failed launch.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -54,9 +56,49 @@ __global__ __launch_bounds__(256) void probe_gather_kernel(const float* __restri
   if (acc.x == 1.2345e38f) sink[0] = acc.x + acc.y + acc.z + acc.w;
 }
 
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Every wavefront issues iters x 4 MFMAs on four independent accumulators (operands stay in
+// registers; nothing is loaded).  The sum is stored only if it equals a value it cannot take.
+__global__ __launch_bounds__(256) void probe_mfma_f16_kernel(int iters, float* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  f16x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = (_Float16)(0.001f * (lane + i)), b[i] = (_Float16)(0.002f * (lane - i));
+  f32x16 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+#pragma unroll 1
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[t], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sum += acc[t][v];
+  if (sum == 1.2345e38f) sink[0] = sum;
+}
+
 }  // namespace
 
 extern "C" {
+
+// waves_per_simd (1..8) wavefronts on every SIMD of `cus` compute units, each issuing iters x 4
+// MFMAs of 32x32x16 (2*32*32*16 flop each); *flop receives the flop of the whole launch.
+int bench_probe_mfma_f16(int32_t cus, int32_t waves_per_simd, int32_t iters, float* d_sink, double* flop,
+                         void* stream) {
+  if (!(cus > 0 && waves_per_simd >= 1 && waves_per_simd <= 8 && iters > 0 && d_sink && flop)) return -1;
+  const int blocks = cus * waves_per_simd;  // four wavefronts each, one per SIMD
+  *flop = (double)blocks * 4 * (double)iters * 4 * (2.0 * 32 * 32 * 16);
+  hipLaunchKernelGGL(probe_mfma_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     iters, d_sink);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
 
 // Copies `bytes` (a multiple of 16) from d_src to d_dst.
 int bench_probe_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream) {
