@@ -201,6 +201,77 @@ __global__ __launch_bounds__(256) void csr_spmm_kernel(int m, int feat, int spli
   }
 }
 
+// Feature rows narrower than a wavefront (G < 64 lanes): a wavefront owns 64 / G consecutive rows
+// of the matrix, one per lane group.  A group walks its own row -- G nonzeros per index load, up
+// to eight gathers in flight per lane -- and stores it without any exchange between lanes; the
+// wavefront writes 64 / G consecutive rows of C.  With one wavefront per row (the kernel above) a
+// row of seven nonzeros at 32 features keeps one lane group in eight busy for one step and still
+// pays the index round trip, the cross-lane sum and the store.  Rows of more than 2 * G nonzeros
+// would hold the other groups up: the wavefront takes those one by one afterwards, all groups
+// sharing the row as in the kernel above (and leaves rows above kLongRow zero-filled for
+// csr_long_rows_kernel when split_long is set).
+template <int G>
+__global__ __launch_bounds__(256) void csr_spmm_rows_kernel(int m, int feat, int split_long,
+                                                            const float* __restrict__ A,
+                                                            const float* __restrict__ B,
+                                                            float* __restrict__ C,
+                                                            const int32_t* __restrict__ indptr,
+                                                            const int32_t* __restrict__ indices) {
+  constexpr int NG = kWave / G;
+  constexpr int CH = G < 8 ? G : 8;  // gathers in flight per lane
+  constexpr int kGroupRow = 2 * G;   // longest row a lane group takes alone (1 to 4 * G measure the same)
+  const int lane = threadIdx.x & 63;
+  const int g = lane / G, gl = lane % G;
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * NG;
+  if (row0 >= m) return;
+  const int64_t row = row0 + g;
+  int start = 0, end = 0;
+  if (row < m) start = indptr[row], end = indptr[row + 1];
+  const bool alone = end - start <= kGroupRow;
+  const int my_end = alone ? end : start;
+  const bool chunk_live = gl * 4 < feat;
+  const float* Bl = B + gl * 4;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int base = start; base < my_end; base += G) {
+    const int p = base + gl;
+    const int my_col = p < my_end ? __builtin_nontemporal_load(indices + p) : 0;
+    const float my_val = p < my_end ? __builtin_nontemporal_load(A + p) : 0.f;
+    const int cnt = min(G, my_end - base);
+#pragma unroll 1
+    for (int c = 0; c < cnt; c += CH) {
+      float4 x[CH];
+      float v[CH];
+#pragma unroll
+      for (int u = 0; u < CH; ++u) {
+        const int sl = g * G + c + u;  // a lane of this group: it is in this loop as well
+        const int col = __shfl(my_col, sl, kWave);
+        v[u] = __shfl(my_val, sl, kWave);
+        x[u] = (c + u < cnt && chunk_live) ? ld4(Bl + (int64_t)col * feat) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < CH; ++u) fma4(acc, v[u], x[u]);
+    }
+  }
+  if (row < m && alone && chunk_live) {
+    float* q = C + row * feat + gl * 4;
+    __builtin_nontemporal_store(acc.x, q);
+    __builtin_nontemporal_store(acc.y, q + 1);
+    __builtin_nontemporal_store(acc.z, q + 2);
+    __builtin_nontemporal_store(acc.w, q + 3);
+  }
+  // the longer rows, one after the other, by the whole wavefront
+  uint64_t todo = __ballot(row < m && !alone && gl == 0);
+  while (todo) {
+    const int src = __ffsll((long long)todo) - 1;
+    todo &= todo - 1;
+    const int s = __shfl(start, src, kWave), e = __shfl(end, src, kWave);
+    float4 sum[1] = {make_float4(0.f, 0.f, 0.f, 0.f)};
+    if (!(split_long && e - s > kLongRow)) csr_accumulate<G, 1>(sum, s, e, feat, A, B, indices, lane);
+    reduce_groups<G, 1>(sum, kWave);
+    if (g == 0) write_row<G, 1>(C, row0 + src / G, feat, lane, sum, 0, nullptr);
+  }
+}
+
 // One wavefront per kLongPiece consecutive nonzeros: the parts of rows longer than kLongRow that
 // fall into the piece are summed and added to C (cleared by csr_spmm_kernel) with atomics.
 // Pieces that touch no long row -- nearly all of them -- end after looking at their rows.
@@ -855,16 +926,31 @@ int stir_csr_spmm_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const flo
   }
   // feature widths that are a multiple of 4 take the vectorised kernel with the smallest lane
   // group that covers them (lanes beyond feat / 4 idle); anything else the generic one
+  // lane groups narrower than the wavefront: a lane group per row (csr_spmm_rows_kernel)
+#define STIR_CSR_ROWS(G)                                                                                   \
+  {                                                                                                        \
+    const dim3 row_grid((unsigned)stir::ceil_div(m, 4 * (kWave / G)));                                     \
+    hipLaunchKernelGGL((csr_spmm_rows_kernel<G>), row_grid, block, 0, st, m, feat, split_long, d_A, d_B,   \
+                       d_C, d_indptr, d_indices);                                                          \
+    if (split_long)                                                                                        \
+      hipLaunchKernelGGL((csr_long_rows_kernel<G, 1>), pieces, block, 0, st, m, feat, (int64_t)0, nnz, d_A, \
+                         d_B, d_C, d_indptr, d_indices);                                                   \
+  }
   switch (vector_class(feat)) {
-    case 0: STIR_CSR(4, 1); break;
-    case 1: STIR_CSR(8, 1); break;
-    case 2: STIR_CSR(16, 1); break;
-    case 3: STIR_CSR(32, 1); break;
+    case 0: STIR_CSR_ROWS(4); break;
+    case 1: STIR_CSR_ROWS(8); break;
+    case 2: STIR_CSR_ROWS(16); break;
+    case 3:
+      // two rows per wavefront pay when rows are short: config 2 (7 nonzeros per row) 125 -> 119 us,
+      // config 3 (25 per row) 5.06 -> 5.14 ms
+      if (nnz < 16 * (int64_t)m) STIR_CSR_ROWS(32) else STIR_CSR(32, 1);
+      break;
     case 4: STIR_CSR(64, 1); break;
     case 5: STIR_CSR(64, 2); break;
     default:
       hipLaunchKernelGGL(csr_spmm_generic_kernel, grid, block, 0, st, m, feat, d_A, d_B, d_C, d_indptr, d_indices);
   }
+#undef STIR_CSR_ROWS
 #undef STIR_CSR
   STIR_LAUNCH_CHECK();
   return 0;

@@ -100,6 +100,41 @@ def test_csr_spmm_hub_rows_are_split(dev, feat):
     _check(got, indptr, indices, vals, x, f"hub rows feat={feat}")
 
 
+@pytest.mark.parametrize("feat", [4, 8, 12, 32, 40, 64, 128])
+@pytest.mark.parametrize("split", [False, True])
+def test_csr_spmm_lane_group_per_row(dev, feat, split):
+    """Feature rows narrower than a wavefront: a wavefront owns several rows, one per lane group.
+    Row lengths around every limit of that kernel -- 0, 1, the group width G, 2G (the longest row a
+    group takes alone), 2G + 1 (left to the whole wavefront), 64, 65, 256, 257 and a hub row --
+    next to each other in one wavefront's rows, a row count that is no multiple of the rows per
+    wavefront, and (split) enough nonzeros for the second launch that adds up rows above 256."""
+    G = next(g for g in (4, 8, 16, 32) if 4 * g >= feat)
+    rng = np.random.default_rng(100 * feat + split)
+    special = [0, 1, G - 1, G, G + 1, 2 * G, 2 * G + 1, 3 * G, 63, 64, 65, 255, 256, 257, 0, 1500]
+    # 128 features take this kernel below 16 nonzeros per row on average
+    m, n = (64 * 300 + 5 if feat == 128 and split else 64 * 37 + 5), 9000
+    deg = rng.integers(0, 12, m)
+    for k, d in enumerate(special):
+        deg[k] = d                              # all in the first wavefronts, side by side
+        deg[(k * 97 + 300) % m] = d             # and scattered
+    deg[m - 1] = 2 * G + 1
+    if split:
+        deg[m // 2] = 6000
+        deg[m // 3] = n
+        big = np.nonzero(deg <= 12)[0]
+        while deg.sum() < (1 << 18) + 1000:     # rows of 250 .. 400 until the second launch is on
+            deg[rng.choice(big)] = rng.integers(250, 400)
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    assert (indptr[-1] >= 1 << 18) == split
+    assert feat != 128 or indptr[-1] < 16 * m
+    indices = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
+    vals = rng.random(len(indices), dtype=np.float32) - 0.4
+    x = rng.standard_normal((n, feat), dtype=np.float32)
+    got = _run_csr(dev, indptr, indices, vals, x, feat)
+    assert np.all(got[deg == 0] == 0.0)
+    _check(got, indptr, indices, vals, x, f"lane group per row, feat={feat}, split={split}")
+
+
 def test_csr_spmm_argument_checks(dev):
     f = ops.build_csrmm(4, 4, 32, 3)
     z = lambda k, dt=torch.float32: torch.zeros(k, dtype=dt, device=dev)
