@@ -168,8 +168,11 @@ __device__ __forceinline__ void csr_accumulate(float4 (&acc)[REP], int start, in
 
 // Rows with more nonzeros than this are not left to a single wavefront (a 17k-entry hub row
 // costs one wavefront milliseconds): the row kernel only clears them and csr_long_rows_kernel,
-// launched after it, adds them up in pieces of kLongPiece nonzeros.
-constexpr int kLongRow = 256;
+// launched after it, adds them up in pieces of kLongPiece nonzeros.  64 rather than 256: the
+// piece kernel keeps every lane busy whatever the row, a wavefront on a row of its own does not
+// (169 k-node power-law graph, half of its nonzeros in rows above 256: 46 -> 41 us at 32 features,
+// 223 -> 203 us at 256; 2.45 M-node graph, 128 features: 5.05 -> 5.01 ms; 32 is slower again).
+constexpr int kLongRow = 64;
 constexpr int kLongPiece = 256;
 
 // One wavefront per row.  With split_long the rows above kLongRow are zero-filled here.

@@ -83,13 +83,14 @@ def test_csr_spmm_long_row(dev):
 
 @pytest.mark.parametrize("feat", [32, 128, 512, 96])
 def test_csr_spmm_hub_rows_are_split(dev, feat):
-    """Enough nonzeros for the second launch that adds up rows longer than 256 entries in
+    """Enough nonzeros for the second launch that adds up rows longer than 64 entries in
     256-entry pieces: hub rows of different lengths (piece boundaries inside, at the start and at
     the end of rows), rows just below and above the limit, the output pre-filled with NaN."""
     m, n = 4500, 40000
     rng = np.random.default_rng(feat)
     deg = rng.integers(0, 120, m)
-    for row, d in [(0, 257), (1, 256), (2, 2049), (7, 30000), (8, 2560), (1500, 12345), (m - 1, 5000)]:
+    for row, d in [(0, 257), (1, 256), (2, 2049), (3, 64), (4, 65), (5, 63), (7, 30000), (8, 2560), (1500, 12345),
+                   (m - 1, 5000)]:
         deg[row] = d
     indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
     assert indptr[-1] >= 1 << 18
@@ -107,7 +108,7 @@ def test_csr_spmm_lane_group_per_row(dev, feat, split):
     Row lengths around every limit of that kernel -- 0, 1, the group width G, 2G (the longest row a
     group takes alone), 2G + 1 (left to the whole wavefront), 64, 65, 256, 257 and a hub row --
     next to each other in one wavefront's rows, a row count that is no multiple of the rows per
-    wavefront, and (split) enough nonzeros for the second launch that adds up rows above 256."""
+    wavefront, and (split) enough nonzeros for the second launch that adds up rows above 64."""
     G = next(g for g in (4, 8, 16, 32) if 4 * g >= feat)
     rng = np.random.default_rng(100 * feat + split)
     special = [0, 1, G - 1, G, G + 1, 2 * G, 2 * G + 1, 3 * G, 63, 64, 65, 255, 256, 257, 0, 1500]
