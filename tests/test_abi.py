@@ -45,3 +45,23 @@ def test_no_product_file_touches_the_oracle():
                 text = open(os.path.join(base, f), errors="ignore").read()
                 assert "import oracle" not in text and "from oracle" not in text, f
                 assert "sparsetir_oracle" not in text, f
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: any other --gpus ends at once with a message that says so."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 2
+    assert "one GPU" in (r.stdout + r.stderr)
+
+
+def test_probe_library_exports_its_entry_points():
+    """The benchmark's own probe library (built by __graft_entry__.build) loads and exports the
+    three probes bench.py binds; nothing is launched here."""
+    path = os.path.join(ROOT, "libbench_probes.so")
+    assert os.path.exists(path), "build with `python -c 'import __graft_entry__ as g; g.build()'`"
+    lib = ctypes.CDLL(path)
+    for name in ("bench_probe_copy", "bench_probe_gather", "bench_probe_mfma_f16"):
+        assert hasattr(lib, name), name
