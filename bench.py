@@ -355,9 +355,27 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     # the reference's own form of this operator writes fp16 (bench_tc_spmm.py: fp16 accumulator fragments)
     tc16 = ops.build_tcspmm(mb2, nnzb2, f2, 32, 16, g2["n"], torch.float16)
     c16 = torch.zeros(mb2 * 32 * f2, device=dev, dtype=torch.float16)
+    t0 = time.perf_counter()
+    tc16(a2, b2, c16, gp, ti)  # makes the operator's plan (the long row tiles, longest first, in pieces)
+    torch.cuda.synchronize()
+    first_ms = (time.perf_counter() - t0) * 1e3
     tm = time_small(lambda: tc16(a2, b2, c16, gp, ti), 50, 5, torch)
     out["tcspmm_config2_feat128_f16_out"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"],
-                                             "us": tm["us_back_to_back"]}
+                                             "us": tm["us_back_to_back"], "first_call_ms": first_ms,
+                                             "useful_gflops": 2.0 * nnz2 * f2 / tm["us_back_to_back"] / 1e3,
+                                             "plan": "made from the group counts at the first call"}
+    # the entry point without a plan, as a TVM process binds it
+    from sparsetir_amd import _lib as stlib
+    L16 = stlib.lib()
+    vp = lambda v: ctypes.c_void_p(v.data_ptr())
+
+    def plain():
+        stlib.check(L16.stir_tc_spmm_f16(0, mb2, 32, 16, f2, nnzb2, vp(a2), vp(b2), vp(c16), vp(gp), vp(ti),
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+    tm = time_small(plain, 50, 5, torch)
+    out["tcspmm_config2_feat128_f16_out_no_plan"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"],
+                                                     "us": tm["us_back_to_back"]}
 
     # fp32 forms: ELL3D buckets with 32-slot groups (the reference's composable fp32 setting) and the
     # CSF traversal; W is [R, fout, fin]

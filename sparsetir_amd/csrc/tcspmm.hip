@@ -20,6 +20,12 @@
 // two ways: the launches run in turn.  Running them side by side on two streams was tried for
 // fp16 output and lost: workgroups of 16 wavefronts wait for room beside the other launch, and
 // the hub tile's chain runs slower on a shared compute unit than the overlap gains.)
+// With a plan (stir_tc_plan: the long tiles listed once, longest first, in pieces of at most
+// kPieceSteps steps) the second launch has a workgroup per piece and the hub tiles are spread
+// over many compute units; fp32 partial tiles in the plan's memory, one rounding at the end.
+#include <algorithm>
+#include <vector>
+
 #include "common.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -175,61 +181,36 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   }
 }
 
-// fp16 output: the tiles the kernel above skips.  A workgroup owns (row tile, 32 * NTL features)
-// and has 32 / NTL wavefronts: 8 with all four 32-feature accumulators of a 128-feature slice, or
-// (what is launched) 16 with two -- 64 features; half the accumulators and half the staged bytes
-// per wavefront, so that 16 fit the register file.  Wavefront w takes steps w, w + WAVES, ... of the
-// tile, gathers the step's 32 rows of B itself (lane: k pairs kp, kp + KP, ... and 8-feature chunk
+// The steps [s_begin, s_end) of row tile io for the features [f0, f0 + 32 * NTL), by a workgroup of
+// 32 / NTL wavefronts: 8 with all four 32-feature accumulators of a 128-feature slice, or (what is
+// launched) 16 with two -- 64 features; half the accumulators and half the staged bytes per
+// wavefront, so that 16 fit the register file.  Wavefront w takes steps s_begin + w, + WAVES, ...,
+// gathers the step's 32 rows of B itself (lane: k pairs kp, kp + KP, ... and 8-feature chunk
 // fc) into its own piece of LDS -- no workgroup barrier in the loop, the LDS operations of one
 // wavefront execute in order -- and the partial results are added through LDS, one 32-feature
-// tile at a time.  The steps of a tile are a chain per wavefront (a step is a round trip to
-// memory): more wavefronts per tile shorten the launch, whose length is that of its longest tile.
-// Dynamic LDS: WAVES * 16 * 32 * NTL words (64 KB either way).
-template <int NTL>
-__global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, int64_t mb, int f_tiles,
-                                                                      const uint16_t* __restrict__ A,
-                                                                      const uint16_t* __restrict__ B,
-                                                                      void* __restrict__ C,
-                                                                      const int32_t* __restrict__ indptr,
-                                                                      const int32_t* __restrict__ indices) {
+// tile at a time; store(row in tile, feature, sum) receives every sum once.  The steps are a chain
+// per wavefront (a step is a round trip to memory): more wavefronts per tile shorten it.
+// lds: WAVES * 16 * 32 * NTL words (64 KB either way).  Ends with LDS reads: a caller that goes on
+// to another tile puts a workgroup barrier in between.
+template <int NTL, class Store>
+__device__ __forceinline__ void tcspmm_long_steps(uint32_t* __restrict__ lds, int feat, int64_t io, int f0,
+                                                  int s_begin, int s_end, const uint16_t* __restrict__ A,
+                                                  const uint16_t* __restrict__ B,
+                                                  const int32_t* __restrict__ indptr,
+                                                  const int32_t* __restrict__ indices, Store store) {
   constexpr int WAVES = 32 / NTL;  // wavefronts per workgroup
   constexpr int TF = 32 * NTL;     // features per workgroup
   constexpr int CH = TF / 8;       // 8-feature chunks of a staged row
   constexpr int KP = 64 / CH;      // k pairs a wavefront stages at once
   constexpr int Q = 16 / KP;       // ... times Q = the 16 k pairs of a step
-  extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, h = lane >> 5;
-  const int f_tile = (int)(blockIdx.x % f_tiles);
-  const int f0 = f_tile * TF;
   const int kp = lane / CH, fc = lane % CH;
   const bool stage_live = f0 + fc * 8 < feat;
   uint32_t(*xs)[TF] = reinterpret_cast<uint32_t(*)[TF]>(lds + wave * (16 * TF));  // [k pair][feature]
-  // A workgroup looks at kLongScan row tiles and works on the long ones among them (most have
-  // none): a workgroup per tile would start tens of thousands that only find out that their tile
-  // is short, each holding 64 KB of LDS while it does.  Its tiles lie a whole grid apart -- long
-  // tiles come in runs (the hub rows of a graph sorted by degree) and would otherwise queue up in
-  // one workgroup.
-  const int64_t io_stride = gridDim.x / f_tiles;
-  // which of them are long: lane k asks for the group range of the k-th tile, all at once
-  uint64_t todo;
-  {
-    const int64_t io = blockIdx.x / f_tiles + (int64_t)lane * io_stride;
-    int64_t groups = 0;
-    if (lane < kLongScan && io < mb) groups = indptr[io + 1] - indptr[io];
-    todo = __ballot((groups * kGroup + 31) / 32 > kLongSteps);
-  }
-  bool used_lds = false;
-  while (todo) {
-  const int k_tile = __ffsll((long long)todo) - 1;
-  todo &= todo - 1;
-  const int64_t io = blockIdx.x / f_tiles + (int64_t)k_tile * io_stride;
   const int64_t g_begin = indptr[io], g_end = indptr[io + 1];
   const int64_t rows_total = (g_end - g_begin) * kGroup;
-  const int steps = (int)((rows_total + 31) / 32);
-  if (used_lds) __syncthreads();       // the sums of the tile before have been read
-  used_lds = true;
   const int32_t* rowlist = indices + g_begin * kGroup;
 
   f32x16 acc[NTL];
@@ -263,15 +244,15 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, 
         r1[q] = *reinterpret_cast<const u32x4*>(B + (int64_t)row_b[q] * feat + f0 + fc * 8);
       }
     }
-    if (it + WAVES < steps) fetch_ids(it + WAVES);
+    if (it + WAVES < s_end) fetch_ids(it + WAVES);
   };
 
-  // a wavefront without a step (steps < WAVES) only takes part in the sums
-  if (wave < steps) {
-    fetch_ids(wave);
-    fetch(wave);
+  // a wavefront without a step (fewer steps than wavefronts) only takes part in the sums
+  if (s_begin + wave < s_end) {
+    fetch_ids(s_begin + wave);
+    fetch(s_begin + wave);
   }
-  for (int it = wave; it < steps; it += WAVES) {
+  for (int it = s_begin + wave; it < s_end; it += WAVES) {
     const u32x4 a0 = a_next[0], a1 = a_next[1];
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
@@ -286,7 +267,7 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, 
       *reinterpret_cast<u32x4*>(&xs[kp + KP * q][fc * 8]) = lo;
       *reinterpret_cast<u32x4*>(&xs[kp + KP * q][fc * 8 + 4]) = hi;
     }
-    if (it + WAVES < steps) fetch(it + WAVES);
+    if (it + WAVES < s_end) fetch(it + WAVES);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -323,15 +304,120 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, 
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) sum += red[(w * 16 + v) * 64 + l];
       const int fcol = f0 + t * 32 + (l & 31);
-      if (fcol < feat) {
-        const int row = (v & 3) + 4 * (l >> 5) + 8 * (v >> 2);
-        const int64_t off = (io * kTile + row) * feat + fcol;
-        const _Float16 hv = (_Float16)sum;
-        static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
-      }
+      if (fcol < feat) store((v & 3) + 4 * (l >> 5) + 8 * (v >> 2), fcol, sum);
     }
   }
-  }  // row tiles of this workgroup
+}
+
+// fp16 output without a plan: the tiles the kernel above skips (more than kLongSteps steps).
+template <int NTL>
+__global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, int64_t mb, int f_tiles,
+                                                                      const uint16_t* __restrict__ A,
+                                                                      const uint16_t* __restrict__ B,
+                                                                      void* __restrict__ C,
+                                                                      const int32_t* __restrict__ indptr,
+                                                                      const int32_t* __restrict__ indices) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int f0 = (int)(blockIdx.x % f_tiles) * (32 * NTL);
+  // A workgroup looks at kLongScan row tiles and works on the long ones among them (most have
+  // none): a workgroup per tile would start tens of thousands that only find out that their tile
+  // is short, each holding 64 KB of LDS while it does.  Its tiles lie a whole grid apart -- long
+  // tiles come in runs (the hub rows of a graph sorted by degree) and would otherwise queue up in
+  // one workgroup.
+  const int64_t io_stride = gridDim.x / f_tiles;
+  // which of them are long: lane k asks for the group range of the k-th tile, all at once
+  uint64_t todo;
+  {
+    const int64_t io = blockIdx.x / f_tiles + (int64_t)lane * io_stride;
+    int64_t groups = 0;
+    if (lane < kLongScan && io < mb) groups = indptr[io + 1] - indptr[io];
+    todo = __ballot((groups * kGroup + 31) / 32 > kLongSteps);
+  }
+  bool used_lds = false;
+  while (todo) {
+    const int k_tile = __ffsll((long long)todo) - 1;
+    todo &= todo - 1;
+    const int64_t io = blockIdx.x / f_tiles + (int64_t)k_tile * io_stride;
+    if (used_lds) __syncthreads();  // the sums of the tile before have been read
+    used_lds = true;
+    tcspmm_long_steps<NTL>(lds, feat, io, f0, 0, tile_steps(indptr, io), A, B, indptr, indices,
+                           [&](int row, int fcol, float sum) {
+                             const _Float16 hv = (_Float16)sum;
+                             static_cast<uint16_t*>(C)[(io * kTile + row) * feat + fcol] = __builtin_bit_cast(uint16_t, hv);
+                           });
+  }
+}
+
+// ---- fp16 output with a plan (stir_tc_plan): the long tiles are listed once, longest first, and
+// cut into pieces of at most kPieceSteps steps, a workgroup of 16 wavefronts each, so that the
+// hub tiles of a power-law graph are spread over many compute units from the start of the launch
+// and no workgroup is started only to find its tile short.  A tile that is one piece is written
+// as fp16 by its workgroup; the pieces of a longer tile leave fp32 partial tiles in the plan's
+// scratch memory, which tcspmm_pieces_sum_kernel adds up and rounds once.
+constexpr int kPieceSteps = 128;
+
+struct TcPiece {
+  int32_t tile, step_begin, step_end;
+  int32_t slot;  // partial tile in the scratch memory, or -1: the piece is the whole tile
+};
+struct TcMulti {
+  int32_t tile, first_slot, pieces, pad;
+};
+
+template <int NTL>
+__global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat, int f_tiles,
+                                                                        const TcPiece* __restrict__ pieces,
+                                                                        const uint16_t* __restrict__ A,
+                                                                        const uint16_t* __restrict__ B,
+                                                                        void* __restrict__ C,
+                                                                        float* __restrict__ scratch,
+                                                                        const int32_t* __restrict__ indptr,
+                                                                        const int32_t* __restrict__ indices) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+  const TcPiece pc = pieces[blockIdx.x / f_tiles];
+  const int f0 = (int)(blockIdx.x % f_tiles) * (32 * NTL);
+  const int64_t io = pc.tile;
+  // a plan made from other contents of indptr: stay inside the tile as it is now
+  const int s_end = min(pc.step_end, tile_steps(indptr, io));
+  if (pc.slot < 0) {
+    tcspmm_long_steps<NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
+                           [&](int row, int fcol, float sum) {
+                             const _Float16 hv = (_Float16)sum;
+                             static_cast<uint16_t*>(C)[(io * kTile + row) * feat + fcol] = __builtin_bit_cast(uint16_t, hv);
+                           });
+  } else {
+    float* part = scratch + (int64_t)pc.slot * kTile * feat;
+    tcspmm_long_steps<NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
+                           [&](int row, int fcol, float sum) { part[(int64_t)row * feat + fcol] = sum; });
+  }
+}
+
+// C[tile] = fp16(sum of the tile's partial tiles); grid (tiles cut into several pieces) x
+// (32 * feat / 1024): a thread owns four consecutive elements (feat is a multiple of 32)
+__global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int feat, int chunks, const TcMulti* __restrict__ multi,
+                                                                const float* __restrict__ scratch,
+                                                                uint16_t* __restrict__ C) {
+  const TcMulti mt = multi[blockIdx.x / chunks];
+  const int64_t elems = (int64_t)kTile * feat;
+  const int64_t e = ((int64_t)(blockIdx.x % chunks) * 256 + threadIdx.x) * 4;
+  if (e >= elems) return;
+  const float* part = scratch + (int64_t)mt.first_slot * elems + e;
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int p0 = 0; p0 < mt.pieces; p0 += 4) {
+    float4 x[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      x[u] = p0 + u < mt.pieces ? *reinterpret_cast<const float4*>(part + (p0 + u) * elems)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sum.x += x[u].x, sum.y += x[u].y, sum.z += x[u].z, sum.w += x[u].w;
+  }
+  const _Float16 h0 = (_Float16)sum.x, h1 = (_Float16)sum.y, h2 = (_Float16)sum.z, h3 = (_Float16)sum.w;
+  uint2 out;
+  out.x = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+  out.y = (uint32_t)__builtin_bit_cast(uint16_t, h2) | ((uint32_t)__builtin_bit_cast(uint16_t, h3) << 16);
+  *reinterpret_cast<uint2*>(C + (int64_t)mt.tile * elems + e) = out;
 }
 
 }  // namespace
@@ -374,3 +460,129 @@ extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size
   STIR_LAUNCH_CHECK();
   return 0;
 }
+
+struct stir_tc_plan {
+  int32_t mb = 0;
+  int device = 0;
+  int64_t n_pieces = 0, n_multi = 0, slots = 0;
+  TcPiece* d_pieces = nullptr;
+  TcMulti* d_multi = nullptr;
+  float* d_scratch = nullptr;  // slots x 32 x feat floats, grown by the launch that needs more
+  size_t scratch_bytes = 0;
+};
+
+extern "C" int stir_tc_plan_destroy(stir_tc_plan* plan) {
+  if (!plan) return 0;
+  if (plan->d_pieces) (void)hipFree(plan->d_pieces);
+  if (plan->d_multi) (void)hipFree(plan->d_multi);
+  if (plan->d_scratch) (void)hipFree(plan->d_scratch);
+  delete plan;
+  return 0;
+}
+
+extern "C" int stir_tc_plan_create(stir_tc_plan** plan, int32_t mb, const int32_t* d_indptr, void* stream) {
+  STIR_REQUIRE(plan, "tc_plan_create: plan is null");
+  STIR_REQUIRE(mb >= 0 && (mb == 0 || d_indptr), "tc_plan_create: bad arguments");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  std::vector<int32_t> ptr(size_t(mb) + 1, 0);
+  if (mb > 0) {
+    STIR_HIP(hipMemcpyAsync(ptr.data(), d_indptr, sizeof(int32_t) * ptr.size(), hipMemcpyDeviceToHost, st));
+    STIR_HIP(hipStreamSynchronize(st));
+  }
+  // the long tiles, longest first (ties in tile order)
+  std::vector<std::pair<int32_t, int32_t>> longs;  // (steps, tile)
+  for (int32_t io = 0; io < mb; ++io) {
+    STIR_REQUIRE(ptr[io] <= ptr[io + 1], "tc_plan_create: indptr decreases at tile %d", io);
+    const int64_t steps = ((int64_t)(ptr[io + 1] - ptr[io]) * kGroup + 31) / 32;
+    if (steps > kLongSteps) longs.emplace_back((int32_t)steps, io);
+  }
+  std::stable_sort(longs.begin(), longs.end(),
+                   [](const std::pair<int32_t, int32_t>& a, const std::pair<int32_t, int32_t>& b) { return a.first > b.first; });
+  std::vector<TcPiece> pieces;
+  std::vector<TcMulti> multi;
+  int64_t slots = 0;
+  for (const auto& lt : longs) {
+    const int32_t steps = lt.first, io = lt.second;
+    const int32_t n = (steps + kPieceSteps - 1) / kPieceSteps;  // pieces of equal length
+    const int32_t len = (steps + n - 1) / n;
+    STIR_REQUIRE(slots + n < (int64_t(1) << 31), "tc_plan_create: too many pieces");
+    if (n > 1) multi.push_back(TcMulti{io, (int32_t)slots, n, 0});
+    for (int32_t p = 0; p < n; ++p)
+      pieces.push_back(TcPiece{io, p * len, std::min(steps, (p + 1) * len), n > 1 ? (int32_t)(slots + p) : -1});
+    if (n > 1) slots += n;
+  }
+  stir_tc_plan* p = new stir_tc_plan();
+  p->mb = mb;
+  p->n_pieces = (int64_t)pieces.size();
+  p->n_multi = (int64_t)multi.size();
+  p->slots = slots;
+  hipError_t e = hipGetDevice(&p->device);
+  if (e == hipSuccess && !pieces.empty()) {
+    e = hipMalloc(reinterpret_cast<void**>(&p->d_pieces), sizeof(TcPiece) * pieces.size());
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(p->d_pieces, pieces.data(), sizeof(TcPiece) * pieces.size(), hipMemcpyHostToDevice, st);
+  }
+  if (e == hipSuccess && !multi.empty()) {
+    e = hipMalloc(reinterpret_cast<void**>(&p->d_multi), sizeof(TcMulti) * multi.size());
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(p->d_multi, multi.data(), sizeof(TcMulti) * multi.size(), hipMemcpyHostToDevice, st);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(st);  // the host vectors go away
+  if (e != hipSuccess) {
+    stir_tc_plan_destroy(p);
+    return stir::fail("tc_plan_create: %s", hipGetErrorString(e));
+  }
+  *plan = p;
+  return 0;
+}
+
+extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t mb, int32_t tile_size, int32_t group_size,
+                                        int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,
+                                        const int32_t* d_indptr, const int32_t* d_indices, void* stream) {
+  STIR_REQUIRE(plan, "tc_spmm_planned: plan is null");
+  STIR_REQUIRE(plan->mb == mb, "tc_spmm_planned: the plan was made for %d row tiles, not %d", plan->mb, mb);
+  STIR_REQUIRE(tile_size == kTile && group_size == kGroup,
+               "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t=32, g=16", tile_size, group_size);
+  STIR_REQUIRE(mb >= 0 && nnzb >= 0, "tc_spmm: bad sizes");
+  STIR_REQUIRE(feat > 0 && feat % 32 == 0, "tc_spmm: feat=%d must be a multiple of 32", feat);
+  if (mb == 0) return 0;
+  STIR_REQUIRE(d_B && d_C && d_indptr && (nnzb == 0 || (d_A && d_indices)), "tc_spmm: null pointer argument");
+  const int f_tiles = (int)stir::ceil_div(feat, kTileF);
+  const int64_t blocks = (int64_t)mb * f_tiles;
+  STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint16_t* A = static_cast<const uint16_t*>(d_A);
+  const uint16_t* B = static_cast<const uint16_t*>(d_B);
+  // the partial tiles of this feature width
+  const size_t need = size_t(plan->slots) * kTile * size_t(feat) * sizeof(float);
+  if (need > plan->scratch_bytes) {
+    if (plan->d_scratch) STIR_HIP(hipFree(plan->d_scratch));
+    plan->d_scratch = nullptr;
+    plan->scratch_bytes = 0;
+    STIR_HIP(hipMalloc(reinterpret_cast<void**>(&plan->d_scratch), need));
+    plan->scratch_bytes = need;
+  }
+  // the tiles of up to kLongSteps steps
+  hipLaunchKernelGGL((tcspmm_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb, f_tiles,
+                     A, B, d_C, d_indptr, d_indices);
+  STIR_LAUNCH_CHECK();
+  if (plan->n_pieces > 0) {
+    constexpr int kLongTF = 32 * kLongNT, kLongWaves = 32 / kLongNT;
+    constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kLongTF * sizeof(uint32_t);
+    const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
+    const int64_t long_blocks = plan->n_pieces * long_f_tiles;
+    STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many pieces for one launch");
+    hipLaunchKernelGGL(tcspmm_pieces_kernel<kLongNT>, dim3((unsigned)long_blocks), dim3(64 * kLongWaves), kLongLds, st,
+                       feat, long_f_tiles, plan->d_pieces, A, B, d_C, plan->d_scratch, d_indptr, d_indices);
+    STIR_LAUNCH_CHECK();
+    if (plan->n_multi > 0) {
+      const int chunks = (int)stir::ceil_div((int64_t)kTile * feat, 1024);
+      STIR_REQUIRE(plan->n_multi * chunks < (int64_t(1) << 31), "tc_spmm: too many partial tiles for one launch");
+      hipLaunchKernelGGL(tcspmm_pieces_sum_kernel, dim3((unsigned)(plan->n_multi * chunks)), dim3(256), 0, st, feat,
+                         chunks, plan->d_multi, plan->d_scratch, static_cast<uint16_t*>(d_C));
+      STIR_LAUNCH_CHECK();
+    }
+  }
+  return 0;
+}
+

@@ -288,7 +288,14 @@ class DBsrMM(_Operator):
 
 
 class TcSpMM(_Operator):
-    """SpMM over the condensed (t x 1 tiles, g per group) format on the matrix cores."""
+    """SpMM over the condensed (t x 1 tiles, g per group) format on the matrix cores.
+
+    With fp16 output (the reference's form) the operator keeps a plan made from the group counts
+    on the first call with a given ``indptr`` array (keyed by its address): the row tiles with many
+    groups, longest first, cut into pieces.  After rewriting ``indptr`` in place call
+    :meth:`invalidate` (the reference's operator reads the array on every call).  The first call
+    of a plan allocates and synchronises the stream, so it cannot be part of a captured graph;
+    later calls can."""
     name = "tcspmm"
 
     def __init__(self, mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=torch.float16):
@@ -296,6 +303,23 @@ class TcSpMM(_Operator):
         self.t, self.g, self.brows = int(tile_size), int(group_size), int(num_b_rows)
         self.out_dtype = out_dtype
         self.L = _lib.lib()
+        self._plan, self._key = None, None
+
+    def _drop_plan(self):
+        if self._plan is not None:
+            self.L.stir_tc_plan_destroy(self._plan)
+            self._plan = None
+
+    def invalidate(self):
+        """Forget the plan made from the contents ``indptr`` had at the last call."""
+        self._drop_plan()
+        self._key = None
+
+    def __del__(self):
+        try:
+            self._drop_plan()
+        except Exception:
+            pass
 
     def __call__(self, *args):
         f16, i32 = torch.float16, torch.int32
@@ -304,9 +328,20 @@ class TcSpMM(_Operator):
                                  ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb * self.g)])
         a, b, c, indptr, indices = args
         with torch.cuda.device(dev):
-            _lib.check(self.L.stir_tc_spmm_f16(_DT[self.out_dtype], self.mb, self.t, self.g, self.feat,
-                                               self.nnzb, _ptr(a), _ptr(b), _ptr(c), _ptr(indptr),
-                                               _ptr(indices), _stream()))
+            if self.out_dtype != torch.float16 or (self.t, self.g) != (32, 16):
+                _lib.check(self.L.stir_tc_spmm_f16(_DT[self.out_dtype], self.mb, self.t, self.g, self.feat,
+                                                   self.nnzb, _ptr(a), _ptr(b), _ptr(c), _ptr(indptr),
+                                                   _ptr(indices), _stream()))
+                return
+            key = (dev, indptr.data_ptr())
+            if key != self._key:
+                self._drop_plan()
+                plan = ctypes.c_void_p()
+                _lib.check(self.L.stir_tc_plan_create(ctypes.byref(plan), self.mb, _ptr(indptr), _stream()))
+                self._plan, self._key = plan, key
+            _lib.check(self.L.stir_tc_spmm_f16_planned(self._plan, self.mb, self.t, self.g, self.feat, self.nnzb,
+                                                       _ptr(a), _ptr(b), _ptr(c), _ptr(indptr), _ptr(indices),
+                                                       _stream()))
 
 
 class Rgms(_Operator):

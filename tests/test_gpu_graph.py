@@ -94,3 +94,28 @@ def test_graph_hyb_and_rgms_tiles(dev):
         # bit-equal except in the few tiles that are cut into units and meet in atomics
         assert torch.allclose(y, y_want, rtol=1e-6, atol=1e-6), f"rgms replay {k}"
         assert float((y != y_want).float().mean()) < 0.01
+
+
+def test_graph_tcspmm_with_plan(dev):
+    """TC-SpMM with fp16 output: the plan and its memory for partial tiles exist after the eager
+    first call, so the three launches of a later call can be recorded."""
+    g = datasets.config2()
+    gptr, tiles, mask = st.condense(g["indptr"], g["indices"], 32, 16)
+    mb, nnzb, feat = len(gptr) - 1, tiles.shape[0], 64
+    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    a, b = t(mask.astype(np.float16).ravel()), torch.randn(g["n"] * feat, device=dev).half()
+    gp, ti = t(gptr), t(tiles.ravel())
+    f = ops.build_tcspmm(mb, nnzb, feat, 32, 16, g["n"], torch.float16)
+    want = torch.empty(mb * 32 * feat, dtype=torch.float16, device=dev)
+    f(a, b, want, gp, ti)  # makes the plan
+    torch.cuda.synchronize()
+    c = torch.zeros_like(want)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        f(a, b, c, gp, ti)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        f(a, b, c, gp, ti)
+    _replays(dev, graph, c, want, lambda: c.fill_(1.0))

@@ -4,13 +4,16 @@ import numpy as np
 import pytest
 import torch
 
+import ctypes
+
 import oracle
 import sparsetir_amd as st
-from sparsetir_amd import datasets, ops
+from sparsetir_amd import _lib, datasets, ops
 from sparsetir_amd._lib import SparseTIRError
 from helpers import random_csr, spmm_f64
 
 pytestmark = pytest.mark.gpu
+STIR_F16 = 0  # include/sparsetir_amd.h
 
 
 def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0):
@@ -35,16 +38,33 @@ def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0):
                 rl, sl = np.nonzero(mask[grp])
                 a[grp, rl, sl] = dense[tile * t + rl, tiles[grp, sl]]
     td = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
-    c = torch.full((mb * t * feat,), float("nan"), dtype=out_dtype, device=dev)
-    f = ops.build_tcspmm(mb, tiles.shape[0], feat, t, g, n, out_dtype)
-    f(td(a.ravel()), td(x.ravel()), c, td(gptr), td(tiles.ravel()))
-    torch.cuda.synchronize()
-    got = c.float().cpu().numpy().reshape(mb * t, feat)
     want = spmm_f64(indptr, indices, vals, x.astype(np.float32))
     scale = spmm_f64(indptr, indices, np.abs(vals), np.abs(x.astype(np.float32)))
-    assert np.all(got[m:] == 0)  # rows added to fill the last tile
     bound = 1e-5 * scale + (2e-2 * np.abs(want) if out_dtype == torch.float16 else 0) + 1e-30
-    assert np.all(np.abs(got[:m] - want) <= bound)
+    d_a, d_x, d_ptr, d_tiles = td(a.ravel()), td(x.ravel()), td(gptr), td(tiles.ravel())
+
+    def check(c, what):
+        torch.cuda.synchronize()
+        got = c.float().cpu().numpy().reshape(mb * t, feat)
+        assert np.all(got[m:] == 0), what  # rows added to fill the last tile
+        assert np.all(np.abs(got[:m] - want) <= bound), what
+
+    # the built operator: with fp16 output it makes a plan from the group counts at its first call
+    c = torch.full((mb * t * feat,), float("nan"), dtype=out_dtype, device=dev)
+    f = ops.build_tcspmm(mb, tiles.shape[0], feat, t, g, n, out_dtype)
+    f(d_a, d_x, c, d_ptr, d_tiles)
+    check(c, "operator, first call")
+    if out_dtype == torch.float16:
+        c.fill_(float("nan"))
+        f(d_a, d_x, c, d_ptr, d_tiles)
+        check(c, "operator, with its plan")
+        # and the entry point that takes no plan
+        c.fill_(float("nan"))
+        vp = lambda v: ctypes.c_void_p(v.data_ptr() if v.numel() else 0)
+        _lib.check(_lib.lib().stir_tc_spmm_f16(STIR_F16, mb, t, g, feat, tiles.shape[0], vp(d_a), vp(d_x), vp(c),
+                                               vp(d_ptr), vp(d_tiles),
+                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        check(c, "without a plan")
 
 
 @pytest.mark.parametrize("feat", [32, 64, 128, 256, 160])
@@ -98,3 +118,71 @@ def test_tcspmm_every_tile_long(dev, tiles, feat, out_dtype):
     m, n = tiles * 32 - 5, 3000
     indptr, indices = random_csr(m, n, 40 * m, tiles, skew=0.0)
     _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=tiles)
+
+
+def test_tcspmm_plan_entry_points(dev):
+    """stir_tc_plan_create / stir_tc_spmm_f16_planned through the C ABI: one plan used at three
+    feature widths in turn (its memory for partial tiles grows with the widest), a plan for a
+    matrix without long tiles, the row-tile count checked against the plan's, and an in-place
+    change of the group counts followed by the operator's invalidate()."""
+    L = _lib.lib()
+    t, g = 32, 16
+    m, n = 300, 12000
+    rng = np.random.default_rng(41)
+    deg = rng.integers(0, 10, m)
+    deg[5], deg[130], deg[131], deg[299] = 7000, 2200, 300, 4100   # tiles of 219, 76 and 129 steps
+    indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    indices = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
+    gptr, tiles, mask = st.condense(indptr, indices, t, g)
+    mb, nnzb = len(gptr) - 1, tiles.shape[0]
+    td = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
+    vp = lambda v: ctypes.c_void_p(v.data_ptr() if v.numel() else 0)
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    d_a, d_ptr, d_tiles = td(mask.astype(np.float16).ravel()), td(gptr), td(tiles.ravel())
+    plan = ctypes.c_void_p()
+    _lib.check(L.stir_tc_plan_create(ctypes.byref(plan), mb, vp(d_ptr), stream()))
+    try:
+        for feat in (64, 256, 96, 256):
+            x = rng.standard_normal((n, feat)).astype(np.float16)
+            c = torch.full((mb * t * feat,), float("nan"), dtype=torch.float16, device=dev)
+            _lib.check(L.stir_tc_spmm_f16_planned(plan, mb, t, g, feat, nnzb, vp(d_a), vp(td(x.ravel())), vp(c),
+                                                  vp(d_ptr), vp(d_tiles), stream()))
+            torch.cuda.synchronize()
+            got = c.float().cpu().numpy().reshape(mb * t, feat)[:m]
+            ones = np.ones(len(indices), np.float32)
+            want = spmm_f64(indptr, indices, ones, x.astype(np.float32))
+            scale = spmm_f64(indptr, indices, ones, np.abs(x.astype(np.float32)))
+            assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), feat
+        assert L.stir_tc_spmm_f16_planned(plan, mb + 1, t, g, 64, nnzb, vp(d_a), vp(d_a), vp(d_a), vp(d_ptr),
+                                          vp(d_tiles), stream()) == -1
+        assert b"row tiles" in L.stir_last_error()
+    finally:
+        L.stir_tc_plan_destroy(plan)
+
+    # no long tile at all: the plan is empty and the launch is the first kernel alone
+    indptr2, indices2 = random_csr(200, 500, 1500, 7, skew=0.0)
+    _run(dev, indptr2, indices2, 500, 64, weighted=False, out_dtype=torch.float16)
+
+    # the operator after its indptr array was rewritten in place: invalidate() makes a new plan
+    feat = 64
+    x = rng.standard_normal((n, feat)).astype(np.float16)
+    f = ops.build_tcspmm(mb, nnzb, feat, t, g, n, torch.float16)
+    c = torch.zeros(mb * t * feat, dtype=torch.float16, device=dev)
+    f(d_a, td(x.ravel()), c, d_ptr, d_tiles)
+    # the rows of tile 0 (the longest) and of tile 6 change places: the same groups, other tiles long
+    rows = [*range(192, 224), *range(32, 192), *range(0, 32), *range(224, m)]
+    indptr3 = np.concatenate([[0], np.cumsum(deg[rows])]).astype(np.int32)
+    indices3 = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in rows])
+    gptr3, tiles3, mask3 = st.condense(indptr3, indices3, t, g)
+    assert tiles3.shape[0] == nnzb  # the same number of groups: the arrays can be rewritten in place
+    d_ptr.copy_(td(gptr3)), d_tiles.copy_(td(tiles3.ravel())), d_a.copy_(td(mask3.astype(np.float16).ravel()))
+    f.invalidate()
+    c.fill_(float("nan"))
+    f(d_a, td(x.ravel()), c, d_ptr, d_tiles)
+    torch.cuda.synchronize()
+    got = c.float().cpu().numpy().reshape(mb * t, feat)[:m]
+    ones = np.ones(len(indices3), np.float32)
+    want = spmm_f64(indptr3, indices3, ones, x.astype(np.float32))
+    scale = spmm_f64(indptr3, indices3, ones, np.abs(x.astype(np.float32)))
+    assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30)
+
