@@ -301,12 +301,12 @@ int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t g
                      const int32_t* d_indptr, const int32_t* d_indices, void* stream);
 
 /*
- * The same operator with fp16 output and a plan made once from the group counts (the reference
+ * The same operator with a plan made once from the group counts (the reference
  * has no counterpart: its built operator, examples/spmm/bench_tc_spmm.py:650-656, reads nothing
  * ahead of the launch).  stir_tc_plan_create reads d_indptr (mb+1 entries) on `stream`,
  * synchronises it, and lists the row tiles of more than 16 steps (32 gathered rows each), longest
- * first, cut into pieces of at most 64 steps.  stir_tc_spmm_f16_planned then takes the arguments
- * of stir_tc_spmm_f16 (out_dtype is STIR_F16): the short tiles as there, then one workgroup per
+ * first, cut into pieces of at most 128 steps.  stir_tc_spmm_f16_planned then takes the arguments
+ * of stir_tc_spmm_f16: the short tiles as there, then one workgroup per
  * piece -- none is started only to find its tile short, and the hub tiles of a power-law graph
  * are spread over many compute units from the start of the launch -- and, for the tiles of several
  * pieces, a launch that adds their fp32 partial tiles and rounds once (the sums are those of
@@ -317,9 +317,9 @@ int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t g
  */
 typedef struct stir_tc_plan stir_tc_plan;
 int stir_tc_plan_create(stir_tc_plan** plan, int32_t mb, const int32_t* d_indptr, void* stream);
-int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t mb, int32_t tile_size, int32_t group_size,
-                             int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,
-                             const int32_t* d_indptr, const int32_t* d_indices, void* stream);
+int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, int32_t mb, int32_t tile_size,
+                             int32_t group_size, int32_t feat, int64_t nnzb, const void* d_A, const void* d_B,
+                             void* d_C, const int32_t* d_indptr, const int32_t* d_indices, void* stream);
 int stir_tc_plan_destroy(stir_tc_plan* plan);
 
 /*

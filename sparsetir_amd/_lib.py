@@ -50,7 +50,7 @@ SIGNATURES = {
     "stir_dbsr_spmm": (I32, [I32, I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP, VP]),
     "stir_tc_spmm_f16": (I32, [I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
     "stir_tc_plan_create": (I32, [VP, I32, VP, VP]),
-    "stir_tc_spmm_f16_planned": (I32, [VP, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
+    "stir_tc_spmm_f16_planned": (I32, [VP, I32, I32, I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
     "stir_tc_plan_destroy": (I32, [VP]),
     "stir_rgms_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),

@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void tcspmm_clear_long_kernel(int feat, int64_
 
 // OUT: 0 = fp16 output, 1 = fp32 output.  SPLIT: grid is (mb * f_tiles, kSplit); the units of a
 // long tile take equal shares of its steps and add with atomics, unit 0 of a short tile stores.
-template <int OUT, bool SPLIT>
+template <int OUT, bool SPLIT, bool SKIP_LONG = (OUT == 0)>
 __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f_tiles,
                                                      const uint16_t* __restrict__ A,
                                                      const uint16_t* __restrict__ B, void* __restrict__ C,
@@ -90,8 +90,8 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   const int64_t rows_total = (g_end - g_begin) * kGroup;  // gathered rows of B for this tile
   const int steps = (int)((rows_total + 31) / 32);
   const int32_t* rowlist = indices + g_begin * kGroup;
-  if constexpr (OUT == 0) {
-    if (steps > kLongSteps) return;  // left to tcspmm_long_kernel; uniform over the workgroup
+  if constexpr (SKIP_LONG) {
+    if (steps > kLongSteps) return;  // left to the launch for long tiles; uniform over the workgroup
   }
   int it_begin = 0, it_end = steps;
   bool add = false;
@@ -365,7 +365,7 @@ struct TcMulti {
   int32_t tile, first_slot, pieces, pad;
 };
 
-template <int NTL>
+template <int NTL, int OUT>
 __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat, int f_tiles,
                                                                         const TcPiece* __restrict__ pieces,
                                                                         const uint16_t* __restrict__ A,
@@ -383,8 +383,13 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat
   if (pc.slot < 0) {
     tcspmm_long_steps<NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
                            [&](int row, int fcol, float sum) {
-                             const _Float16 hv = (_Float16)sum;
-                             static_cast<uint16_t*>(C)[(io * kTile + row) * feat + fcol] = __builtin_bit_cast(uint16_t, hv);
+                             const int64_t off = (io * kTile + row) * feat + fcol;
+                             if constexpr (OUT == 1) {
+                               static_cast<float*>(C)[off] = sum;
+                             } else {
+                               const _Float16 hv = (_Float16)sum;
+                               static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
+                             }
                            });
   } else {
     float* part = scratch + (int64_t)pc.slot * kTile * feat;
@@ -395,9 +400,10 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat
 
 // C[tile] = fp16(sum of the tile's partial tiles); grid (tiles cut into several pieces) x
 // (32 * feat / 1024): a thread owns four consecutive elements (feat is a multiple of 32)
+template <int OUT>
 __global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int feat, int chunks, const TcMulti* __restrict__ multi,
                                                                 const float* __restrict__ scratch,
-                                                                uint16_t* __restrict__ C) {
+                                                                void* __restrict__ C) {
   const TcMulti mt = multi[blockIdx.x / chunks];
   const int64_t elems = (int64_t)kTile * feat;
   const int64_t e = ((int64_t)(blockIdx.x % chunks) * 256 + threadIdx.x) * 4;
@@ -413,11 +419,15 @@ __global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int feat, int ch
 #pragma unroll
     for (int u = 0; u < 4; ++u) sum.x += x[u].x, sum.y += x[u].y, sum.z += x[u].z, sum.w += x[u].w;
   }
-  const _Float16 h0 = (_Float16)sum.x, h1 = (_Float16)sum.y, h2 = (_Float16)sum.z, h3 = (_Float16)sum.w;
-  uint2 out;
-  out.x = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
-  out.y = (uint32_t)__builtin_bit_cast(uint16_t, h2) | ((uint32_t)__builtin_bit_cast(uint16_t, h3) << 16);
-  *reinterpret_cast<uint2*>(C + (int64_t)mt.tile * elems + e) = out;
+  if constexpr (OUT == 1) {
+    *reinterpret_cast<float4*>(static_cast<float*>(C) + (int64_t)mt.tile * elems + e) = sum;
+  } else {
+    const _Float16 h0 = (_Float16)sum.x, h1 = (_Float16)sum.y, h2 = (_Float16)sum.z, h3 = (_Float16)sum.w;
+    uint2 out;
+    out.x = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+    out.y = (uint32_t)__builtin_bit_cast(uint16_t, h2) | ((uint32_t)__builtin_bit_cast(uint16_t, h3) << 16);
+    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(C) + (int64_t)mt.tile * elems + e) = out;
+  }
 }
 
 }  // namespace
@@ -536,10 +546,12 @@ extern "C" int stir_tc_plan_create(stir_tc_plan** plan, int32_t mb, const int32_
   return 0;
 }
 
-extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t mb, int32_t tile_size, int32_t group_size,
-                                        int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,
-                                        const int32_t* d_indptr, const int32_t* d_indices, void* stream) {
+extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, int32_t mb, int32_t tile_size,
+                                        int32_t group_size, int32_t feat, int64_t nnzb, const void* d_A,
+                                        const void* d_B, void* d_C, const int32_t* d_indptr,
+                                        const int32_t* d_indices, void* stream) {
   STIR_REQUIRE(plan, "tc_spmm_planned: plan is null");
+  STIR_REQUIRE(out_dtype == STIR_F16 || out_dtype == STIR_F32, "tc_spmm: out_dtype must be STIR_F16 or STIR_F32");
   STIR_REQUIRE(plan->mb == mb, "tc_spmm_planned: the plan was made for %d row tiles, not %d", plan->mb, mb);
   STIR_REQUIRE(tile_size == kTile && group_size == kGroup,
                "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t=32, g=16", tile_size, group_size);
@@ -563,8 +575,13 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t mb, int32_t 
     plan->scratch_bytes = need;
   }
   // the tiles of up to kLongSteps steps
-  hipLaunchKernelGGL((tcspmm_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb, f_tiles,
-                     A, B, d_C, d_indptr, d_indices);
+  const bool out32 = out_dtype == STIR_F32;
+  if (out32)
+    hipLaunchKernelGGL((tcspmm_kernel<1, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
+                       f_tiles, A, B, d_C, d_indptr, d_indices);
+  else
+    hipLaunchKernelGGL((tcspmm_kernel<0, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
+                       f_tiles, A, B, d_C, d_indptr, d_indices);
   STIR_LAUNCH_CHECK();
   if (plan->n_pieces > 0) {
     constexpr int kLongTF = 32 * kLongNT, kLongWaves = 32 / kLongNT;
@@ -572,14 +589,24 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t mb, int32_t 
     const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
     const int64_t long_blocks = plan->n_pieces * long_f_tiles;
     STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many pieces for one launch");
-    hipLaunchKernelGGL(tcspmm_pieces_kernel<kLongNT>, dim3((unsigned)long_blocks), dim3(64 * kLongWaves), kLongLds, st,
-                       feat, long_f_tiles, plan->d_pieces, A, B, d_C, plan->d_scratch, d_indptr, d_indices);
+    if (out32)
+      hipLaunchKernelGGL((tcspmm_pieces_kernel<kLongNT, 1>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
+                         kLongLds, st, feat, long_f_tiles, plan->d_pieces, A, B, d_C, plan->d_scratch, d_indptr,
+                         d_indices);
+    else
+      hipLaunchKernelGGL((tcspmm_pieces_kernel<kLongNT, 0>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
+                         kLongLds, st, feat, long_f_tiles, plan->d_pieces, A, B, d_C, plan->d_scratch, d_indptr,
+                         d_indices);
     STIR_LAUNCH_CHECK();
     if (plan->n_multi > 0) {
       const int chunks = (int)stir::ceil_div((int64_t)kTile * feat, 1024);
       STIR_REQUIRE(plan->n_multi * chunks < (int64_t(1) << 31), "tc_spmm: too many partial tiles for one launch");
-      hipLaunchKernelGGL(tcspmm_pieces_sum_kernel, dim3((unsigned)(plan->n_multi * chunks)), dim3(256), 0, st, feat,
-                         chunks, plan->d_multi, plan->d_scratch, static_cast<uint16_t*>(d_C));
+      if (out32)
+        hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<1>, dim3((unsigned)(plan->n_multi * chunks)), dim3(256), 0, st, feat,
+                           chunks, plan->d_multi, plan->d_scratch, d_C);
+      else
+        hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<0>, dim3((unsigned)(plan->n_multi * chunks)), dim3(256), 0, st, feat,
+                           chunks, plan->d_multi, plan->d_scratch, d_C);
       STIR_LAUNCH_CHECK();
     }
   }

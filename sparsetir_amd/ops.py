@@ -290,9 +290,9 @@ class DBsrMM(_Operator):
 class TcSpMM(_Operator):
     """SpMM over the condensed (t x 1 tiles, g per group) format on the matrix cores.
 
-    With fp16 output (the reference's form) the operator keeps a plan made from the group counts
-    on the first call with a given ``indptr`` array (keyed by its address): the row tiles with many
-    groups, longest first, cut into pieces.  After rewriting ``indptr`` in place call
+    The operator keeps a plan made from the group counts on the first call with a given ``indptr``
+    array (keyed by its address): the row tiles with many groups, longest first, cut into pieces
+    that are summed in fp32 and rounded once.  After rewriting ``indptr`` in place call
     :meth:`invalidate` (the reference's operator reads the array on every call).  The first call
     of a plan allocates and synchronises the stream, so it cannot be part of a captured graph;
     later calls can."""
@@ -328,7 +328,7 @@ class TcSpMM(_Operator):
                                  ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb * self.g)])
         a, b, c, indptr, indices = args
         with torch.cuda.device(dev):
-            if self.out_dtype != torch.float16 or (self.t, self.g) != (32, 16):
+            if (self.t, self.g) != (32, 16):  # refused by the library with its own message
                 _lib.check(self.L.stir_tc_spmm_f16(_DT[self.out_dtype], self.mb, self.t, self.g, self.feat,
                                                    self.nnzb, _ptr(a), _ptr(b), _ptr(c), _ptr(indptr),
                                                    _ptr(indices), _stream()))
@@ -339,7 +339,8 @@ class TcSpMM(_Operator):
                 plan = ctypes.c_void_p()
                 _lib.check(self.L.stir_tc_plan_create(ctypes.byref(plan), self.mb, _ptr(indptr), _stream()))
                 self._plan, self._key = plan, key
-            _lib.check(self.L.stir_tc_spmm_f16_planned(self._plan, self.mb, self.t, self.g, self.feat, self.nnzb,
+            _lib.check(self.L.stir_tc_spmm_f16_planned(self._plan, _DT[self.out_dtype], self.mb, self.t, self.g,
+                                                       self.feat, self.nnzb,
                                                        _ptr(a), _ptr(b), _ptr(c), _ptr(indptr), _ptr(indices),
                                                        _stream()))
 

@@ -13,7 +13,7 @@ from sparsetir_amd._lib import SparseTIRError
 from helpers import random_csr, spmm_f64
 
 pytestmark = pytest.mark.gpu
-STIR_F16 = 0  # include/sparsetir_amd.h
+STIR_F16, STIR_F32 = 0, 2  # include/sparsetir_amd.h
 
 
 def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0):
@@ -49,22 +49,21 @@ def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0):
         assert np.all(got[m:] == 0), what  # rows added to fill the last tile
         assert np.all(np.abs(got[:m] - want) <= bound), what
 
-    # the built operator: with fp16 output it makes a plan from the group counts at its first call
+    # the built operator: it makes a plan from the group counts at its first call
     c = torch.full((mb * t * feat,), float("nan"), dtype=out_dtype, device=dev)
     f = ops.build_tcspmm(mb, tiles.shape[0], feat, t, g, n, out_dtype)
     f(d_a, d_x, c, d_ptr, d_tiles)
     check(c, "operator, first call")
-    if out_dtype == torch.float16:
-        c.fill_(float("nan"))
-        f(d_a, d_x, c, d_ptr, d_tiles)
-        check(c, "operator, with its plan")
-        # and the entry point that takes no plan
-        c.fill_(float("nan"))
-        vp = lambda v: ctypes.c_void_p(v.data_ptr() if v.numel() else 0)
-        _lib.check(_lib.lib().stir_tc_spmm_f16(STIR_F16, mb, t, g, feat, tiles.shape[0], vp(d_a), vp(d_x), vp(c),
-                                               vp(d_ptr), vp(d_tiles),
-                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
-        check(c, "without a plan")
+    c.fill_(float("nan"))
+    f(d_a, d_x, c, d_ptr, d_tiles)
+    check(c, "operator, with its plan")
+    # and the entry point that takes no plan
+    c.fill_(float("nan"))
+    vp = lambda v: ctypes.c_void_p(v.data_ptr() if v.numel() else 0)
+    _lib.check(_lib.lib().stir_tc_spmm_f16(STIR_F16 if out_dtype == torch.float16 else STIR_F32, mb, t, g, feat,
+                                           tiles.shape[0], vp(d_a), vp(d_x), vp(c), vp(d_ptr), vp(d_tiles),
+                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    check(c, "without a plan")
 
 
 @pytest.mark.parametrize("feat", [32, 64, 128, 256, 160])
@@ -142,20 +141,25 @@ def test_tcspmm_plan_entry_points(dev):
     plan = ctypes.c_void_p()
     _lib.check(L.stir_tc_plan_create(ctypes.byref(plan), mb, vp(d_ptr), stream()))
     try:
-        for feat in (64, 256, 96, 256):
+        for feat, dt in ((64, torch.float16), (256, torch.float32), (96, torch.float16), (256, torch.float16)):
             x = rng.standard_normal((n, feat)).astype(np.float16)
-            c = torch.full((mb * t * feat,), float("nan"), dtype=torch.float16, device=dev)
-            _lib.check(L.stir_tc_spmm_f16_planned(plan, mb, t, g, feat, nnzb, vp(d_a), vp(td(x.ravel())), vp(c),
-                                                  vp(d_ptr), vp(d_tiles), stream()))
+            c = torch.full((mb * t * feat,), float("nan"), dtype=dt, device=dev)
+            _lib.check(L.stir_tc_spmm_f16_planned(plan, STIR_F16 if dt == torch.float16 else STIR_F32, mb, t, g, feat,
+                                                  nnzb, vp(d_a), vp(td(x.ravel())), vp(c), vp(d_ptr), vp(d_tiles),
+                                                  stream()))
             torch.cuda.synchronize()
             got = c.float().cpu().numpy().reshape(mb * t, feat)[:m]
             ones = np.ones(len(indices), np.float32)
             want = spmm_f64(indptr, indices, ones, x.astype(np.float32))
             scale = spmm_f64(indptr, indices, ones, np.abs(x.astype(np.float32)))
-            assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30), feat
-        assert L.stir_tc_spmm_f16_planned(plan, mb + 1, t, g, 64, nnzb, vp(d_a), vp(d_a), vp(d_a), vp(d_ptr),
-                                          vp(d_tiles), stream()) == -1
+            rtol = 2e-2 if dt == torch.float16 else 0.0
+            assert np.all(np.abs(got - want) <= rtol * np.abs(want) + 1e-5 * scale + 1e-30), (feat, dt)
+        assert L.stir_tc_spmm_f16_planned(plan, STIR_F16, mb + 1, t, g, 64, nnzb, vp(d_a), vp(d_a), vp(d_a),
+                                          vp(d_ptr), vp(d_tiles), stream()) == -1
         assert b"row tiles" in L.stir_last_error()
+        assert L.stir_tc_spmm_f16_planned(plan, 1, mb, t, g, 64, nnzb, vp(d_a), vp(d_a), vp(d_a), vp(d_ptr),
+                                          vp(d_tiles), stream()) == -1  # bf16 output does not exist
+        assert b"out_dtype" in L.stir_last_error()
     finally:
         L.stir_tc_plan_destroy(plan)
 
