@@ -292,8 +292,10 @@ class TcSpMM(_Operator):
 
     The operator keeps a plan made from the group counts on the first call with a given ``indptr``
     array (keyed by its address): the row tiles with many groups, longest first, cut into pieces
-    that are summed in fp32 and rounded once.  After rewriting ``indptr`` in place call
-    :meth:`invalidate` (the reference's operator reads the array on every call).  The first call
+    that are summed in fp32 and rounded once.  In-place changes of ``indptr`` made through torch
+    are noticed (its version counter is part of the key); after rewriting it by other means (a
+    kernel of the caller's, another library) call :meth:`invalidate` -- the reference's operator
+    reads the array on every call.  The first call
     of a plan allocates and synchronises the stream, so it cannot be part of a captured graph;
     later calls can."""
     name = "tcspmm"
@@ -333,7 +335,8 @@ class TcSpMM(_Operator):
                                                    self.nnzb, _ptr(a), _ptr(b), _ptr(c), _ptr(indptr),
                                                    _ptr(indices), _stream()))
                 return
-            key = (dev, indptr.data_ptr())
+            # torch counts the in-place changes it knows of: rewriting indptr with torch calls makes a new plan
+            key = (dev, indptr.data_ptr(), indptr._version)
             if key != self._key:
                 self._drop_plan()
                 plan = ctypes.c_void_p()

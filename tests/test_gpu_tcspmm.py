@@ -179,14 +179,34 @@ def test_tcspmm_plan_entry_points(dev):
     indices3 = np.concatenate([indices[indptr[r]:indptr[r + 1]] for r in rows])
     gptr3, tiles3, mask3 = st.condense(indptr3, indices3, t, g)
     assert tiles3.shape[0] == nnzb  # the same number of groups: the arrays can be rewritten in place
+    ones = np.ones(len(indices3), np.float32)
+    want3 = spmm_f64(indptr3, indices3, ones, x.astype(np.float32))
+    scale3 = spmm_f64(indptr3, indices3, ones, np.abs(x.astype(np.float32)))
+
+    def agrees():
+        c.fill_(float("nan"))
+        f(d_a, td(x.ravel()), c, d_ptr, d_tiles)
+        torch.cuda.synchronize()
+        got = c.float().cpu().numpy().reshape(mb * t, feat)[:m]
+        return np.all(np.abs(got - want3) <= 2e-2 * np.abs(want3) + 1e-5 * scale3 + 1e-30)
+
+    # rewritten through torch: the operator notices by itself
     d_ptr.copy_(td(gptr3)), d_tiles.copy_(td(tiles3.ravel())), d_a.copy_(td(mask3.astype(np.float16).ravel()))
+    assert agrees()
+    # rewritten behind torch's back (a plain hipMemcpy to the array's address): invalidate() is the
+    # caller's part
+    import ctypes as ct
+    hip = ct.CDLL("libamdhip64.so")
+    back = np.ascontiguousarray(gptr)
+    assert hip.hipMemcpy(ct.c_void_p(d_ptr.data_ptr()), back.ctypes.data_as(ct.c_void_p), ct.c_size_t(back.nbytes), 1) == 0
+    d_tiles.copy_(td(tiles.ravel())), d_a.copy_(td(mask.astype(np.float16).ravel()))
     f.invalidate()
     c.fill_(float("nan"))
     f(d_a, td(x.ravel()), c, d_ptr, d_tiles)
     torch.cuda.synchronize()
     got = c.float().cpu().numpy().reshape(mb * t, feat)[:m]
-    ones = np.ones(len(indices3), np.float32)
-    want = spmm_f64(indptr3, indices3, ones, x.astype(np.float32))
-    scale = spmm_f64(indptr3, indices3, ones, np.abs(x.astype(np.float32)))
+    ones = np.ones(len(indices), np.float32)
+    want = spmm_f64(indptr, indices, ones, x.astype(np.float32))
+    scale = spmm_f64(indptr, indices, ones, np.abs(x.astype(np.float32)))
     assert np.all(np.abs(got - want) <= 2e-2 * np.abs(want) + 1e-5 * scale + 1e-30)
 
