@@ -565,6 +565,10 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* B = static_cast<const uint16_t*>(d_B);
+  // the sums of the partial tiles leave four to a thread, as one 8- or 16-byte store
+  const bool out32 = out_dtype == STIR_F32;
+  STIR_REQUIRE(plan->n_multi == 0 || reinterpret_cast<uintptr_t>(d_C) % (out32 ? 16 : 8) == 0,
+               "tc_spmm: C must be %d-byte aligned", out32 ? 16 : 8);
   // the partial tiles of this feature width
   const size_t need = size_t(plan->slots) * kTile * size_t(feat) * sizeof(float);
   if (need > plan->scratch_bytes) {
@@ -575,7 +579,6 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
     plan->scratch_bytes = need;
   }
   // the tiles of up to kLongSteps steps
-  const bool out32 = out_dtype == STIR_F32;
   if (out32)
     hipLaunchKernelGGL((tcspmm_kernel<1, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
                        f_tiles, A, B, d_C, d_indptr, d_indices);
