@@ -37,8 +37,10 @@ struct TileLds {
 
 // Phase 1: S[r, :] = sum over the edges p in [range(r).x, range(r).y) of A[p] * X[cols[p], :] for
 // the 32 rows of the tile (zero for r >= nrows).  A row belongs to one lane group (G lanes, one
-// float4 each): group g takes rows g, g + NG, ..., and requests the first edges of up to eight
-// of its rows together before it adds anything.  Rows with more than kLongRow edges are left to
+// float4 each): group g takes rows g, g + NG, ...; the columns and weights of a row arrive a
+// chunk of at least 16 edges at a time, fetched by the group's lanes side by side and handed round
+// with cross-lane reads, the first chunks of up to eight of its rows requested together before it
+// adds anything.  Rows with more than kLongRow edges are left to
 // a second pass in which all lane groups share the row's edges and combine their partial sums
 // with cross-lane adds.  Nothing here is atomic (LDS float atomics run at a fraction of the rate
 // of plain LDS stores on this chip), and every S entry is written exactly once.
@@ -49,75 +51,88 @@ __device__ __forceinline__ void accumulate_rows(float* S, const float* __restric
                                                 const int32_t* __restrict__ cols, int fin, int lane, int nrows,
                                                 Range range) {
   constexpr int G = FP / 4, NG = kWave / G;
-  constexpr int RPG = kTileRows / NG;       // rows per lane group
-  constexpr int RB = RPG < 8 ? RPG : 8;     // rows whose first edges are in flight together
-  constexpr int U0 = 8 / RB;                // first edges per row requested up front
-  constexpr int U = 4;                      // edges per step after that
+  constexpr int RPG = kTileRows / NG;        // rows per lane group
+  constexpr int PER = G >= 16 ? 1 : 16 / G;  // edges whose column and weight one lane fetches per chunk
+  constexpr int CHUNK = G * PER;             // edges of a row per chunk (at least 16)
+  constexpr int CH = G < 4 ? G : 4;          // gathers in flight per lane (8 cost a wavefront of occupancy: 165 against 158 us)
   const int g = lane / G, gl = lane % G;
+  // Every gather is unconditional (no register cleared first, no lane branches): an edge of weight
+  // zero -- the padding of an ELL row, column 0 -- fetches row 0 of X and adds 0 * X[0, :], as the
+  // reference's kernel does; lanes whose features lie beyond feat_in fetch the first features
+  // instead and their sums are replaced by zeros before they are stored.
   const bool chunk_live = 4 * gl < fin;
-  const float* Xl = X + 4 * gl;
-  auto ld_x = [&](int c, float w) {
-    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (w != 0.f && chunk_live) x = *reinterpret_cast<const float4*>(Xl + (int64_t)c * fin);
-    return x;
-  };
+  const float* Xl = X + (chunk_live ? 4 * gl : 0);
+  auto ld_x = [&](int c, float) { return *reinterpret_cast<const float4*>(Xl + (int64_t)c * fin); };
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
   auto fma4 = [](float4& acc, float w, const float4& x) {
     acc.x += w * x.x, acc.y += w * x.y, acc.z += w * x.z, acc.w += w * x.w;
   };
+  // The edges of a row are fetched by the row's lane group, one chunk per round trip (lane gl takes
+  // edges gl, gl + G, ... of the chunk: coalesced), and handed round inside the group; the first
+  // chunk of every row of the group is requested before anything else, so that a tile of rows
+  // of up to CHUNK edges costs one round trip for its columns and weights.
+  constexpr int RB = RPG < 8 ? RPG : 8;  // rows of a lane group whose first chunks are in flight together
 #pragma unroll 1
   for (int k0 = 0; k0 < RPG; k0 += RB) {
-    int rb[RB], re[RB];
-    int col[RB][U0];
-    float w[RB][U0];
-    bool keep[RB];
+  int rb[RB], re[RB];
+  int col[RB][PER];
+  float w[RB][PER];
+  bool keep[RB];
 #pragma unroll
-    for (int k = 0; k < RB; ++k) {
-      const int r = g + NG * (k0 + k);
-      int2 be = make_int2(0, 0);
-      if (r < nrows) be = range(r);
-      keep[k] = be.y - be.x <= kLongRow;
-      rb[k] = be.x;
-      re[k] = keep[k] ? be.y : be.x;
+  for (int k = 0; k < RB; ++k) {
+    const int r = g + NG * (k0 + k);
+    int2 be = make_int2(0, 0);
+    if (r < nrows) be = range(r);
+    keep[k] = be.y - be.x <= kLongRow;
+    rb[k] = be.x;
+    re[k] = keep[k] ? be.y : be.x;
 #pragma unroll
-      for (int u = 0; u < U0; ++u) {
-        const bool live = rb[k] + u < re[k];
-        col[k][u] = live ? cols[rb[k] + u] : 0;
-        w[k][u] = live ? A[rb[k] + u] : 0.f;
-      }
-    }
-    float4 x[RB][U0];
-#pragma unroll
-    for (int k = 0; k < RB; ++k)
-#pragma unroll
-      for (int u = 0; u < U0; ++u) x[k][u] = ld_x(col[k][u], w[k][u]);
-#pragma unroll
-    for (int k = 0; k < RB; ++k) {
-      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-      for (int u = 0; u < U0; ++u) fma4(acc, w[k][u], x[k][u]);
-#pragma unroll 1
-      for (int p = rb[k] + U0; p < re[k]; p += U) {
-        int c2[U];
-        float w2[U];
-        float4 x2[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const bool live = p + u < re[k];
-          c2[u] = live ? cols[p + u] : 0;
-          w2[u] = live ? A[p + u] : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) x2[u] = ld_x(c2[u], w2[u]);
-#pragma unroll
-        for (int u = 0; u < U; ++u) fma4(acc, w2[u], x2[u]);
-      }
-      if (keep[k]) {
-        float* s = S + (g + NG * (k0 + k)) * (FP + 1) + 4 * gl;
-        s[0] = acc.x, s[1] = acc.y, s[2] = acc.z, s[3] = acc.w;
-      }
+    for (int i = 0; i < PER; ++i) {
+      const int p = rb[k] + i * G + gl;
+      col[k][i] = p < re[k] ? cols[p] : 0;
+      w[k][i] = p < re[k] ? A[p] : 0.f;
     }
   }
+#pragma unroll
+  for (int k = 0; k < RB; ++k) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int base = rb[k]; base < re[k]; base += CHUNK) {
+      if (base != rb[k]) {  // a row of more than CHUNK edges: its next chunk
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int p = base + i * G + gl;
+          col[k][i] = p < re[k] ? cols[p] : 0;
+          w[k][i] = p < re[k] ? A[p] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+#pragma unroll
+        for (int c = 0; c < G; c += CH) {
+          if (base + i * G + c >= re[k]) continue;  // the same for every lane of the group
+          float4 x[CH];
+          float wv[CH];
+#pragma unroll
+          for (int u = 0; u < CH; ++u) {
+            const int src = g * G + c + u;  // a lane of this group
+            const int cc = __shfl(col[k][i], src, kWave);
+            wv[u] = __shfl(w[k][i], src, kWave);  // zero beyond the row's end and on padding
+            x[u] = ld_x(cc, wv[u]);
+          }
+#pragma unroll
+          for (int u = 0; u < CH; ++u) fma4(acc, wv[u], x[u]);
+        }
+      }
+    }
+    if (keep[k]) {
+      if (!chunk_live) acc = zero4;
+      float* s = S + (g + NG * (k0 + k)) * (FP + 1) + 4 * gl;
+      s[0] = acc.x, s[1] = acc.y, s[2] = acc.z, s[3] = acc.w;
+    }
+  }
+  }  // batches of rows
   // long rows: lane l < nrows knows whether row l is one
+  constexpr int U = 4;  // edges per lane group and step
   int2 mine = make_int2(0, 0);
   if (lane < nrows) mine = range(lane);
   uint64_t todo = __ballot(mine.y - mine.x > kLongRow);
@@ -150,6 +165,7 @@ __device__ __forceinline__ void accumulate_rows(float* S, const float* __restric
       acc.w += __shfl_xor(acc.w, off, kWave);
     }
     if (g == 0) {
+      if (!chunk_live) acc = zero4;
       float* s = S + r * (FP + 1) + 4 * gl;
       s[0] = acc.x, s[1] = acc.y, s[2] = acc.z, s[3] = acc.w;
     }

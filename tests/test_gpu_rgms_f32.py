@@ -37,7 +37,7 @@ def test_rgms_csf_f32(dev, fin, fout):
     x = rng.standard_normal((n, fin), dtype=np.float32)
     w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
     a = (0.5 + rng.random(len(csf[3]), dtype=np.float32))
-    a[::7] = 0.0  # zero-weight edges are skipped by the kernel
+    a[::7] = 0.0  # zero-weight edges add nothing
     f = ops.build_rgms_csf(n, n, R, fin, fout, len(csf[1]), len(csf[3]))
     y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
     f(_t(dev, a), _t(dev, w.ravel()), _t(dev, x.ravel()), y, *[_t(dev, c) for c in csf])
