@@ -313,7 +313,8 @@ int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t g
  * stir_tc_spmm_f16 up to the order of the fp32 additions).  The partial tiles live in memory the
  * plan owns, sized by the first launch with a given feat (that launch allocates): launches with
  * one plan must not overlap on the GPU.  The plan describes the contents of d_indptr at its
- * creation; make a new one when they change.
+ * creation; make a new one when they change.  It belongs to the device that was current at
+ * its creation, and a launch with another device current is refused.
  */
 typedef struct stir_tc_plan stir_tc_plan;
 int stir_tc_plan_create(stir_tc_plan** plan, int32_t mb, const int32_t* d_indptr, void* stream);

@@ -553,6 +553,10 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
   STIR_REQUIRE(plan, "tc_spmm_planned: plan is null");
   STIR_REQUIRE(out_dtype == STIR_F16 || out_dtype == STIR_F32, "tc_spmm: out_dtype must be STIR_F16 or STIR_F32");
   STIR_REQUIRE(plan->mb == mb, "tc_spmm_planned: the plan was made for %d row tiles, not %d", plan->mb, mb);
+  int device = 0;
+  STIR_HIP(hipGetDevice(&device));
+  STIR_REQUIRE(device == plan->device, "tc_spmm_planned: the plan lives on device %d, the current device is %d",
+               plan->device, device);
   STIR_REQUIRE(tile_size == kTile && group_size == kGroup,
                "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t=32, g=16", tile_size, group_size);
   STIR_REQUIRE(mb >= 0 && nnzb >= 0, "tc_spmm: bad sizes");
