@@ -62,7 +62,7 @@ __device__ __forceinline__ void accumulate_rows(float* S, const float* __restric
   // instead and their sums are replaced by zeros before they are stored.
   const bool chunk_live = 4 * gl < fin;
   const float* Xl = X + (chunk_live ? 4 * gl : 0);
-  auto ld_x = [&](int c, float) { return *reinterpret_cast<const float4*>(Xl + (int64_t)c * fin); };
+  auto ld_x = [&](int c) { return *reinterpret_cast<const float4*>(Xl + (int64_t)c * fin); };
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
   auto fma4 = [](float4& acc, float w, const float4& x) {
     acc.x += w * x.x, acc.y += w * x.y, acc.z += w * x.z, acc.w += w * x.w;
@@ -74,62 +74,62 @@ __device__ __forceinline__ void accumulate_rows(float* S, const float* __restric
   constexpr int RB = RPG < 8 ? RPG : 8;  // rows of a lane group whose first chunks are in flight together
 #pragma unroll 1
   for (int k0 = 0; k0 < RPG; k0 += RB) {
-  int rb[RB], re[RB];
-  int col[RB][PER];
-  float w[RB][PER];
-  bool keep[RB];
+    int rb[RB], re[RB];
+    int col[RB][PER];
+    float w[RB][PER];
+    bool keep[RB];
 #pragma unroll
-  for (int k = 0; k < RB; ++k) {
-    const int r = g + NG * (k0 + k);
-    int2 be = make_int2(0, 0);
-    if (r < nrows) be = range(r);
-    keep[k] = be.y - be.x <= kLongRow;
-    rb[k] = be.x;
-    re[k] = keep[k] ? be.y : be.x;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int p = rb[k] + i * G + gl;
-      col[k][i] = p < re[k] ? cols[p] : 0;
-      w[k][i] = p < re[k] ? A[p] : 0.f;
-    }
-  }
-#pragma unroll
-  for (int k = 0; k < RB; ++k) {
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int base = rb[k]; base < re[k]; base += CHUNK) {
-      if (base != rb[k]) {  // a row of more than CHUNK edges: its next chunk
-#pragma unroll
-        for (int i = 0; i < PER; ++i) {
-          const int p = base + i * G + gl;
-          col[k][i] = p < re[k] ? cols[p] : 0;
-          w[k][i] = p < re[k] ? A[p] : 0.f;
-        }
-      }
+    for (int k = 0; k < RB; ++k) {
+      const int r = g + NG * (k0 + k);
+      int2 be = make_int2(0, 0);
+      if (r < nrows) be = range(r);
+      keep[k] = be.y - be.x <= kLongRow;
+      rb[k] = be.x;
+      re[k] = keep[k] ? be.y : be.x;
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
-#pragma unroll
-        for (int c = 0; c < G; c += CH) {
-          if (base + i * G + c >= re[k]) continue;  // the same for every lane of the group
-          float4 x[CH];
-          float wv[CH];
-#pragma unroll
-          for (int u = 0; u < CH; ++u) {
-            const int src = g * G + c + u;  // a lane of this group
-            const int cc = __shfl(col[k][i], src, kWave);
-            wv[u] = __shfl(w[k][i], src, kWave);  // zero beyond the row's end and on padding
-            x[u] = ld_x(cc, wv[u]);
-          }
-#pragma unroll
-          for (int u = 0; u < CH; ++u) fma4(acc, wv[u], x[u]);
-        }
+        const int p = rb[k] + i * G + gl;
+        col[k][i] = p < re[k] ? cols[p] : 0;
+        w[k][i] = p < re[k] ? A[p] : 0.f;
       }
     }
-    if (keep[k]) {
-      if (!chunk_live) acc = zero4;
-      float* s = S + (g + NG * (k0 + k)) * (FP + 1) + 4 * gl;
-      s[0] = acc.x, s[1] = acc.y, s[2] = acc.z, s[3] = acc.w;
+#pragma unroll
+    for (int k = 0; k < RB; ++k) {
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int base = rb[k]; base < re[k]; base += CHUNK) {
+        if (base != rb[k]) {  // a row of more than CHUNK edges: its next chunk
+#pragma unroll
+          for (int i = 0; i < PER; ++i) {
+            const int p = base + i * G + gl;
+            col[k][i] = p < re[k] ? cols[p] : 0;
+            w[k][i] = p < re[k] ? A[p] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+#pragma unroll
+          for (int c = 0; c < G; c += CH) {
+            if (base + i * G + c >= re[k]) continue;  // the same for every lane of the group
+            float4 x[CH];
+            float wv[CH];
+#pragma unroll
+            for (int u = 0; u < CH; ++u) {
+              const int src = g * G + c + u;  // a lane of this group
+              const int cc = __shfl(col[k][i], src, kWave);
+              wv[u] = __shfl(w[k][i], src, kWave);  // zero beyond the row's end and on padding
+              x[u] = ld_x(cc);
+            }
+#pragma unroll
+            for (int u = 0; u < CH; ++u) fma4(acc, wv[u], x[u]);
+          }
+        }
+      }
+      if (keep[k]) {
+        if (!chunk_live) acc = zero4;
+        float* s = S + (g + NG * (k0 + k)) * (FP + 1) + 4 * gl;
+        s[0] = acc.x, s[1] = acc.y, s[2] = acc.z, s[3] = acc.w;
+      }
     }
-  }
   }  // batches of rows
   // long rows: lane l < nrows knows whether row l is one
   constexpr int U = 4;  // edges per lane group and step
@@ -153,7 +153,7 @@ __device__ __forceinline__ void accumulate_rows(float* S, const float* __restric
         w2[u] = live ? A[p + u * NG] : 0.f;
       }
 #pragma unroll
-      for (int u = 0; u < U; ++u) x2[u] = ld_x(c2[u], w2[u]);
+      for (int u = 0; u < U; ++u) x2[u] = ld_x(c2[u]);
 #pragma unroll
       for (int u = 0; u < U; ++u) fma4(acc, w2[u], x2[u]);
     }
