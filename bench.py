@@ -48,8 +48,8 @@ PROBES_LIB = os.path.join(ROOT, "libbench_probes.so")
 
 def build_probes():
     cmd = [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "-O3", "-std=c++17", "-fPIC", "-shared",
-           "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-x", "hip", PROBES_SRC, "-o", PROBES_LIB]
+           "--offload-arch=gfx950", "-munsafe-fp-atomics", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-x", "hip", PROBES_SRC, "-o", PROBES_LIB]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed on bench_probes.hip:\n" + r.stdout + r.stderr)
@@ -63,6 +63,7 @@ def load_probes():
     VP, I64, I32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
     L.bench_probe_copy.restype, L.bench_probe_copy.argtypes = I32, [VP, VP, I64, VP]
     L.bench_probe_gather.restype, L.bench_probe_gather.argtypes = I32, [VP, I64, I32, I64, VP, VP]
+    L.bench_probe_atomic_rows.restype, L.bench_probe_atomic_rows.argtypes = I32, [VP, I64, I64, VP]
     L.bench_probe_mfma_f16.restype = I32
     L.bench_probe_mfma_f16.argtypes = [I32, I32, I32, VP, ctypes.POINTER(ctypes.c_double), VP]
     return L
@@ -400,6 +401,22 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     out["rgms_f32_ell3d_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
                                      "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
                                      "ell_rows": int(sum(r.size for r in rows))}
+    # every ELL row adds feat_out floats to Y with one atomic each: the launch's bound.  Beside
+    # it, what the same number of row additions to hashed rows of Y takes with nothing else going on
+    er = out["rgms_f32_ell3d_config5"]["ell_rows"]
+    out["rgms_f32_ell3d_config5"]["atomic_adds"] = er * fout
+    out["rgms_f32_ell3d_config5"]["atomic_adds_G_per_s"] = er * fout / d / 1e9
+    if fout == 32:
+        P = load_probes()
+        st0 = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        yp = ctypes.c_void_p(y.data_ptr())
+
+        def scatter_only():
+            if P.bench_probe_atomic_rows(yp, n, er, st0) != 0:
+                raise RuntimeError("atomic probe failed")
+        tp = time_small(scatter_only, 20, 2, torch)
+        out["rgms_f32_ell3d_config5"]["probe_atomic_rows_us"] = tp["us_back_to_back"]
+        out["rgms_f32_ell3d_config5"]["probe_atomic_adds_G_per_s"] = er * fout / tp["us_back_to_back"] / 1e3
     csf = [t(cfg[k]) for k in ("indptr0", "indices0", "indptr1", "indices1")]
     ones = torch.ones(E, device=dev)
     fc = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E)

@@ -56,6 +56,21 @@ __global__ __launch_bounds__(256) void probe_gather_kernel(const float* __restri
   if (acc.x == 1.2345e38f) sink[0] = acc.x + acc.y + acc.z + acc.w;
 }
 
+// Every half wavefront adds 1.0 to the 32 floats of `per_group` rows at hashed indices, one
+// fp32 atomic per lane and row (no return value, device scope): the scatter of an operator that
+// adds 128-byte rows to its output, without the rest of that operator.
+__global__ __launch_bounds__(256) void probe_atomic_rows_kernel(float* __restrict__ table, int64_t rows,
+                                                                int per_group) {
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 5, gl = lane & 31;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t seed = (uint32_t)(wave * 2 + g) * 2654435761u;
+  for (int i = 0; i < per_group; ++i) {
+    const int64_t row = mix32(seed + i) % (uint64_t)rows;
+    __hip_atomic_fetch_add(table + row * 32 + gl, 1.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -123,6 +138,19 @@ int bench_probe_gather(const float* d_table, int64_t rows, int32_t row_floats, i
   if (blocks >= (int64_t(1) << 31)) return -1;
   hipLaunchKernelGGL(probe_gather_kernel, dim3((unsigned)blocks), dim3(256), 0,
                      static_cast<hipStream_t>(stream), d_table, rows, row_floats, lanes, per_group, d_sink);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// num_rows (rounded up to whole workgroups' worth) additions of a row of 32 floats of 1.0 to
+// hashed rows of d_table (rows x 32 floats): 32 fp32 atomics each.
+int bench_probe_atomic_rows(float* d_table, int64_t rows, int64_t num_rows, void* stream) {
+  if (!(d_table && rows > 0 && num_rows > 0)) return -1;
+  const int per_group = 32;
+  const int64_t per_block = (int64_t)per_group * 2 * 4;
+  const int64_t blocks = (num_rows + per_block - 1) / per_block;
+  if (blocks >= (int64_t(1) << 31)) return -1;
+  hipLaunchKernelGGL(probe_atomic_rows_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), d_table, rows, per_group);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -63,5 +63,5 @@ def test_probe_library_exports_its_entry_points():
     path = os.path.join(ROOT, "libbench_probes.so")
     assert os.path.exists(path), "build with `python -c 'import __graft_entry__ as g; g.build()'`"
     lib = ctypes.CDLL(path)
-    for name in ("bench_probe_copy", "bench_probe_gather", "bench_probe_mfma_f16"):
+    for name in ("bench_probe_copy", "bench_probe_gather", "bench_probe_mfma_f16", "bench_probe_atomic_rows"):
         assert hasattr(lib, name), name
