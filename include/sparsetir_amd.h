@@ -292,7 +292,9 @@ int stir_dbsr_spmm(int32_t dtype, int32_t out_dtype, int32_t nnz_rows, int32_t n
  * (operator :538-565).  A: nnzb*t*g (the 0/1 mask of ConDense as fp16, or edge weights),
  * B: dense features, at least max(indices)+1 rows of feat, C: mb*t*feat of out_dtype (STIR_F16
  * as in the reference, or STIR_F32), indptr: group_indptr (mb+1), indices: tile_indices
- * (nnzb*g).  The MFMA path needs tile_size t = 32 and group_size g = 16.  C is written, not
+ * (nnzb*g).  The MFMA path takes tile_size t = 8 or 16 (the two sizes the reference condenses
+ * with, examples/spmm/bench_tc_spmm.py:584-585,670: t = mma_m of m8n32k16 / m16n16k16) or 32, and
+ * group_size g = 16 (= mma_k).  C is written, not
  * accumulated into; with fp32 output this takes two launches (row tiles with very many groups
  * are cleared, then summed by several workgroups).
  */

@@ -1,14 +1,19 @@
 // SpMM on the gfx950 matrix cores over the condensed format of ConDense: the rows of the
-// sparse matrix are cut into tiles of t = 32 rows; inside a tile the distinct columns are
-// gathered g = 16 at a time into dense 32 x 16 blocks A[jo] (zero where the row has no entry):
-//   C[io*32 + ii, f] = sum over groups jo of tile io, ji < 16:  A[jo, ii, ji] * B[indices[jo, ji], f]
+// sparse matrix are cut into tiles of t rows (t = 8, 16 -- the two sizes the reference's
+// examples/spmm/bench_tc_spmm.py:584-585,670 condenses with -- or 32); inside a tile the distinct
+// columns are gathered g = 16 at a time into dense t x 16 blocks A[jo] (zero where the row has no
+// entry):
+//   C[io*t + ii, f] = sum over groups jo of tile io, ji < 16:  A[jo, ii, ji] * B[indices[jo, ji], f]
 // fp16 inputs, fp32 accumulation, fp16 or fp32 output.
 //
 // Same tiling as the BSR kernel: a workgroup of four wavefronts owns (row tile, 128 features),
-// a wavefront a 32x32 accumulator.  A step covers two groups (32 gathered rows of B): A[jo] is
+// a wavefront t rows x 32 features.  A step covers two groups (32 gathered rows of B): A[jo] is
 // already in MFMA A-operand order (a lane's 8 k values are contiguous), the 32 gathered rows of
 // B go through LDS, interleaved into (k, k+1) pairs on the way, double-buffered, with the next
-// step's gathers in flight during the multiply.
+// step's gathers in flight during the multiply.  Tiles of 32 rows multiply with two
+// v_mfma_f32_32x32x16_f16 per step (one per group); tiles of 16 rows with v_mfma_f32_16x16x32_f16,
+// whose k extent of 32 is the step's two groups, once per 16 features; tiles of 8 rows are the
+// upper half of a 16-row operand whose other rows are zero.
 //
 // A row tile that touches thousands of distinct columns (a hub row of a power-law graph) would be
 // one long serial chain in one workgroup.  With fp32 output such tiles are cut into up to kSplit
@@ -35,8 +40,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 constexpr int kTileF = 128;
-constexpr int kTile = 32;   // t
 constexpr int kGroup = 16;  // g
 constexpr int kUnitSteps = 16;  // steps (of two groups) per unit of a long tile
 constexpr int kSplit = 16;      // most units per tile (second grid dimension of the split launch)
@@ -49,42 +55,131 @@ __device__ __forceinline__ int tile_steps(const int32_t* __restrict__ indptr, in
   return (int)((rows_total + 31) / 32);
 }
 
+// ---- what differs between the row-tile sizes: the accumulators of a wavefront for (T rows) x
+// (32 features), the A operand of a step, and the multiply of a step out of the staged rows of B.
+// WIDE = 32-row tiles on the 32x32x16 instruction; otherwise 16-row operands on 16x16x32.
+template <bool WIDE>
+struct TcAcc;
+template <>
+struct TcAcc<true> {
+  static constexpr int kRegs = 16;
+  f32x16 r;
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) r[v] = 0.f;
+  }
+  __device__ __forceinline__ float get(int v) const { return r[v]; }
+  // register v of lane l is this row / feature of the wavefront's tile
+  static __device__ __forceinline__ int row(int v, int l) { return (v & 3) + 4 * (l >> 5) + 8 * (v >> 2); }
+  static __device__ __forceinline__ int col(int v, int l) { return l & 31; }
+};
+template <>
+struct TcAcc<false> {
+  static constexpr int kRegs = 8;  // two 16x16 tiles side by side
+  f32x4 r[2];
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int v = 0; v < 8; ++v) r[v >> 2][v & 3] = 0.f;
+  }
+  __device__ __forceinline__ float get(int v) const { return r[v >> 2][v & 3]; }
+  static __device__ __forceinline__ int row(int v, int l) { return 4 * (l >> 4) + (v & 3); }
+  static __device__ __forceinline__ int col(int v, int l) { return 16 * (v >> 2) + (l & 15); }
+};
+
+// A[jo] and A[jo + 1] as the A operand(s) of a step (zero past the tile's last group).
+// T = 32: lane (n = l % 32, h = l / 32) holds A[jo + d][n][8h .. 8h+7] in a[d].
+// T <= 16: lane (i = l % 16, q = l / 16) holds k = 8q .. 8q+7 of the step's 32, i.e.
+// A[jo + q/2][i][8(q%2) ..], in a[0]; rows i >= T of the operand are zero.
+template <int T>
+__device__ __forceinline__ void tc_load_a(u32x4 (&a)[2], const uint16_t* __restrict__ A, int64_t jo, int64_t g_end,
+                                          int lane) {
+  a[0] = a[1] = u32x4{0, 0, 0, 0};
+  if constexpr (T == 32) {
+    const int n = lane & 31, h = lane >> 5;
+    a[0] = *reinterpret_cast<const u32x4*>(A + (jo * 32 + n) * kGroup + 8 * h);
+    if (jo + 1 < g_end) a[1] = *reinterpret_cast<const u32x4*>(A + ((jo + 1) * 32 + n) * kGroup + 8 * h);
+  } else {
+    const int i = lane & 15, q = lane >> 4;
+    const int64_t grp = jo + (q >> 1);
+    if (i < T && grp < g_end) a[0] = *reinterpret_cast<const u32x4*>(A + (grp * T + i) * kGroup + 8 * (q & 1));
+  }
+}
+
+// Where 16-byte-aligned feature offset `col` of k pair `kp` lives inside its staged row of STRIDE
+// words (a power of two).  The 16-row multiply reads rows 4q .. 4q+3 for q = l / 16 at 16
+// consecutive features: rotating a row by 16 (kp / 4) words puts the four q on different banks.
+template <int T, int STRIDE>
+__device__ __forceinline__ int tc_stage_col(int kp, int col) {
+  if constexpr (T == 32) return col;
+  else return (col + 16 * (kp >> 2)) & (STRIDE - 1);
+}
+
+// acc += A-operand(s) x the 32 staged rows of B, features col0 .. col0+31 of the staged rows
+// xs[16 k pairs][STRIDE]
+template <int T, int STRIDE>
+__device__ __forceinline__ void tc_multiply(TcAcc<T == 32>& acc, const u32x4 (&a)[2], const uint32_t* xs, int col0,
+                                            int lane) {
+  if constexpr (T == 32) {
+    const int n = lane & 31, h = lane >> 5;
+    u32x4 b0, b1;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      b0[d] = xs[(4 * h + d) * STRIDE + col0 + n];      // rows 8h .. 8h+7 of the first group
+      b1[d] = xs[(8 + 4 * h + d) * STRIDE + col0 + n];  // rows 8h .. 8h+7 of the second group
+    }
+    acc.r = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[0]), __builtin_bit_cast(f16x8, b0),
+                                                  acc.r, 0, 0, 0);
+    acc.r = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[1]), __builtin_bit_cast(f16x8, b1),
+                                                  acc.r, 0, 0, 0);
+  } else {
+    const int n = lane & 15, q = lane >> 4;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int c = tc_stage_col<T, STRIDE>(4 * q, col0 + 16 * nt) + n;
+      u32x4 b;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) b[d] = xs[(4 * q + d) * STRIDE + c];  // rows 8q .. 8q+7 of the step
+      acc.r[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[0]),
+                                                        __builtin_bit_cast(f16x8, b), acc.r[nt], 0, 0, 0);
+    }
+  }
+}
+
 // Clears the fp32 rows of the tiles that the split launch accumulates into.  grid (mb * f_tiles)
-__global__ __launch_bounds__(256) void tcspmm_clear_long_kernel(int feat, int64_t mb, int f_tiles,
+__global__ __launch_bounds__(256) void tcspmm_clear_long_kernel(int tile, int feat, int64_t mb, int f_tiles,
                                                                 float* __restrict__ C,
                                                                 const int32_t* __restrict__ indptr) {
   const int f_tile = (int)(blockIdx.x % f_tiles);
   const int64_t io = blockIdx.x / f_tiles;
   if (io >= mb || tile_steps(indptr, io) <= kUnitSteps) return;
   const int f0 = f_tile * kTileF;
-  for (int e = threadIdx.x; e < kTile * kTileF; e += 256) {
+  for (int e = threadIdx.x; e < tile * kTileF; e += 256) {
     const int row = e / kTileF, f = f0 + e % kTileF;
-    if (f < feat) C[(io * kTile + row) * feat + f] = 0.f;
+    if (f < feat) C[(io * tile + row) * feat + f] = 0.f;
   }
 }
 
 // OUT: 0 = fp16 output, 1 = fp32 output.  SPLIT: grid is (mb * f_tiles, kSplit); the units of a
 // long tile take equal shares of its steps and add with atomics, unit 0 of a short tile stores.
-template <int OUT, bool SPLIT, bool SKIP_LONG = (OUT == 0)>
+template <int T, int OUT, bool SPLIT, bool SKIP_LONG = (OUT == 0)>
 __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f_tiles,
                                                      const uint16_t* __restrict__ A,
                                                      const uint16_t* __restrict__ B, void* __restrict__ C,
                                                      const int32_t* __restrict__ indptr,
                                                      const int32_t* __restrict__ indices) {
-  __shared__ uint32_t xs[2][16][kTileF];  // [buffer][k pair][feature]
+  __shared__ __attribute__((aligned(16))) uint32_t xs[2][16 * kTileF];  // [buffer][k pair][feature]
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int n = lane & 31, h = lane >> 5;
   const int f_tile = (int)(blockIdx.x % f_tiles);
   const int64_t io = blockIdx.x / f_tiles;
   if (io >= mb) return;
   const int f0 = f_tile * kTileF;
   const int kp = tid >> 4, fc = tid & 15;  // staging role: k pair, 8-feature chunk
   const bool stage_live = f0 + fc * 8 < feat;
+  const int stage_at = kp * kTileF + tc_stage_col<T, kTileF>(kp, fc * 8);
 
-  f32x16 acc;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  TcAcc<T == 32> acc;
+  acc.clear();
 
   const int64_t g_begin = indptr[io], g_end = indptr[io + 1];
   const int64_t rows_total = (g_end - g_begin) * kGroup;  // gathered rows of B for this tile
@@ -118,11 +213,7 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   };
   u32x4 r0, r1, a_next[2];
   auto fetch = [&](int it) {
-    // A[jo][n][8h .. 8h+7] for the step's two groups (zero when the tile has an odd group count)
-    const int64_t jo = g_begin + 2 * it;
-    a_next[0] = *reinterpret_cast<const u32x4*>(A + (jo * kTile + n) * kGroup + 8 * h);
-    a_next[1] = u32x4{0, 0, 0, 0};
-    if (jo + 1 < g_end) a_next[1] = *reinterpret_cast<const u32x4*>(A + ((jo + 1) * kTile + n) * kGroup + 8 * h);
+    tc_load_a<T>(a_next, A, g_begin + 2 * it, g_end, lane);
     r0 = r1 = u32x4{0, 0, 0, 0};
     const int64_t k = (int64_t)it * 32 + 2 * kp;
     if (stage_live && k < rows_total) {
@@ -138,7 +229,7 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
   }
   for (int it = it_begin; it < it_end; ++it) {
     const int buf = it & 1;
-    const u32x4 a0 = a_next[0], a1 = a_next[1];
+    const u32x4 a_now[2] = {a_next[0], a_next[1]};
     u32x4 lo, hi;
 #pragma unroll
     for (int d = 0; d < 2; ++d) {
@@ -147,35 +238,26 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
       hi[2 * d] = __builtin_amdgcn_perm(r1[d + 2], r0[d + 2], 0x05040100);
       hi[2 * d + 1] = __builtin_amdgcn_perm(r1[d + 2], r0[d + 2], 0x07060302);
     }
-    *reinterpret_cast<u32x4*>(&xs[buf][kp][fc * 8]) = lo;
-    *reinterpret_cast<u32x4*>(&xs[buf][kp][fc * 8 + 4]) = hi;
+    *reinterpret_cast<u32x4*>(&xs[buf][stage_at]) = lo;
+    *reinterpret_cast<u32x4*>(&xs[buf][stage_at + 4]) = hi;
     if (it + 1 < it_end) fetch(it + 1);
     __syncthreads();
-    const int col = wave * 32 + n;
-    u32x4 b0, b1;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      b0[d] = xs[buf][4 * h + d][col];      // rows 8h .. 8h+7 of the first group
-      b1[d] = xs[buf][8 + 4 * h + d][col];  // rows 8h .. 8h+7 of the second group
-    }
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a0), __builtin_bit_cast(f16x8, b0),
-                                                acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a1), __builtin_bit_cast(f16x8, b1),
-                                                acc, 0, 0, 0);
+    tc_multiply<T, kTileF>(acc, a_now, xs[buf], wave * 32, lane);
   }
   const int fcol = f0 + wave * 32;
   if (fcol >= feat) return;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int row = (v & 3) + 4 * h + 8 * (v >> 2);
-    const int64_t off = (io * kTile + row) * feat + fcol + n;
+  for (int v = 0; v < TcAcc<T == 32>::kRegs; ++v) {
+    const int row = TcAcc<T == 32>::row(v, lane);
+    if (T < 16 && row >= T) continue;
+    const int64_t off = (io * T + row) * feat + fcol + TcAcc<T == 32>::col(v, lane);
     if constexpr (OUT == 1) {
       if (add)
-        __hip_atomic_fetch_add(static_cast<float*>(C) + off, acc[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(static_cast<float*>(C) + off, acc.get(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else
-        static_cast<float*>(C)[off] = acc[v];
+        static_cast<float*>(C)[off] = acc.get(v);
     } else {
-      const _Float16 hv = (_Float16)acc[v];
+      const _Float16 hv = (_Float16)acc.get(v);
       static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
     }
   }
@@ -192,12 +274,13 @@ __global__ __launch_bounds__(256) void tcspmm_kernel(int feat, int64_t mb, int f
 // per wavefront (a step is a round trip to memory): more wavefronts per tile shorten it.
 // lds: WAVES * 16 * 32 * NTL words (64 KB either way).  Ends with LDS reads: a caller that goes on
 // to another tile puts a workgroup barrier in between.
-template <int NTL, class Store>
+template <int T, int NTL, class Store>
 __device__ __forceinline__ void tcspmm_long_steps(uint32_t* __restrict__ lds, int feat, int64_t io, int f0,
                                                   int s_begin, int s_end, const uint16_t* __restrict__ A,
                                                   const uint16_t* __restrict__ B,
                                                   const int32_t* __restrict__ indptr,
                                                   const int32_t* __restrict__ indices, Store store) {
+  using Acc = TcAcc<T == 32>;
   constexpr int WAVES = 32 / NTL;  // wavefronts per workgroup
   constexpr int TF = 32 * NTL;     // features per workgroup
   constexpr int CH = TF / 8;       // 8-feature chunks of a staged row
@@ -205,19 +288,16 @@ __device__ __forceinline__ void tcspmm_long_steps(uint32_t* __restrict__ lds, in
   constexpr int Q = 16 / KP;       // ... times Q = the 16 k pairs of a step
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n = lane & 31, h = lane >> 5;
   const int kp = lane / CH, fc = lane % CH;
   const bool stage_live = f0 + fc * 8 < feat;
-  uint32_t(*xs)[TF] = reinterpret_cast<uint32_t(*)[TF]>(lds + wave * (16 * TF));  // [k pair][feature]
+  uint32_t* xs = lds + wave * (16 * TF);  // [k pair][feature]
   const int64_t g_begin = indptr[io], g_end = indptr[io + 1];
   const int64_t rows_total = (g_end - g_begin) * kGroup;
   const int32_t* rowlist = indices + g_begin * kGroup;
 
-  f32x16 acc[NTL];
+  Acc acc[NTL];
 #pragma unroll
-  for (int t = 0; t < NTL; ++t)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+  for (int t = 0; t < NTL; ++t) acc[t].clear();
 
   // row ids one step (of this wavefront) before the rows of B, as in the kernel above
   int row_a[Q], row_b[Q];
@@ -231,10 +311,7 @@ __device__ __forceinline__ void tcspmm_long_steps(uint32_t* __restrict__ lds, in
   };
   u32x4 r0[Q], r1[Q], a_next[2];
   auto fetch = [&](int it) {
-    const int64_t jo = g_begin + 2 * it;
-    a_next[0] = *reinterpret_cast<const u32x4*>(A + (jo * kTile + n) * kGroup + 8 * h);
-    a_next[1] = u32x4{0, 0, 0, 0};
-    if (jo + 1 < g_end) a_next[1] = *reinterpret_cast<const u32x4*>(A + ((jo + 1) * kTile + n) * kGroup + 8 * h);
+    tc_load_a<T>(a_next, A, g_begin + 2 * it, g_end, lane);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
       r0[q] = r1[q] = u32x4{0, 0, 0, 0};
@@ -253,7 +330,7 @@ __device__ __forceinline__ void tcspmm_long_steps(uint32_t* __restrict__ lds, in
     fetch(s_begin + wave);
   }
   for (int it = s_begin + wave; it < s_end; it += WAVES) {
-    const u32x4 a0 = a_next[0], a1 = a_next[1];
+    const u32x4 a_now[2] = {a_next[0], a_next[1]};
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
       u32x4 lo, hi;
@@ -264,53 +341,43 @@ __device__ __forceinline__ void tcspmm_long_steps(uint32_t* __restrict__ lds, in
         hi[2 * d] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x05040100);
         hi[2 * d + 1] = __builtin_amdgcn_perm(r1[q][d + 2], r0[q][d + 2], 0x07060302);
       }
-      *reinterpret_cast<u32x4*>(&xs[kp + KP * q][fc * 8]) = lo;
-      *reinterpret_cast<u32x4*>(&xs[kp + KP * q][fc * 8 + 4]) = hi;
+      const int at = (kp + KP * q) * TF + tc_stage_col<T, TF>(kp + KP * q, fc * 8);
+      *reinterpret_cast<u32x4*>(xs + at) = lo;
+      *reinterpret_cast<u32x4*>(xs + at + 4) = hi;
     }
     if (it + WAVES < s_end) fetch(it + WAVES);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int t = 0; t < NTL; ++t) {
-      const int col = t * 32 + n;
-      u32x4 b0, b1;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        b0[d] = xs[4 * h + d][col];
-        b1[d] = xs[8 + 4 * h + d][col];
-      }
-      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a0), __builtin_bit_cast(f16x8, b0),
-                                                     acc[t], 0, 0, 0);
-      acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a1), __builtin_bit_cast(f16x8, b1),
-                                                     acc[t], 0, 0, 0);
-    }
+    for (int t = 0; t < NTL; ++t) tc_multiply<T, TF>(acc[t], a_now, xs, t * 32, lane);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     __builtin_amdgcn_wave_barrier();  // the next step's stores come after these reads
   }
 
   // ---- the partial tiles, one 32-feature tile at a time: a thread sums register v of lane l
-  // over the wavefronts; that is row (v%4) + 4(l/32) + 8(v/4), feature l%32 of the tile.
-  float* red = reinterpret_cast<float*>(lds);  // [wavefront][register][lane], 4 KB per wavefront
+  // over the wavefronts
+  constexpr int REGS = Acc::kRegs;
+  float* red = reinterpret_cast<float*>(lds);  // [wavefront][register][lane], at most 4 KB per wavefront
 #pragma unroll
   for (int t = 0; t < NTL; ++t) {
     __syncthreads();  // staging pieces (t = 0) or the sums of the tile before are done with
 #pragma unroll
-    for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[t][v];
+    for (int v = 0; v < REGS; ++v) red[(wave * REGS + v) * 64 + lane] = acc[t].get(v);
     __syncthreads();
-#pragma unroll
-    for (int e = tid; e < 16 * 64; e += 64 * WAVES) {
+    for (int e = tid; e < REGS * 64; e += 64 * WAVES) {
       const int v = e >> 6, l = e & 63;
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) sum += red[(w * 16 + v) * 64 + l];
-      const int fcol = f0 + t * 32 + (l & 31);
-      if (fcol < feat) store((v & 3) + 4 * (l >> 5) + 8 * (v >> 2), fcol, sum);
+      for (int w = 0; w < WAVES; ++w) sum += red[(w * REGS + v) * 64 + l];
+      const int row = Acc::row(v, l);
+      const int fcol = f0 + t * 32 + Acc::col(v, l);
+      if (fcol < feat && row < T) store(row, fcol, sum);
     }
   }
 }
 
 // fp16 output without a plan: the tiles the kernel above skips (more than kLongSteps steps).
-template <int NTL>
+template <int T, int NTL>
 __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, int64_t mb, int f_tiles,
                                                                       const uint16_t* __restrict__ A,
                                                                       const uint16_t* __restrict__ B,
@@ -341,11 +408,11 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, 
     const int64_t io = blockIdx.x / f_tiles + (int64_t)k_tile * io_stride;
     if (used_lds) __syncthreads();  // the sums of the tile before have been read
     used_lds = true;
-    tcspmm_long_steps<NTL>(lds, feat, io, f0, 0, tile_steps(indptr, io), A, B, indptr, indices,
-                           [&](int row, int fcol, float sum) {
-                             const _Float16 hv = (_Float16)sum;
-                             static_cast<uint16_t*>(C)[(io * kTile + row) * feat + fcol] = __builtin_bit_cast(uint16_t, hv);
-                           });
+    tcspmm_long_steps<T, NTL>(lds, feat, io, f0, 0, tile_steps(indptr, io), A, B, indptr, indices,
+                              [&](int row, int fcol, float sum) {
+                                const _Float16 hv = (_Float16)sum;
+                                static_cast<uint16_t*>(C)[(io * T + row) * feat + fcol] = __builtin_bit_cast(uint16_t, hv);
+                              });
   }
 }
 
@@ -365,7 +432,7 @@ struct TcMulti {
   int32_t tile, first_slot, pieces, pad;
 };
 
-template <int NTL, int OUT>
+template <int T, int NTL, int OUT>
 __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat, int f_tiles,
                                                                         const TcPiece* __restrict__ pieces,
                                                                         const uint16_t* __restrict__ A,
@@ -381,31 +448,32 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat
   // a plan made from other contents of indptr: stay inside the tile as it is now
   const int s_end = min(pc.step_end, tile_steps(indptr, io));
   if (pc.slot < 0) {
-    tcspmm_long_steps<NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
-                           [&](int row, int fcol, float sum) {
-                             const int64_t off = (io * kTile + row) * feat + fcol;
-                             if constexpr (OUT == 1) {
-                               static_cast<float*>(C)[off] = sum;
-                             } else {
-                               const _Float16 hv = (_Float16)sum;
-                               static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
-                             }
-                           });
+    tcspmm_long_steps<T, NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
+                              [&](int row, int fcol, float sum) {
+                                const int64_t off = (io * T + row) * feat + fcol;
+                                if constexpr (OUT == 1) {
+                                  static_cast<float*>(C)[off] = sum;
+                                } else {
+                                  const _Float16 hv = (_Float16)sum;
+                                  static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
+                                }
+                              });
   } else {
-    float* part = scratch + (int64_t)pc.slot * kTile * feat;
-    tcspmm_long_steps<NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
-                           [&](int row, int fcol, float sum) { part[(int64_t)row * feat + fcol] = sum; });
+    float* part = scratch + (int64_t)pc.slot * T * feat;
+    tcspmm_long_steps<T, NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
+                              [&](int row, int fcol, float sum) { part[(int64_t)row * feat + fcol] = sum; });
   }
 }
 
 // C[tile] = fp16(sum of the tile's partial tiles); grid (tiles cut into several pieces) x
-// (32 * feat / 1024): a thread owns four consecutive elements (feat is a multiple of 32)
+// (tile * feat / 1024): a thread owns four consecutive elements (feat is a multiple of 32)
 template <int OUT>
-__global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int feat, int chunks, const TcMulti* __restrict__ multi,
+__global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int tile, int feat, int chunks,
+                                                                const TcMulti* __restrict__ multi,
                                                                 const float* __restrict__ scratch,
                                                                 void* __restrict__ C) {
   const TcMulti mt = multi[blockIdx.x / chunks];
-  const int64_t elems = (int64_t)kTile * feat;
+  const int64_t elems = (int64_t)tile * feat;
   const int64_t e = ((int64_t)(blockIdx.x % chunks) * 256 + threadIdx.x) * 4;
   if (e >= elems) return;
   const float* part = scratch + (int64_t)mt.first_slot * elems + e;
@@ -430,45 +498,104 @@ __global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int feat, int ch
   }
 }
 
+constexpr int kLongTF = 32 * kLongNT, kLongWaves = 32 / kLongNT;
+constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kLongTF * sizeof(uint32_t);
+
+int check_args(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t group_size, int32_t feat, int64_t nnzb,
+               const void* d_A, const void* d_B, void* d_C, const int32_t* d_indptr, const int32_t* d_indices) {
+  STIR_REQUIRE(out_dtype == STIR_F16 || out_dtype == STIR_F32, "tc_spmm: out_dtype must be STIR_F16 or STIR_F32");
+  STIR_REQUIRE((tile_size == 8 || tile_size == 16 || tile_size == 32) && group_size == kGroup,
+               "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t in {8, 16, 32} and g=16", tile_size,
+               group_size);
+  STIR_REQUIRE(mb >= 0 && nnzb >= 0, "tc_spmm: bad sizes");
+  STIR_REQUIRE(feat > 0 && feat % 32 == 0, "tc_spmm: feat=%d must be a multiple of 32", feat);
+  STIR_REQUIRE(mb == 0 || (d_B && d_C && d_indptr && (nnzb == 0 || (d_A && d_indices))),
+               "tc_spmm: null pointer argument");
+  return 0;
+}
+
+template <int T>
+int launch_unplanned(bool out32, int32_t mb, int32_t feat, const uint16_t* A, const uint16_t* B, void* d_C,
+                     const int32_t* d_indptr, const int32_t* d_indices, hipStream_t st) {
+  const int f_tiles = (int)stir::ceil_div(feat, kTileF);
+  const int64_t blocks = (int64_t)mb * f_tiles;
+  STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
+  if (out32) {
+    hipLaunchKernelGGL(tcspmm_clear_long_kernel, dim3((unsigned)blocks), dim3(256), 0, st, T, feat, (int64_t)mb,
+                       f_tiles, static_cast<float*>(d_C), d_indptr);
+    STIR_LAUNCH_CHECK();
+    hipLaunchKernelGGL((tcspmm_kernel<T, 1, true>), dim3((unsigned)blocks, kSplit), dim3(256), 0, st, feat,
+                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
+  } else {
+    // the two launches write different row tiles
+    const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
+    const int64_t long_blocks = stir::ceil_div((int64_t)mb, kLongScan) * long_f_tiles;
+    STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
+    hipLaunchKernelGGL((tcspmm_kernel<T, 0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
+                       f_tiles, A, B, d_C, d_indptr, d_indices);
+    STIR_LAUNCH_CHECK();
+    hipLaunchKernelGGL((tcspmm_long_kernel<T, kLongNT>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves), kLongLds,
+                       st, feat, (int64_t)mb, long_f_tiles, A, B, d_C, d_indptr, d_indices);
+  }
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int T>
+int launch_planned(bool out32, int32_t mb, int32_t feat, int64_t n_pieces, int64_t n_multi, const TcPiece* d_pieces,
+                   const TcMulti* d_multi, float* d_scratch, const uint16_t* A, const uint16_t* B, void* d_C,
+                   const int32_t* d_indptr, const int32_t* d_indices, hipStream_t st) {
+  const int f_tiles = (int)stir::ceil_div(feat, kTileF);
+  const int64_t blocks = (int64_t)mb * f_tiles;
+  STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
+  // the tiles of up to kLongSteps steps
+  if (out32)
+    hipLaunchKernelGGL((tcspmm_kernel<T, 1, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat,
+                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
+  else
+    hipLaunchKernelGGL((tcspmm_kernel<T, 0, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat,
+                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
+  STIR_LAUNCH_CHECK();
+  if (n_pieces == 0) return 0;
+  const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
+  const int64_t long_blocks = n_pieces * long_f_tiles;
+  STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many pieces for one launch");
+  if (out32)
+    hipLaunchKernelGGL((tcspmm_pieces_kernel<T, kLongNT, 1>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
+                       kLongLds, st, feat, long_f_tiles, d_pieces, A, B, d_C, d_scratch, d_indptr, d_indices);
+  else
+    hipLaunchKernelGGL((tcspmm_pieces_kernel<T, kLongNT, 0>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
+                       kLongLds, st, feat, long_f_tiles, d_pieces, A, B, d_C, d_scratch, d_indptr, d_indices);
+  STIR_LAUNCH_CHECK();
+  if (n_multi == 0) return 0;
+  const int chunks = (int)stir::ceil_div((int64_t)T * feat, 1024);
+  STIR_REQUIRE(n_multi * chunks < (int64_t(1) << 31), "tc_spmm: too many partial tiles for one launch");
+  if (out32)
+    hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<1>, dim3((unsigned)(n_multi * chunks)), dim3(256), 0, st, T, feat,
+                       chunks, d_multi, d_scratch, d_C);
+  else
+    hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<0>, dim3((unsigned)(n_multi * chunks)), dim3(256), 0, st, T, feat,
+                       chunks, d_multi, d_scratch, d_C);
+  STIR_LAUNCH_CHECK();
+  return 0;
+}
+
 }  // namespace
 
 extern "C" int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t group_size,
                                 int32_t feat, int64_t nnzb, const void* d_A, const void* d_B, void* d_C,
                                 const int32_t* d_indptr, const int32_t* d_indices, void* stream) {
-  STIR_REQUIRE(out_dtype == STIR_F16 || out_dtype == STIR_F32, "tc_spmm: out_dtype must be STIR_F16 or STIR_F32");
-  STIR_REQUIRE(tile_size == kTile && group_size == kGroup,
-               "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t=32, g=16", tile_size, group_size);
-  STIR_REQUIRE(mb >= 0 && nnzb >= 0, "tc_spmm: bad sizes");
-  STIR_REQUIRE(feat > 0 && feat % 32 == 0, "tc_spmm: feat=%d must be a multiple of 32", feat);
+  if (check_args(out_dtype, mb, tile_size, group_size, feat, nnzb, d_A, d_B, d_C, d_indptr, d_indices)) return -1;
   if (mb == 0) return 0;
-  STIR_REQUIRE(d_B && d_C && d_indptr && (nnzb == 0 || (d_A && d_indices)), "tc_spmm: null pointer argument");
-  const int f_tiles = (int)stir::ceil_div(feat, kTileF);
-  const int64_t blocks = (int64_t)mb * f_tiles;
-  STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* B = static_cast<const uint16_t*>(d_B);
-  if (out_dtype == STIR_F32) {
-    hipLaunchKernelGGL(tcspmm_clear_long_kernel, dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
-                       f_tiles, static_cast<float*>(d_C), d_indptr);
-    STIR_LAUNCH_CHECK();
-    hipLaunchKernelGGL((tcspmm_kernel<1, true>), dim3((unsigned)blocks, kSplit), dim3(256), 0, st, feat,
-                       (int64_t)mb, f_tiles, A, B, d_C, d_indptr, d_indices);
-  } else {
-    // the two launches write different row tiles
-    constexpr int kLongTF = 32 * kLongNT, kLongWaves = 32 / kLongNT;
-    constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kLongTF * sizeof(uint32_t);
-    const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
-    const int64_t long_blocks = stir::ceil_div((int64_t)mb, kLongScan) * long_f_tiles;
-    STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
-    hipLaunchKernelGGL((tcspmm_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
-                       f_tiles, A, B, d_C, d_indptr, d_indices);
-    STIR_LAUNCH_CHECK();
-    hipLaunchKernelGGL(tcspmm_long_kernel<kLongNT>, dim3((unsigned)long_blocks), dim3(64 * kLongWaves), kLongLds, st,
-                       feat, (int64_t)mb, long_f_tiles, A, B, d_C, d_indptr, d_indices);
+  const bool out32 = out_dtype == STIR_F32;
+  switch (tile_size) {
+    case 8: return launch_unplanned<8>(out32, mb, feat, A, B, d_C, d_indptr, d_indices, st);
+    case 16: return launch_unplanned<16>(out32, mb, feat, A, B, d_C, d_indptr, d_indices, st);
+    default: return launch_unplanned<32>(out32, mb, feat, A, B, d_C, d_indptr, d_indices, st);
   }
-  STIR_LAUNCH_CHECK();
-  return 0;
 }
 
 struct stir_tc_plan {
@@ -551,21 +678,13 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
                                         const void* d_B, void* d_C, const int32_t* d_indptr,
                                         const int32_t* d_indices, void* stream) {
   STIR_REQUIRE(plan, "tc_spmm_planned: plan is null");
-  STIR_REQUIRE(out_dtype == STIR_F16 || out_dtype == STIR_F32, "tc_spmm: out_dtype must be STIR_F16 or STIR_F32");
+  if (check_args(out_dtype, mb, tile_size, group_size, feat, nnzb, d_A, d_B, d_C, d_indptr, d_indices)) return -1;
   STIR_REQUIRE(plan->mb == mb, "tc_spmm_planned: the plan was made for %d row tiles, not %d", plan->mb, mb);
   int device = 0;
   STIR_HIP(hipGetDevice(&device));
   STIR_REQUIRE(device == plan->device, "tc_spmm_planned: the plan lives on device %d, the current device is %d",
                plan->device, device);
-  STIR_REQUIRE(tile_size == kTile && group_size == kGroup,
-               "tc_spmm: tile_size=%d group_size=%d; the MFMA path needs t=32, g=16", tile_size, group_size);
-  STIR_REQUIRE(mb >= 0 && nnzb >= 0, "tc_spmm: bad sizes");
-  STIR_REQUIRE(feat > 0 && feat % 32 == 0, "tc_spmm: feat=%d must be a multiple of 32", feat);
   if (mb == 0) return 0;
-  STIR_REQUIRE(d_B && d_C && d_indptr && (nnzb == 0 || (d_A && d_indices)), "tc_spmm: null pointer argument");
-  const int f_tiles = (int)stir::ceil_div(feat, kTileF);
-  const int64_t blocks = (int64_t)mb * f_tiles;
-  STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* A = static_cast<const uint16_t*>(d_A);
   const uint16_t* B = static_cast<const uint16_t*>(d_B);
@@ -573,8 +692,8 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
   const bool out32 = out_dtype == STIR_F32;
   STIR_REQUIRE(plan->n_multi == 0 || reinterpret_cast<uintptr_t>(d_C) % (out32 ? 16 : 8) == 0,
                "tc_spmm: C must be %d-byte aligned", out32 ? 16 : 8);
-  // the partial tiles of this feature width
-  const size_t need = size_t(plan->slots) * kTile * size_t(feat) * sizeof(float);
+  // the partial tiles of this tile size and feature width
+  const size_t need = size_t(plan->slots) * size_t(tile_size) * size_t(feat) * sizeof(float);
   if (need > plan->scratch_bytes) {
     if (plan->d_scratch) STIR_HIP(hipFree(plan->d_scratch));
     plan->d_scratch = nullptr;
@@ -582,41 +701,15 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
     STIR_HIP(hipMalloc(reinterpret_cast<void**>(&plan->d_scratch), need));
     plan->scratch_bytes = need;
   }
-  // the tiles of up to kLongSteps steps
-  if (out32)
-    hipLaunchKernelGGL((tcspmm_kernel<1, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
-                       f_tiles, A, B, d_C, d_indptr, d_indices);
-  else
-    hipLaunchKernelGGL((tcspmm_kernel<0, false, true>), dim3((unsigned)blocks), dim3(256), 0, st, feat, (int64_t)mb,
-                       f_tiles, A, B, d_C, d_indptr, d_indices);
-  STIR_LAUNCH_CHECK();
-  if (plan->n_pieces > 0) {
-    constexpr int kLongTF = 32 * kLongNT, kLongWaves = 32 / kLongNT;
-    constexpr size_t kLongLds = size_t(kLongWaves) * 16 * kLongTF * sizeof(uint32_t);
-    const int long_f_tiles = (int)stir::ceil_div(feat, kLongTF);
-    const int64_t long_blocks = plan->n_pieces * long_f_tiles;
-    STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many pieces for one launch");
-    if (out32)
-      hipLaunchKernelGGL((tcspmm_pieces_kernel<kLongNT, 1>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
-                         kLongLds, st, feat, long_f_tiles, plan->d_pieces, A, B, d_C, plan->d_scratch, d_indptr,
-                         d_indices);
-    else
-      hipLaunchKernelGGL((tcspmm_pieces_kernel<kLongNT, 0>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
-                         kLongLds, st, feat, long_f_tiles, plan->d_pieces, A, B, d_C, plan->d_scratch, d_indptr,
-                         d_indices);
-    STIR_LAUNCH_CHECK();
-    if (plan->n_multi > 0) {
-      const int chunks = (int)stir::ceil_div((int64_t)kTile * feat, 1024);
-      STIR_REQUIRE(plan->n_multi * chunks < (int64_t(1) << 31), "tc_spmm: too many partial tiles for one launch");
-      if (out32)
-        hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<1>, dim3((unsigned)(plan->n_multi * chunks)), dim3(256), 0, st, feat,
-                           chunks, plan->d_multi, plan->d_scratch, d_C);
-      else
-        hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<0>, dim3((unsigned)(plan->n_multi * chunks)), dim3(256), 0, st, feat,
-                           chunks, plan->d_multi, plan->d_scratch, d_C);
-      STIR_LAUNCH_CHECK();
-    }
+  switch (tile_size) {
+    case 8:
+      return launch_planned<8>(out32, mb, feat, plan->n_pieces, plan->n_multi, plan->d_pieces, plan->d_multi,
+                               plan->d_scratch, A, B, d_C, d_indptr, d_indices, st);
+    case 16:
+      return launch_planned<16>(out32, mb, feat, plan->n_pieces, plan->n_multi, plan->d_pieces, plan->d_multi,
+                                plan->d_scratch, A, B, d_C, d_indptr, d_indices, st);
+    default:
+      return launch_planned<32>(out32, mb, feat, plan->n_pieces, plan->n_multi, plan->d_pieces, plan->d_multi,
+                                plan->d_scratch, A, B, d_C, d_indptr, d_indices, st);
   }
-  return 0;
 }
-

@@ -305,12 +305,13 @@ class TcSpMM(_Operator):
         self.t, self.g, self.brows = int(tile_size), int(group_size), int(num_b_rows)
         self.out_dtype = out_dtype
         self.L = _lib.lib()
-        self._plan, self._key = None, None
+        self._plan, self._key, self._keep = None, None, None
 
     def _drop_plan(self):
         if self._plan is not None:
             self.L.stir_tc_plan_destroy(self._plan)
             self._plan = None
+        self._keep = None
 
     def invalidate(self):
         """Forget the plan made from the contents ``indptr`` had at the last call."""
@@ -330,7 +331,7 @@ class TcSpMM(_Operator):
                                  ("indptr", i32, self.mb + 1), ("indices", i32, self.nnzb * self.g)])
         a, b, c, indptr, indices = args
         with torch.cuda.device(dev):
-            if (self.t, self.g) != (32, 16):  # refused by the library with its own message
+            if self.t not in (8, 16, 32) or self.g != 16:  # refused by the library with its own message
                 _lib.check(self.L.stir_tc_spmm_f16(_DT[self.out_dtype], self.mb, self.t, self.g, self.feat,
                                                    self.nnzb, _ptr(a), _ptr(b), _ptr(c), _ptr(indptr),
                                                    _ptr(indices), _stream()))
@@ -341,7 +342,9 @@ class TcSpMM(_Operator):
                 self._drop_plan()
                 plan = ctypes.c_void_p()
                 _lib.check(self.L.stir_tc_plan_create(ctypes.byref(plan), self.mb, _ptr(indptr), _stream()))
-                self._plan, self._key = plan, key
+                # the array stays alive with the plan: its address cannot be handed to another
+                # indptr array (same size, version 0) that the key would take for this one
+                self._plan, self._key, self._keep = plan, key, indptr
             _lib.check(self.L.stir_tc_spmm_f16_planned(self._plan, _DT[self.out_dtype], self.mb, self.t, self.g,
                                                        self.feat, self.nnzb,
                                                        _ptr(a), _ptr(b), _ptr(c), _ptr(indptr), _ptr(indices),

@@ -16,8 +16,8 @@ pytestmark = pytest.mark.gpu
 STIR_F16, STIR_F32 = 0, 2  # include/sparsetir_amd.h
 
 
-def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0):
-    t, g = 32, 16
+def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0, t=32):
+    g = 16
     gptr, tiles, mask = st.condense(indptr, indices, t, g)
     want_fmt = oracle.condense(indptr, indices, t, g)
     for a, b in zip((gptr, tiles, mask), want_fmt):
@@ -66,17 +66,25 @@ def _run(dev, indptr, indices, n, feat, weighted, out_dtype, seed=0):
     check(c, "without a plan")
 
 
+# tile sizes: 8 and 16 are what the reference condenses with (tile_size = mma_m of m8n32k16 and
+# m16n16k16, examples/spmm/bench_tc_spmm.py:584-585,670), 32 fills the 32x32x16 instruction
+TILES = [8, 16, 32]
+
+
+@pytest.mark.parametrize("t", TILES)
 @pytest.mark.parametrize("feat", [32, 64, 128, 256, 160])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
-def test_tcspmm_small(dev, feat, out_dtype):
-    m, n = 1000, 777
+def test_tcspmm_small(dev, feat, out_dtype, t):
+    m, n = 1000 + t // 8, 777  # the last tile is partial at every tile size
     indptr, indices = random_csr(m, n, 20000, feat, skew=1.0)
-    _run(dev, indptr, indices, n, feat, weighted=(feat % 64 == 0), out_dtype=out_dtype, seed=feat)
+    _run(dev, indptr, indices, n, feat, weighted=(feat % 64 == 0), out_dtype=out_dtype, seed=feat, t=t)
 
 
-def test_tcspmm_config2_graph(dev):
+@pytest.mark.parametrize("t,out_dtype", [(8, torch.float16), (16, torch.float16), (32, torch.float32),
+                                         (16, torch.float32)])
+def test_tcspmm_config2_graph(dev, t, out_dtype):
     g = datasets.config2()
-    _run(dev, g["indptr"], g["indices"], g["n"], 128, weighted=False, out_dtype=torch.float32)
+    _run(dev, g["indptr"], g["indices"], g["n"], 128, weighted=False, out_dtype=out_dtype, t=t)
 
 
 def test_tcspmm_empty_tiles_and_errors(dev):
@@ -86,13 +94,19 @@ def test_tcspmm_empty_tiles_and_errors(dev):
     indices = np.asarray([1, 7, 9], np.int32)
     _run(dev, indptr, indices, n, 64, weighted=False, out_dtype=torch.float16)
     z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
-    f = ops.build_tcspmm(1, 1, 32, 16, 16, 4)
-    with pytest.raises(SparseTIRError, match="t=32"):
-        f(z(256, torch.float16), z(128, torch.float16), z(512, torch.float16), z(2, torch.int32), z(16, torch.int32))
+    _run(dev, indptr, indices, n, 64, weighted=False, out_dtype=torch.float16, t=8)
+    _run(dev, indptr, indices, n, 32, weighted=False, out_dtype=torch.float32, t=16)
+    # a tile size without a matrix-core shape, and a group size other than the k extent
+    for t, g in ((4, 16), (16, 8)):
+        f = ops.build_tcspmm(1, 1, 32, t, g, 4)
+        with pytest.raises(SparseTIRError, match="t in"):
+            f(z(t * g, torch.float16), z(128, torch.float16), z(t * 32, torch.float16), z(2, torch.int32),
+              z(g, torch.int32))
 
 
+@pytest.mark.parametrize("t", TILES)
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
-def test_tcspmm_hub_tile(dev, out_dtype):
+def test_tcspmm_hub_tile(dev, out_dtype, t):
     """One row with 9000 distinct columns: its tile has 563 groups = 282 steps, which the fp32
     path cuts into equal units that meet in atomics; C starts as NaN, so the rows of that tile
     must be cleared first.  Another tile lies just above the length of one unit.  Two feature
@@ -104,28 +118,30 @@ def test_tcspmm_hub_tile(dev, out_dtype):
     deg[150] = 530   # 34 groups = 17 steps: just above one unit
     indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
     indices = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
-    _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=9)
+    _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=9, t=t)
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("tiles,feat", [(40, 96), (9, 64), (67, 32)])
-def test_tcspmm_every_tile_long(dev, tiles, feat, out_dtype):
+@pytest.mark.parametrize("tiles,feat,t", [(40, 96, 32), (9, 64, 32), (67, 32, 32), (40, 96, 16), (67, 32, 16)])
+def test_tcspmm_every_tile_long(dev, tiles, feat, out_dtype, t):
     """Rows of about 40 entries over 3000 columns: every row tile has more than a thousand
     distinct columns, i.e. 35 to 40 steps.  With fp16 output a workgroup of the launch for long
     tiles then works on several tiles in turn (it looks at eight, a whole grid apart); tile counts
     that are and are not multiples of eight, and a last tile with fewer than 32 rows."""
     m, n = tiles * 32 - 5, 3000
-    indptr, indices = random_csr(m, n, 40 * m, tiles, skew=0.0)
-    _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=tiles)
+    per_row = 40 * 32 // t  # 16-row tiles of 80 entries per row reach the same 35 to 40 steps
+    indptr, indices = random_csr(m, n, per_row * m, tiles, skew=0.0)
+    _run(dev, indptr, indices, n, feat, weighted=False, out_dtype=out_dtype, seed=tiles, t=t)
 
 
-def test_tcspmm_plan_entry_points(dev):
+@pytest.mark.parametrize("t", [32, 8])
+def test_tcspmm_plan_entry_points(dev, t):
     """stir_tc_plan_create / stir_tc_spmm_f16_planned through the C ABI: one plan used at three
     feature widths in turn (its memory for partial tiles grows with the widest), a plan for a
     matrix without long tiles, the row-tile count checked against the plan's, and an in-place
     change of the group counts followed by the operator's invalidate()."""
     L = _lib.lib()
-    t, g = 32, 16
+    g = 16
     m, n = 300, 12000
     rng = np.random.default_rng(41)
     deg = rng.integers(0, 10, m)
@@ -165,7 +181,7 @@ def test_tcspmm_plan_entry_points(dev):
 
     # no long tile at all: the plan is empty and the launch is the first kernel alone
     indptr2, indices2 = random_csr(200, 500, 1500, 7, skew=0.0)
-    _run(dev, indptr2, indices2, 500, 64, weighted=False, out_dtype=torch.float16)
+    _run(dev, indptr2, indices2, 500, 64, weighted=False, out_dtype=torch.float16, t=t)
 
     # the operator after its indptr array was rewritten in place: invalidate() makes a new plan
     feat = 64
