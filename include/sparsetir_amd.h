@@ -223,6 +223,19 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
                          int32_t num_buckets, const int32_t* bucket_widths,
                          const int64_t* nrows, const float* const* d_A,
                          const int32_t* const* d_rows, const int32_t* const* d_cols);
+/*
+ * The same with flags.  STIR_PLAN_ADDRESSES_ONLY: the plan holds the addresses and sizes of the
+ * arrays and nothing derived from what they contain -- always one launch with atomics in every
+ * adding bucket (the rule of examples/spmm/bench_spmm.py:170), whatever the partition count --
+ * so the arrays may be rewritten in place between launches, as with the reference's built
+ * operator, which reads them at every call.  It is what the PackedFunc layer uses until the
+ * caller promises static index arrays ("sparsetir.static_structure").
+ */
+#define STIR_PLAN_ADDRESSES_ONLY 1u
+int stir_hyb_plan_create_ex(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,
+                            int32_t num_buckets, const int32_t* bucket_widths,
+                            const int64_t* nrows, const float* const* d_A,
+                            const int32_t* const* d_rows, const int32_t* const* d_cols, uint32_t flags);
 int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B, float* d_C,
                       void* stream);
 int stir_hyb_plan_destroy(stir_hyb_plan* plan);
@@ -362,6 +375,15 @@ int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_
  * plan has been launched with the other setting.
  */
 int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on);
+/*
+ * The opposite choice, made before the first launch: the plan never builds an edge index, so
+ * nothing in it depends on what the index arrays hold and they may be rewritten in place between
+ * launches (the reference's built operator reads them at every call,
+ * examples/rgms/rgcn/bench_rgcn_tensorcore.py:852).  Every launch is then the kernel of the small
+ * inputs at any size: one fp32 atomic per (ELL row, output feature), about four times the run
+ * time of the indexed form at 2M edges.  Fails once the plan has built its index.
+ */
+int stir_rgms_plan_set_addresses_only(stir_rgms_plan* plan, int32_t on);
 /* The same with bf16 W, X and slot weights (the reference has an fp16 example only). */
 int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
                    int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,

@@ -105,22 +105,35 @@ enum {
  *      examples/rgms/rgcn/bench_rgcn_composable.py:208-221
  * "sparsetir.rgms_csf"       (A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j, feat_in, feat_out)
  *      examples/rgms/rgcn/bench_rgcn_non_composable.py:109         fp32, W [R, feat_out, feat_in]
- * "sparsetir.invalidate_plans" ()
+ * "sparsetir.static_structure" (on)
  *      no counterpart in the reference, whose built operators read their index arrays on every
- *      call.  Here "sparsetir.hyb_csrmm", "sparsetir.rgms" and "sparsetir.rgms_f32" keep one plan
- *      each per process, reused while the array addresses and sizes of a call equal those of the
- *      previous one.  A plan holds what was derived from the index arrays' contents (rgms: the
- *      edge index built by the first launch over 8192 slots or more; hyb_csrmm with 2 to 4
- *      partitions: whether its buckets need atomics).  A caller that rewrites rows / cols / mids
- *      in place, or frees them and gets arrays of the same sizes at the same addresses, calls
- *      this first; the next operator call then builds a fresh plan.  Edge weights (A_k), W, X, B
- *      may change freely.
+ *      call.  Default off: "sparsetir.hyb_csrmm" and "sparsetir.rgms" then do the same -- their
+ *      cached plans hold the addresses and sizes of the arrays and nothing derived from their
+ *      contents (hyb: one launch, atomics in every adding bucket, the rule of
+ *      examples/spmm/bench_spmm.py:170; rgms: one fp32 atomic per ELL row and output feature), so
+ *      rows / cols / mids may be rewritten in place, or freed and replaced by arrays of the same
+ *      sizes at the same addresses, at any time.  on != 0 is the promise that these index arrays
+ *      keep their contents for as long as they keep their addresses, which is how every script of
+ *      the reference uses them (decomposed once, then timed).  Plans made from then on keep what
+ *      they derive from the contents: rgms the edge index by destination tile that its first
+ *      launch over 8192 slots or more builds (about four times faster at 2M edges), hyb_csrmm with
+ *      2 to 4 partitions whether its buckets need atomics, with more than 4 the slot list of every
+ *      output row.  Changing the setting drops the cached plans.  Edge weights (A_k), W, X, B may
+ *      change freely under either setting.
+ * "sparsetir.invalidate_plans" ()
+ *      no counterpart in the reference.  "sparsetir.hyb_csrmm", "sparsetir.rgms" and
+ *      "sparsetir.rgms_f32" each keep the eight plans used last, found again by the addresses and
+ *      sizes of a call's arrays (a ninth plan replaces the one whose last use lies furthest back),
+ *      so a caller that alternates between a few graphs builds each plan once.  This call
+ *      destroys them all.  A caller that has promised static structure and then does rewrite
+ *      rows / cols / mids in place calls it before the next operator call.
  * "sparsetir.rgms_static_weights" (on)
  *      no counterpart in the reference.  on != 0: the plans "sparsetir.rgms" makes from now on carry
  *      the promise of stir_rgms_plan_set_static_weights -- the A_k keep the values they have at the
  *      plan's first call (the reference's A_k is the 0/1 mask of CSFToELL3D, written once) -- and
- *      leave the zero-weight padding slots out of their edge index.  Drops the cached plan when the
- *      setting changes.  Default off.
+ *      leave the zero-weight padding slots out of their edge index.  Takes effect together with
+ *      "sparsetir.static_structure"(1): without that promise no index is kept.  Drops the cached
+ *      plans when the setting changes.  Default off.
  *
  * Format pass (host tensors, kDLCPU, as in the reference, or device tensors; the reference returns
  * nested Array<NDArray>, which needs libtvm objects, so here a sizing call is followed by a fill
@@ -154,12 +167,17 @@ int stir_packed_rgms_f32(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms_csf(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_invalidate_plans(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_rgms_static_weights(TVMValue*, int*, int, TVMRetValueHandle, void*);
+int stir_packed_static_structure(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_column_part_hyb_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_csf_to_ell3d_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_csf_to_ell3d_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_condense_sizes(TVMValue*, int*, int, TVMRetValueHandle, void*);
 int stir_packed_condense_fill(TVMValue*, int*, int, TVMRetValueHandle, void*);
+
+/* Plans the packed operators have made since the library was loaded (a call that finds its
+ * plan among the cached ones makes none): lets a caller see that alternating graphs reuse plans. */
+int64_t stir_packed_plan_builds(void);
 
 /* Number of packed operators, and the i-th one's global name / function. */
 int stir_packed_count(void);

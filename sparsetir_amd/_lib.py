@@ -40,6 +40,7 @@ SIGNATURES = {
     "stir_csr_to_bsr_fill": (I32, [I32, I32, I32, VP, VP, VP, VP, VP, VP, VP, I32, I64, VP]),
     "stir_csr_spmm_f32": (I32, [I32, I32, I32, I64, VP, VP, VP, VP, VP, VP]),
     "stir_hyb_plan_create": (I32, [VP, I32, I32, I32, I32, VP, VP, VP, VP, VP]),
+    "stir_hyb_plan_create_ex": (I32, [VP, I32, I32, I32, I32, VP, VP, VP, VP, VP, ctypes.c_uint32]),
     "stir_hyb_spmm_f32": (I32, [VP, I32, VP, VP, VP]),
     "stir_hyb_plan_destroy": (I32, [VP]),
     "stir_hyb_spmm_f32_noalloc": (I32, [I32, I32, I32, I32, VP, VP, VP, VP, VP, I32, VP, VP, VP]),
@@ -56,6 +57,7 @@ SIGNATURES = {
     "stir_rgms_f16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
     "stir_rgms_bf16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
     "stir_rgms_plan_set_static_weights": (I32, [VP, I32]),
+    "stir_rgms_plan_set_addresses_only": (I32, [VP, I32]),
     "stir_rgms_plan_destroy": (I32, [VP]),
     "stir_rgms_f32_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f32": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),

@@ -168,20 +168,64 @@ struct DeviceGuard {
 
 bool fits_i32(int64_t x) { return x >= 0 && x <= INT32_MAX; }
 
-// ---- cached plans for the plan-based kernels: rebuilt when any pointer or size changes
+// ---- cached plans for the plan-based kernels.  A plan is found again by the addresses and sizes
+// of the arrays it was made from; each operator keeps the kPlanCacheEntries plans used last, so a
+// caller that alternates between a few graphs (mini-batches, training and validation sets) builds
+// each plan once.  Making a plan beyond that number destroys the one whose last use lies furthest
+// back.
 struct HybKey {
   std::vector<uintptr_t> ptrs;
   std::vector<int64_t> nums;
   bool operator==(const HybKey& o) const { return ptrs == o.ptrs && nums == o.nums; }
 };
-std::mutex g_plan_mutex;
-HybKey g_hyb_key;
-stir_hyb_plan* g_hyb_plan = nullptr;
-HybKey g_rgms_key;
-stir_rgms_plan* g_rgms_plan = nullptr;
-bool g_rgms_static_weights = false;  // promise for the plans "sparsetir.rgms" makes from now on
-HybKey g_rgms_f32_key;
-stir_rgms_f32_plan* g_rgms_f32_plan = nullptr;
+constexpr size_t kPlanCacheEntries = 8;
+std::mutex g_plan_mutex;   // guards the caches, the promises and the counter below
+int64_t g_plan_builds = 0;  // plans made by the PackedFuncs since the library was loaded
+
+template <class Plan>
+struct PlanCache {
+  struct Entry {
+    HybKey key;
+    Plan* plan;
+    uint64_t used;
+  };
+  int (*destroy)(Plan*);
+  std::vector<Entry> entries;
+  uint64_t clock = 0;
+  explicit PlanCache(int (*d)(Plan*)) : destroy(d) {}
+  Plan* find(const HybKey& key) {
+    for (Entry& e : entries)
+      if (e.key == key) {
+        e.used = ++clock;
+        return e.plan;
+      }
+    return nullptr;
+  }
+  void insert(const HybKey& key, Plan* plan) {
+    if (entries.size() >= kPlanCacheEntries) {
+      size_t oldest = 0;
+      for (size_t i = 1; i < entries.size(); ++i)
+        if (entries[i].used < entries[oldest].used) oldest = i;
+      destroy(entries[oldest].plan);
+      entries.erase(entries.begin() + (std::ptrdiff_t)oldest);
+    }
+    entries.push_back(Entry{key, plan, ++clock});
+    ++g_plan_builds;
+  }
+  void clear() {
+    for (Entry& e : entries) destroy(e.plan);
+    entries.clear();
+  }
+};
+PlanCache<stir_hyb_plan> g_hyb_plans(stir_hyb_plan_destroy);
+PlanCache<stir_rgms_plan> g_rgms_plans(stir_rgms_plan_destroy);
+PlanCache<stir_rgms_f32_plan> g_rgms_f32_plans(stir_rgms_f32_plan_destroy);
+// Promises of the caller for the plans made from now on.  Without the first, a cached plan holds
+// addresses and sizes only and every call reads the index arrays afresh, as the reference's built
+// operators do; with it, plans may keep what they derive from the contents of the index arrays
+// (the verdict that drops atomics and the slot lists of hyb, the edge index of RGMS).
+bool g_static_structure = false;
+bool g_rgms_static_weights = false;
 
 }  // namespace
 
@@ -262,17 +306,19 @@ int stir_packed_hyb_csrmm(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*)
   }
   for (int b = 0; b < nb; ++b) key.nums.push_back(widths[b]);
   key.nums.push_back(parts);
+  key.nums.push_back(C.len / feat);
+  key.nums.push_back(B.len / feat);
   key.nums.push_back(a.dev_id);
   std::lock_guard<std::mutex> lock(g_plan_mutex);
-  if (!g_hyb_plan || !(key == g_hyb_key)) {
-    if (g_hyb_plan) stir_hyb_plan_destroy(g_hyb_plan);
-    g_hyb_plan = nullptr;
-    if (stir_hyb_plan_create(&g_hyb_plan, (int32_t)(C.len / feat), (int32_t)(B.len / feat), (int32_t)parts, nb,
-                             widths.data(), nrows.data(), Ak.data(), Rk.data(), Ck.data()))
+  stir_hyb_plan* plan = g_hyb_plans.find(key);
+  if (!plan) {
+    if (stir_hyb_plan_create_ex(&plan, (int32_t)(C.len / feat), (int32_t)(B.len / feat), (int32_t)parts, nb,
+                                widths.data(), nrows.data(), Ak.data(), Rk.data(), Ck.data(),
+                                g_static_structure ? 0u : STIR_PLAN_ADDRESSES_ONLY))
       return forward(-1);
-    g_hyb_key = key;
+    g_hyb_plans.insert(key, plan);
   }
-  return forward(stir_hyb_spmm_f32(g_hyb_plan, (int32_t)feat, (const float*)B.data, (float*)C.data, g_stream));
+  return forward(stir_hyb_spmm_f32(plan, (int32_t)feat, (const float*)B.data, (float*)C.data, g_stream));
 }
 
 static int sddmm_common(const char* fn, bool preproc, TVMValue* v, int* tc, int n) {
@@ -454,34 +500,37 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
   std::lock_guard<std::mutex> lock(g_plan_mutex);
   const int32_t mm = (int32_t)(Y.len / fout), nn = (int32_t)(X.len / fin), rr = (int32_t)(W.len / (fin * fout));
   if (f32) {
-    if (!g_rgms_f32_plan || !(key == g_rgms_f32_key)) {
-      if (g_rgms_f32_plan) stir_rgms_f32_plan_destroy(g_rgms_f32_plan);
-      g_rgms_f32_plan = nullptr;
+    stir_rgms_f32_plan* plan = g_rgms_f32_plans.find(key);
+    if (!plan) {
       std::vector<const float*> Af(nb);
       for (int b = 0; b < nb; ++b) Af[b] = (const float*)Ak[b];
-      if (stir_rgms_f32_plan_create(&g_rgms_f32_plan, nb, rb.data(), cb.data(), groups.data(), Af.data(),
-                                    Rk.data(), Ck.data(), Mk.data()))
+      if (stir_rgms_f32_plan_create(&plan, nb, rb.data(), cb.data(), groups.data(), Af.data(), Rk.data(), Ck.data(),
+                                    Mk.data()))
         return forward(-1);
-      g_rgms_f32_key = key;
+      g_rgms_f32_plans.insert(key, plan);
     }
-    return forward(stir_rgms_f32(g_rgms_f32_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, (const float*)W.data,
+    return forward(stir_rgms_f32(plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, (const float*)W.data,
                                  (const float*)X.data, (float*)Y.data, g_stream));
   }
-  if (!g_rgms_plan || !(key == g_rgms_key)) {
-    if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
-    g_rgms_plan = nullptr;
-    if (stir_rgms_plan_create(&g_rgms_plan, nb, rb.data(), cb.data(), groups.data(), Ak.data(), Rk.data(),
-                              Ck.data(), Mk.data()))
+  // an edge index also depends on the sizes the launch is given
+  key.nums.push_back(mm);
+  key.nums.push_back(nn);
+  key.nums.push_back(rr);
+  stir_rgms_plan* plan = g_rgms_plans.find(key);
+  if (!plan) {
+    if (stir_rgms_plan_create(&plan, nb, rb.data(), cb.data(), groups.data(), Ak.data(), Rk.data(), Ck.data(),
+                              Mk.data()))
       return forward(-1);
-    if (g_rgms_static_weights && stir_rgms_plan_set_static_weights(g_rgms_plan, 1)) {
-      stir_rgms_plan_destroy(g_rgms_plan);
-      g_rgms_plan = nullptr;
+    // weights inside the index only when the structure may be kept at all
+    if ((!g_static_structure && stir_rgms_plan_set_addresses_only(plan, 1)) ||
+        (g_static_structure && g_rgms_static_weights && stir_rgms_plan_set_static_weights(plan, 1))) {
+      stir_rgms_plan_destroy(plan);
       return forward(-1);
     }
-    g_rgms_key = key;
+    g_rgms_plans.insert(key, plan);
   }
-  return forward((bf ? stir_rgms_bf16 : stir_rgms_f16)(g_rgms_plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data,
-                                                       X.data, (float*)Y.data, g_stream));
+  return forward((bf ? stir_rgms_bf16 : stir_rgms_f16)(plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data, X.data,
+                                                       (float*)Y.data, g_stream));
 }
 
 int stir_packed_rgms(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
@@ -495,13 +544,32 @@ int stir_packed_rgms_f32(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) 
 int stir_packed_invalidate_plans(TVMValue*, int*, int n, TVMRetValueHandle, void*) {
   if (n != 0) return packed_fail("sparsetir.invalidate_plans: num_args should be 0");
   std::lock_guard<std::mutex> lock(g_plan_mutex);
-  if (g_hyb_plan) stir_hyb_plan_destroy(g_hyb_plan);
-  if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
-  if (g_rgms_f32_plan) stir_rgms_f32_plan_destroy(g_rgms_f32_plan);
-  g_hyb_plan = nullptr;
-  g_rgms_plan = nullptr;
-  g_rgms_f32_plan = nullptr;
+  g_hyb_plans.clear();
+  g_rgms_plans.clear();
+  g_rgms_f32_plans.clear();
   return 0;
+}
+
+// "sparsetir.static_structure"(on): the promise that the index arrays (rows_k, cols_k, mids_k)
+// handed to hyb_csrmm / rgms keep their contents for as long as they keep their addresses
+int stir_packed_static_structure(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
+  Args a{"sparsetir.static_structure", v, tc, n};
+  if (!a.count(1)) return -1;
+  const int64_t on = a.integer(0, "on");
+  if (!a.ok) return -1;
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  if (g_static_structure != (on != 0)) {
+    // the cached plans were made under the other setting
+    g_hyb_plans.clear();
+    g_rgms_plans.clear();
+  }
+  g_static_structure = on != 0;
+  return 0;
+}
+
+int64_t stir_packed_plan_builds(void) {
+  std::lock_guard<std::mutex> lock(g_plan_mutex);
+  return g_plan_builds;
 }
 
 int stir_packed_rgms_static_weights(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) {
@@ -510,11 +578,7 @@ int stir_packed_rgms_static_weights(TVMValue* v, int* tc, int n, TVMRetValueHand
   const int64_t on = a.integer(0, "on");
   if (!a.ok) return -1;
   std::lock_guard<std::mutex> lock(g_plan_mutex);
-  if (g_rgms_static_weights != (on != 0)) {
-    // the cached plan was made under the other setting
-    if (g_rgms_plan) stir_rgms_plan_destroy(g_rgms_plan);
-    g_rgms_plan = nullptr;
-  }
+  if (g_rgms_static_weights != (on != 0)) g_rgms_plans.clear();  // made under the other setting
   g_rgms_static_weights = on != 0;
   return 0;
 }
@@ -548,13 +612,26 @@ int stir_packed_rgms_csf(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) 
 // ----------------------------------------------------------------------------- format pass
 
 // Scratch of a device format pass, kept per thread between its sizing and its fill call.  It
-// belongs to the device it was allocated on: a call for another device starts over.
+// belongs to the device it was allocated on: a call for another device starts over.  The sizing
+// call leaves the layout of the scratch behind, and that layout follows from its arguments: the
+// fill call must come with the same input (`key`: addresses, sizes, bucket lists) and with
+// outputs of the lengths the sizing call returned (`counts`), or its kernels would read offsets
+// and write lengths that belong to another input.
 struct FormatScratch {
   void* ptr = nullptr;
   size_t bytes = 0;
   int dev = -1;
+  bool sized = false;
+  std::vector<int64_t> key, counts;
+  void forget() { sized = false, key.clear(), counts.clear(); }
+  void remember(std::vector<int64_t> k, const int64_t* c, size_t n) {
+    key = std::move(k);
+    counts.assign(c, c + n);
+    sized = true;
+  }
   // at least `need` bytes on device `dev_id` (which must be current), nullptr when that fails
   void* reserve(int dev_id, size_t need) {
+    forget();
     if (ptr && (dev != dev_id || need > bytes)) {
       (void)hipFree(ptr);
       ptr = nullptr;
@@ -571,8 +648,16 @@ struct FormatScratch {
     return ptr;
   }
   // what the sizing call left for device `dev_id`, or nullptr
-  void* get(int dev_id) const { return dev == dev_id ? ptr : nullptr; }
+  void* get(int dev_id) const { return dev == dev_id && sized ? ptr : nullptr; }
+  // the fill call's own key against the sizing call's; false with a recorded message
+  bool same_input(const char* fn, const std::vector<int64_t>& k) const {
+    if (k == key) return true;
+    packed_fail("%s: the arguments differ from those of the .sizes call before it on this thread "
+                "(arrays, sizes or bucket lists)", fn);
+    return false;
+  }
 };
+static int64_t addr_of(const void* p) { return (int64_t)(uintptr_t)p; }
 static thread_local FormatScratch g_hyb_scratch, g_csf_scratch, g_condense_scratch;
 
 static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
@@ -591,6 +676,11 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
   if (!a.ok) return -1;
   const int nb = (int)Bk.len;
   const int64_t nk = parts * nb;
+  auto hyb_key = [&]() {
+    std::vector<int64_t> k = {num_rows, num_cols, addr_of(P.data), addr_of(I.data), I.len, parts, nb, a.dev_id};
+    for (int b = 0; b < nb; ++b) k.push_back(((const int32_t*)Bk.data)[b]);
+    return k;
+  };
   DeviceGuard g;
   if (dev && g.enter(a.dev_id)) return forward(-1);
   if (!fill) {
@@ -604,9 +694,11 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
     const size_t need = stir_column_part_hyb_device_workspace_bytes((int32_t)num_rows, (int32_t)parts, nb, I.len);
     void* ws = g_hyb_scratch.reserve(a.dev_id, need);
     if (!ws) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
-    return forward(stir_column_part_hyb_device_sizes((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
+    const int rc = stir_column_part_hyb_device_sizes((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
                                                      (const int32_t*)I.data, (int32_t)parts,
-                                                     (const int32_t*)Bk.data, nb, ws, (int64_t*)N.data, g_stream));
+                                                     (const int32_t*)Bk.data, nb, ws, (int64_t*)N.data, g_stream);
+    if (rc == 0) g_hyb_scratch.remember(hyb_key(), (const int64_t*)N.data, (size_t)nk);
+    return forward(rc);
   }
   if (!a.count(6 + 3 * (int)nk)) return -1;
   std::vector<int32_t*> R(nk), C(nk), M(nk);
@@ -628,6 +720,14 @@ static int hyb_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
                                              R.data(), C.data(), M.data()));
   void* ws = g_hyb_scratch.get(a.dev_id);
   if (!ws) return packed_fail("%s: call tir.sparse.ColumnPartHyb.sizes first on this thread", fn);
+  if (!g_hyb_scratch.same_input(fn, hyb_key())) return -1;
+  // R[k] has r.len entries; the lengths were read above, so recover them from the arguments
+  for (int64_t k = 0; k < nk; ++k) {
+    const DLTensor* rk = static_cast<const DLTensor*>(v[6 + 3 * (int)k].v_handle);
+    if (rk->shape[0] != g_hyb_scratch.counts[(size_t)k])
+      return packed_fail("%s: rows_%lld has %lld entries, the .sizes call returned %lld", fn, (long long)k,
+                         (long long)rk->shape[0], (long long)g_hyb_scratch.counts[(size_t)k]);
+  }
   int rc = stir_column_part_hyb_device_fill((int32_t)num_rows, (int32_t)num_cols, (const int32_t*)P.data,
                                             (const int32_t*)I.data, (int32_t)parts, (const int32_t*)Bk.data, nb,
                                             ws, R.data(), C.data(), M.data(), g_stream);
@@ -659,6 +759,11 @@ static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
                 *i1 = (const int32_t*)I1.data, *rb = (const int32_t*)RB.data, *cb = (const int32_t*)CB.data;
   if (dev && P1.len != I0.len + 1)
     return packed_fail("%s: csf_indptr_1 must have one entry more than csf_indices_0", fn);
+  auto csf_key = [&]() {
+    std::vector<int64_t> k = {rels, addr_of(p0), addr_of(i0), addr_of(p1), addr_of(i1), I0.len, I1.len, nb, a.dev_id};
+    for (int b = 0; b < nb; ++b) k.push_back(rb[b]), k.push_back(cb[b]);
+    return k;
+  };
   DeviceGuard g;
   if (dev && g.enter(a.dev_id)) return forward(-1);
   if (!fill) {
@@ -669,8 +774,10 @@ static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
     const size_t need = stir_csf_to_ell3d_device_workspace_bytes((int32_t)rels, I0.len, nb);
     void* ws = g_csf_scratch.reserve(a.dev_id, need);
     if (!ws) return packed_fail("%s: cannot allocate %zu bytes of scratch", fn, need);
-    return forward(stir_csf_to_ell3d_device_sizes((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
-                                                  (int64_t*)G.data, g_stream));
+    const int rc = stir_csf_to_ell3d_device_sizes((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
+                                                  (int64_t*)G.data, g_stream);
+    if (rc == 0) g_csf_scratch.remember(csf_key(), (const int64_t*)G.data, (size_t)nb);
+    return forward(rc);
   }
   if (!a.count(6 + 4 * nb)) return -1;
   std::vector<int32_t*> OP(nb), R(nb), C(nb), M(nb);
@@ -695,6 +802,11 @@ static int csf_format(const char* fn, bool fill, TVMValue* v, int* tc, int n) {
                                           M.data()));
   void* ws = g_csf_scratch.get(a.dev_id);
   if (!ws) return packed_fail("%s: call tir.sparse.CSFToELL3D.sizes first on this thread", fn);
+  if (!g_csf_scratch.same_input(fn, csf_key())) return -1;
+  for (int b = 0; b < nb; ++b)
+    if (groups[b] != g_csf_scratch.counts[(size_t)b])
+      return packed_fail("%s: rows_%d holds %lld groups, the .sizes call returned %lld", fn, b, (long long)groups[b],
+                         (long long)g_csf_scratch.counts[(size_t)b]);
   return forward(stir_csf_to_ell3d_device_fill((int32_t)rels, I0.len, I1.len, p0, i0, p1, i1, rb, cb, nb, ws,
                                                groups.data(), OP.data(), R.data(), C.data(), M.data(), g_stream));
 }
@@ -729,9 +841,13 @@ int stir_packed_condense_sizes(TVMValue* v, int* tc, int n, TVMRetValueHandle, v
   const size_t need = stir_condense_device_workspace_bytes((int32_t)rows, I.len, (int32_t)t);
   void* g_condense_ws = g_condense_scratch.reserve(a.dev_id, need);
   if (!g_condense_ws) return packed_fail("%s: cannot allocate %zu bytes of scratch", a.fn, need);
-  return forward(stir_condense_device_sizes((int32_t)rows, I.len, (const int32_t*)P.data, (const int32_t*)I.data,
+  const int rc = stir_condense_device_sizes((int32_t)rows, I.len, (const int32_t*)P.data, (const int32_t*)I.data,
                                             (int32_t)t, (int32_t)g, g_condense_ws, (int32_t*)GP.data,
-                                            (int64_t*)NG.data, g_stream));
+                                            (int64_t*)NG.data, g_stream);
+  if (rc == 0)
+    g_condense_scratch.remember({rows, addr_of(P.data), addr_of(I.data), I.len, t, g, a.dev_id},
+                                (const int64_t*)NG.data, 1);
+  return forward(rc);
 }
 
 // Device form: (indptr, indices, t, g, tile_indices_out, mask_out, group_indptr) -- the seventh
@@ -756,6 +872,10 @@ int stir_packed_condense_fill(TVMValue* v, int* tc, int n, TVMRetValueHandle, vo
   if (!a.ok || !a.len(GP, "group_indptr", (rows + t - 1) / t + 1)) return -1;
   void* g_condense_ws = g_condense_scratch.get(a.dev_id);
   if (!g_condense_ws) return packed_fail("%s: call tir.sparse.ConDense.sizes first on this thread", a.fn);
+  if (!g_condense_scratch.same_input(a.fn, {rows, addr_of(P.data), addr_of(I.data), I.len, t, g, a.dev_id})) return -1;
+  if (TI.len / g != g_condense_scratch.counts[0])
+    return packed_fail("%s: tile_indices_out holds %lld groups, the .sizes call returned %lld", a.fn,
+                       (long long)(TI.len / g), (long long)g_condense_scratch.counts[0]);
   DeviceGuard guard;
   if (guard.enter(a.dev_id)) return forward(-1);
   return forward(stir_condense_device_fill((int32_t)rows, I.len, (const int32_t*)P.data, (const int32_t*)I.data,
@@ -782,6 +902,7 @@ static const PackedEntry kTable[] = {
     {"sparsetir.rgms_csf", stir_packed_rgms_csf},
     {"sparsetir.invalidate_plans", stir_packed_invalidate_plans},
     {"sparsetir.rgms_static_weights", stir_packed_rgms_static_weights},
+    {"sparsetir.static_structure", stir_packed_static_structure},
     {"tir.sparse.ColumnPartHyb.sizes", stir_packed_column_part_hyb_sizes},
     {"tir.sparse.ColumnPartHyb.fill", stir_packed_column_part_hyb_fill},
     {"tir.sparse.CSFToELL3D.sizes", stir_packed_csf_to_ell3d_sizes},

@@ -259,6 +259,7 @@ struct stir_rgms_plan {
   std::vector<stir::TileBucket> tile_buckets;
   int64_t slots;
   bool static_weights;  // promise of the caller, see stir_rgms_plan_set_static_weights
+  bool addresses_only;  // see stir_rgms_plan_set_addresses_only: no edge index, every launch reads the arrays
   stir::TileIndexSet tiles;
 };
 
@@ -313,6 +314,7 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   p->tile_buckets = tile_buckets;
   p->slots = slots;
   p->static_weights = false;
+  p->addresses_only = false;
   hipError_t err = hipSuccess;
   if (nk > 0) {
     err = hipMalloc(reinterpret_cast<void**>(&p->d_table), sizeof(RgmsBucket) * nk);
@@ -344,7 +346,7 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
   hipStream_t st = static_cast<hipStream_t>(stream);
   const uint16_t* W = static_cast<const uint16_t*>(d_W);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
-  if (plan->slots >= kTileMinSlots && plan->slots < (int64_t(1) << 31)) {
+  if (!plan->addresses_only && plan->slots >= kTileMinSlots && plan->slots < (int64_t(1) << 31)) {
     // the plan's edge index and packed copy of W are filled in by the launches: a plan serves
     // one call at a time
     stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
@@ -391,6 +393,14 @@ int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on) {
   STIR_REQUIRE(plan->tiles.m < 0 || plan->static_weights == (on != 0),
                "rgms_plan_set_static_weights: the plan has been launched already");
   plan->static_weights = on != 0;
+  return 0;
+}
+
+int stir_rgms_plan_set_addresses_only(stir_rgms_plan* plan, int32_t on) {
+  STIR_REQUIRE(plan, "rgms_plan_set_addresses_only: plan is null");
+  STIR_REQUIRE(plan->tiles.m < 0 || plan->addresses_only == (on != 0),
+               "rgms_plan_set_addresses_only: the plan has built its edge index already");
+  plan->addresses_only = on != 0;
   return 0;
 }
 

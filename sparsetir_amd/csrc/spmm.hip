@@ -963,11 +963,22 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
                          int32_t num_buckets, const int32_t* bucket_widths, const int64_t* nrows,
                          const float* const* d_A, const int32_t* const* d_rows,
                          const int32_t* const* d_cols) {
+  return stir_hyb_plan_create_ex(plan, m, n, num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols, 0);
+}
+
+int stir_hyb_plan_create_ex(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num_col_parts,
+                            int32_t num_buckets, const int32_t* bucket_widths, const int64_t* nrows,
+                            const float* const* d_A, const int32_t* const* d_rows,
+                            const int32_t* const* d_cols, uint32_t flags) {
   STIR_REQUIRE(plan, "hyb_plan_create: plan is null");
+  STIR_REQUIRE((flags & ~uint32_t(STIR_PLAN_ADDRESSES_ONLY)) == 0, "hyb_plan_create: unknown flags 0x%x", flags);
   if (check_hyb_arguments("hyb_plan_create", m, n, num_col_parts, num_buckets, bucket_widths, nrows, d_A, d_rows,
                           d_cols) != 0)
     return -1;
-  bool phased = num_col_parts > 1 && num_col_parts <= kMaxPhases;
+  // nothing of the plan may depend on what the arrays hold: one launch, atomics in every adding
+  // bucket (the reference's rule), no list of slots per output row
+  const bool addresses_only = (flags & STIR_PLAN_ADDRESSES_ONLY) != 0;
+  bool phased = !addresses_only && num_col_parts > 1 && num_col_parts <= kMaxPhases;
   if (phased && phases_have_single_writers(m, num_col_parts, num_buckets, nrows, d_rows, &phased) != 0) return -1;
   stir_hyb_plan* p = new stir_hyb_plan();
   p->m = m;
@@ -976,7 +987,7 @@ int stir_hyb_plan_create(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t num
   p->num_buckets = num_buckets;
   p->d_tables = nullptr;
   p->merged = false;
-  if (num_col_parts > kMaxPhases &&
+  if (!addresses_only && num_col_parts > kMaxPhases &&
       build_merged_rows(m, num_col_parts * num_buckets, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols,
                         &p->rows, &p->merged) != 0) {
     delete p;

@@ -25,6 +25,7 @@ one dimension, exact dtype, exact length, contiguous, all on one device.  Operat
 mean of ``number`` back-to-back launches between device events
 (src/runtime/profiling.cc:742-797).
 """
+import collections
 import ctypes
 
 import torch
@@ -38,6 +39,47 @@ def _ptr(t):
 
 def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class _PlanCache:
+    """The plans an operator used last, found again by key (addresses and torch version counters
+    of the arrays a plan was made from).  At most ``capacity`` are kept: one more destroys the plan
+    whose last use lies furthest back, so a caller that alternates between a few graphs
+    (mini-batches, training and validation sets) builds each plan once.  ``builds`` counts the
+    plans made.  An entry keeps its arrays alive: their addresses cannot be handed to other arrays
+    while a plan made from them exists."""
+    capacity = 8
+
+    def __init__(self, destroy):
+        self._destroy = destroy
+        self._plans = collections.OrderedDict()  # key -> (plan, arrays kept alive)
+        self.builds = 0
+
+    def get(self, key):
+        hit = self._plans.get(key)
+        if hit is None:
+            return None
+        self._plans.move_to_end(key)
+        return hit[0]
+
+    def put(self, key, plan, keep):
+        while len(self._plans) >= self.capacity:
+            _, (old, _) = self._plans.popitem(last=False)
+            self._destroy(old)
+        self._plans[key] = (plan, keep)
+        self.builds += 1
+
+    def clear(self):
+        while self._plans:
+            _, (old, _) = self._plans.popitem()
+            self._destroy(old)
+
+    def __len__(self):
+        return len(self._plans)
+
+
+def _addr(t):
+    return t.data_ptr() if t.numel() else 0
 
 
 class _Operator:
@@ -121,7 +163,16 @@ class CsrMM(_Operator):
 class HybCsrMM(_Operator):
     """All ELL buckets of all column partitions in one launch.  ``nrows`` lists the ELL rows
     of every bucket, partition-major, the quantity the reference specialises the kernel with
-    (examples/spmm/bench_spmm.py:146-152)."""
+    (examples/spmm/bench_spmm.py:146-152).
+
+    The operator keeps the plans of the array sets it was called with last (see :class:`_PlanCache`),
+    keyed by the addresses of the (A_k, rows_k, cols_k) arrays and the version counters torch keeps
+    for rows_k and cols_k: with 2 to 4 column partitions a plan remembers whether the row arrays
+    allowed dropping atomics, with more than 4 it holds a list of every output row's slots made from
+    the row and column arrays (the weights A_k are read at every call).  In-place changes made
+    through torch are therefore noticed; after rewriting row or column arrays by other means (a
+    kernel of the caller's, another library) call :meth:`invalidate` -- the reference's operator
+    reads them afresh on every call."""
     name = "hyb_csrmm"
 
     def __init__(self, m, n, feat, num_col_parts, buckets, nrows):
@@ -131,10 +182,12 @@ class HybCsrMM(_Operator):
         if len(self.nrows) != self.parts * len(self.buckets):
             raise _lib.SparseTIRError("hyb_csrmm: nrows must have num_col_parts*len(buckets) entries")
         self.L = _lib.lib()
-        self._plan = None
-        self._key = None
-        self._keep = None
+        self._plans = _PlanCache(self.L.stir_hyb_plan_destroy)
         self._spec_cache = None
+
+    @property
+    def plan_builds(self):
+        return self._plans.builds
 
     def _spec(self):
         f32, i32 = torch.float32, torch.int32
@@ -146,24 +199,13 @@ class HybCsrMM(_Operator):
             spec += [(f"A_{tag}", f32, r * w), (f"rows_{tag}", i32, r), (f"cols_{tag}", i32, r * w)]
         return spec
 
-    def _drop_plan(self):
-        if self._plan is not None:
-            self.L.stir_hyb_plan_destroy(self._plan)
-            self._plan = None
-
     def invalidate(self):
-        """Forget the plan made from the arrays of the last call.  The plan is reused while the
-        (A_k, rows_k, cols_k) arrays keep their addresses; with 2 to 4 column partitions it also
-        remembers whether the row arrays allowed dropping atomics, and with more than 4 it holds a
-        list of every output row's slots made from the row and column arrays (the weights A_k are
-        read at every call).  Call this after rewriting row or column arrays in place (the
-        reference's operator reads them afresh on every call)."""
-        self._drop_plan()
-        self._key = None
+        """Forget every plan made from the arrays of earlier calls."""
+        self._plans.clear()
 
     def __del__(self):
         try:
-            self._drop_plan()
+            self._plans.clear()
         except Exception:
             pass
 
@@ -172,22 +214,21 @@ class HybCsrMM(_Operator):
             self._spec_cache = self._spec()
         dev = self._check(args, self._spec_cache)
         b, c, triples = args[0], args[1], args[2:]
-        key = (dev,) + tuple(t.data_ptr() for t in triples)
+        key = (dev,) + tuple(_addr(t) if i % 3 == 0 else (_addr(t), t._version) for i, t in enumerate(triples))
         with torch.cuda.device(dev):
-            if key != self._key:
-                self._drop_plan()
+            plan = self._plans.get(key)
+            if plan is None:
                 nk = len(self.nrows)
                 widths = (ctypes.c_int32 * len(self.buckets))(*self.buckets)
                 nrows = (ctypes.c_int64 * max(nk, 1))(*self.nrows)
                 plan = ctypes.c_void_p()
-                A = _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in triples[0::3]])
-                R = _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in triples[1::3]])
-                Cc = _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in triples[2::3]])
+                A = _lib.ptr_table([_addr(t) for t in triples[0::3]])
+                R = _lib.ptr_table([_addr(t) for t in triples[1::3]])
+                Cc = _lib.ptr_table([_addr(t) for t in triples[2::3]])
                 _lib.check(self.L.stir_hyb_plan_create(ctypes.byref(plan), self.m, self.n, self.parts,
                                                        len(self.buckets), widths, nrows, A, R, Cc))
-                self._plan, self._key = plan, key
-                self._keep = triples  # the plan stores pointers into these arrays
-            _lib.check(self.L.stir_hyb_spmm_f32(self._plan, self.feat, _ptr(b), _ptr(c), _stream()))
+                self._plans.put(key, plan, triples)  # the plan stores pointers into these arrays
+            _lib.check(self.L.stir_hyb_spmm_f32(plan, self.feat, _ptr(b), _ptr(c), _stream()))
 
 
 class SddmmPreproc(_Operator):
@@ -305,22 +346,19 @@ class TcSpMM(_Operator):
         self.t, self.g, self.brows = int(tile_size), int(group_size), int(num_b_rows)
         self.out_dtype = out_dtype
         self.L = _lib.lib()
-        self._plan, self._key, self._keep = None, None, None
+        self._plans = _PlanCache(self.L.stir_tc_plan_destroy)
 
-    def _drop_plan(self):
-        if self._plan is not None:
-            self.L.stir_tc_plan_destroy(self._plan)
-            self._plan = None
-        self._keep = None
+    @property
+    def plan_builds(self):
+        return self._plans.builds
 
     def invalidate(self):
-        """Forget the plan made from the contents ``indptr`` had at the last call."""
-        self._drop_plan()
-        self._key = None
+        """Forget the plans made from the contents ``indptr`` arrays had at earlier calls."""
+        self._plans.clear()
 
     def __del__(self):
         try:
-            self._drop_plan()
+            self._plans.clear()
         except Exception:
             pass
 
@@ -338,14 +376,14 @@ class TcSpMM(_Operator):
                 return
             # torch counts the in-place changes it knows of: rewriting indptr with torch calls makes a new plan
             key = (dev, indptr.data_ptr(), indptr._version)
-            if key != self._key:
-                self._drop_plan()
+            plan = self._plans.get(key)
+            if plan is None:
                 plan = ctypes.c_void_p()
                 _lib.check(self.L.stir_tc_plan_create(ctypes.byref(plan), self.mb, _ptr(indptr), _stream()))
                 # the array stays alive with the plan: its address cannot be handed to another
                 # indptr array (same size, version 0) that the key would take for this one
-                self._plan, self._key, self._keep = plan, key, indptr
-            _lib.check(self.L.stir_tc_spmm_f16_planned(self._plan, _DT[self.out_dtype], self.mb, self.t, self.g,
+                self._plans.put(key, plan, indptr)
+            _lib.check(self.L.stir_tc_spmm_f16_planned(plan, _DT[self.out_dtype], self.mb, self.t, self.g,
                                                        self.feat, self.nnzb,
                                                        _ptr(a), _ptr(b), _ptr(c), _ptr(indptr), _ptr(indices),
                                                        _stream()))
@@ -355,10 +393,12 @@ class Rgms(_Operator):
     """RGMS on ELL3D buckets.  ``groups`` lists the group count of every bucket, ``rows_bkt`` /
     ``cols_bkt`` the ELL rows per group and slots per ELL row.
 
-    The operator keeps a plan made on the first call with a given set of bucket arrays (keyed by
-    their addresses).  From 8192 slots on, that plan holds an edge index derived from the contents
-    of the rows / cols / mids arrays: after changing those in place call :meth:`invalidate`, or the
-    old structure keeps being used (the reference's operator reads the arrays on every call).  The
+    The operator keeps the plans of the array sets it was called with last (see :class:`_PlanCache`),
+    keyed by the arrays' addresses and the version counters torch keeps for the index arrays.  From
+    8192 slots on, a plan holds an edge index derived from the contents of the rows / cols / mids
+    arrays: in-place changes made through torch are noticed, after changing them by other means
+    call :meth:`invalidate`, or the old structure keeps being used (the reference's operator reads
+    the arrays on every call).  The
     edge weights ``A_k``, ``W`` and ``X`` are read on every call -- unless the operator was built
     with ``static_weights=True``, the promise that the ``A_k`` keep the values of the first call
     (the reference's use: its ``A_k`` is the 0/1 mask); zero-weight padding slots are then left out
@@ -383,10 +423,12 @@ class Rgms(_Operator):
         self.rb, self.cb = [int(v) for v in rows_bkt], [int(v) for v in cols_bkt]
         self.groups = [int(v) for v in groups]
         self.L = _lib.lib()
-        self._plan = None
-        self._key = None
-        self._keep = None
+        self._plans = _PlanCache(getattr(self.L, self._fns[2]))
         self._spec_cache = None
+
+    @property
+    def plan_builds(self):
+        return self._plans.builds
 
     def _spec(self):
         f16, f32, i32 = self._in_dtype, torch.float32, torch.int32
@@ -399,19 +441,13 @@ class Rgms(_Operator):
             spec.append((f"mids_{k}", i32, g))
         return spec
 
-    def _drop_plan(self):
-        if self._plan is not None:
-            getattr(self.L, self._fns[2])(self._plan)
-            self._plan = None
-
     def invalidate(self):
-        """Forget the plan (and the edge index) made from the arrays of the last call."""
-        self._drop_plan()
-        self._key = None
+        """Forget the plans (and edge indices) made from the arrays of earlier calls."""
+        self._plans.clear()
 
     def __del__(self):
         try:
-            self._drop_plan()
+            self._plans.clear()
         except Exception:
             pass
 
@@ -422,22 +458,25 @@ class Rgms(_Operator):
         w, x, y, rest = args[0], args[1], args[2], args[3:]
         nb = len(self.groups)
         triples, mids = rest[:3 * nb], rest[3 * nb:]
-        key = (dev,) + tuple(t.data_ptr() for t in rest)
+        # index arrays: address and torch's count of in-place changes; weights: address only, unless
+        # the plan keeps them inside its index
+        key = (dev,) + tuple(_addr(t) if (i < 3 * nb and i % 3 == 0 and not self._static) else (_addr(t), t._version)
+                             for i, t in enumerate(rest))
         with torch.cuda.device(dev):
-            if key != self._key:
-                self._drop_plan()
+            plan = self._plans.get(key)
+            if plan is None:
                 plan = ctypes.c_void_p()
                 rb = (ctypes.c_int32 * nb)(*self.rb)
                 cb = (ctypes.c_int32 * nb)(*self.cb)
                 groups = (ctypes.c_int64 * nb)(*self.groups)
-                tab = lambda ts: _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in ts])
+                tab = lambda ts: _lib.ptr_table([_addr(t) for t in ts])
                 _lib.check(getattr(self.L, self._fns[0])(ctypes.byref(plan), nb, rb, cb, groups,
                                                          tab(triples[0::3]), tab(triples[1::3]),
                                                          tab(triples[2::3]), tab(mids)))
-                self._plan, self._key, self._keep = plan, key, rest
+                self._plans.put(key, plan, rest)
                 if self._static and self._in_dtype is not torch.float32:
                     _lib.check(self.L.stir_rgms_plan_set_static_weights(plan, 1))
-            _lib.check(getattr(self.L, self._fns[1])(self._plan, self.m, self.n, self.R, self.fin, self.fout,
+            _lib.check(getattr(self.L, self._fns[1])(plan, self.m, self.n, self.R, self.fin, self.fout,
                                                      _ptr(w), _ptr(x), _ptr(y), _stream()))
 
 

@@ -126,3 +126,11 @@ def set_stream(stream_handle):
     L.stir_set_stream.argtypes = [ctypes.c_void_p]
     L.stir_set_stream.restype = None
     L.stir_set_stream(ctypes.c_void_p(stream_handle))
+
+
+def plan_builds():
+    """Plans made by the packed operators since the library was loaded."""
+    L = _lib.lib()
+    L.stir_packed_plan_builds.restype = ctypes.c_int64
+    L.stir_packed_plan_builds.argtypes = []
+    return int(L.stir_packed_plan_builds())

@@ -204,54 +204,6 @@ def test_packed_dbsrmm_tcspmm_and_fp32_rgms_match_operator_objects(dev):
                                                      fin, fout)
 
 
-def test_index_arrays_rewritten_in_place_need_invalidate(dev):
-    """The RGMS plan over 8192 slots or more holds an edge index made from the contents of the
-    row / column / relation arrays.  The reference reads those arrays on every call; here a
-    caller that rewrites them in place tells the library (ops: .invalidate(); packed:
-    "sparsetir.invalidate_plans") and then gets the result for the new contents."""
-    R, n, fin, fout, group, buckets = 6, 3000, 32, 32, 32, [1, 2, 4, 8]
-    csf = random_csf(R, n, 30000, seed=8)
-    rb = [group // b for b in buckets]
-    iptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
-    assert sum(c.size for c in cols) >= 8192
-    t = lambda v: torch.from_numpy(np.ascontiguousarray(v)).to(dev)
-    rng = np.random.default_rng(8)
-    w = t(rng.standard_normal(R * fin * fout).astype(np.float16) * 0.1)
-    xx = t(rng.standard_normal(n * fin).astype(np.float16))
-    triples, mids = [], []
-    for k in range(len(buckets)):
-        triples += [t(mask[k].astype(np.float16).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
-        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(iptr[k]))))
-    groups = [c.shape[0] for c in cols]
-
-    def fresh_result():  # a new operator object sees the arrays as they are now
-        y = torch.zeros(n * fout, device=dev)
-        ops.build_rgms(n, n, R, fin, fout, rb, buckets, groups)(w, xx, y, *triples, *mids)
-        torch.cuda.synchronize()
-        return y
-
-    f = ops.build_rgms(n, n, R, fin, fout, rb, buckets, groups)
-    g = packed.get_global_func("sparsetir.rgms")
-    y0, y0p = torch.zeros(n * fout, device=dev), torch.zeros(n * fout, device=dev)
-    f(w, xx, y0, *triples, *mids)
-    g(w, xx, y0p, *triples, *mids, fin, fout)
-    before = fresh_result()
-    assert torch.allclose(y0, before, rtol=1e-5, atol=1e-5) and torch.allclose(y0p, before, rtol=1e-5, atol=1e-5)
-    # new structure at the same addresses: every source node shifted by one
-    for k in range(len(buckets)):
-        triples[3 * k + 2].copy_((triples[3 * k + 2] + 1) % n)
-    after = fresh_result()
-    assert not torch.allclose(after, before, rtol=1e-3, atol=1e-3)
-    f.invalidate()
-    packed.get_global_func("sparsetir.invalidate_plans")()
-    y1, y1p = torch.zeros(n * fout, device=dev), torch.zeros(n * fout, device=dev)
-    f(w, xx, y1, *triples, *mids)
-    g(w, xx, y1p, *triples, *mids, fin, fout)
-    torch.cuda.synchronize()
-    assert torch.allclose(y1, after, rtol=1e-5, atol=1e-5)
-    assert torch.allclose(y1p, after, rtol=1e-5, atol=1e-5)
-
-
 def test_packed_rgms_static_weights(dev):
     """"sparsetir.rgms_static_weights"(1) makes the packed RGMS operator build its plans with the
     promise that the slot weights stay as they are: same result as without it, for weights that
@@ -272,6 +224,8 @@ def test_packed_rgms_static_weights(dev):
         mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(iptr[k]))))
     g = packed.get_global_func("sparsetir.rgms")
     promise = packed.get_global_func("sparsetir.rgms_static_weights")
+    structure = packed.get_global_func("sparsetir.static_structure")
+    structure(1)  # weights live inside the edge index, which is only kept under this promise
     results = []
     try:
         for on in (0, 1, 0):
@@ -283,6 +237,7 @@ def test_packed_rgms_static_weights(dev):
             results.append(y)
     finally:
         promise(0)
+        structure(0)
     assert results[0].abs().sum() > 0
     assert torch.allclose(results[0], results[1], rtol=1e-5, atol=1e-5)
     assert torch.allclose(results[0], results[2], rtol=1e-5, atol=1e-5)

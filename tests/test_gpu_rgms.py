@@ -143,7 +143,7 @@ def test_rgms_static_weights_edge_cases(dev):
     torch.cuda.synchronize()
     assert ya.abs().sum() > 0 and torch.allclose(ya, yb, rtol=1e-5, atol=1e-5)
     with pytest.raises(SparseTIRError, match="launched already"):
-        check(lib().stir_rgms_plan_set_static_weights(fa._plan, 0))
+        check(lib().stir_rgms_plan_set_static_weights(next(iter(fa._plans._plans.values()))[0], 0))
 
 
 def test_rgms_tiled_repeat_calls_accumulate(dev):
