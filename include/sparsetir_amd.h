@@ -282,7 +282,8 @@ int stir_sddmm_scaled_f32(int32_t m, int32_t n, int32_t feat, int64_t nnz, const
  * BSR SpMM on MFMA, 16-bit inputs, fp32 accumulation; argument list [A, X, Y, indptr,
  * indices] of examples/blocksparse/bsr_spmm.py:427-432.  A: nnzb*blk*blk, X: nb*blk*feat,
  * Y: mb*blk*feat.  dtype: STIR_F16 or STIR_BF16 for A and X; out_dtype: the same 16-bit
- * type or STIR_F32.  blk must be 16 or 32 and feat a multiple of 32.
+ * type or STIR_F32.  blk: a multiple of 16 (the reference's schedule splits both block axes by 16,
+ * bsr_spmm.py:379-380); feat: a multiple of 32.
  */
 int stir_bsr_spmm(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk,
                   int32_t feat, int64_t nnzb, const void* d_A, const void* d_X, void* d_Y,

@@ -81,11 +81,15 @@ __device__ __forceinline__ bool decode_tile(int64_t L, int64_t slices, int f_til
 // and the 32*RS x 32 piece of the block into LDS -- each thread loads 16-byte chunks, consecutive
 // lanes consecutive chunks of a row of X -- while the previous step is multiplied (two LDS
 // stages, one barrier per step).  LDS keeps X feature-contiguous, in 16-byte units of 8 features:
-// unit (k, c) sits at (k/4)*4*FCN + (k%4)*FCN + (c ^ 2*(k%4)), FCN = units per row.  The MFMA B
+// unit (k, c) sits at (k/4)*4*FCN + (k%4)*FCN + (c ^ 4*(k%4)), FCN = units per row.  The MFMA B
 // operand (8 consecutive k for one feature per lane) comes out of that image through the
 // transposing read ds_read_b64_tr_b16, which hands lane i of a block of 16 lanes four consecutive
-// k of column i when the lanes address rows k .. k+3, four features each; the XOR keeps both the
-// 16-byte stores of a row (8 lanes, one k) and those reads (4 rows x 2 units) on distinct banks.
+// k of column i when the lanes address rows k .. k+3, four features each.  The LDS serves such a
+// read 32 lanes at a time from 64 banks: two blocks of 16 lanes, each reading two units in each of
+// four rows whose stride is a multiple of all banks, so the XOR has to move the four rows of a
+// block to four different groups of four units (c ^ 4*(k%4); with c ^ 2*(k%4) two rows of the two
+// blocks met in the same banks and every read took twice its cycles).  The 16-byte stores of a row
+// (8 lanes and 8 consecutive units per cycle) stay on distinct banks under either XOR.
 // The block piece is fetched once per workgroup (8*RS bytes per thread) and laid out by k chunk so
 // that a lane's A operand is one 16-byte read.
 // lds: 2 * (64*128*NT + 2048*RS) bytes.
@@ -110,7 +114,7 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
   for (int q = 0; q < 2 * NT; ++q) {
     const int idx = 64 * (wave * 2 * NT + q) + lane, c = idx % FCN, k = idx / FCN;
     xoff[q] = (uint32_t)(k * feat + 8 * c);  // in elements, from the tile's first element
-    xdst[q] = (uint32_t)(((k >> 2) * 4 * FCN + (k & 3) * FCN + (c ^ (2 * (k & 3)))) * 16);
+    xdst[q] = (uint32_t)(((k >> 2) * 4 * FCN + (k & 3) * FCN + (c ^ (4 * (k & 3)))) * 16);
     xlive[q] = f0 + 8 * c < feat;  // feat is a multiple of 32, so chunks are whole
   }
   // ... and 8*RS bytes of the block: RS = 1: half of the unit (chunk tid/64, row (tid/2)%32);
@@ -126,7 +130,7 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int kr = sl >> 2, c = (wave * NT + t) * 4 + 2 * half16 + ((sl & 3) >> 1);
-    bread[t] = (uint32_t)(((2 * h) * 4 * FCN + kr * FCN + (c ^ (2 * kr))) * 16 + (sl & 1) * 8);
+    bread[t] = (uint32_t)(((2 * h) * 4 * FCN + kr * FCN + (c ^ (4 * kr))) * 16 + (sl & 1) * 8);
   }
   const uint32_t aread = XB + (h * 32 + n) * 16;
 
@@ -516,6 +520,124 @@ __global__ __launch_bounds__(256) void bsr_spmm_ksplit_kernel(int blk, int feat,
   }
 }
 
+// ------------------------------------------------------------------ blocks of 16 k+16 rows
+// Block sides that are a multiple of 16 but not of 32 (the reference's schedule splits both block
+// axes by 16, examples/blocksparse/bsr_spmm.py:379-380): 16-row slices on v_mfma_f32_16x16x32,
+// whose k extent of 32 is two 16-column chunks of the block row's blocks in storage order.  A
+// workgroup of four wavefronts owns (block row, 16-row slice, 128 features), a wavefront 16 rows
+// x 32 features (two accumulators of four registers).  The A operand -- 8 consecutive k of one row
+// per lane -- is one 16-byte load from the block; the 32 rows of X of a step go through LDS as
+// (k, k+1) pairs, double-buffered, the next step's loads in flight during the multiply.  Rows of
+// the staged image are rotated by 16 (k pair / 4) words so that the four k groups a multiply
+// reads lie on different banks.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <bool BF16>
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                  0, 0);
+}
+
+template <bool BF16, int OUT>
+__global__ __launch_bounds__(256) void bsr16_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles,
+                                                         const uint16_t* __restrict__ A,
+                                                         const uint16_t* __restrict__ X, void* __restrict__ Y,
+                                                         const int32_t* __restrict__ indptr,
+                                                         const int32_t* __restrict__ indices,
+                                                         const int32_t* __restrict__ row_ids) {
+  __shared__ __attribute__((aligned(16))) uint32_t xs[2][16 * kTileF];  // [buffer][k pair][feature]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int f_tile = (int)(blockIdx.x % f_tiles);
+  const int64_t slice = blockIdx.x / f_tiles;
+  if (slice >= slices) return;
+  const int sub = blk / 16;  // 16-row slices per block row = 16-column chunks per block
+  const int i = (int)(slice / sub), s = (int)(slice % sub);
+  const int i_out = row_ids ? row_ids[i] : i;
+  const int f0 = f_tile * kTileF;
+  // staging role: k pair kp (rows 2kp, 2kp+1 of the step's 32), 8-feature chunk fc
+  const int kp = tid >> 4, fc = tid & 15;
+  const bool stage_live = f0 + fc * 8 < feat;
+  const int stage_at = kp * kTileF + ((fc * 8 + 16 * (kp >> 2)) & (kTileF - 1));
+  // operand role: row ii of the slice, k group q (8 of the step's 32 k)
+  const int ii = lane & 15, q = lane >> 4;
+
+  const int p_begin = indptr[i];
+  const int chunks = (indptr[i + 1] - p_begin) * sub;
+  const int steps = (chunks + 1) / 2;
+
+  f32x4 acc[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // the block column of a step's chunk is requested one step before its rows of X
+  int j_stage = 0;
+  auto fetch_ids = [&](int it) {
+    const int c = 2 * it + (kp >> 3);
+    j_stage = c < chunks ? indices[p_begin + c / sub] : 0;
+  };
+  u32x4 r0, r1, a_next;
+  auto fetch = [&](int it) {
+    a_next = r0 = r1 = u32x4{0, 0, 0, 0};
+    const int ca = 2 * it + (q >> 1);
+    if (ca < chunks)
+      a_next = *reinterpret_cast<const u32x4*>(A + ((int64_t)(p_begin + ca / sub) * blk + s * 16 + ii) * blk +
+                                               (ca % sub) * 16 + 8 * (q & 1));
+    const int c = 2 * it + (kp >> 3);
+    if (stage_live && c < chunks) {
+      const uint16_t* xp = X + ((int64_t)j_stage * blk + (c % sub) * 16 + 2 * (kp & 7)) * feat + f0 + fc * 8;
+      r0 = *reinterpret_cast<const u32x4*>(xp);
+      r1 = *reinterpret_cast<const u32x4*>(xp + feat);
+    }
+    if (it + 1 < steps) fetch_ids(it + 1);
+  };
+
+  if (steps > 0) {
+    fetch_ids(0);
+    fetch(0);
+  }
+  for (int it = 0; it < steps; ++it) {
+    const int buf = it & 1;
+    const u32x4 a_now = a_next;
+    u32x4 lo, hi;
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      lo[2 * d] = __builtin_amdgcn_perm(r1[d], r0[d], 0x05040100);
+      lo[2 * d + 1] = __builtin_amdgcn_perm(r1[d], r0[d], 0x07060302);
+      hi[2 * d] = __builtin_amdgcn_perm(r1[d + 2], r0[d + 2], 0x05040100);
+      hi[2 * d + 1] = __builtin_amdgcn_perm(r1[d + 2], r0[d + 2], 0x07060302);
+    }
+    *reinterpret_cast<u32x4*>(&xs[buf][stage_at]) = lo;
+    *reinterpret_cast<u32x4*>(&xs[buf][stage_at + 4]) = hi;
+    if (it + 1 < steps) fetch(it + 1);
+    __syncthreads();
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int c = ((wave * 32 + 16 * nt + 16 * q) & (kTileF - 1)) + ii;
+      u32x4 b;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) b[d] = xs[buf][(4 * q + d) * kTileF + c];  // rows 8q .. 8q+7 of the step
+      acc[nt] = mfma16<BF16>(a_now, b, acc[nt]);
+    }
+  }
+  const int fcol = f0 + wave * 32;
+  if (fcol >= feat) return;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int64_t off = ((int64_t)i_out * blk + s * 16 + 4 * q + v) * feat + fcol + 16 * nt + ii;
+      if constexpr (OUT == 1)
+        static_cast<float*>(Y)[off] = acc[nt][v];
+      else
+        static_cast<uint16_t*>(Y)[off] = to16<BF16>(acc[nt][v]);
+    }
+}
+
 }  // namespace
 
 static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, int32_t blk, int32_t feat,
@@ -524,10 +646,29 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   STIR_REQUIRE(dtype == STIR_F16 || dtype == STIR_BF16, "bsr_spmm: dtype must be STIR_F16 or STIR_BF16");
   STIR_REQUIRE(out_dtype == dtype || out_dtype == STIR_F32, "bsr_spmm: out_dtype must equal dtype or be STIR_F32");
   STIR_REQUIRE(mb >= 0 && nb >= 0 && nnzb >= 0, "bsr_spmm: bad sizes mb=%d nb=%d", mb, nb);
-  STIR_REQUIRE(blk > 0 && blk % 32 == 0, "bsr_spmm: blk=%d must be a multiple of 32", blk);
+  STIR_REQUIRE(blk > 0 && blk % 16 == 0, "bsr_spmm: blk=%d must be a multiple of 16", blk);
   STIR_REQUIRE(feat > 0 && feat % 32 == 0, "bsr_spmm: feat=%d must be a multiple of 32", feat);
   if (mb == 0) return 0;
   STIR_REQUIRE(d_X && d_Y && d_indptr && (nnzb == 0 || (d_A && d_indices)), "bsr_spmm: null pointer argument");
+  hipStream_t st16 = static_cast<hipStream_t>(stream);
+  if (blk % 32 != 0) {
+    const int f_tiles16 = (int)stir::ceil_div(feat, kTileF);
+    const int64_t slices16 = (int64_t)mb * (blk / 16);
+    STIR_REQUIRE(slices16 * f_tiles16 < (int64_t(1) << 31), "bsr_spmm: too many tiles for one launch");
+    dim3 grid16((unsigned)(slices16 * f_tiles16)), block16(256);
+#define STIR_BSR_16(BF, OUT)                                                                                    \
+  hipLaunchKernelGGL((bsr16_spmm_kernel<BF, OUT>), grid16, block16, 0, st16, blk, feat, slices16, f_tiles16,     \
+                     static_cast<const uint16_t*>(d_A), static_cast<const uint16_t*>(d_X), d_Y, d_indptr, d_indices, \
+                     d_row_ids)
+    if (dtype == STIR_BF16) {
+      if (out_dtype == STIR_F32) STIR_BSR_16(true, 1); else STIR_BSR_16(true, 0);
+    } else {
+      if (out_dtype == STIR_F32) STIR_BSR_16(false, 1); else STIR_BSR_16(false, 0);
+    }
+#undef STIR_BSR_16
+    STIR_LAUNCH_CHECK();
+    return 0;
+  }
   // two 32-row slices per workgroup when the block height allows it
   const int rs = (blk % 64 == 0) ? 2 : 1;
   const int64_t slices = (int64_t)mb * (blk / (32 * rs));

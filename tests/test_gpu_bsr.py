@@ -146,11 +146,26 @@ def test_bsr_launch_swept_in_step(dev, dtype, out32, varied):
     assert bool((got[empty] == 0).all())
 
 
+@pytest.mark.parametrize("blk,feat,dtype,out32", [
+    (16, 512, torch.float16, False),    # the reference's schedule splits both block axes by 16
+    (16, 160, torch.bfloat16, True),    # an odd number of 16-column chunks in most block rows, a partial feature tile
+    (48, 96, torch.float16, True),      # a multiple of 16 that is not one of 32: three slices, three chunks per block
+    (80, 256, torch.bfloat16, False),
+])
+def test_bsr_blocks_of_16_rows(dev, blk, feat, dtype, out32):
+    """Block sides that are multiples of 16 (examples/blocksparse/bsr_spmm.py:379-380 splits the
+    block axes by 16): the 16-row slices run on the 16x16x32 matrix-core instruction, two
+    16-column chunks per step."""
+    cfg = datasets.config4(seed=blk + feat, mb=11, nb=13, blk=blk, density=0.3, feat=feat)
+    got, a32, x32 = _run(dev, cfg, dtype, torch.float32 if out32 else None)
+    _check(got, cfg, a32, x32, not out32, f"blk={blk} feat={feat} {dtype}")
+
+
 def test_bsr_rejects_unsupported(dev):
     z = lambda k, dt: torch.zeros(k, dtype=dt, device=dev)
-    f = ops.build_bsrmm(1, 1, 1, 16, 32)
+    f = ops.build_bsrmm(1, 1, 1, 8, 32)
     with pytest.raises(SparseTIRError, match="blk"):
-        f(z(256, torch.float16), z(512, torch.float16), z(512, torch.float16), z(2, torch.int32), z(1, torch.int32))
+        f(z(64, torch.float16), z(256, torch.float16), z(256, torch.float16), z(2, torch.int32), z(1, torch.int32))
 
 
 def test_dbsr_doubly_compressed(dev):
