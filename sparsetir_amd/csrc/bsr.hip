@@ -109,14 +109,17 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
 
   // staging role: 2*NT chunks of X per thread
   uint32_t xoff[2 * NT], xdst[2 * NT];
-  bool xlive[2 * NT];
 #pragma unroll
   for (int q = 0; q < 2 * NT; ++q) {
     const int idx = 64 * (wave * 2 * NT + q) + lane, c = idx % FCN, k = idx / FCN;
     xoff[q] = (uint32_t)(k * feat + 8 * c);  // in elements, from the tile's first element
     xdst[q] = (uint32_t)(((k >> 2) * 4 * FCN + (k & 3) * FCN + (c ^ (4 * (k & 3)))) * 16);
-    xlive[q] = f0 + 8 * c < feat;  // feat is a multiple of 32, so chunks are whole
   }
+  // a lane's chunks all lie in the same feature column (FCN divides 64): one test for all of
+  // them; feat is a multiple of 32, so chunks are whole.  A lane beyond feat never loads and
+  // keeps staging the zeros its registers start with.
+  static_assert(64 % FCN == 0, "a lane's chunks share their feature column");
+  const bool xlive = f0 + 8 * (lane % FCN) < feat;
   // ... and 8*RS bytes of the block: RS = 1: half of the unit (chunk tid/64, row (tid/2)%32);
   // RS = 2: the unit (slice tid/128, chunk (tid/32)%4, row tid%32)
   uint32_t aoff;
@@ -153,13 +156,16 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
   int j_cur = nblk > 0 ? indices[p_begin] : 0;
   int j_nxt = nblk > 1 ? indices[p_begin + 1] : 0;
   u32x4 xr[2 * NT];
+#pragma unroll
+  for (int q = 0; q < 2 * NT; ++q) xr[q] = u32x4{0, 0, 0, 0};
   u32x4 ar;  // RS = 1 uses the first two words
   auto fetch = [&]() {
     const uint16_t* xb = X + ((int64_t)j_cur * blk + k0) * feat + f0;
     const uint16_t* ab = A + (int64_t)(p_begin + pb) * blk * blk + (int64_t)bi0 * blk + k0;
+    if (xlive) {
 #pragma unroll
-    for (int q = 0; q < 2 * NT; ++q)
-      xr[q] = xlive[q] ? *reinterpret_cast<const u32x4*>(xb + xoff[q]) : u32x4{0, 0, 0, 0};
+      for (int q = 0; q < 2 * NT; ++q) xr[q] = *reinterpret_cast<const u32x4*>(xb + xoff[q]);
+    }
     if constexpr (RS == 1) {
       const u32x2 v = *reinterpret_cast<const u32x2*>(ab + aoff);
       ar[0] = v[0], ar[1] = v[1];
@@ -230,9 +236,24 @@ __device__ __forceinline__ void bsr_tile(char* __restrict__ lds, int blk, int fe
   }
 }
 
+// The other order, for tall blocks (by_rows): XCD x owns the block rows i = x, x + 8, ... and
+// walks, for each, the slices of the block row inside every feature tile before the next feature
+// tile.  The workgroups that are resident together on an XCD then share the blocks of A of their
+// block row (fetched into that L2 once instead of once per feature tile) and, between the slices
+// of a block row, its tiles of X.
+__device__ __forceinline__ bool decode_tile_by_rows(int64_t L, int64_t block_rows, int sub, int f_tiles,
+                                                    int64_t& slice, int& f_tile) {
+  const int xcd = (int)(L & 7);
+  const int64_t t = L >> 3;
+  const int64_t i = xcd + 8 * (t / ((int64_t)sub * f_tiles));
+  f_tile = (int)((t / sub) % f_tiles);
+  slice = i * sub + t % sub;
+  return i < block_rows;
+}
+
 // One workgroup per tile, 1-D grid (see decode_tile).
 template <bool BF16, int OUT, int NT, int RS>
-__global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles,
+__global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_t slices, int f_tiles, int by_rows,
                                                        const uint16_t* __restrict__ A,
                                                        const uint16_t* __restrict__ X, void* __restrict__ Y,
                                                        const int32_t* __restrict__ indptr,
@@ -242,8 +263,12 @@ __global__ __launch_bounds__(256) void bsr_spmm_kernel(int blk, int feat, int64_
   __shared__ __attribute__((aligned(16))) char xs[2 * (kTileK * TF * 2 + 2048 * RS)];
   int64_t slice;
   int f_tile;
-  if (!decode_tile(blockIdx.x, slices, f_tiles, slice, f_tile)) return;
   const int sub = blk / (32 * RS);  // slices of 32*RS rows per block row
+  if (by_rows) {
+    if (!decode_tile_by_rows(blockIdx.x, slices / sub, sub, f_tiles, slice, f_tile)) return;
+  } else if (!decode_tile(blockIdx.x, slices, f_tiles, slice, f_tile)) {
+    return;
+  }
   const int i = (int)(slice / sub), bi0 = (int)(slice % sub) * (32 * RS);
   // doubly-compressed form: stored block row i is block row row_ids[i] of the output
   const int i_out = row_ids ? row_ids[i] : i;
@@ -728,14 +753,21 @@ static int bsr_launch(int32_t dtype, int32_t out_dtype, int32_t mb, int32_t nb, 
   // with fewer than 8 feature tiles or two slices per workgroup the plain order is faster)
   const bool sweep = cus >= 8 && cus % 8 == 0 && rs == 1 && f_tiles >= 8 && x_tile_bytes > (3 << 20) &&
                      slices <= kSweepMaxSlices;
-  const int64_t blocks = f_tiles >= 8 ? 8 * stir::ceil_div(f_tiles, 8) * slices : (int64_t)f_tiles * slices;
+  // Blocks of 128 rows and more: block rows dealt to XCDs (decode_tile_by_rows).  Measured at
+  // 16384^2, 10 %, 4096 features: 128 x 128 blocks 387 -> 365 us; 64 x 64 blocks (one slice per
+  // block row, so only A is shared) 443 -> 514 us and 32 x 32 blocks 600 -> 950 us: there the
+  // feature tile per XCD, which keeps an XCD on one slice of X, is worth more.
+  const int sub_rows = blk / (32 * rs);
+  const int by_rows = (rs == 2 && sub_rows >= 2 && f_tiles >= 2) ? 1 : 0;
+  const int64_t blocks = by_rows ? 8 * stir::ceil_div((int64_t)mb, 8) * sub_rows * f_tiles
+                         : f_tiles >= 8 ? 8 * stir::ceil_div(f_tiles, 8) * slices : (int64_t)f_tiles * slices;
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "bsr_spmm: too many tiles for one launch");
   dim3 grid((unsigned)blocks);
 #define STIR_BSR_L(BF, OUT, NTV, RSV)                                                                      \
   {                                                                                                        \
-    if (sweep) STIR_BSR_SWEEP(BF, OUT, NTV, RSV);                                                          \
+    if (sweep && !by_rows) STIR_BSR_SWEEP(BF, OUT, NTV, RSV);                                                        \
     hipLaunchKernelGGL((bsr_spmm_kernel<BF, OUT, NTV, RSV>), grid, block, 0, st, blk, feat, slices, f_tiles, \
-                       A, X, d_Y, d_indptr, d_indices, d_row_ids);                                         \
+                       by_rows, A, X, d_Y, d_indptr, d_indices, d_row_ids);                                \
   }
 #define STIR_BSR(BF, OUT)                                                          \
   do {                                                                             \

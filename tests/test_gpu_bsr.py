@@ -71,10 +71,14 @@ def test_bsr_block64_and_empty_rows(dev):
     (64, 1056, torch.bfloat16, False),   # two slices per workgroup, two accumulators per wavefront
     (128, 160, torch.float16, True),     # two slices per workgroup, four k steps per block
     (96, 64, torch.float16, False),      # 96 rows: one slice per workgroup
+    (128, 1280, torch.float16, False),   # block rows dealt to XCDs, five feature tiles of 256
+    (256, 384, torch.bfloat16, True),    # four slices per block row in that order, a partial second feature tile
 ])
 def test_bsr_tall_blocks(dev, blk, feat, dtype, out32):
-    """Blocks of 64 rows and more: a workgroup takes two 32-row slices when blk is a multiple of 64."""
-    cfg = datasets.config4(seed=blk, mb=5, nb=6, blk=blk, density=0.35, feat=feat)
+    """Blocks of 64 rows and more: a workgroup takes two 32-row slices when blk is a multiple of 64;
+    from 128 rows on (and more than one feature tile) the block rows are dealt to XCDs, 13 block
+    rows here: neither a multiple of 8 nor below it."""
+    cfg = datasets.config4(seed=blk, mb=13 if blk >= 128 else 5, nb=6, blk=blk, density=0.35, feat=feat)
     got, a32, x32 = _run(dev, cfg, dtype, torch.float32 if out32 else None)
     _check(got, cfg, a32, x32, not out32, f"blk={blk} feat={feat} {dtype}")
 
