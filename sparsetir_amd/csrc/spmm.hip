@@ -642,6 +642,13 @@ int phases_have_single_writers(int32_t m, int num_col_parts, int num_buckets, co
 }  // namespace
 
 constexpr int kMaxPhases = 4;
+// With 2 to kMaxPhases partitions a plan holds both forms and the launch picks by feature width:
+// phases below this width, merged rows from it on.  Measured on the 169k-node graph with two
+// partitions (CSR row-split 39 / 64 / 112 / 203 us at 32 / 64 / 128 / 256 features): phases
+// 44 / 60 / 119 / 254 us, merged rows 81 / 98 / 136 / 235 us -- a phase reads and writes C once
+// more, which at 256 features (173 MB each way) costs more than the merged list's indirect loads.
+constexpr int kMergedFromFeat = 256;
+constexpr size_t kMergedOptionalBytes = size_t(1) << 30;  // ... when the slot list stays below this
 
 namespace {
 
@@ -987,7 +994,13 @@ int stir_hyb_plan_create_ex(stir_hyb_plan** plan, int32_t m, int32_t n, int32_t 
   p->num_buckets = num_buckets;
   p->d_tables = nullptr;
   p->merged = false;
-  if (!addresses_only && num_col_parts > kMaxPhases &&
+  bool want_merged = !addresses_only && num_col_parts > kMaxPhases;
+  if (!addresses_only && num_col_parts > 1 && num_col_parts <= kMaxPhases) {
+    size_t slots = 0;
+    for (int k = 0; k < num_col_parts * num_buckets; ++k) slots += size_t(nrows[k]) * size_t(bucket_widths[k % num_buckets]);
+    want_merged = slots * 12 <= kMergedOptionalBytes;
+  }
+  if (want_merged &&
       build_merged_rows(m, num_col_parts * num_buckets, num_buckets, bucket_widths, nrows, d_A, d_rows, d_cols,
                         &p->rows, &p->merged) != 0) {
     delete p;
@@ -1020,7 +1033,7 @@ int stir_hyb_spmm_f32(const stir_hyb_plan* plan, int32_t feat, const float* d_B,
   const size_t nk = plan->tables.tiles.size();
   if (nk == 0) return 0;
   STIR_REQUIRE(d_B && d_C, "hyb_spmm: null pointer argument");
-  if (plan->merged && vector_class(feat) >= 0)
+  if (plan->merged && vector_class(feat) >= 0 && (plan->num_col_parts > kMaxPhases || feat >= kMergedFromFeat))
     return launch_merged(plan->rows, plan->m, feat, d_B, d_C, static_cast<hipStream_t>(stream));
   return launch_hyb(plan->tables, plan->d_tables, plan->d_tables + nk, feat, d_B, d_C,
                     static_cast<hipStream_t>(stream));

@@ -140,6 +140,36 @@ def _column_part_hyb_device(num_rows, num_cols, indptr, indices, num_col_parts, 
     return nest(rows), nest(cols), nest(mask)
 
 
+def suggest_decomposition(num_rows, num_cols, nnz, feat):
+    """``(num_col_parts, buckets)`` to hand to :func:`column_part_hyb` for hyb SpMM on an MI355X:
+    the counterpart of the per-graph tables ``col_part_config`` / ``bucketing_config`` of the
+    reference (examples/spmm/bench_spmm.py:233-253), which were tuned by hand for another GPU.
+
+    The rule is what was measured on MI355X, at every size and feature width tried: **one column
+    partition, widths 1, 2, 4, ... 512**.
+
+    * Column partitions never pay.  A partition's slice of the dense operand would have to fit the
+      4 MB L2 of an XCD to raise the hit rate, i.e. hundreds of partitions for a graph of millions
+      of nodes, while every partition beyond the first reads and writes the output once more.
+      2.45 M nodes / 61.8 M edges, 128 features: 1 / 2 / 4 / 8 / 16 partitions take
+      5.07 / 5.29 / 5.62 / 5.23 / 5.21 ms with uniform columns and 4.04 / 4.03 / 4.11 / 4.27 / 4.29 ms
+      with power-law columns; 169 k nodes / 1.16 M edges: 24 / 32 / 47 / 83 / 83 us at 32 features,
+      189 / 237 / 232 / 236 / 236 us at 256 (CSR row-split: 39 and 202 us).
+    * The widest bucket should reach a few hundred slots: rows above it are cut into several ELL
+      rows that meet in atomics.  Widest bucket 32 / 64 / 128 / 256 / 512 / 1024 on the large
+      graph: 6.2 / 4.4 / 4.1 / 4.0 / 4.0 / 4.0 ms.  Empty buckets cost nothing.
+
+    ``num_rows``, ``nnz`` and ``feat`` do not change the answer today; they are part of the
+    signature because the rule is a measured one and may come to depend on them.  The widths stop
+    at the first power of two that covers ``num_cols`` (no row has more distinct columns)."""
+    if min(int(num_rows), int(num_cols), int(feat)) <= 0 or int(nnz) < 0:
+        raise _lib.SparseTIRError("suggest_decomposition: sizes must be positive")
+    buckets = [1]
+    while buckets[-1] < 512 and buckets[-1] < int(num_cols):
+        buckets.append(buckets[-1] * 2)
+    return 1, buckets
+
+
 def csr_to_bsr(indptr, indices, values, shape, blocksize, dtype=None):
     """Pack a CSR matrix (CUDA tensors: int32 indptr/indices, float32 values, no duplicate
     entries) into BSR with ``blocksize x blocksize`` blocks on the GPU.

@@ -218,3 +218,22 @@ def test_on_disk_cache_ignores_a_damaged_file(tmp_path):
     again = cached_column_part_hyb(str(tmp_path), 50, 40, indptr, indices, 1, [1, 2])  # rewritten and readable
     for a, c in zip(again, want):
         _same(a, c)
+
+
+def test_suggest_decomposition():
+    """The decomposition chooser (counterpart of the reference's col_part_config / bucketing_config
+    tables, examples/spmm/bench_spmm.py:233-253): one partition, power-of-two widths up to 512 or
+    the first one that covers the column count; its output feeds column_part_hyb as it is."""
+    import sparsetir_amd as st
+    from sparsetir_amd._lib import SparseTIRError
+    assert st.suggest_decomposition(2449029, 2449029, 61833585, 128) == (1, [1, 2, 4, 8, 16, 32, 64, 128, 256, 512])
+    assert st.suggest_decomposition(100, 5, 200, 32) == (1, [1, 2, 4, 8])
+    assert st.suggest_decomposition(3, 1, 3, 4) == (1, [1])
+    with pytest.raises(SparseTIRError):
+        st.suggest_decomposition(10, 0, 5, 32)
+    m, n = 40, 37
+    indptr, indices = random_csr(m, n, 300, 3)
+    parts, buckets = st.suggest_decomposition(m, n, len(indices), 64)
+    rows, cols, mask = st.column_part_hyb(m, n, indptr, indices, parts, buckets)
+    assert len(rows) == 1 and len(rows[0]) == len(buckets)
+    assert sum(int(k.sum()) for k in mask[0]) == len(indices)
