@@ -110,7 +110,8 @@ enum {
  *      call.  Default off: "sparsetir.hyb_csrmm" and "sparsetir.rgms" then do the same -- their
  *      cached plans hold the addresses and sizes of the arrays and nothing derived from their
  *      contents (hyb: one launch, atomics in every adding bucket, the rule of
- *      examples/spmm/bench_spmm.py:170; rgms: one fp32 atomic per ELL row and output feature), so
+ *      examples/spmm/bench_spmm.py:170; rgms: one fp32 atomic per ELL row and output feature;
+ *      rgms_f32 plans never hold more, rgms_csf has no plan), so
  *      rows / cols / mids may be rewritten in place, or freed and replaced by arrays of the same
  *      sizes at the same addresses, at any time.  on != 0 is the promise that these index arrays
  *      keep their contents for as long as they keep their addresses, which is how every script of

@@ -61,7 +61,11 @@ SIGNATURES = {
     "stir_rgms_plan_destroy": (I32, [VP]),
     "stir_rgms_f32_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f32": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
+    "stir_rgms_f32_plan_set_deterministic": (I32, [VP, I32]),
     "stir_rgms_f32_plan_destroy": (I32, [VP]),
+    "stir_rgms_csf_f32_plan_create": (I32, [VP, I64, I64, VP, VP, VP, VP, VP]),
+    "stir_rgms_csf_f32_planned": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
+    "stir_rgms_csf_f32_plan_destroy": (I32, [VP]),
     "stir_rgms_csf_f32": (I32, [I32, I32, I32, I32, I32, I64, I64, VP, VP, VP, VP, VP, VP, VP, VP, VP]),
 }
 

@@ -220,6 +220,7 @@ struct PlanCache {
 PlanCache<stir_hyb_plan> g_hyb_plans(stir_hyb_plan_destroy);
 PlanCache<stir_rgms_plan> g_rgms_plans(stir_rgms_plan_destroy);
 PlanCache<stir_rgms_f32_plan> g_rgms_f32_plans(stir_rgms_f32_plan_destroy);
+
 // Promises of the caller for the plans made from now on.  Without the first, a cached plan holds
 // addresses and sizes only and every call reads the index arrays afresh, as the reference's built
 // operators do; with it, plans may keep what they derive from the contents of the index arrays
@@ -499,6 +500,10 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
   key.nums.push_back(a.dev_id);
   std::lock_guard<std::mutex> lock(g_plan_mutex);
   const int32_t mm = (int32_t)(Y.len / fout), nn = (int32_t)(X.len / fin), rr = (int32_t)(W.len / (fin * fout));
+  // an edge index also depends on the sizes the launch is given
+  key.nums.push_back(mm);
+  key.nums.push_back(nn);
+  key.nums.push_back(rr);
   if (f32) {
     stir_rgms_f32_plan* plan = g_rgms_f32_plans.find(key);
     if (!plan) {
@@ -512,10 +517,6 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
     return forward(stir_rgms_f32(plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, (const float*)W.data,
                                  (const float*)X.data, (float*)Y.data, g_stream));
   }
-  // an edge index also depends on the sizes the launch is given
-  key.nums.push_back(mm);
-  key.nums.push_back(nn);
-  key.nums.push_back(rr);
   stir_rgms_plan* plan = g_rgms_plans.find(key);
   if (!plan) {
     if (stir_rgms_plan_create(&plan, nb, rb.data(), cb.data(), groups.data(), Ak.data(), Rk.data(), Ck.data(),

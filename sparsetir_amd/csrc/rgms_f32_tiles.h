@@ -1,0 +1,59 @@
+// Destination-tiled fp32 RGMS: every 64-row tile of Y is summed on chip and written once, without
+// atomics.  Serves both fp32 front ends (ELL3D buckets and the CSF arrays).
+//
+// The edges (slots) of the operator are re-indexed once per plan, sorted by (destination tile of
+// 64 rows, relation, destination row); runs of equal key are the (relation, row) pairs, whose
+// weighted sums of X rows meet the relation's W on the matrix cores 16 pairs at a time
+// (v_mfma_f32_16x16x4_f32), and the products are added into a partial tile in LDS.
+#pragma once
+#include <cstdint>
+#include <vector>
+
+#include "common.h"
+
+namespace stir {
+
+struct F32Bucket {
+  const float* A;       // device: slot weights, groups*rb*cb
+  const int32_t* rows;  // device: groups*rb
+  const int32_t* cols;  // device: groups*rb*cb
+  const int32_t* mids;  // device: groups
+  int64_t groups;
+  int32_t rb, cb;
+};
+
+// Where the edges come from: ELL3D buckets, or (csf) the four CSF arrays and their edge values.
+struct F32Source {
+  bool csf = false;
+  std::vector<F32Bucket> buckets;
+  const float* A = nullptr;
+  const int32_t* indptr_i = nullptr;
+  const int32_t* indices_i = nullptr;
+  const int32_t* indptr_j = nullptr;
+  const int32_t* indices_j = nullptr;
+  int64_t nnz_i = 0, nnz_j = 0;
+};
+
+struct F32TileIndex {
+  int32_t m = -1, n = -1, num_rels = -1;  // what the index was built for
+  int64_t edges = 0, pairs = 0, batches = 0, tiles = 0;
+  void* d_edges = nullptr;       // edges x 16 bytes, sorted
+  void* d_pairs = nullptr;       // pairs x 16 bytes, sorted
+  void* d_batches = nullptr;     // batches x 16 bytes: up to 16 pairs of one (tile, relation) each
+  void* d_tile_pairs = nullptr;  // tiles + 1 offsets into d_batches
+  void* d_wpack = nullptr;       // W in the multiply's operand order, rewritten by every launch
+  size_t wpack_bytes = 0;
+};
+
+// True when the kernel serves these feature sizes (else the caller keeps its other kernel).
+bool f32_tiles_serves(int32_t feat_in, int32_t feat_out);
+// Builds the index on `stream` (synchronises; allocates).  A no-op when it exists for the same m,
+// n and num_rels.  Fails when a row id, column id or relation id is out of range.
+int f32_tiles_prepare(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, int32_t num_rels,
+                      hipStream_t stream);
+// Y += RGMS(W, X) over the indexed edges.  W: [R, feat_out, feat_in], X: [n, feat_in], fp32.
+int f32_tiles_launch(F32TileIndex& idx, int32_t feat_in, int32_t feat_out, const float* d_W, const float* d_X,
+                     float* d_Y, hipStream_t stream);
+void f32_tiles_free(F32TileIndex& idx);
+
+}  // namespace stir

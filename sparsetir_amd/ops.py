@@ -520,27 +520,60 @@ class Rgms(_Operator):
                 self._plans.put(key, plan, rest)
                 if self._static and self._in_dtype is not torch.float32:
                     _lib.check(self.L.stir_rgms_plan_set_static_weights(plan, 1))
+                if getattr(self, "_deterministic", False):
+                    _lib.check(self.L.stir_rgms_f32_plan_set_deterministic(plan, 1))
             _lib.check(getattr(self.L, self._fns[1])(plan, self.m, self.n, self.R, self.fin, self.fout,
                                                      _ptr(w), _ptr(x), _ptr(y), _stream()))
 
 
 class RgmsF32(Rgms):
     """fp32 RGMS on ELL3D buckets with W laid out [R, feat_out, feat_in]: the composable operator of
-    examples/rgms/rgcn/bench_rgcn_composable.py:208-221, same argument order as :class:`Rgms`."""
+    examples/rgms/rgcn/bench_rgcn_composable.py:208-221, same argument order as :class:`Rgms`.
+    Adds to Y with atomics; ``deterministic=True`` (no counterpart in the reference) instead sums
+    every 64-row tile of Y on chip in a fixed order, from an edge index its plans build at their
+    first call: the same bits on every run, at about 1.5 times the run time."""
     name = "rgms_f32"
     _in_dtype = torch.float32
     _fns = ("stir_rgms_f32_plan_create", "stir_rgms_f32", "stir_rgms_f32_plan_destroy")
 
+    def __init__(self, *args, deterministic=False, **kwargs):
+        super().__init__(*args, **kwargs)
+        self._deterministic = bool(deterministic)
+
 
 class RgmsCsf(_Operator):
     """fp32 RGMS over the CSF arrays: f(A, W, X, Y, indptr_i, indices_i, indptr_j, indices_j), the
-    non-composable operator of examples/rgms/rgcn/bench_rgcn_non_composable.py:82-112."""
+    non-composable operator of examples/rgms/rgcn/bench_rgcn_non_composable.py:82-112.
+
+    By default stateless, like the reference's operator: every call reads the arrays and adds to Y
+    with atomics.  ``deterministic=True`` (no counterpart in the reference) gives sums that come
+    out the same, bit for bit, on every run, at the same speed: the operator then keeps plans,
+    keyed by the addresses of the five graph arrays and torch's version counters of the four index
+    arrays; from 8192 edges on a plan holds an edge index by 64-row tile of Y (built by the first
+    call: it allocates and synchronises) and Y is accumulated into without atomics.  The edge
+    values ``A`` are read on every call either way."""
     name = "rgms_csf"
 
-    def __init__(self, m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j):
+    def __init__(self, m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j, deterministic=False):
         self.m, self.n, self.R = int(m), int(n), int(num_rels)
         self.fin, self.fout, self.nnz_i, self.nnz_j = int(feat_in), int(feat_out), int(nnz_i), int(nnz_j)
+        self.deterministic = bool(deterministic)
         self.L = _lib.lib()
+        self._plans = _PlanCache(self.L.stir_rgms_csf_f32_plan_destroy)
+
+    @property
+    def plan_builds(self):
+        return self._plans.builds
+
+    def invalidate(self):
+        """Forget the plans (and edge indices) made from the arrays of earlier calls."""
+        self._plans.clear()
+
+    def __del__(self):
+        try:
+            self._plans.clear()
+        except Exception:
+            pass
 
     def __call__(self, *args):
         f32, i32 = torch.float32, torch.int32
@@ -549,10 +582,23 @@ class RgmsCsf(_Operator):
                                  ("indptr_i", i32, self.R + 1), ("indices_i", i32, self.nnz_i),
                                  ("indptr_j", i32, self.nnz_i + 1), ("indices_j", i32, self.nnz_j)])
         a, w, x, y, pi, ii, pj, ij = args
+        if not self.deterministic:
+            with torch.cuda.device(dev):
+                _lib.check(self.L.stir_rgms_csf_f32(self.m, self.n, self.R, self.fin, self.fout, self.nnz_i,
+                                                    self.nnz_j, _ptr(a), _ptr(w), _ptr(x), _ptr(y), _ptr(pi),
+                                                    _ptr(ii), _ptr(pj), _ptr(ij), _stream()))
+            return
+        graph = (a, pi, ii, pj, ij)
+        key = (dev, tuple(map(_data_ptrs, graph)), tuple(map(_version_of, graph[1:])))
         with torch.cuda.device(dev):
-            _lib.check(self.L.stir_rgms_csf_f32(self.m, self.n, self.R, self.fin, self.fout, self.nnz_i,
-                                                self.nnz_j, _ptr(a), _ptr(w), _ptr(x), _ptr(y), _ptr(pi),
-                                                _ptr(ii), _ptr(pj), _ptr(ij), _stream()))
+            plan = self._plans.get(key)
+            if plan is None:
+                plan = ctypes.c_void_p()
+                _lib.check(self.L.stir_rgms_csf_f32_plan_create(ctypes.byref(plan), self.nnz_i, self.nnz_j, _ptr(a),
+                                                                _ptr(pi), _ptr(ii), _ptr(pj), _ptr(ij)))
+                self._plans.put(key, plan, graph)
+            _lib.check(self.L.stir_rgms_csf_f32_planned(plan, self.m, self.n, self.R, self.fin, self.fout, _ptr(w),
+                                                        _ptr(x), _ptr(y), _stream()))
 
 
 def build_csrmm(m, n, feat, nnz):
@@ -592,9 +638,9 @@ def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dt
     return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype, static_weights)
 
 
-def build_rgms_f32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups):
-    return RgmsF32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups)
+def build_rgms_f32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, deterministic=False):
+    return RgmsF32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, deterministic=deterministic)
 
 
-def build_rgms_csf(m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j):
-    return RgmsCsf(m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j)
+def build_rgms_csf(m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j, deterministic=False):
+    return RgmsCsf(m, n, num_rels, feat_in, feat_out, nnz_i, nnz_j, deterministic)

@@ -78,7 +78,7 @@ def test_rgms_csf_f32_empty(dev):
     assert torch.all(y == 3.0)
 
 
-def _run_ell3d(dev, csf, n, x, w, group, buckets, weighted, seed=0):
+def _run_ell3d(dev, csf, n, x, w, group, buckets, weighted, seed=0, deterministic=False):
     R, fout, fin = w.shape
     rows_bkt = [max(1, group // b) for b in buckets]
     ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
@@ -92,7 +92,8 @@ def _run_ell3d(dev, csf, n, x, w, group, buckets, weighted, seed=0):
         bk.append((a, rows[b], cols[b], mid))
         triples += [_t(dev, a.ravel()), _t(dev, rows[b].ravel()), _t(dev, cols[b].ravel())]
         mids.append(_t(dev, mid))
-    f = ops.build_rgms_f32(n, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols])
+    f = ops.build_rgms_f32(n, n, R, fin, fout, rows_bkt, buckets, [c.shape[0] for c in cols],
+                           deterministic=deterministic)
     y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
     f(_t(dev, w.ravel()), _t(dev, x.ravel()), y, *triples, *mids)
     torch.cuda.synchronize()
@@ -139,3 +140,108 @@ def test_rgms_f32_config5_reduced_both_forms_agree(dev):
     torch.cuda.synchronize()
     _check(y.cpu().numpy().reshape(n, 32), want, scale, oracle.rgms_csf_f32(ones, w, cfg["x"], *csf, n), "config5 csf")
 
+
+
+# ---- deterministic=True, from 8192 slots on: the destination-tiled kernel (an edge index by 64-row
+# tile of Y, the (relation, row) pairs multiplied 16 at a time on the 16x16x4 fp32 instruction, no
+# atomics: the same bits on every run)
+
+@pytest.mark.parametrize("fin,fout,R,n", [
+    (32, 32, 7, 1000),    # the RGCN layer's sizes; the last tile has 40 rows
+    (20, 40, 3, 777),     # inputs and outputs that fill neither a k group nor an output tile
+    (64, 64, 5, 640),     # two input halves per lane, four output tiles
+    (48, 16, 40, 500),    # more relations than pairs in a product: most products hold one to three pairs
+    (4, 4, 2, 129),
+])
+def test_rgms_f32_tiled_both_front_ends(dev, fin, fout, R, n):
+    edges = 12000
+    csf = random_csf(R, n, edges, seed=fin * 100 + fout)
+    rng = np.random.default_rng(fin + R)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
+    a = (0.5 + rng.random(len(csf[3]), dtype=np.float32))
+    a[::5] = 0.0
+    assert len(csf[3]) >= 8192
+    want, scale = _closed_forms(csf, a, x, w, n)
+    # CSF front end, twice: the second call adds to Y, and both calls give the same bits
+    f = ops.build_rgms_csf(n, n, R, fin, fout, len(csf[1]), len(csf[3]), deterministic=True)
+    d = [_t(dev, a), _t(dev, w.ravel()), _t(dev, x.ravel())]
+    d_csf = [_t(dev, c) for c in csf]
+    y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
+    f(d[0], d[1], d[2], y, *d_csf)
+    torch.cuda.synchronize()
+    first = y.clone()
+    _check(first.cpu().numpy().reshape(n, fout), want, scale, oracle.rgms_csf_f32(a, w, x, *csf, n), "tiled csf")
+    y2 = torch.zeros_like(y)
+    f(d[0], d[1], d[2], y2, *d_csf)
+    f(d[0], d[1], d[2], y, *d_csf)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, first)  # no atomics: the same sums in the same order
+    assert np.all(np.abs(y.cpu().numpy().reshape(n, fout) - 2 * want) <= 2e-5 * np.abs(want) + 2e-5 * scale + 1e-30)
+    assert f.plan_builds == 1
+    # edge values rewritten in place are read by the next call (the plan holds their addresses)
+    d[0].mul_(2.0)
+    y3 = torch.zeros_like(y)
+    f(d[0], d[1], d[2], y3, *d_csf)
+    torch.cuda.synchronize()
+    assert np.all(np.abs(y3.cpu().numpy().reshape(n, fout) - 2 * want) <= 2e-5 * np.abs(want) + 2e-5 * scale + 1e-30)
+    # ELL3D front end on the same graph (weights 1)
+    ones = np.ones(len(csf[3]), np.float32)
+    want1, scale1 = _closed_forms(csf, ones, x, w, n)
+    got, bk = _run_ell3d(dev, csf, n, x, w, 32, [1, 2, 4, 8, 16], False, deterministic=True)
+    assert sum(b[0].size for b in bk) >= 8192
+    _check(got, want1, scale1, oracle.rgms_ell3d_f32(w, x, bk, n), "tiled ell3d")
+    again, _ = _run_ell3d(dev, csf, n, x, w, 32, [1, 2, 4, 8, 16], False, deterministic=True)
+    assert np.array_equal(got, again)
+
+
+def test_rgms_f32_tiled_hub_row_and_empty_relations(dev):
+    """A destination row with 9000 edges of one relation (one pair whose edges a lane group walks
+    four at a time), relations without rows, a tile of Y without edges, m != n."""
+    m, n, fin, fout, R = 700, 9500, 32, 32, 6
+    rng = np.random.default_rng(5)
+    rows_per_rel = [np.asarray([3, 650], np.int32), np.zeros(0, np.int32), np.asarray([3, 4, 5, 699], np.int32),
+                    np.zeros(0, np.int32), np.zeros(0, np.int32), np.asarray([650], np.int32)]
+    counts = {(0, 3): 9000, (0, 650): 40, (2, 3): 5, (2, 4): 1, (2, 5): 70, (2, 699): 17, (5, 650): 300}
+    p0, i0, p1, i1 = [0], [], [0], []
+    for r in range(R):
+        for row in rows_per_rel[r]:
+            i0.append(int(row))
+            cols = np.sort(rng.choice(n, counts[(r, int(row))], replace=False))
+            i1.extend(cols.tolist())
+            p1.append(len(i1))
+        p0.append(len(i0))
+    csf = tuple(np.asarray(v, np.int32) for v in (p0, i0, p1, i1))
+    assert len(csf[3]) >= 8192
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
+    a = rng.standard_normal(len(csf[3])).astype(np.float32)
+    f = ops.build_rgms_csf(m, n, R, fin, fout, len(csf[1]), len(csf[3]), deterministic=True)
+    y = torch.zeros(m * fout, dtype=torch.float32, device=dev)
+    f(_t(dev, a), _t(dev, w.ravel()), _t(dev, x.ravel()), y, *[_t(dev, c) for c in csf])
+    torch.cuda.synchronize()
+    want, scale = _closed_forms(csf, a, x, w, m)
+    got = y.cpu().numpy().reshape(m, fout)
+    _check(got, want, scale, oracle.rgms_csf_f32(a, w, x, *csf, m), "hub row")
+    untouched = np.setdiff1d(np.arange(m), [3, 4, 5, 650, 699])
+    assert np.all(got[untouched] == 0)
+
+
+def test_rgms_f32_tiled_rejects_bad_ids(dev):
+    """Row, column and relation ids are checked when the index of the deterministic form is built."""
+    from sparsetir_amd._lib import SparseTIRError
+    R, n, fin, fout = 3, 500, 32, 32
+    csf = list(random_csf(R, n, 30000, seed=77))
+    assert len(csf[3]) >= 8192  # below that the kernel with atomics runs, which reads no index ahead
+    x = torch.zeros(n * fin, device=dev)
+    w = torch.zeros(R * fout * fin, device=dev)
+    a = torch.ones(len(csf[3]), device=dev)
+    bad_cols = csf[3].copy()
+    bad_cols[123] = n
+    f = ops.build_rgms_csf(n, n, R, fin, fout, len(csf[1]), len(csf[3]), deterministic=True)
+    with pytest.raises(SparseTIRError, match="column id"):
+        f(a, w, x, torch.zeros(n * fout, device=dev), _t(dev, csf[0]), _t(dev, csf[1]), _t(dev, csf[2]), _t(dev, bad_cols))
+    bad_rows = csf[1].copy()
+    bad_rows[7] = n + 5
+    with pytest.raises(SparseTIRError, match="row id"):
+        f(a, w, x, torch.zeros(n * fout, device=dev), _t(dev, csf[0]), _t(dev, bad_rows), _t(dev, csf[2]), _t(dev, csf[3]))
