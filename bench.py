@@ -38,6 +38,7 @@ import time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 ROOT = os.path.dirname(os.path.abspath(__file__))
 
 # ---- bandwidth probes: a small library of this benchmark's own (bench_probes.hip), not part of
@@ -56,8 +57,19 @@ def build_probes():
     return PROBES_LIB
 
 
+PROBE_SYMBOLS = ("bench_probe_copy", "bench_probe_gather", "bench_probe_atomic_rows", "bench_probe_mfma_f16")
+
+
 def load_probes():
-    if not os.path.exists(PROBES_LIB):
+    """The probe library, built first when it is missing, older than its source, or lacks a symbol
+    this file binds (a checkout that kept a library from an older bench_probes.hip)."""
+    stale = (not os.path.exists(PROBES_LIB)
+             or os.path.getmtime(PROBES_LIB) < os.path.getmtime(PROBES_SRC))
+    if not stale:
+        have = ctypes.CDLL(PROBES_LIB)
+        stale = not all(hasattr(have, name) for name in PROBE_SYMBOLS)
+        del have
+    if stale:
         build_probes()
     L = ctypes.CDLL(PROBES_LIB)
     VP, I64, I32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
@@ -70,24 +82,36 @@ def load_probes():
 
 
 def measured_traffic(workload):
-    """HBM-side bytes per launch of the headline kernel as measured with rocprofv3 --pmc
-    (FETCH_SIZE, WRITE_SIZE, scaled by a plain copy of known size).  The summaries under
-    profiles/ carry one line per measured workload,
-        traffic-bytes-per-launch: workload=<signature> bytes=<float> kernel-source-sha1=<sha1>
-    where the sha1 is that of sparsetir_amd/csrc/spmm.hip when the counters were taken.  Returns
-    (bytes, note); bytes is None when nothing was measured for this workload or the kernel source
-    has changed since."""
-    with open(os.path.join(ROOT, "sparsetir_amd", "csrc", "spmm.hip"), "rb") as f:
-        now = hashlib.sha1(f.read()).hexdigest()
-    pat = re.compile(r"traffic-bytes-per-launch:\s+workload=(\S+)\s+bytes=(\S+)\s+kernel-source-sha1=(\w+)")
+    """HBM-side bytes per launch of a kernel as measured with rocprofv3 --pmc (FETCH_SIZE,
+    WRITE_SIZE, scaled by a plain copy of known size).  The summaries under profiles/ carry one
+    line per measured workload,
+        traffic-bytes-per-launch: workload=<signature> bytes=<float> kernel-source-sha1=<sha1> [kernel-source=<file>]
+    where the sha1 is that of the kernel's source file under sparsetir_amd/csrc/ (spmm.hip when the
+    line names none) when the counters were taken.  Returns (bytes, note); bytes is None when
+    nothing was measured for this workload or the kernel source has changed since."""
+    pat = re.compile(r"traffic-bytes-per-launch:\s+workload=(\S+)\s+bytes=(\S+)\s+kernel-source-sha1=(\w+)"
+                     r"(?:\s+kernel-source=(\S+))?")
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
         for line in open(path):
             mt = pat.search(line)
             if mt and mt.group(1) == workload:
+                src = mt.group(4) or "spmm.hip"
+                with open(os.path.join(ROOT, "sparsetir_amd", "csrc", src), "rb") as f:
+                    now = hashlib.sha1(f.read()).hexdigest()
                 if mt.group(3) != now:
-                    return None, f"stale: spmm.hip changed since {os.path.basename(path)} was taken"
+                    return None, f"stale: {src} changed since {os.path.basename(path)} was taken"
                 return float(mt.group(2)), os.path.basename(path)
     return None, "not measured for this workload"
+
+
+def side_roofline(bound, achieved, tag):
+    """The roofline block of a side kernel: `achieved` in TFLOP/s against the dense fp16 MFMA peak
+    (bound "mfma") or in GB/s of algorithmic bytes against the HBM peak (bound "hbm"); traffic
+    from the profile line of workload `tag`, if one exists for the kernel source as it is now."""
+    peak = MFMA_F16_PEAK_TFLOPS if bound == "mfma" else HBM_PEAK_GBS
+    traffic, note = measured_traffic(tag)
+    return {"bound": bound, "achieved": achieved, "peak": peak, "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
+            "frac": achieved / peak, "traffic": traffic, "traffic_source": note}
 
 
 def parse():
@@ -178,7 +202,6 @@ def time_small(fn, calls, warmup, torch, graph=True):
     return out
 
 
-MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
 def config2_sweep(torch, dev, ops, st, datasets, time_steps):
@@ -194,19 +217,31 @@ def config2_sweep(torch, dev, ops, st, datasets, time_steps):
         for b in range(len(buckets)):
             triples += [mask[p][b].reshape(-1).float(), rows[p][b], cols[p][b].reshape(-1)]
             nrows.append(int(rows[p][b].shape[0]))
+    # ... and the decomposition format.suggest_decomposition gives for this GPU (one partition)
+    sparts, sbuckets = st.suggest_decomposition(m, n, nnz, 128)
+    srows, scols, smask = st.column_part_hyb(m, n, d_ptr, d_idx, sparts, sbuckets)
+    striples, snrows = [], []
+    for b in range(len(sbuckets)):
+        striples += [smask[0][b].reshape(-1).float(), srows[0][b], scols[0][b].reshape(-1)]
+        snrows.append(int(srows[0][b].shape[0]))
     ones = torch.ones(nnz, device=dev)
-    out = {"nodes": m, "edges": nnz, "num_col_parts": parts}
+    out = {"nodes": m, "edges": nnz, "num_col_parts": parts,
+           "suggested_decomposition": {"num_col_parts": sparts, "buckets": sbuckets}}
     for feat in (32, 64, 128, 256):
         x = torch.randn(n * feat, device=dev)
         c = torch.zeros(m * feat, device=dev)
         hyb = ops.build_hyb_csrmm(m, n, feat, parts, buckets, nrows)
+        shyb = ops.build_hyb_csrmm(m, n, feat, sparts, sbuckets, snrows)
         csr = ops.build_csrmm(m, n, feat, nnz)
         reps = 3 if PROFILE_RUN else 50
         _, dh, _ = time_steps(lambda: hyb(x, c, *triples), reps, 2, torch)
+        _, ds, _ = time_steps(lambda: shyb(x, c, *striples), reps, 2, torch)
         _, dc, _ = time_steps(lambda: csr(ones, x, c, d_ptr, d_idx), reps, 2, torch)
         byts = 8.0 * nnz + 4.0 * (m + 1) + 4.0 * n * feat + 4.0 * m * feat
         out[f"feat{feat}"] = {"hyb_us": dh * 1e6, "csr_us": dc * 1e6, "hyb_gflops": 2.0 * nnz * feat / dh / 1e9,
-                              "hyb_alg_GBps": byts / dh / 1e9}
+                              "hyb_alg_GBps": byts / dh / 1e9, "hyb_suggested_us": ds * 1e6,
+                              "hyb_suggested_alg_GBps": byts / ds / 1e9,
+                              "roofline": side_roofline("hbm", byts / dh / 1e9, f"config2/p{parts}/f{feat}")}
     return out
 
 
@@ -230,8 +265,9 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
         byts = 2.0 * nnzb * blk * blk + 4 * nnzb + 4 * (mb + 1) + 2.0 * nb * blk * feat + 2.0 * mb * blk * feat
         out[tag] = dict(tm, us=d * 1e6, tflops=flops / d / 1e12,
                         frac_of_mfma_peak=flops / d / 1e12 / MFMA_F16_PEAK_TFLOPS, alg_GBps=byts / d / 1e9,
-                        frac_of_hbm_peak=byts / d / 1e9 / HBM_PEAK_GBS, nnzb=nnzb,
-                        shape=[mb * blk, nb * blk, feat], blk=blk, dtype=str(dtype).split(".")[-1])
+                        frac_of_hbm_peak=byts / d / 1e9 / HBM_PEAK_GBS, nnzb=nnzb, algorithmic_bytes=byts,
+                        shape=[mb * blk, nb * blk, feat], blk=blk, dtype=str(dtype).split(".")[-1],
+                        roofline=side_roofline("mfma", flops / d / 1e12, tag))
 
     bsr("bsr_config4_f16", 128, 128, 32, 0.10, 512, torch.float16)
     bsr("bsr_config4_bf16", 128, 128, 32, 0.10, 512, torch.bfloat16)
@@ -240,6 +276,8 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     bsr("bsr_16384x16384_f4096_f16", 512, 512, 32, 0.10, 4096, torch.float16, calls=20)
     bsr("bsr_16384x16384_blk64_f4096_f16", 256, 256, 64, 0.10, 4096, torch.float16, calls=20)
     bsr("bsr_16384x16384_blk128_f4096_f16", 128, 128, 128, 0.10, 4096, torch.float16, calls=20)
+    # 16 x 16 blocks, the granularity of the reference's schedule (bsr_spmm.py:379-380): 16-row slices on 16x16x32
+    bsr("bsr_16384x16384_blk16_f4096_f16", 1024, 1024, 16, 0.10, 4096, torch.float16, calls=10)
 
     cfg = datasets.config5()
     R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
@@ -294,6 +332,7 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
         d = tm["us_back_to_back"] / 1e6
         out[tag] = dict(tm, us=d * 1e6, first_call_ms=first_s * 1e3, tflops=flops / d / 1e12,
                         alg_GBps=byts / d / 1e9, frac_of_hbm_peak=byts / d / 1e9 / HBM_PEAK_GBS, edges=E,
+                        algorithmic_bytes=byts, roofline=side_roofline("mfma", flops / d / 1e12, tag),
                         ell_rows=int(sum(r.size for r in rows)), static_weights=static,
                         accumulation="32-row output tiles written once; tiles cut by a share boundary add with atomics")
 
@@ -315,9 +354,10 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     f(w_r, x_r, y, *triples_r, *mids_r)
     tm = time_small(lambda: f(w_r, x_r, y, *triples_r, *mids_r), 50, 3, torch)
     Er = int(cfg_r["indices1"].shape[0])
+    tf_r = (2.0 * Er * fin * fout + 2.0 * Er * fout) / tm["us_back_to_back"] / 1e6
     out["rgms_130_relations"] = dict(tm, us=tm["us_back_to_back"], edges=Er, num_rels=Rr, static_weights=True,
-                                     tflops=(2.0 * Er * fin * fout + 2.0 * Er * fout) / tm["us_back_to_back"] / 1e6,
-                                     launches_per_call=2)
+                                     tflops=tf_r, launches_per_call=2,
+                                     roofline=side_roofline("mfma", tf_r, "rgms_130_relations"))
     del d_csf, triples_r, mids_r, w_r, x_r, f
 
     # SpMM over the condensed format (t = 32, g = 16) on the config-2 graph, fp16 in, fp32 out
@@ -354,7 +394,9 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     nnz2 = len(g2["indices"])
     out["tcspmm_config2_feat128"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "useful_gflops": 2.0 * nnz2 * f2 / d / 1e9,
                                      "mfma_tflops": 2.0 * nnzb2 * 32 * 16 * f2 / d / 1e12, "groups": int(nnzb2),
-                                     "mask_density": float(nnz2) / (nnzb2 * 32 * 16)}
+                                     "mask_density": float(nnz2) / (nnzb2 * 32 * 16),
+                                     "roofline": side_roofline("mfma", 2.0 * nnzb2 * 32 * 16 * f2 / d / 1e12,
+                                                               "tcspmm_config2_feat128")}
     # the reference's own form of this operator writes fp16 (bench_tc_spmm.py: fp16 accumulator fragments)
     tc16 = ops.build_tcspmm(mb2, nnzb2, f2, 32, 16, g2["n"], torch.float16)
     c16 = torch.zeros(mb2 * 32 * f2, device=dev, dtype=torch.float16)
@@ -366,7 +408,32 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     out["tcspmm_config2_feat128_f16_out"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"],
                                              "us": tm["us_back_to_back"], "first_call_ms": first_ms,
                                              "useful_gflops": 2.0 * nnz2 * f2 / tm["us_back_to_back"] / 1e3,
-                                             "plan": "made from the group counts at the first call"}
+                                             "plan": "made from the group counts at the first call",
+                                             "roofline": side_roofline(
+                                                 "mfma", 2.0 * nnzb2 * 32 * 16 * f2 / tm["us_back_to_back"] / 1e6,
+                                                 "tcspmm_config2_feat128_f16_out")}
+    # the tile sizes the reference condenses with (tile_size = mma_m: 8 by default, 16;
+    # examples/spmm/bench_tc_spmm.py:584-585,670) beside 32, fp16 out, condensed on the GPU
+    d_ptr2, d_idx2 = t(g2["indptr"]), t(g2["indices"])
+    sizes = {}
+    for tsz in (8, 16, 32):
+        gptr_t, tiles_t, mask_t = st.condense(d_ptr2, d_idx2, tsz, 16)
+        mb_t, nnzb_t = int(gptr_t.shape[0]) - 1, int(tiles_t.shape[0])
+        f_t = ops.build_tcspmm(mb_t, nnzb_t, f2, tsz, 16, g2["n"], torch.float16)
+        a_t, ti_t = mask_t.reshape(-1).half(), tiles_t.reshape(-1)
+        c_t = torch.zeros(mb_t * tsz * f2, device=dev, dtype=torch.float16)
+        f_t(a_t, b2, c_t, gptr_t, ti_t)
+        tm = time_small(lambda: f_t(a_t, b2, c_t, gptr_t, ti_t), 50, 5, torch)
+        us = tm["us_back_to_back"]
+        # the matrix cores multiply 16-row operands for tiles of 8 rows
+        mfma_tf = 2.0 * nnzb_t * max(tsz, 16) * 16 * f2 / us / 1e6
+        sizes[f"tile{tsz}"] = {"us": us, "us_graph": tm["us_graph"], "row_tiles": mb_t, "groups": nnzb_t,
+                               "mask_density": float(nnz2) / (nnzb_t * tsz * 16),
+                               "useful_gflops": 2.0 * nnz2 * f2 / us / 1e3, "mfma_tflops": mfma_tf,
+                               "roofline": side_roofline("mfma", mfma_tf, f"tcspmm_config2_tile{tsz}")}
+        del f_t, a_t, ti_t, c_t, gptr_t, tiles_t, mask_t
+    out["tcspmm_config2_tile_sizes"] = sizes
+    del d_ptr2, d_idx2
     # the entry point without a plan, as a TVM process binds it
     from sparsetir_amd import _lib as stlib
     L16 = stlib.lib()
@@ -400,7 +467,15 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     d = tm["us_back_to_back"] / 1e6
     out["rgms_f32_ell3d_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
                                      "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
+                                     "algorithmic_bytes": byts32,
+                                     "roofline": side_roofline("hbm", byts32 / d / 1e9, "rgms_f32_ell3d_config5"),
                                      "ell_rows": int(sum(r.size for r in rows))}
+    # the optional form without atomics (the same bits on every run)
+    f32d = ops.build_rgms_f32(n, n, R, fin, fout, rb32, buckets, [c.shape[0] for c in cols], deterministic=True)
+    f32d(w32, x32, y, *triples, *mids)  # builds its edge index
+    tm_d = time_small(lambda: f32d(w32, x32, y, *triples, *mids), 20, 2, torch)
+    out["rgms_f32_ell3d_config5"]["deterministic_us"] = tm_d["us_back_to_back"]
+    del f32d
     # every ELL row adds feat_out floats to Y with one atomic each: the launch's bound.  Beside
     # it, what the same number of row additions to hashed rows of Y takes with nothing else going on
     er = out["rgms_f32_ell3d_config5"]["ell_rows"]
@@ -408,11 +483,10 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     out["rgms_f32_ell3d_config5"]["atomic_adds_G_per_s"] = er * fout / d / 1e9
     if fout == 32:
         P = load_probes()
-        st0 = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         yp = ctypes.c_void_p(y.data_ptr())
 
-        def scatter_only():
-            if P.bench_probe_atomic_rows(yp, n, er, st0) != 0:
+        def scatter_only():  # on the stream that is current when it is called (a capture has its own)
+            if P.bench_probe_atomic_rows(yp, n, er, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) != 0:
                 raise RuntimeError("atomic probe failed")
         tp = time_small(scatter_only, 20, 2, torch)
         out["rgms_f32_ell3d_config5"]["probe_atomic_rows_us"] = tp["us_back_to_back"]
@@ -424,7 +498,14 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     d = tm["us_back_to_back"] / 1e6
     out["rgms_f32_csf_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
                                    "frac_of_hbm_peak": byts32 / d / 1e9 / HBM_PEAK_GBS,
+                                   "algorithmic_bytes": byts32,
+                                   "roofline": side_roofline("hbm", byts32 / d / 1e9, "rgms_f32_csf_config5"),
                                    "stored_rows": int(len(cfg["indices0"]))}
+    fcd = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E, deterministic=True)
+    fcd(ones, w32, x32, y, *csf)  # builds its edge index
+    tm_d = time_small(lambda: fcd(ones, w32, x32, y, *csf), 20, 2, torch)
+    out["rgms_f32_csf_config5"]["deterministic_us"] = tm_d["us_back_to_back"]
+    del fcd
     return out
 
 
@@ -622,7 +703,9 @@ def main():
         extra = {}
         steps = max(3, min(args.steps, 10))
         w2, d2, _ = time_steps(lambda: csr(ones, x, c_csr, d_indptr, d_indices), steps, 1, torch)
-        extra["csr_spmm"] = {"gflops": flops / w2 / 1e9, "ms": d2 * 1e3, "alg_GBps": alg_bytes / d2 / 1e9}
+        extra["csr_spmm"] = {"gflops": flops / w2 / 1e9, "ms": d2 * 1e3, "alg_GBps": alg_bytes / d2 / 1e9,
+                             "roofline": side_roofline("hbm", alg_bytes / d2 / 1e9,
+                                                       f"csr/{args.columns}/f{feat}/s{args.scale}")}
         del c_csr, ones
         f2 = 64
         gen = wl["gen"]
@@ -641,6 +724,9 @@ def main():
         extra["sddmm_feat64_scaled"] = {"gflops": (2.0 * f2 + 1.0) * nnz / w4 / 1e9, "ms": d4 * 1e3,
                                         "alg_GBps": sd_bytes / d4 / 1e9,
                                         "frac_of_hbm_peak": sd_bytes / d4 / 1e9 / HBM_PEAK_GBS,
+                                        "algorithmic_bytes": sd_bytes,
+                                        "roofline": side_roofline("hbm", sd_bytes / d4 / 1e9,
+                                                                  f"sddmm/{args.columns}/f{f2}/s{args.scale}"),
                                         "preproc_ms": d3 * 1e3}
         del edge, a2, b2, out, mid, sargs
         if args.parts is None and args.buckets is None and not getattr(args, "profile", False):

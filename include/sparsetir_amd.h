@@ -251,7 +251,10 @@ int stir_hyb_plan_destroy(stir_hyb_plan* plan);
  * SpMM kernel (plus one small launch per 32 buckets that writes the descriptors): with several
  * partitions every bucket adds with atomics, as in the reference (examples/spmm/bench_spmm.py:170).
  * Calls on one GPU share that array: calls that overlap in time on one GPU (different streams or
- * threads) race; calls on one stream are ordered and safe.
+ * threads) race; calls on one stream are ordered and safe.  The first call on a device looks up
+ * the array's address (hipGetDevice, hipGetSymbolAddress) and must happen outside a stream
+ * capture; later calls may be recorded into a graph -- the descriptors travel inside the recorded
+ * fill kernels' arguments, so every replay writes them again before its SpMM kernel reads them.
  */
 int stir_hyb_spmm_f32_noalloc(int32_t m, int32_t n, int32_t num_col_parts, int32_t num_buckets,
                               const int32_t* bucket_widths, const int64_t* nrows,

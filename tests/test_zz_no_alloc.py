@@ -104,3 +104,66 @@ def test_noalloc_rejects_more_buckets_than_the_fixed_array_holds(dev):
     assert rc == -1
     assert b"at most 1024" in L.stir_last_error()
     assert bool((y == 0).all())
+
+
+def test_noalloc_inside_a_captured_graph(dev):
+    """What the entry point is for: a call recorded into a HIP graph (after one eager call on the
+    device, which looks up the fixed array's address -- that first call must happen outside a
+    capture).  The graph is replayed twice; between the replays an eager call with another, smaller
+    operator overwrites the descriptors in the fixed array, so the second replay only gives the
+    right sums if the recorded fill kernels write them again.  Every replay is compared with the
+    plan-based pair."""
+    L = _lib.lib()
+    feat, parts, buckets = 64, 2, [1, 2, 4, 8, 16, 32]
+    nb = len(buckets)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+    tab = lambda ts: _lib.ptr_table([t.data_ptr() if t.numel() else 0 for t in ts])
+    widths = (ctypes.c_int32 * nb)(*buckets)
+
+    def operator(m, n, nnz, seed):
+        indptr, indices, vals, A, R, C, nrows = _decompose(dev, m, n, nnz, parts, buckets, seed=seed)
+        x = torch.randn(n * feat, device=dev, generator=torch.Generator(device=dev).manual_seed(seed))
+        counts = (ctypes.c_int64 * len(nrows))(*nrows)
+        return dict(m=m, n=n, indptr=indptr, vals=vals, A=A, R=R, C=C, nrows=nrows, x=x, counts=counts,
+                    tabs=(tab(A), tab(R), tab(C)))
+
+    def launch(op, out):
+        ta, tr, tc = op["tabs"]
+        _lib.check(L.stir_hyb_spmm_f32_noalloc(op["m"], op["n"], parts, nb, widths, op["counts"], ta, tr, tc, feat,
+                                               vp(op["x"]), vp(out),
+                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+    def expected(op):
+        ta, tr, tc = op["tabs"]
+        plan = ctypes.c_void_p()
+        _lib.check(L.stir_hyb_plan_create(ctypes.byref(plan), op["m"], op["n"], parts, nb, widths, op["counts"], ta, tr, tc))
+        want = torch.zeros(op["m"] * feat, device=dev)
+        _lib.check(L.stir_hyb_spmm_f32(plan, feat, vp(op["x"]), vp(want),
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        _lib.check(L.stir_hyb_plan_destroy(plan))
+        return want
+
+    big, small = operator(5000, 4000, 120000, 51), operator(600, 800, 5000, 52)
+    want_big, want_small = expected(big), expected(small)
+    out_big = torch.zeros(big["m"] * feat, device=dev)
+    out_small = torch.zeros(small["m"] * feat, device=dev)
+    launch(big, out_big)  # eager: the first call on this device
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        launch(big, out_big)
+    for replay in range(2):
+        out_big.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        _compare(dev, out_big, want_big, big["m"], feat, big["indptr"], big["vals"], big["x"], big["R"], big["nrows"],
+                 parts, nb, f"replay {replay}")
+        # another operator's descriptors go into the fixed array
+        out_small.zero_()
+        launch(small, out_small)
+        torch.cuda.synchronize()
+        _compare(dev, out_small, want_small, small["m"], feat, small["indptr"], small["vals"], small["x"], small["R"],
+                 small["nrows"], parts, nb, f"eager call after replay {replay}")
