@@ -161,12 +161,21 @@ PROFILE_RUN = False  # set by --profile
 
 
 def time_small(fn, calls, warmup, torch, graph=True):
-    """Three timings of a short kernel, in microseconds: events around every call, one event pair
+    """Three timings of a short kernel, in microseconds: events around every call (the median over
+    the calls: a single call now and then waits tens of milliseconds for the host), one event pair
     around a run of calls (the median of three such runs), and a captured graph of 20 launches
     replayed (device time only)."""
     if PROFILE_RUN:
         calls, warmup, graph = 3, 1, False
-    _, per_call, _ = time_steps(fn, calls, warmup, torch)
+    for _ in range(warmup):
+        fn()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(calls)]
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    per_call = float(np.median([a.elapsed_time(b) for a, b in pairs])) / 1e3
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     batches = []
     for _ in range(1 if PROFILE_RUN else 3):  # the median of three runs: clocks drift between neighbours
@@ -339,6 +348,18 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
                         algorithmic_bytes=byts, roofline=side_roofline("mfma", flops / d / 1e12, tag),
                         ell_rows=int(sum(r.size for r in rows)), static_weights=static,
                         accumulation="32-row output tiles written once; tiles cut by a share boundary add with atomics")
+
+    # an fp16 Y: the reference's operator built with dtype "float16" (bench_rgcn_tensorcore.py:564-607)
+    f = ops.build_rgms(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols], static_weights=True,
+                       out_dtype=torch.float16)
+    y16 = torch.zeros(n * fout, device=dev, dtype=torch.float16)
+    f(w, x, y16, *triples, *mids)
+    tm = time_small(lambda: f(w, x, y16, *triples, *mids), 50, 3, torch)
+    d = tm["us_back_to_back"] / 1e6
+    out["rgms_config5_f16_out"] = dict(tm, us=d * 1e6, tflops=flops / d / 1e12, static_weights=True,
+                                       algorithmic_bytes=byts - 2.0 * n * fout,
+                                       roofline=side_roofline("mfma", flops / d / 1e12, "rgms_config5_f16_out"))
+    del f, y16
 
     # The same layer with 130 relations (the reference's BGS and AM graphs have 200 to 270 with their
     # inverses): W is twice what the LDS of a compute unit holds, so the plan runs two ranges of

@@ -388,6 +388,17 @@ int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on);
  * time of the indexed form at 2M edges.  Fails once the plan has built its index.
  */
 int stir_rgms_plan_set_addresses_only(stir_rgms_plan* plan, int32_t on);
+/*
+ * The same with an fp16 Y: the operator of examples/rgms/rgcn/bench_rgcn_tensorcore.py:564-607
+ * built with dtype "float16" (its main program builds "float32" only, :893).  d_Y is [m, feat_out]
+ * fp16, 4-byte aligned, and is added to.  Sums are kept in fp32 (the reference's WMMA fragments
+ * accumulate in fp16); a row tile is rounded to fp16 once when it is written, and the few tiles
+ * that are cut between workgroups -- or every ELL row, for plans below 8192 slots -- are added
+ * with packed fp16 atomics, rounded once per addition.  Same plans as stir_rgms_f16.
+ */
+int stir_rgms_f16_out_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
+                          int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
+                          void* d_Y, void* stream);
 /* The same with bf16 W, X and slot weights (the reference has an fp16 example only). */
 int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
                    int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,

@@ -55,6 +55,7 @@ SIGNATURES = {
     "stir_tc_plan_destroy": (I32, [VP]),
     "stir_rgms_plan_create": (I32, [VP, I32, VP, VP, VP, VP, VP, VP, VP]),
     "stir_rgms_f16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
+    "stir_rgms_f16_out_f16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
     "stir_rgms_bf16": (I32, [VP, I32, I32, I32, I32, I32, VP, VP, VP, VP]),
     "stir_rgms_plan_set_static_weights": (I32, [VP, I32]),
     "stir_rgms_plan_set_addresses_only": (I32, [VP, I32]),

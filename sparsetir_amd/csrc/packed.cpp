@@ -455,8 +455,13 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
   const uint8_t fcode = bf ? kDLBfloat : kDLFloat;
   if (n < 5 || (n - 5) % 4 != 0) return packed_fail("%s: num_args should be 3 + 4*buckets + 2", a.fn);
   const int nb = (n - 5) / 4;
+  // the fp16 form also writes an fp16 Y (the reference's operator built with dtype "float16")
+  const DLTensor* d2 = (n > 2 && (tc[2] == kTVMDLTensorHandle || tc[2] == kTVMNDArrayHandle ||
+                                  tc[2] == kTVMOpaqueHandle))
+                           ? static_cast<const DLTensor*>(v[2].v_handle) : nullptr;
+  const bool out16 = !f32 && !bf && d2 && d2->dtype.code == kDLFloat && d2->dtype.bits == 16;
   Arr W = a.arr(0, "W", fcode, bits, kDevice), X = a.arr(1, "X", fcode, bits, kDevice),
-      Y = a.arr(2, "Y", kDLFloat, 32, kDevice);
+      Y = a.arr(2, "Y", kDLFloat, out16 ? 16 : 32, kDevice);
   const int64_t fin = a.integer(n - 2, "feat_in"), fout = a.integer(n - 1, "feat_out");
   if (!a.ok) return -1;
   if (fin <= 0 || fout <= 0 || W.len % (fin * fout) != 0 || X.len % fin != 0 || Y.len % fout != 0)
@@ -530,6 +535,9 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
     }
     g_rgms_plans.insert(key, plan);
   }
+  if (out16)
+    return forward(stir_rgms_f16_out_f16(plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data, X.data, Y.data,
+                                         g_stream));
   return forward((bf ? stir_rgms_bf16 : stir_rgms_f16)(plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, W.data, X.data,
                                                        (float*)Y.data, g_stream));
 }

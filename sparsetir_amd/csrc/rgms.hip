@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "common.h"
+#include "rgms_out.h"
 #include "rgms_tiles.h"
 #include "../../include/sparsetir_amd.h"
 
@@ -61,19 +62,15 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
                                                   0, 0);
 }
 
-__device__ __forceinline__ void atomic_addf(float* p, float v) {
-  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // One group (one relation), one wavefront.  KK = feat_in / 16; LCB = log2(cb) for power-of-two
 // cb <= 32, else -1.  The group is processed in chunks of TI tiles (32 slots each): the chunk's
 // column ids, slot weights and row ids are fetched with a few coalesced loads (lane l holds slots
 // l, l+64, ...), then the X rows of all TI tiles are requested at once, so a chunk costs two
 // memory latencies instead of several per tile.
-template <int KK, int LCB, bool BF16>
+template <int KK, int LCB, bool BF16, typename YT>
 __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int chunk, int feat_out,
                                            const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
-                                           float* __restrict__ Y, int lane) {
+                                           YT* __restrict__ Y, int lane) {
   constexpr int FIN = KK * 16;
   constexpr int TI = KK <= 2 ? 4 : 2;  // tiles in flight
   constexpr int MJ = TI / 2;           // 64-slot metadata registers per lane
@@ -96,9 +93,9 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
         wf[kk][d] = (uint32_t)wp[0] | ((uint32_t)wp[feat_out] << 16);
       }
     }
-    float* yb = Y + nt + n;
-    // result of an ELL row with output row `row`
-    auto emit = [&](int row, float v) { atomic_addf(yb + (int64_t)row * feat_out, v); };
+    YT* yb = Y + nt + n;
+    // result of an ELL row with output row `row`, added where `on` holds (the same for every n)
+    auto emit = [&](bool on, int row, float v) { stir::y_atomic_add(yb + (int64_t)row * feat_out, v, on, lane); };
     const int s_end = min(gsize, (chunk + 1) * kChunkSlots);
 #pragma unroll 1
     for (int s_base = chunk * kChunkSlots; s_base < s_end; s_base += 32 * TI) {
@@ -154,21 +151,21 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int sl = s_base + 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
-            if (wgt[v] != 0.f) atomic_addf(yb + (int64_t)rowg[sl / bk.cb] * feat_out, acc[v]);
+            emit(wgt[v] != 0.f, wgt[v] != 0.f ? rowg[sl / bk.cb] : 0, acc[v]);
           }
         } else if constexpr (LCB == 0) {
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int sl = 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
             const int row = row_of(sl, t >> 1);
-            if (wgt[v] != 0.f) emit(row, acc[v]);
+            emit(wgt[v] != 0.f, row, acc[v]);
           }
         } else if constexpr (LCB == 1) {
 #pragma unroll
           for (int v = 0; v < 16; v += 2) {
             const int sl = 32 * t + (v & 3) + 4 * h + 8 * (v >> 2);
             const int row = row_of(sl >> 1, t >> 2);
-            if (s_base + sl < gsize) emit(row, acc[v] + acc[v + 1]);
+            emit(s_base + sl < gsize, row, acc[v] + acc[v + 1]);
           }
         } else {
           // cb >= 4: the four registers of a quad belong to one ELL row
@@ -180,7 +177,7 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
             for (int u = 0; u < 4; ++u) {
               const int sl = 32 * t + 4 * h + 8 * u;
               const int row = row_of(sl >> 2, 0);
-              if (s_base + sl < gsize) emit(row, q4[u]);
+              emit(s_base + sl < gsize, row, q4[u]);
             }
           } else {
             // cb >= 8: add the other half-wave's quad (slots 8u+4..8u+7 vs 8u..8u+3)
@@ -194,17 +191,17 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
                 const int sl = 32 * t + 8 * tt;
                 const float val = tt == 0 ? q4[0] : tt == 1 ? q4[1] : tt == 2 ? q4[2] : q4[3];
                 const int row = row_of(sl >> 3, 0);
-                if (s_base + sl < gsize) emit(row, val);
+                emit(s_base + sl < gsize, row, val);
               }
             } else if constexpr (LCB == 4) {
               const float val = h == 0 ? q4[0] + q4[1] : q4[2] + q4[3];
               const int sl = 32 * t + 16 * h;
               const int row = row_of(sl >> 4, 0);
-              if (s_base + sl < gsize) emit(row, val);
+              emit(s_base + sl < gsize, row, val);
             } else {  // cb == 32: the whole tile is one ELL row
               const float val = (q4[0] + q4[1]) + (q4[2] + q4[3]);
               const int row = row_of(t, 0);
-              if (h == 0 && tile_live) emit(row, val);
+              emit(h == 0 && tile_live, row, val);
             }
           }
         }
@@ -216,11 +213,11 @@ __device__ __forceinline__ void rgms_group(const RgmsBucket& bk, int64_t g, int 
 
 // grid: one wavefront per work unit (kChunkSlots slots of one group), 4 per workgroup; feat_out
 // tiles of 32 are walked inside.
-template <int KK, bool BF16>
+template <int KK, bool BF16, typename YT>
 __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict__ table, int nb,
                                                    int64_t total_units, int feat_out,
                                                    const uint16_t* __restrict__ W,
-                                                   const uint16_t* __restrict__ X, float* __restrict__ Y) {
+                                                   const uint16_t* __restrict__ X, YT* __restrict__ Y) {
   const int lane = threadIdx.x & 63;
   const int64_t gid = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   if (gid >= total_units) return;
@@ -234,13 +231,13 @@ __global__ __launch_bounds__(256) void rgms_kernel(const RgmsBucket* __restrict_
   const int64_t g = unit / bk.chunks;
   const int chunk = (int)(unit % bk.chunks);
   switch (bk.log2cb) {
-    case 0: rgms_group<KK, 0, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
-    case 1: rgms_group<KK, 1, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
-    case 2: rgms_group<KK, 2, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
-    case 3: rgms_group<KK, 3, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
-    case 4: rgms_group<KK, 4, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
-    case 5: rgms_group<KK, 5, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
-    default: rgms_group<KK, -1, BF16>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 0: rgms_group<KK, 0, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 1: rgms_group<KK, 1, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 2: rgms_group<KK, 2, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 3: rgms_group<KK, 3, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 4: rgms_group<KK, 4, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    case 5: rgms_group<KK, 5, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
+    default: rgms_group<KK, -1, BF16, YT>(bk, g, chunk, feat_out, W, X, Y, lane); break;
   }
 }
 
@@ -330,8 +327,9 @@ int stir_rgms_plan_create(stir_rgms_plan** plan, int32_t num_buckets, const int3
   return 0;
 }
 
-static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
-                       int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X, float* d_Y,
+// out16: Y holds fp16 values (fp16 inputs only); otherwise fp32.
+static int rgms_launch(bool bf16, bool out16, const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels,
+                       int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X, void* d_Y,
                        void* stream) {
   STIR_REQUIRE(plan, "rgms: plan is null");
   STIR_REQUIRE(m >= 0 && n >= 0 && num_rels >= 0, "rgms: bad sizes");
@@ -340,6 +338,7 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
   STIR_REQUIRE(feat_out > 0 && feat_out % 32 == 0, "rgms: feat_out=%d must be a multiple of 32", feat_out);
   if (plan->nk == 0) return 0;
   STIR_REQUIRE(d_W && d_X && d_Y, "rgms: null pointer argument");
+  STIR_REQUIRE(!out16 || reinterpret_cast<uintptr_t>(d_Y) % 4 == 0, "rgms: an fp16 Y must be 4-byte aligned");
   const int64_t blocks = stir::ceil_div(plan->total_units, 4);
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "rgms: too many groups for one launch");
   dim3 grid((unsigned)blocks), block(256);
@@ -352,16 +351,19 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
     stir_rgms_plan* mp = const_cast<stir_rgms_plan*>(plan);
     if (stir::tile_set_prepare(mp->tiles, mp->tile_buckets, m, n, num_rels, feat_in, feat_out, mp->static_weights, st))
       return -1;
-    return stir::tile_set_launch(bf16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
+    return stir::tile_set_launch(bf16, out16, mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
   }
-#define STIR_RGMS(KK)                                                                              \
-  case KK:                                                                                         \
-    if (bf16)                                                                                      \
-      hipLaunchKernelGGL((rgms_kernel<KK, true>), grid, block, 0, st, plan->d_table, plan->nk,     \
-                         plan->total_units, feat_out, W, X, d_Y);                              \
-    else                                                                                           \
-      hipLaunchKernelGGL((rgms_kernel<KK, false>), grid, block, 0, st, plan->d_table, plan->nk,    \
-                         plan->total_units, feat_out, W, X, d_Y);                              \
+#define STIR_RGMS_GO(KK, BF, YT)                                                               \
+  hipLaunchKernelGGL((rgms_kernel<KK, BF, YT>), grid, block, 0, st, plan->d_table, plan->nk,   \
+                     plan->total_units, feat_out, W, X, static_cast<YT*>(d_Y))
+#define STIR_RGMS(KK)                                     \
+  case KK:                                                \
+    if (out16)                                            \
+      STIR_RGMS_GO(KK, false, _Float16);                  \
+    else if (bf16)                                        \
+      STIR_RGMS_GO(KK, true, float);                      \
+    else                                                  \
+      STIR_RGMS_GO(KK, false, float);                     \
     break
   switch (feat_in / 16) {
     STIR_RGMS(1);
@@ -374,18 +376,24 @@ static int rgms_launch(bool bf16, const stir_rgms_plan* plan, int32_t m, int32_t
     STIR_RGMS(8);
   }
 #undef STIR_RGMS
+#undef STIR_RGMS_GO
   STIR_LAUNCH_CHECK();
   return 0;
 }
 
 int stir_rgms_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels, int32_t feat_in,
                   int32_t feat_out, const void* d_W, const void* d_X, float* d_Y, void* stream) {
-  return rgms_launch(false, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
+  return rgms_launch(false, false, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
+}
+
+int stir_rgms_f16_out_f16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels, int32_t feat_in,
+                          int32_t feat_out, const void* d_W, const void* d_X, void* d_Y, void* stream) {
+  return rgms_launch(false, true, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
 }
 
 int stir_rgms_bf16(const stir_rgms_plan* plan, int32_t m, int32_t n, int32_t num_rels, int32_t feat_in,
                    int32_t feat_out, const void* d_W, const void* d_X, float* d_Y, void* stream) {
-  return rgms_launch(true, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
+  return rgms_launch(true, false, plan, m, n, num_rels, feat_in, feat_out, d_W, d_X, d_Y, stream);
 }
 
 int stir_rgms_plan_set_static_weights(stir_rgms_plan* plan, int32_t on) {

@@ -61,8 +61,9 @@ struct TileIndexSet {
 int tile_set_prepare(TileIndexSet& set, const std::vector<TileBucket>& buckets, int32_t m, int32_t n,
                      int32_t num_rels, int32_t feat_in, int32_t feat_out, bool static_weights, hipStream_t stream);
 // Y += RGMS(W, X) over the indexed edges.  W: [R, feat_in, feat_out], X: [n, feat_in], 16-bit.
-int tile_set_launch(bool bf16, TileIndexSet& set, int32_t feat_in, int32_t feat_out, const void* d_W,
-                    const void* d_X, float* d_Y, hipStream_t stream);
+// Y: [m, feat_out] fp32, or fp16 with out16 (fp16 inputs only; 4-byte aligned).
+int tile_set_launch(bool bf16, bool out16, TileIndexSet& set, int32_t feat_in, int32_t feat_out, const void* d_W,
+                    const void* d_X, void* d_Y, hipStream_t stream);
 void tile_set_free(TileIndexSet& set);
 
 }  // namespace stir

@@ -11,6 +11,7 @@
 // keeps fp32 accuracy.  S is assembled in a per-wavefront LDS tile: the lane of edge e stores
 // weight_e at (row_e, e), every lane reads its operand row, then the entry is cleared again.
 #include "rgms_tiles.h"
+#include "rgms_out.h"
 
 #include <hipcub/hipcub.hpp>
 
@@ -289,11 +290,11 @@ __device__ __forceinline__ f32x16 scatter_step(uint16_t* S, int dl, int jcol, in
 // steps w, w + 4, ...: more wavefronts in flight per tile, since a step costs a full memory
 // round trip), each with its own accumulator tile; the four tiles are added through LDS and the
 // workgroup writes the 32 rows of Y once.  KK = feat_in / 16.
-template <int KK, bool BF16, typename Rec>
+template <int KK, bool BF16, typename Rec, typename YT>
 __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* __restrict__ units,
                                                         const Rec* __restrict__ edges, int m, int feat_out,
                                                         const u32x4* __restrict__ Wp, const uint16_t* __restrict__ X,
-                                                        float* __restrict__ Y) {
+                                                        YT* __restrict__ Y) {
   constexpr int FIN = KK * 16;
   constexpr bool kPacked = sizeof(Rec) == sizeof(PackedEdge);
   constexpr int PW = KK <= 4 ? 2 : 1;  // relations whose W fragments are requested together
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
     for (int k = 0; k < kSumIters; ++k) {
       const int elem = threadIdx.x + kThreads * k;
       const int64_t yrow = (int64_t)tile * kTileRows + (elem >> 5);
-      yold[k] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + (elem & 31)] : 0.f;
+      yold[k] = (!atomic && yrow < m) ? y_load(Y + yrow * feat_out + 32 * nti + (elem & 31)) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -432,13 +433,10 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
 #pragma unroll
       for (int w = 1; w < kUnitWaves; ++w) sum += partial[w][at];
       const int64_t yrow = (int64_t)tile * kTileRows + row;
-      if (yrow < m) {
-        float* y = Y + yrow * feat_out + 32 * nti + col;
-        if (atomic)
-          __hip_atomic_fetch_add(y, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else
-          *y = yold[k] + sum;
-      }
+      // (a row belongs to 32 consecutive threads: the two lanes of a pair share `yrow`)
+      YT* y = Y + yrow * feat_out + 32 * nti + col;
+      y_atomic_add(y, sum, atomic && yrow < m, threadIdx.x);
+      if (!atomic && yrow < m) y_store(y, yold[k] + sum);
     }
     if (nti + 1 < ntiles) __syncthreads();  // the partial sums are rewritten by the next pass
   }
@@ -466,11 +464,11 @@ constexpr int kTeamWaves = 2;  // wavefronts that share a unit in the resident k
 // distinct banks, and so do the eight writers of one column phase (see the fill loop)
 __device__ __forceinline__ int w_slot(int lane) { return lane ^ ((lane >> 3) & 7); }
 
-template <int KK, bool BF16, typename Rec, int T>
+template <int KK, bool BF16, typename Rec, int T, typename YT>
 __global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
     const int32_t* __restrict__ share_ptr, const Unit* __restrict__ share_units, const Rec* __restrict__ edges, int m,
     int feat_out, int num_rels, const uint16_t* __restrict__ W, const uint16_t* __restrict__ X,
-    float* __restrict__ Y) {
+    YT* __restrict__ Y) {
   constexpr int FIN = KK * 16;
   constexpr bool kPacked = sizeof(Rec) == sizeof(PackedEdge);
   constexpr int UW = kTeamWaves;
@@ -608,7 +606,7 @@ __global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
 #pragma unroll
       for (int v = 0; v < 8; ++v) {
         const int64_t yrow = (int64_t)tile * kTileRows + 16 * tw + (v & 3) + 4 * h + 8 * (v >> 2);
-        yold[v] = (!atomic && yrow < m) ? Y[yrow * feat_out + 32 * nti + mrow] : 0.f;
+        yold[v] = (!atomic && yrow < m) ? y_load(Y + yrow * feat_out + 32 * nti + mrow) : 0.f;
       }
       f32x16 acc2;
 #pragma unroll
@@ -707,13 +705,9 @@ __global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
 #pragma unroll
       for (int v = 0; v < 8; ++v) {
         const int64_t yrow = (int64_t)tile * kTileRows + 16 * tw + (v & 3) + 4 * h + 8 * (v >> 2);
-        if (yrow < m) {
-          float* y = Y + yrow * feat_out + 32 * nti + mrow;
-          if (atomic)
-            __hip_atomic_fetch_add(y, own[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          else
-            *y = yold[v] + own[v];
-        }
+        YT* y = Y + yrow * feat_out + 32 * nti + mrow;  // lanes 2k and 2k + 1: the same row, features 2k, 2k + 1
+        y_atomic_add(y, own[v], atomic && yrow < m, lane);
+        if (!atomic && yrow < m) y_store(y, yold[v] + own[v]);
       }
       team_arrive();  // waited for where the next pass first writes to its S tile
     }
@@ -747,10 +741,10 @@ constexpr int kResidentMaxQuads = 3;
 constexpr int kMaxRelationParts = 3;
 
 // Launches the resident kernel with `quads` x 4 wavefronts per workgroup.
-template <int KK, bool BF16, typename Rec>
+template <int KK, bool BF16, typename Rec, typename YT>
 int launch_resident(int quads, dim3 grid, size_t lds, hipStream_t stream, const int32_t* share_ptr,
                     const Unit* share_units, const Rec* edges, int m, int feat_out, int num_rels, const uint16_t* W,
-                    const uint16_t* X, float* Y) {
+                    const uint16_t* X, YT* Y) {
   auto go = [&](auto* fn) -> int {
     if (int rc = allow_lds(reinterpret_cast<const void*>(fn))) return rc;
     hipLaunchKernelGGL(fn, grid, dim3(256 * quads), lds, stream, share_ptr, share_units, edges, m, feat_out, num_rels, W,
@@ -758,8 +752,8 @@ int launch_resident(int quads, dim3 grid, size_t lds, hipStream_t stream, const 
     return 0;
   };
   constexpr int kTeamsPerQuad = 4 / kTeamWaves;
-  if (quads == 2) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 2 * kTeamsPerQuad>);
-  if (quads == 3) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 3 * kTeamsPerQuad>);
+  if (quads == 2) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 2 * kTeamsPerQuad, YT>);
+  if (quads == 3) return go(rgms_tile_lds_kernel<KK, BF16, Rec, 3 * kTeamsPerQuad, YT>);
   return fail("rgms: no kernel for %d wavefronts per workgroup", 4 * quads);
 }
 
@@ -966,8 +960,9 @@ int tile_index_build(TileIndex& ix, const std::vector<TileBucket>& buckets, int3
 }
 
 // Y += RGMS(W, X) over the edges of one index; W starts at the index's first relation.
-int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
-                     float* d_Y, hipStream_t stream) {
+// out16: Y is fp16 (fp16 inputs only), else fp32.
+int tile_rgms_launch(bool bf16, bool out16, TileIndex& ix, int32_t feat_in, int32_t feat_out, const void* d_W,
+                     const void* d_X, void* d_Y, hipStream_t stream) {
   STIR_REQUIRE(ix.m >= 0, "rgms: the edge index has not been built");
   if (ix.units == 0) return 0;
   STIR_REQUIRE(feat_in % 16 == 0 && feat_in / 16 <= kMaxKK && feat_out % 32 == 0, "rgms: unsupported feature sizes");
@@ -979,6 +974,9 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
   const PackedEdge* pedges = static_cast<const PackedEdge*>(ix.d_edges);
   const uint16_t* X = static_cast<const uint16_t*>(d_X);
   const uint16_t* W = static_cast<const uint16_t*>(d_W);
+  float* Y32 = static_cast<float*>(d_Y);
+  _Float16* Y16 = static_cast<_Float16*>(d_Y);
+  STIR_REQUIRE(!(bf16 && out16), "rgms: fp16 output takes fp16 inputs");
 
   // W resident in LDS when it fits beside the S tiles of at least two teams
   const size_t w_bytes = size_t(frags) * 64 * sizeof(u32x4);
@@ -1000,17 +998,25 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
     const dim3 grid((unsigned)wgs);
     const int32_t* share_ptr = static_cast<const int32_t*>(ix.d_share_ptr);
     const Unit* share_units = static_cast<const Unit*>(ix.d_share_units);
-#define STIR_LDS_R(KKV, BF, REC, PTR)                                                                   \
+#define STIR_LDS_R(KKV, BF, REC, PTR, YP)                                                               \
   if (int rc = launch_resident<KKV, BF, REC>(quads, grid, lds, stream, share_ptr, share_units, PTR, ix.m, feat_out, \
-                                             ix.num_rels, W, X, d_Y))                                  \
+                                             ix.num_rels, W, X, YP))                                       \
     return rc
-#define STIR_LDS(KKV)                                                                          \
-  case KKV:                                                                                    \
-    if (ix.packed_records) {                                                                   \
-      if (bf16) { STIR_LDS_R(KKV, true, PackedEdge, pedges); } else { STIR_LDS_R(KKV, false, PackedEdge, pedges); } \
-    } else {                                                                                   \
-      if (bf16) { STIR_LDS_R(KKV, true, Edge, edges); } else { STIR_LDS_R(KKV, false, Edge, edges); } \
-    }                                                                                          \
+#define STIR_LDS_Y(KKV, REC, PTR)                           \
+  if (out16) {                                              \
+    STIR_LDS_R(KKV, false, REC, PTR, Y16);                  \
+  } else if (bf16) {                                        \
+    STIR_LDS_R(KKV, true, REC, PTR, Y32);                   \
+  } else {                                                  \
+    STIR_LDS_R(KKV, false, REC, PTR, Y32);                  \
+  }
+#define STIR_LDS(KKV)                        \
+  case KKV:                                  \
+    if (ix.packed_records) {                 \
+      STIR_LDS_Y(KKV, PackedEdge, pedges)    \
+    } else {                                 \
+      STIR_LDS_Y(KKV, Edge, edges)           \
+    }                                        \
     break
     switch (kk_count) {
       STIR_LDS(1);
@@ -1019,6 +1025,7 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
       STIR_LDS(4);
     }
 #undef STIR_LDS
+#undef STIR_LDS_Y
 #undef STIR_LDS_R
     STIR_LAUNCH_CHECK();
     return 0;
@@ -1037,15 +1044,22 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
                      W, Wp, frags, kk_count, feat_out);
   STIR_LAUNCH_CHECK();
   const dim3 grid((unsigned)ix.units), block(64 * kUnitWaves);
-#define STIR_TILES_R(KKV, BF, REC, PTR) \
-  hipLaunchKernelGGL((rgms_tile_kernel<KKV, BF, REC>), grid, block, 0, stream, units, PTR, ix.m, feat_out, Wp, X, d_Y)
-#define STIR_TILES(KKV)                                                                          \
-  case KKV:                                                                                      \
-    if (ix.packed_records) {                                                                     \
-      if (bf16) STIR_TILES_R(KKV, true, PackedEdge, pedges); else STIR_TILES_R(KKV, false, PackedEdge, pedges); \
-    } else {                                                                                     \
-      if (bf16) STIR_TILES_R(KKV, true, Edge, edges); else STIR_TILES_R(KKV, false, Edge, edges); \
-    }                                                                                            \
+#define STIR_TILES_R(KKV, BF, REC, PTR, YT, YP) \
+  hipLaunchKernelGGL((rgms_tile_kernel<KKV, BF, REC, YT>), grid, block, 0, stream, units, PTR, ix.m, feat_out, Wp, X, YP)
+#define STIR_TILES_Y(KKV, REC, PTR)                       \
+  if (out16)                                              \
+    STIR_TILES_R(KKV, false, REC, PTR, _Float16, Y16);    \
+  else if (bf16)                                          \
+    STIR_TILES_R(KKV, true, REC, PTR, float, Y32);        \
+  else                                                    \
+    STIR_TILES_R(KKV, false, REC, PTR, float, Y32)
+#define STIR_TILES(KKV)                       \
+  case KKV:                                   \
+    if (ix.packed_records) {                  \
+      STIR_TILES_Y(KKV, PackedEdge, pedges);  \
+    } else {                                  \
+      STIR_TILES_Y(KKV, Edge, edges);         \
+    }                                         \
     break
   switch (kk_count) {
     STIR_TILES(1);
@@ -1058,6 +1072,7 @@ int tile_rgms_launch(bool bf16, TileIndex& ix, int32_t feat_in, int32_t feat_out
     STIR_TILES(8);
   }
 #undef STIR_TILES
+#undef STIR_TILES_Y
 #undef STIR_TILES_R
   STIR_LAUNCH_CHECK();
   return 0;
@@ -1111,12 +1126,12 @@ int tile_set_prepare(TileIndexSet& set, const std::vector<TileBucket>& buckets, 
   return 0;
 }
 
-int tile_set_launch(bool bf16, TileIndexSet& set, int32_t feat_in, int32_t feat_out, const void* d_W, const void* d_X,
-                    float* d_Y, hipStream_t stream) {
+int tile_set_launch(bool bf16, bool out16, TileIndexSet& set, int32_t feat_in, int32_t feat_out, const void* d_W,
+                    const void* d_X, void* d_Y, hipStream_t stream) {
   STIR_REQUIRE(set.m >= 0, "rgms: the edge index has not been built");
   for (TileIndex& ix : set.parts) {
     const uint16_t* W = static_cast<const uint16_t*>(d_W) + (int64_t)ix.rel_lo * feat_in * feat_out;
-    if (int rc = tile_rgms_launch(bf16, ix, feat_in, feat_out, W, d_X, d_Y, stream)) return rc;
+    if (int rc = tile_rgms_launch(bf16, out16, ix, feat_in, feat_out, W, d_X, d_Y, stream)) return rc;
   }
   return 0;
 }

@@ -437,8 +437,10 @@ class Rgms(_Operator):
     _in_dtype = torch.float16
     _fns = ("stir_rgms_plan_create", "stir_rgms_f16", "stir_rgms_plan_destroy")
 
+    _out_dtype = torch.float32
+
     def __init__(self, m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=None,
-                 static_weights=False):
+                 static_weights=False, out_dtype=None):
         self._static = bool(static_weights)
         if dtype is not None and self._in_dtype is torch.float16:
             if dtype not in (torch.float16, torch.bfloat16):
@@ -446,6 +448,12 @@ class Rgms(_Operator):
             if dtype is torch.bfloat16:  # same kernel on the bf16 matrix-core instruction
                 self._in_dtype = dtype
                 self._fns = ("stir_rgms_plan_create", "stir_rgms_bf16", "stir_rgms_plan_destroy")
+        if out_dtype not in (None, torch.float32):
+            # the reference's operator built with dtype "float16" (bench_rgcn_tensorcore.py:564-607)
+            if out_dtype is not torch.float16 or self._in_dtype is not torch.float16:
+                raise _lib.SparseTIRError("rgms: out_dtype must be torch.float32, or torch.float16 with fp16 inputs")
+            self._out_dtype = out_dtype
+            self._fns = ("stir_rgms_plan_create", "stir_rgms_f16_out_f16", "stir_rgms_plan_destroy")
         self.m, self.n, self.R = int(m), int(n), int(num_rels)
         self.fin, self.fout = int(feat_in), int(feat_out)
         self.rb, self.cb = [int(v) for v in rows_bkt], [int(v) for v in cols_bkt]
@@ -462,7 +470,7 @@ class Rgms(_Operator):
     def _spec(self):
         f16, f32, i32 = self._in_dtype, torch.float32, torch.int32
         spec = [("W", f16, self.R * self.fin * self.fout), ("X", f16, self.n * self.fin),
-                ("Y", f32, self.m * self.fout)]
+                ("Y", self._out_dtype, self.m * self.fout)]
         for k, g in enumerate(self.groups):
             spec += [(f"A_{k}", f16, g * self.rb[k] * self.cb[k]), (f"rows_{k}", i32, g * self.rb[k]),
                      (f"cols_{k}", i32, g * self.rb[k] * self.cb[k])]
@@ -634,8 +642,8 @@ def build_tcspmm(mb, nnzb, feat, tile_size, group_size, num_b_rows, out_dtype=to
 
 
 def build_rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype=torch.float16,
-               static_weights=False):
-    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype, static_weights)
+               static_weights=False, out_dtype=torch.float32):
+    return Rgms(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, dtype, static_weights, out_dtype)
 
 
 def build_rgms_f32(m, n, num_rels, feat_in, feat_out, rows_bkt, cols_bkt, groups, deterministic=False):
