@@ -14,6 +14,7 @@
 #include "rgms_out.h"
 
 #include <hipcub/hipcub.hpp>
+#include <type_traits>
 
 
 namespace stir {
@@ -219,10 +220,21 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 }
 
 // acc += S-operand @ (8 rows of T held as fp32 in t[0..7]), T split into 16-bit terms whose sum
-// carries at least 21 significant bits.
-template <bool BF16>
+// carries at least 21 significant bits -- or, with ONE_TERM (an fp16 Y, which keeps 11 bits),
+// rounded to fp16 once.
+template <bool BF16, bool ONE_TERM>
 __device__ __forceinline__ f32x16 stage2(u32x4 sa, const float* t, f32x16 acc) {
-  if constexpr (BF16) {
+  if constexpr (ONE_TERM) {
+    static_assert(!BF16, "one term: fp16 only");
+    typedef _Float16 r2 __attribute__((ext_vector_type(2)));
+    u32x4 b;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const r2 pair = {(_Float16)t[2 * d], (_Float16)t[2 * d + 1]};  // round to nearest
+      b[d] = __builtin_bit_cast(uint32_t, pair);
+    }
+    acc = mfma32<false>(sa, b, acc);
+  } else if constexpr (BF16) {
     float r[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = t[i];
@@ -266,7 +278,7 @@ constexpr int kSStride = 40;  // 16-bit elements per row of the S tile (32 used;
 // (dl, jcol) of the wavefront's all-zero S tile, every lane reads its operand row, and the entry
 // is cleared again; LDS operations of one wavefront execute in order, so no barrier is needed.
 // Steps of at most 16 edges skip the second half of k.
-template <bool BF16>
+template <bool BF16, bool ONE_TERM>
 __device__ __forceinline__ f32x16 scatter_step(uint16_t* S, int dl, int jcol, int mrow, int h, uint16_t weight,
                                                int left, const f32x16& acc1, f32x16 acc2) {
   if (h == 0) S[dl * kSStride + jcol] = weight;
@@ -281,8 +293,8 @@ __device__ __forceinline__ f32x16 scatter_step(uint16_t* S, int dl, int jcol, in
   float t[16];
 #pragma unroll
   for (int v = 0; v < 16; ++v) t[v] = acc1[v];
-  acc2 = stage2<BF16>(sa0, t, acc2);
-  if (left > 16) acc2 = stage2<BF16>(sa1, t + 8, acc2);
+  acc2 = stage2<BF16, ONE_TERM>(sa0, t, acc2);
+  if (left > 16) acc2 = stage2<BF16, ONE_TERM>(sa1, t + 8, acc2);
   return acc2;
 }
 
@@ -409,7 +421,7 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
       }
 
       // ---- stage 2
-      acc2 = scatter_step<BF16>(S, dl, jcol, mrow, h, live ? wbits : (uint16_t)0, left, acc1, acc2);
+      acc2 = scatter_step<BF16, std::is_same<YT, _Float16>::value>(S, dl, jcol, mrow, h, live ? wbits : (uint16_t)0, left, acc1, acc2);
     }
 
     // ---- add the four tiles and write back.  acc2[v] of lane (n, h) is row (v%4) + 4h + 8(v/4)
@@ -654,7 +666,7 @@ __global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
 
         // ---- stage 2
         if (e0 == e_first) team_wait();  // the sums of the pass before have been read out of the S tiles
-        acc2 = scatter_step<BF16>(S, dl, jcol, mrow, h, live ? wbits : (uint16_t)0, left, acc1, acc2);
+        acc2 = scatter_step<BF16, std::is_same<YT, _Float16>::value>(S, dl, jcol, mrow, h, live ? wbits : (uint16_t)0, left, acc1, acc2);
       };
       // Two steps per turn of the loop, so that the two sets of X registers swap roles without
       // copies: while a step is computed, the rows of X of the step after it are on their way,
