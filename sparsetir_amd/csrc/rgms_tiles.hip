@@ -447,8 +447,10 @@ __global__ __launch_bounds__(64 * kUnitWaves) void rgms_tile_kernel(const Unit* 
       const int64_t yrow = (int64_t)tile * kTileRows + row;
       // (a row belongs to 32 consecutive threads: the two lanes of a pair share `yrow`)
       YT* y = Y + yrow * feat_out + 32 * nti + col;
-      y_atomic_add(y, sum, atomic && yrow < m, threadIdx.x);
-      if (!atomic && yrow < m) y_store(y, yold[k] + sum);
+      if (atomic)  // uniform over the workgroup
+        y_atomic_add(y, sum, yrow < m, threadIdx.x);
+      else if (yrow < m)
+        y_store(y, yold[k] + sum);
     }
     if (nti + 1 < ntiles) __syncthreads();  // the partial sums are rewritten by the next pass
   }
@@ -718,8 +720,10 @@ __global__ __launch_bounds__(64 * kTeamWaves * T) void rgms_tile_lds_kernel(
       for (int v = 0; v < 8; ++v) {
         const int64_t yrow = (int64_t)tile * kTileRows + 16 * tw + (v & 3) + 4 * h + 8 * (v >> 2);
         YT* y = Y + yrow * feat_out + 32 * nti + mrow;  // lanes 2k and 2k + 1: the same row, features 2k, 2k + 1
-        y_atomic_add(y, own[v], atomic && yrow < m, lane);
-        if (!atomic && yrow < m) y_store(y, yold[v] + own[v]);
+        if (atomic)  // uniform over the wavefront
+          y_atomic_add(y, own[v], yrow < m, lane);
+        else if (yrow < m)
+          y_store(y, yold[v] + own[v]);
       }
       team_arrive();  // waited for where the next pass first writes to its S tile
     }
