@@ -487,7 +487,9 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     for k in range(len(buckets)):
         triples += [t(mask[k].astype(np.float32).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
         mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
+    # the operator's default: every 64-row tile of Y summed on chip from an edge index, no atomics
     f32 = ops.build_rgms_f32(n, n, R, fin, fout, rb32, buckets, [c.shape[0] for c in cols])
+    f32(w32, x32, y, *triples, *mids)  # builds its edge index
     tm = time_small(lambda: f32(w32, x32, y, *triples, *mids), 20, 2, torch)
     d = tm["us_back_to_back"] / 1e6
     out["rgms_f32_ell3d_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
@@ -495,17 +497,17 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
                                      "algorithmic_bytes": byts32,
                                      "roofline": side_roofline("hbm", byts32 / d / 1e9, "rgms_f32_ell3d_config5"),
                                      "ell_rows": int(sum(r.size for r in rows))}
-    # the optional form without atomics (the same bits on every run)
-    f32d = ops.build_rgms_f32(n, n, R, fin, fout, rb32, buckets, [c.shape[0] for c in cols], deterministic=True)
-    f32d(w32, x32, y, *triples, *mids)  # builds its edge index
-    tm_d = time_small(lambda: f32d(w32, x32, y, *triples, *mids), 20, 2, torch)
-    out["rgms_f32_ell3d_config5"]["deterministic_us"] = tm_d["us_back_to_back"]
-    del f32d
-    # every ELL row adds feat_out floats to Y with one atomic each: the launch's bound.  Beside
+    # the form that holds nothing derived from the index arrays: one atomic per (ELL row, output)
+    f32a = ops.build_rgms_f32(n, n, R, fin, fout, rb32, buckets, [c.shape[0] for c in cols], deterministic=False)
+    tm_a = time_small(lambda: f32a(w32, x32, y, *triples, *mids), 20, 2, torch)
+    da = tm_a["us_back_to_back"] / 1e6
+    out["rgms_f32_ell3d_config5"]["atomic_form_us"] = da * 1e6
+    del f32a
+    # every ELL row adds feat_out floats to Y with one atomic each: that form's bound.  Beside
     # it, what the same number of row additions to hashed rows of Y takes with nothing else going on
     er = out["rgms_f32_ell3d_config5"]["ell_rows"]
     out["rgms_f32_ell3d_config5"]["atomic_adds"] = er * fout
-    out["rgms_f32_ell3d_config5"]["atomic_adds_G_per_s"] = er * fout / d / 1e9
+    out["rgms_f32_ell3d_config5"]["atomic_adds_G_per_s"] = er * fout / da / 1e9
     if fout == 32:
         P = load_probes()
         yp = ctypes.c_void_p(y.data_ptr())
@@ -519,6 +521,7 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
     csf = [t(cfg[k]) for k in ("indptr0", "indices0", "indptr1", "indices1")]
     ones = torch.ones(E, device=dev)
     fc = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E)
+    fc(ones, w32, x32, y, *csf)  # builds its edge index
     tm = time_small(lambda: fc(ones, w32, x32, y, *csf), 20, 2, torch)
     d = tm["us_back_to_back"] / 1e6
     out["rgms_f32_csf_config5"] = {"us_per_call": tm["us_per_call"], "us_graph": tm["us_graph"], "us": d * 1e6, "tflops": flops / d / 1e12, "alg_GBps": byts32 / d / 1e9,
@@ -526,11 +529,10 @@ def side_kernels(torch, dev, ops, st, datasets, time_steps):
                                    "algorithmic_bytes": byts32,
                                    "roofline": side_roofline("hbm", byts32 / d / 1e9, "rgms_f32_csf_config5"),
                                    "stored_rows": int(len(cfg["indices0"]))}
-    fcd = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E, deterministic=True)
-    fcd(ones, w32, x32, y, *csf)  # builds its edge index
-    tm_d = time_small(lambda: fcd(ones, w32, x32, y, *csf), 20, 2, torch)
-    out["rgms_f32_csf_config5"]["deterministic_us"] = tm_d["us_back_to_back"]
-    del fcd
+    fca = ops.build_rgms_csf(n, n, R, fin, fout, len(cfg["indices0"]), E, deterministic=False)  # stateless, atomics
+    tm_a = time_small(lambda: fca(ones, w32, x32, y, *csf), 20, 2, torch)
+    out["rgms_f32_csf_config5"]["atomic_form_us"] = tm_a["us_back_to_back"]
+    del fca
     return out
 
 

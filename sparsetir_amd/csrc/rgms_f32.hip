@@ -475,10 +475,11 @@ int stir_rgms_f32(const stir_rgms_f32_plan* plan, int32_t m, int32_t n, int32_t 
   STIR_REQUIRE(d_W && d_X && d_Y, "rgms_f32: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (plan->deterministic && plan->slots >= kF32TileMinSlots && plan->slots < (int64_t(1) << 31) &&
-      stir::f32_tiles_serves(feat_in, feat_out) && m > 0 && n > 0 && num_rels > 0) {
+      stir::f32_tiles_serves(feat_in, feat_out) && stir::f32_tiles_fits(n, feat_in, plan->slots) && m > 0 && n > 0 &&
+      num_rels > 0) {
     // the plan's edge index is made by the first launch: a plan serves one call at a time
     stir_rgms_f32_plan* mp = const_cast<stir_rgms_f32_plan*>(plan);
-    if (stir::f32_tiles_prepare(mp->tiles, mp->source, m, n, num_rels, st)) return -1;
+    if (stir::f32_tiles_prepare(mp->tiles, mp->source, m, n, num_rels, feat_in, st)) return -1;
     return stir::f32_tiles_launch(mp->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
   }
 #define STIR_LAUNCH(FP, WAVES)                                                                            \
@@ -549,11 +550,12 @@ int stir_rgms_csf_f32_planned(stir_rgms_csf_f32_plan* plan, int32_t m, int32_t n
   const stir::F32Source& s = plan->source;
   if (s.nnz_j == 0) return 0;
   STIR_REQUIRE(d_W && d_X && d_Y, "rgms_csf_f32: null pointer argument");
-  if (!stir::f32_tiles_serves(feat_in, feat_out) || s.nnz_j < kF32TileMinSlots)
+  if (!stir::f32_tiles_serves(feat_in, feat_out) || !stir::f32_tiles_fits(n, feat_in, s.nnz_j) ||
+      s.nnz_j < kF32TileMinSlots || m <= 0 || n <= 0 || num_rels <= 0)
     return stir_rgms_csf_f32(m, n, num_rels, feat_in, feat_out, s.nnz_i, s.nnz_j, s.A, d_W, d_X, d_Y, s.indptr_i,
                              s.indices_i, s.indptr_j, s.indices_j, stream);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (stir::f32_tiles_prepare(plan->tiles, s, m, n, num_rels, st)) return -1;
+  if (stir::f32_tiles_prepare(plan->tiles, s, m, n, num_rels, feat_in, st)) return -1;
   return stir::f32_tiles_launch(plan->tiles, feat_in, feat_out, d_W, d_X, d_Y, st);
 }
 

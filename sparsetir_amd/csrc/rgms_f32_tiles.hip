@@ -1,32 +1,39 @@
-// Destination-tiled fp32 RGMS declared in rgms_f32_tiles.h: index construction and the kernel.
+// Destination-tiled fp32 RGMS declared in rgms_f32_tiles.h: index construction and the kernels.
 //
 // Index (once per plan): every slot of the ELL3D buckets -- or every stored column of the CSF
 // arrays -- is an edge with the key (destination row / 64, relation, destination row % 64).  One
-// stable radix sort orders the edges by key; runs of equal key are the (relation, row) pairs
-// (run-length encoding of the sorted keys), and a binary search per tile finds where its pairs
-// begin.  An edge record holds the source row and the address of the edge's weight (weights are
-// read at every launch); a pair record its relation, its row inside the tile and its run of edges.
+// stable radix sort orders the edges by key; runs of equal key are the (relation, row) pairs, cut
+// into pieces of at most EMAX = 32 / KS edges (a second key: key << 20 | position in the run /
+// EMAX, run-length encoded).  The pairs of one (tile, relation) run are cut into batches of at
+// most 16 pairs and at most EMAX edges, listed per tile; a tile with many more batches than the
+// average is cut into several units, whose partial tiles go to memory of the plan and are added
+// up, in order, by a second small launch.
+// An edge record holds the source row and the address of the edge's weight (weights are read at
+// every launch); a pair is one word: row inside the tile, edges, first edge inside its batch.
 //
-// The pairs of one (tile, relation) run are cut into batches of at most 16, listed per tile.
-//
-// Kernel: one workgroup of four wavefronts per 64-row tile of Y; wavefront w takes the tile's
-// batches w, w + 4, ... and sums into a partial tile of its own in LDS.  Per batch (up to 16 pairs
-// of one relation):
-//   1. S[i, :] = sum over the edges e of pair i of weight_e * X[src_e, :], in registers: lane
-//      (i = l % 16, q = l / 16) holds inputs 8q .. 8q+7 (+32 per further 32 inputs) of pair i and
-//      walks the pair's edges;
-//   2. P = S @ W[rel]^T on v_mfma_f32_16x16x4_f32.  The instruction's k index is lane / 16; the
+// Kernel: one workgroup of four wavefronts per unit; wavefront w takes the unit's batches w,
+// w + 4, ... and sums into a partial tile of its own in LDS.  Per batch:
+//   1. the rows of X of the batch's edges, times their weights, go to a tile of LDS, eight rows
+//      (128 bytes each) per load instruction: every lane useful whatever the pairs look like;
+//   2. lane (i = l % 16, q = l / 16) adds up the rows of pair i from that tile: inputs 8q .. 8q+7
+//      (+32 per further 32 inputs) of S[i, :] = sum over the edges e of pair i of w_e X[src_e, :];
+//   3. P = S @ W[rel]^T on v_mfma_f32_16x16x4_f32.  The instruction's k index is lane / 16; the
 //      t-th instruction takes input 8q + t from lane (., q) in both operands, so S needs no
 //      rearrangement and a lane's W operands are 32 contiguous bytes of a row of W[rel];
-//   3. row i of P is added to row (destination row % 64) of the wavefront's partial tile with a
-//      plain LDS read-modify-write: the pairs of one relation end in different rows, and no other
-//      wavefront touches this partial tile (LDS float atomics run at a third of a lane per clock
-//      and compute unit on this chip, slower than atomics in memory).
-// A batch is a chain of dependent loads (batch record -> pair records -> edge records -> rows of
-// X), so the records run ahead of the arithmetic: batch records three batches ahead, pair records
-// two, the first two edge records of every pair one; only the rows of X are waited for.
-// At the end the four partial tiles are added to the tile's rows of Y, each element once.
+//   4. row i of P is added to row (destination row % 64) of the wavefront's partial tile with a
+//      plain LDS read-modify-write: the pairs of a batch end in different rows or in pieces of
+//      one row that this lane order adds one after the other, and no other wavefront touches
+//      this partial tile (LDS float atomics run at a third of a lane per clock and compute unit
+//      on this chip, slower than atomics in memory).
+// A batch is a chain of dependent loads (batch record -> edge records -> rows of X and weights),
+// so the records run ahead of the arithmetic: batch records four batches ahead, edge records and
+// pair words three, rows of X and weights one; the loop body has no branch around a load, so the
+// compiler's wait counts leave the younger loads in flight.
+// At the end the four partial tiles are added up: into the tile's rows of Y, each element once,
+// or -- for a unit that is a piece of a tile -- into the plan's memory for partial tiles.
 #include "rgms_f32_tiles.h"
+
+#include <algorithm>
 
 #include <hipcub/hipcub.hpp>
 
@@ -37,12 +44,24 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTileRows = 64;
 constexpr int kTileShift = 6;
-constexpr int kBatch = 16;  // pairs per matrix-core product
+constexpr int kBatch = 16;    // pairs per matrix-core product
+constexpr int kSubBits = 20;  // pieces of one (relation, row) run in the second sort key
 
 struct alignas(16) BatchF32 {
-  int64_t pair_begin;
-  int32_t npairs;  // at most kBatch
+  int32_t pair_begin;  // first pair word
+  int32_t edge_begin;  // first sorted edge
+  uint32_t counts;     // pairs (at most kBatch) | edges << 8 (at most EMAX) | most edges of a pair << 16
   int32_t rel;
+};
+
+struct alignas(16) UnitF32 {
+  int32_t tile;
+  int32_t batch_begin, batch_end;
+  int32_t partial;  // -1: the unit is a whole tile and adds to Y; else its place among the partial tiles
+};
+
+struct alignas(16) MultiF32 {  // a tile cut into several units
+  int32_t tile, first_partial, pieces, pad;
 };
 
 struct alignas(16) DevBucketF32 {
@@ -69,11 +88,6 @@ struct alignas(16) EdgeF32 {
   const float* w;  // the edge's weight
 };
 
-struct alignas(16) PairF32 {
-  uint32_t rel_dl;  // relation << 6 | destination row inside its tile
-  int32_t count;    // edges of the pair
-  int64_t first;    // its first sorted edge
-};
 
 __device__ __forceinline__ int bucket_of(const DevBucketF32* __restrict__ tab, int nb, int64_t q) {
   int lo = 0, hi = nb - 1;
@@ -154,42 +168,75 @@ __global__ __launch_bounds__(256) void f32_edge_records_kernel(const DevBucketF3
   edges[p] = e;
 }
 
-__global__ __launch_bounds__(256) void f32_pairs_kernel(const uint64_t* __restrict__ unique, const int32_t* __restrict__ counts,
-                                                        const int32_t* __restrict__ first, int64_t pairs, int num_rels,
-                                                        PairF32* __restrict__ out) {
+// key2[i] = key[i] << kSubBits | (position of sorted edge i in its run of equal key) / emax; `first`
+// holds the first sorted edge of every run.  flags[0] = 3 when a run has more pieces than fit.
+__global__ __launch_bounds__(256) void f32_subkeys_kernel(const uint64_t* __restrict__ keys,
+                                                          const int32_t* __restrict__ first, int64_t runs, int64_t slots,
+                                                          int emax, uint64_t* __restrict__ key2, int32_t* __restrict__ flags) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= pairs) return;
-  const uint64_t key = unique[i];
-  PairF32 p;
-  p.rel_dl = (uint32_t)(((key >> kTileShift) % (uint64_t)num_rels) << kTileShift) | (uint32_t)(key & (kTileRows - 1));
-  p.count = counts[i];
-  p.first = first[i];
-  out[i] = p;
+  if (i >= slots) return;
+  int64_t lo = 0, hi = runs - 1;  // last run whose first edge is not behind i
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if ((int64_t)first[mid] <= i) lo = mid; else hi = mid - 1;
+  }
+  int64_t piece = (i - first[lo]) / emax;
+  if (piece >= (int64_t(1) << kSubBits)) {
+    flags[0] = 3;
+    piece = (int64_t(1) << kSubBits) - 1;
+  }
+  key2[i] = (keys[i] << kSubBits) | (uint64_t)piece;
 }
 
-// batches of run i (a (tile, relation) run of `count` pairs starting at pair `first`)
-__global__ __launch_bounds__(256) void f32_batch_count_kernel(const int32_t* __restrict__ run_pairs, int64_t runs,
-                                                              int32_t* __restrict__ run_batches) {
+// the (tile, relation) part of a pair's second key
+__global__ __launch_bounds__(256) void f32_shift_keys_kernel(const uint64_t* __restrict__ in, int64_t count,
+                                                             uint64_t* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < runs) run_batches[i] = (run_pairs[i] + kBatch - 1) / kBatch;
+  if (i < count) out[i] = in[i] >> (kSubBits + kTileShift);
 }
 
-__global__ __launch_bounds__(256) void f32_batch_fill_kernel(const uint64_t* __restrict__ run_keys,
-                                                             const int32_t* __restrict__ run_pairs,
-                                                             const int32_t* __restrict__ run_first_pair,
-                                                             const int32_t* __restrict__ run_first_batch, int64_t runs,
-                                                             int num_rels, BatchF32* __restrict__ batches) {
+// Run i is a (tile, relation) run of run_pairs[i] pairs starting at pair run_first_pair[i]: its
+// pairs, in order, fill batches of at most kBatch pairs and at most emax edges.  Counts the
+// batches (FILL = false) or writes them and the pairs' words (FILL = true).  A pair has at most
+// emax edges (f32_subkeys_kernel), so every batch takes at least one.
+template <bool FILL>
+__global__ __launch_bounds__(256) void f32_batches_kernel(const uint64_t* __restrict__ run_keys,
+                                                          const int32_t* __restrict__ run_pairs,
+                                                          const int32_t* __restrict__ run_first_pair,
+                                                          const int32_t* __restrict__ run_first_batch, int64_t runs,
+                                                          int num_rels, int emax, const uint64_t* __restrict__ pair_keys,
+                                                          const int32_t* __restrict__ pair_edges,
+                                                          const int32_t* __restrict__ pair_first,
+                                                          int32_t* __restrict__ run_batches,
+                                                          BatchF32* __restrict__ batches, uint32_t* __restrict__ pinfo) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= runs) return;
-  const int count = run_pairs[i];
+  const int np = run_pairs[i], fp = run_first_pair[i];
   const int rel = (int)(run_keys[i] % (uint64_t)num_rels);
-  for (int k = 0; k * kBatch < count; ++k) {
-    BatchF32 b;
-    b.pair_begin = (int64_t)run_first_pair[i] + k * kBatch;
-    b.npairs = min(kBatch, count - k * kBatch);
-    b.rel = rel;
-    batches[run_first_batch[i] + k] = b;
+  int nb = 0;
+  for (int j = 0; j < np;) {
+    const int pb = j;
+    int ne = 0, most = 0;
+    do {
+      const int c = min(pair_edges[fp + j], emax);
+      if (j > pb && (j - pb == kBatch || ne + c > emax)) break;
+      if (FILL) {
+        const uint32_t dl = (uint32_t)((pair_keys[fp + j] >> kSubBits) & (kTileRows - 1));
+        pinfo[fp + j] = dl | ((uint32_t)c << 8) | ((uint32_t)ne << 16);
+      }
+      ne += c, most = max(most, c), ++j;
+    } while (j < np);
+    if (FILL) {
+      BatchF32 b;
+      b.pair_begin = fp + pb;
+      b.edge_begin = pair_first[fp + pb];
+      b.counts = (uint32_t)(j - pb) | ((uint32_t)ne << 8) | ((uint32_t)most << 16);
+      b.rel = rel;
+      batches[run_first_batch[i] + nb] = b;
+    }
+    ++nb;
   }
+  if (!FILL) run_batches[i] = nb;
 }
 
 // begin[t] = first batch of tile t (t = tiles gives the batch count): the first run whose key
@@ -207,12 +254,6 @@ __global__ __launch_bounds__(256) void f32_tile_batches_kernel(const uint64_t* _
     if (run_keys[mid] < target) lo = mid + 1; else hi = mid;
   }
   begin[t] = lo < runs ? run_first_batch[lo] : total_batches;
-}
-
-__global__ __launch_bounds__(256) void f32_shift_keys_kernel(const uint64_t* __restrict__ in, int64_t count,
-                                                             uint64_t* __restrict__ out) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < count) out[i] = in[i] >> kTileShift;
 }
 
 typedef __attribute__((address_space(1))) const float GlobalF32;  // a global-memory load, not a flat one
@@ -244,181 +285,156 @@ __global__ __launch_bounds__(256) void f32_pack_w_kernel(const float* __restrict
 //
 // Two lane layouts.  Gathering: a row of X (or its first 32 KS floats) is spread over CPR = 8 KS
 // neighbouring lanes, four floats each, so that a load instruction reads 64 / CPR whole rows and
-// the texture addresser sees whole lines per quad of lanes; a lane serves the same (pair, chunk)
-// for every edge of the pair and sums in registers.  Multiplying: lane (i = l % 16, q = l / 16)
-// holds inputs 8q .. 8q+7 of pair i.  The sums change layout through a 16 x 32 KS tile of LDS per
-// wavefront, one write and one read per batch; the pairs' rows inside the tile of Y travel the
-// same way.
+// the texture addresser sees whole lines per quad of lanes; the four load instructions of a batch
+// cover its EMAX = 32 / KS edges in order.  Multiplying: lane (i = l % 16, q = l / 16) holds
+// inputs 8q .. 8q+7 of pair i.  The weighted rows change layout through an EMAX x 32 KS tile of
+// LDS per wavefront: written once per edge, read once per edge by the lanes of the edge's pair.
 //
 // The loads of the batch loop are unconditional -- indices are clamped to records that exist and
 // what must not count is multiplied by zero afterwards -- so that the loop body is one basic
-// block: the rows of X of the current batch are requested first and waited for alone, while the
-// records of the next batches, requested behind them, stay in flight during the arithmetic.
-// Offsets into X, the pair records and the edge records are 32-bit byte offsets from scalar bases
-// (the launch checks that they fit).
+// block.  Offsets into X and the edge records are 32-bit byte offsets from scalar bases (the
+// launch checks that they fit).
 template <int KS, int NT>
-__global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int fout, int64_t total_batches,
-                                                               const int64_t* __restrict__ tile_batches,
-                                                               const BatchF32* __restrict__ batches,
-                                                               const PairF32* __restrict__ pairs,
-                                                               const EdgeF32* __restrict__ edges,
-                                                               const float4* __restrict__ Wp,
-                                                               const float* __restrict__ X, float* __restrict__ Y) {
+__global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
+                                                            const UnitF32* __restrict__ units,
+                                                            const BatchF32* __restrict__ batches,
+                                                            const uint32_t* __restrict__ pinfo,
+                                                            const EdgeF32* __restrict__ edges,
+                                                            const float4* __restrict__ Wp,
+                                                            const float* __restrict__ X, float* __restrict__ Y,
+                                                            float* __restrict__ partials) {
   constexpr int FO = 16 * NT;      // floats per row of a partial tile
   constexpr int CPR = 8 * KS;      // lanes (16-byte chunks) per gathered row
   constexpr int RPI = 64 / CPR;    // rows per load instruction
-  constexpr int PASSES = kBatch / RPI;
-  constexpr int SS = 32 * KS + 4;  // floats per row of the S tile: 16 lanes reading 32 bytes each hit 64 banks
-  constexpr int U = 2;             // edges of a pair whose records are fetched a batch ahead
+  constexpr int EMAX = 32 / KS;    // edges per batch
+  constexpr int NLOAD = EMAX / RPI;
+  constexpr int SS = 32 * KS + 4;  // floats per row of the edge tile: 16 lanes reading 32 bytes each hit 64 banks
+  static_assert(NLOAD == 4, "four load instructions per batch");
+  static_assert(NT == 2 || NT == 4, "a lane's outputs are one 8- or 16-byte word of the partial tile");
   __shared__ __attribute__((aligned(16))) float ytile[4][kTileRows * FO];
-  __shared__ __attribute__((aligned(16))) float stile[4][kBatch * SS];
-  __shared__ __attribute__((aligned(16))) int32_t dtile[4][kBatch];
+  __shared__ __attribute__((aligned(16))) float etile[4][(EMAX + 1) * SS];  // the last row stays zero
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int i = lane & 15, q = lane >> 4;  // multiplying
+  const int i = lane & 15, q = lane >> 4;      // multiplying
   const int gr = lane / CPR, gc = lane % CPR;  // gathering
-  const int64_t tile = blockIdx.x;
+  const UnitF32 u = units[blockIdx.x];
   float* yt = ytile[wave];
-  float* st = stile[wave];
-  int32_t* dt = dtile[wave];
+  float* et = etile[wave];
   for (int e = lane; e < kTileRows * FO; e += 64) yt[e] = 0.f;
+  for (int e = lane; e < (EMAX + 1) * SS; e += 64) et[e] = 0.f;
 
-  const int64_t b_end = tile_batches[tile + 1];
-  int64_t b = tile_batches[tile] + wave;
+  const int b_end = u.batch_end;
+  int b = u.batch_begin + wave;
   const bool chunk_live = 4 * gc < fin;  // fin is a multiple of 4: chunks are whole
   const uint32_t x_off = chunk_live ? 16u * gc : 0u;
-  const float x_keep = chunk_live ? 1.f : 0.f;
   const uint32_t row_bytes = 4u * (uint32_t)fin;
   const char* Xb = reinterpret_cast<const char*>(X);
-  const char* Pb = reinterpret_cast<const char*>(pairs);
   const char* Eb = reinterpret_cast<const char*>(edges);
 
-  struct Batch {
-    uint32_t pair_off;  // bytes
-    int npairs, rel;
+  struct Batch {  // the same in every lane
+    uint32_t pair_begin, edge_off;  // edge_off in bytes
+    int npairs, nedges, most, rel;
   };
-  auto load_batch = [&](int64_t bi) {  // the same for every lane: one address per wavefront
-    const BatchF32 t = batches[min(bi, total_batches - 1)];
+  auto raw_batch = [&](int bi) { return batches[min(bi, total_batches - 1)]; };
+  auto scalars = [&](const BatchF32& t, int bi) {  // a batch beyond the unit's last one: no pairs, no edges
     Batch r;
-    r.pair_off = __builtin_amdgcn_readfirstlane((uint32_t)t.pair_begin * 16u);
-    r.npairs = bi < b_end ? __builtin_amdgcn_readfirstlane(t.npairs) : 0;
+    const uint32_t c = bi < b_end ? __builtin_amdgcn_readfirstlane(t.counts) : 0u;
+    r.pair_begin = __builtin_amdgcn_readfirstlane((uint32_t)t.pair_begin);
+    r.edge_off = __builtin_amdgcn_readfirstlane((uint32_t)t.edge_begin) * 16u;
+    r.npairs = (int)(c & 255u), r.nedges = (int)((c >> 8) & 255u), r.most = (int)((c >> 16) & 255u);
     r.rel = __builtin_amdgcn_readfirstlane(t.rel);
     return r;
   };
-  // gathering layout: in pass p the lane serves pair p * RPI + gr of the batch
-  struct PairsG {
-    uint32_t first[PASSES];  // bytes into the edge records
-    int count[PASSES];
-    int dl[PASSES];
+  struct EdgesG {  // gathering layout: load instruction k serves edge k * RPI + gr of the batch
+    int32_t src[NLOAD];
+    const float* w[NLOAD];
   };
-  auto load_pairs = [&](const Batch& bt) {  // a lane without a pair repeats the batch's first one with no edges
-    PairsG r;
+  auto load_edges = [&](const Batch& bt) {  // beyond the batch's last edge: that one again
+    EdgesG r;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int slot = p * RPI + gr;
-      const PairF32 pr = *reinterpret_cast<const PairF32*>(Pb + (bt.pair_off + (slot < bt.npairs ? 16u * slot : 0u)));
-      r.first[p] = (uint32_t)pr.first * 16u;
-      r.count[p] = slot < bt.npairs ? pr.count : 0;
-      r.dl[p] = (int)(pr.rel_dl & (kTileRows - 1));
+    for (int k = 0; k < NLOAD; ++k) {
+      const int e = k * RPI + gr;
+      // (one 16-byte load; taken apart field by field it becomes two)
+      const uint4 rec = *reinterpret_cast<const uint4*>(Eb + (bt.edge_off + 16u * (uint32_t)min(e, max(bt.nedges - 1, 0))));
+      r.src[k] = (int32_t)rec.x;
+      r.w[k] = reinterpret_cast<const float*>((uintptr_t)rec.z | ((uintptr_t)rec.w << 32));
     }
     return r;
   };
-  struct EdgesG {
-    EdgeF32 e[PASSES][U];
+  struct RowsG {
+    float w[NLOAD];
+    float4 x[NLOAD];
   };
-  auto load_edges = [&](const PairsG& pg) {  // beyond the pair's last edge: its first one again
-    EdgesG r;
+  auto load_rows = [&](const EdgesG& eg) {
+    RowsG r;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p)
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        r.e[p][u] = *reinterpret_cast<const EdgeF32*>(Eb + (pg.first[p] + (u < pg.count[p] ? 16u * u : 0u)));
+    for (int k = 0; k < NLOAD; ++k) {
+      r.w[k] = *reinterpret_cast<GlobalF32*>(reinterpret_cast<uintptr_t>(eg.w[k]));
+      r.x[k] = *reinterpret_cast<const float4*>(Xb + ((uint32_t)eg.src[k] * row_bytes + x_off));
+    }
     return r;
   };
-  auto weight_of = [](const EdgeF32& e) { return *reinterpret_cast<GlobalF32*>(reinterpret_cast<uintptr_t>(e.w)); };
-  auto fma4 = [](float4& acc, float w, const float4& x) {
-    acc.x += w * x.x, acc.y += w * x.y, acc.z += w * x.z, acc.w += w * x.w;
-  };
+  auto load_pair = [&](const Batch& bt) { return pinfo[bt.pair_begin + (i < bt.npairs ? (uint32_t)i : 0u)]; };
 
-  // the pipeline: batch records three ahead, pair records two, first edge records one
-  Batch bt0 = load_batch(b), bt1 = load_batch(b + 4), bt2 = load_batch(b + 8);
-  PairsG pg0 = load_pairs(bt0), pg1 = load_pairs(bt1);
-  EdgesG eg0 = load_edges(pg0);
+  // the pipeline: batch records four ahead, edge records and pair words three, rows of X one
+  Batch bt0 = scalars(raw_batch(b), b), bt1 = scalars(raw_batch(b + 4), b + 4), bt2 = scalars(raw_batch(b + 8), b + 8);
+  BatchF32 raw3 = raw_batch(b + 12);
+  EdgesG eg1 = load_edges(bt1), eg2 = load_edges(bt2);
+  uint32_t pw0 = load_pair(bt0), pw1 = load_pair(bt1), pw2 = load_pair(bt2);
+  RowsG rw0;
+  {
+    const EdgesG eg0 = load_edges(bt0);
+    rw0 = load_rows(eg0);
+  }
 
   while (bt0.npairs > 0) {  // the same for every lane
-    const int rel0 = bt0.rel, npairs = bt0.npairs;
-    // the rows of X and the weights of the pairs' first U edges
-    float wv[PASSES][U];
-    float4 xv[PASSES][U];
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p)
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        wv[p][u] = weight_of(eg0.e[p][u]);
-        xv[p][u] = *reinterpret_cast<const float4*>(Xb + ((uint32_t)eg0.e[p][u].src * row_bytes + x_off));
-      }
-    // B operands of rel0, in lane order
+    // requests: the next batch's rows, this batch's W, the records further ahead
+    const RowsG rw1 = load_rows(eg1);
     float4 wq[NT][KS][2];
-    const float4* wrel = Wp + (int64_t)rel0 * (NT * KS * 2 * 64) + lane;
+    const float4* wrel = Wp + (int64_t)bt0.rel * (NT * KS * 2 * 64) + lane;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int s = 0; s < KS; ++s)
 #pragma unroll
         for (int c = 0; c < 2; ++c) wq[nt][s][c] = wrel[((nt * KS + s) * 2 + c) * 64];
-    // the records of the batches to come
-    const Batch bt3 = load_batch(b + 12);
-    const PairsG pg2 = load_pairs(bt2);
-    const EdgesG eg1 = load_edges(pg1);
+    const Batch bt3 = scalars(raw3, b + 12);
+    const BatchF32 raw4 = raw_batch(b + 16);
+    const EdgesG eg3 = load_edges(bt3);
+    const uint32_t pw3 = load_pair(bt3);
 
-    // the weighted sums of the pairs' rows of X, gathering layout
-    float4 sum[PASSES];
+    // 1. the weighted rows of this batch, into the edge tile.  Places behind the batch's last edge
+    // get whatever was read: no pair reads them.  Chunks beyond feat_in are never written and stay
+    // zero.
+    if (chunk_live) {
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      sum[p] = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-      for (int u = 0; u < U; ++u) fma4(sum[p], u < pg0.count[p] ? wv[p][u] : 0.f, xv[p][u]);
+      for (int k = 0; k < NLOAD; ++k) {
+        const float w = rw0.w[k];
+        float4 v = rw0.x[k];
+        v.x *= w, v.y *= w, v.z *= w, v.w *= w;
+        *reinterpret_cast<float4*>(et + (k * RPI + gr) * SS + 4 * gc) = v;
+      }
     }
-    int most = 0;
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p) most = max(most, pg0.count[p]);
-    for (int t0 = U; __ballot(t0 < most) != 0; t0 += U) {  // pairs of more than U edges: two round trips per pass
-      EdgeF32 er[PASSES][U];
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p)
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          er[p][u] = *reinterpret_cast<const EdgeF32*>(Eb + (pg0.first[p] + (t0 + u < pg0.count[p] ? 16u * (t0 + u) : 0u)));
-      float w2[PASSES][U];
-      float4 x2[PASSES][U];
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p)
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          w2[p][u] = weight_of(er[p][u]);
-          x2[p][u] = *reinterpret_cast<const float4*>(Xb + ((uint32_t)er[p][u].src * row_bytes + x_off));
-        }
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p)
-#pragma unroll
-        for (int u = 0; u < U; ++u) fma4(sum[p], t0 + u < pg0.count[p] ? w2[p][u] : 0.f, x2[p][u]);
-    }
-    // through LDS into the multiplying layout (chunks beyond feat_in were read from the row's start: zero)
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int slot = p * RPI + gr;
-      float4 v = sum[p];
-      v.x *= x_keep, v.y *= x_keep, v.z *= x_keep, v.w *= x_keep;
-      *reinterpret_cast<float4*>(st + slot * SS + 4 * gc) = v;
-      if (gc == 0) dt[slot] = pg0.dl[p];
-    }
+    // 2. the sums of the pairs, multiplying layout: lane (i, q) walks the edges of pair i; a lane
+    // whose pair has fewer edges than the batch's longest reads the tile's row of zeros meanwhile
+    const int my_first = (int)((pw0 >> 16) & 255u), my_count = i < bt0.npairs ? (int)((pw0 >> 8) & 255u) : 0;
+    const int my_dl = (int)(pw0 & (kTileRows - 1));
     float4 sq[KS][2];
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int c = 0; c < 2; ++c) sq[s][c] = *reinterpret_cast<const float4*>(st + i * SS + 32 * s + 8 * q + 4 * c);
-    const int4 dl4 = *reinterpret_cast<const int4*>(dt + 4 * q);
-
+      for (int c = 0; c < 2; ++c) sq[s][c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int t = 0; t < bt0.most; ++t) {  // the same for every lane
+      const float* row = et + (t < my_count ? my_first + t : EMAX) * SS + 8 * q;
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const float4 v = *reinterpret_cast<const float4*>(row + 32 * s + 4 * c);
+          sq[s][c].x += v.x, sq[s][c].y += v.y, sq[s][c].z += v.z, sq[s][c].w += v.w;
+        }
+    }
+    // 3. times W[rel]^T
     f32x4 acc[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -434,36 +450,61 @@ __global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int 
           acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sk.z, wk.z, acc[nt], 0, 0, 0);
           acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sk.w, wk.w, acc[nt], 0, 0, 0);
         }
-
-    // acc[nt][v]: pair 4 q + v of the batch, output 16 nt + i.  Rows of the partial tile are 16 NT
-    // floats; the column is rotated by 16 for every second pair of rows, which keeps most of the
-    // four rows an instruction touches on different banks.
-    const int dls[4] = {dl4.x, dl4.y, dl4.z, dl4.w};
+    // 4. acc[nt][v]: pair 4 q + v of the batch, output 16 nt + i, which lives at float NT i + nt of
+    // its row of the partial tile: a lane's NT outputs are neighbours, one read and one write.
+    // The pairs of a batch end in different rows (a row cut into pieces has at most its last,
+    // shorter piece in a batch with other pairs: a full piece fills a batch), so no two lanes
+    // update the same float.
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      if (4 * q + v < npairs) {
-        const int dl = dls[v];
-        float* row = yt + dl * FO;
-        const int rot = 16 * ((dl >> 1) & 1);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) row[((16 * nt + rot) & (FO - 1)) + i] += acc[nt][v];
+      const int dl = __shfl(my_dl, 4 * q + v, 64);
+      if (4 * q + v < bt0.npairs) {
+        float* at = yt + dl * FO + NT * i;
+        if constexpr (NT == 2) {
+          float2 o = *reinterpret_cast<float2*>(at);
+          o.x += acc[0][v], o.y += acc[1][v];
+          *reinterpret_cast<float2*>(at) = o;
+        } else {
+          float4 o = *reinterpret_cast<float4*>(at);
+          o.x += acc[0][v], o.y += acc[1][v], o.z += acc[2][v], o.w += acc[3][v];
+          *reinterpret_cast<float4*>(at) = o;
+        }
       }
     }
     b += 4;
-    bt0 = bt1, bt1 = bt2, bt2 = bt3;
-    pg0 = pg1, pg1 = pg2;
-    eg0 = eg1;
+    bt0 = bt1, bt1 = bt2, bt2 = bt3, raw3 = raw4;
+    eg1 = eg2, eg2 = eg3;
+    pw0 = pw1, pw1 = pw2, pw2 = pw3;
+    rw0 = rw1;
   }
 
   __syncthreads();
-  const int64_t row0 = tile * kTileRows;
+  const int64_t row0 = (int64_t)u.tile * kTileRows;
   for (int e = tid; e < kTileRows * fout; e += 256) {
     const int r = e / fout, c = e - r * fout;
     if (row0 + r >= m) break;
-    const int at = r * FO + ((((c >> 4) * 16 + 16 * ((r >> 1) & 1)) & (FO - 1)) + (c & 15));
+    const int at = r * FO + NT * (c & 15) + (c >> 4);
     const float sum = (ytile[0][at] + ytile[1][at]) + (ytile[2][at] + ytile[3][at]);
-    float* y = Y + (row0 + r) * fout + c;
-    *y += sum;
+    if (u.partial < 0)
+      Y[(row0 + r) * fout + c] += sum;
+    else
+      partials[(int64_t)u.partial * (kTileRows * fout) + e] = sum;
+  }
+}
+
+// The tiles that were cut into several units: their partial tiles, in the order of the units, are
+// added to Y.  One workgroup per such tile.
+__global__ __launch_bounds__(256) void f32_sum_partials_kernel(const MultiF32* __restrict__ multi, int m, int fout,
+                                                               const float* __restrict__ partials,
+                                                               float* __restrict__ Y) {
+  const MultiF32 t = multi[blockIdx.x];
+  const int64_t row0 = (int64_t)t.tile * kTileRows;
+  const int64_t stride = (int64_t)kTileRows * fout;
+  for (int e = threadIdx.x; e < kTileRows * fout; e += 256) {
+    if (row0 + e / fout >= m) break;
+    float sum = 0.f;
+    for (int p = 0; p < t.pieces; ++p) sum += partials[(t.first_partial + p) * stride + e];
+    Y[row0 * fout + e] += sum;
   }
 }
 
@@ -485,28 +526,36 @@ struct Scratch {
 }  // namespace
 
 namespace {
-int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, int32_t num_rels, hipStream_t stream);
+int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, int32_t num_rels, int32_t emax,
+                hipStream_t stream);
 }
 
 bool f32_tiles_serves(int32_t feat_in, int32_t feat_out) {
   return feat_in > 0 && feat_in % 4 == 0 && feat_in <= 64 && feat_out > 0 && feat_out <= 64;
 }
 
+bool f32_tiles_fits(int32_t n, int32_t feat_in, int64_t edges) {
+  return (int64_t)n * feat_in * 4 < (int64_t(1) << 32) && edges * 16 < (int64_t(1) << 32);
+}
+
 void f32_tiles_free(F32TileIndex& idx) {
   if (idx.d_edges) (void)hipFree(idx.d_edges);
   if (idx.d_pairs) (void)hipFree(idx.d_pairs);
   if (idx.d_batches) (void)hipFree(idx.d_batches);
+  if (idx.d_units) (void)hipFree(idx.d_units);
+  if (idx.d_multi) (void)hipFree(idx.d_multi);
+  if (idx.d_partials) (void)hipFree(idx.d_partials);
   if (idx.d_wpack) (void)hipFree(idx.d_wpack);
-  if (idx.d_tile_pairs) (void)hipFree(idx.d_tile_pairs);
   idx = F32TileIndex();
 }
 
 int f32_tiles_prepare(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, int32_t num_rels,
-                      hipStream_t stream) {
-  if (idx.m == m && idx.n == n && idx.num_rels == num_rels) return 0;
+                      int32_t feat_in, hipStream_t stream) {
+  const int32_t emax = feat_in <= 32 ? 32 : 16;
+  if (idx.m == m && idx.n == n && idx.num_rels == num_rels && idx.emax == emax) return 0;
   f32_tiles_free(idx);
   F32TileIndex built;
-  const int rc = build_index(built, src, m, n, num_rels, stream);
+  const int rc = build_index(built, src, m, n, num_rels, emax, stream);
   if (rc != 0) {
     f32_tiles_free(built);  // nothing half-made stays behind
     return rc;
@@ -516,7 +565,8 @@ int f32_tiles_prepare(F32TileIndex& idx, const F32Source& src, int32_t m, int32_
 }
 
 namespace {
-int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, int32_t num_rels, hipStream_t stream) {
+int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, int32_t num_rels, int32_t emax,
+                hipStream_t stream) {
   STIR_REQUIRE(m > 0 && n > 0 && num_rels > 0, "rgms_f32: m, n and num_rels must be positive");
   // edges and their numbering
   std::vector<DevBucketF32> tab;
@@ -532,16 +582,13 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
   }
   STIR_REQUIRE(slots < (int64_t(1) << 31), "rgms_f32: %lld slots exceed 32-bit edge numbers", (long long)slots);
   const int64_t tiles = ceil_div(m, kTileRows);
-  STIR_REQUIRE((double)tiles * num_rels * kTileRows < 9e18, "rgms_f32: sort keys exceed 64 bits");
-  idx.m = m, idx.n = n, idx.num_rels = num_rels;
+  STIR_REQUIRE(tiles < (int64_t(1) << 31), "rgms_f32: too many tiles");
+  int key_bits = kTileShift;
+  while (key_bits < 64 && ((uint64_t)tiles * num_rels) >> (key_bits - kTileShift)) ++key_bits;
+  STIR_REQUIRE(key_bits + kSubBits <= 64, "rgms_f32: sort keys exceed 64 bits");
+  idx.m = m, idx.n = n, idx.num_rels = num_rels, idx.emax = emax;
   idx.edges = slots, idx.tiles = tiles;
-  STIR_HIP(hipMalloc(&idx.d_tile_pairs, sizeof(int64_t) * (size_t)(tiles + 1)));
-  if (slots == 0) {
-    idx.pairs = 0;
-    STIR_HIP(hipMemsetAsync(idx.d_tile_pairs, 0, sizeof(int64_t) * (size_t)(tiles + 1), stream));
-    STIR_HIP(hipStreamSynchronize(stream));
-    return 0;
-  }
+  if (slots == 0) return 0;  // no units: the launch returns at once
   Scratch tmp;
   DevBucketF32* d_tab = nullptr;
   if (!tab.empty()) {
@@ -551,8 +598,10 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
   const CsfArrays csf = {src.A, src.indptr_i, src.indices_i, src.indptr_j, src.indices_j, src.nnz_i};
   uint64_t *keys_in = nullptr, *keys_out = nullptr, *unique = nullptr;
   int32_t *vals_in = nullptr, *vals_out = nullptr, *counts = nullptr, *first = nullptr, *flags = nullptr;
+  int64_t* tile_begin = nullptr;
   if (tmp.get(&keys_in, slots) || tmp.get(&keys_out, slots) || tmp.get(&unique, slots) || tmp.get(&vals_in, slots) ||
-      tmp.get(&vals_out, slots) || tmp.get(&counts, slots) || tmp.get(&first, slots) || tmp.get(&flags, 2))
+      tmp.get(&vals_out, slots) || tmp.get(&counts, slots) || tmp.get(&first, slots) || tmp.get(&flags, 2) ||
+      tmp.get(&tile_begin, tiles + 1))
     return -1;
   STIR_HIP(hipMemsetAsync(flags, 0, sizeof(int32_t) * 2, stream));
   const dim3 grid((unsigned)ceil_div(slots, 256)), block(256);
@@ -564,17 +613,17 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
     hipLaunchKernelGGL(f32_edge_keys_kernel<false>, grid, block, 0, stream, d_tab, nb, csf, slots, m, n, num_rels,
                        keys_in, vals_in, flags);
   STIR_LAUNCH_CHECK();
-  int key_bits = kTileShift;
-  while (key_bits < 64 && ((uint64_t)tiles * num_rels) >> (key_bits - kTileShift)) ++key_bits;
   size_t sort_bytes = 0, rle_bytes = 0, scan_bytes = 0;
   STIR_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, keys_in, keys_out, vals_in, vals_out, (int)slots, 0,
                                               key_bits, stream));
   STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(nullptr, rle_bytes, keys_out, unique, counts, flags + 1, (int)slots,
                                                  stream));
-  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, scan_bytes, counts, first, (int)slots, stream));
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, scan_bytes, counts, first, (int)slots + 1, stream));
   char* cub_tmp = nullptr;
-  if (tmp.get(&cub_tmp, std::max(sort_bytes, std::max(rle_bytes, scan_bytes)))) return -1;
-  STIR_HIP(hipcub::DeviceRadixSort::SortPairs(cub_tmp, sort_bytes, keys_in, keys_out, vals_in, vals_out, (int)slots, 0,
+  const size_t cub_bytes = std::max(sort_bytes, std::max(rle_bytes, scan_bytes));
+  if (tmp.get(&cub_tmp, cub_bytes)) return -1;
+  size_t bytes = sort_bytes;
+  STIR_HIP(hipcub::DeviceRadixSort::SortPairs(cub_tmp, bytes, keys_in, keys_out, vals_in, vals_out, (int)slots, 0,
                                               key_bits, stream));
   STIR_HIP(hipMalloc(&idx.d_edges, sizeof(EdgeF32) * (size_t)slots));
   if (src.csf)
@@ -584,7 +633,9 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
     hipLaunchKernelGGL(f32_edge_records_kernel<false>, grid, block, 0, stream, d_tab, nb, csf, slots, num_rels,
                        vals_out, static_cast<EdgeF32*>(idx.d_edges));
   STIR_LAUNCH_CHECK();
-  STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(cub_tmp, rle_bytes, keys_out, unique, counts, flags + 1, (int)slots,
+  // runs of equal key, cut into pieces of at most emax edges by a second key
+  bytes = rle_bytes;
+  STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(cub_tmp, bytes, keys_out, unique, counts, flags + 1, (int)slots,
                                                  stream));
   int32_t host_flags[2] = {0, 0};
   STIR_HIP(hipMemcpyAsync(host_flags, flags, sizeof(host_flags), hipMemcpyDeviceToHost, stream));
@@ -592,17 +643,26 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
   if (host_flags[0] != 0)
     return fail(host_flags[0] == 1 ? "rgms_f32: a row id or relation id lies outside [0, m) / [0, num_rels)"
                                    : "rgms_f32: a column id lies outside [0, n)");
+  const int64_t key_runs = host_flags[1];
+  bytes = scan_bytes;
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, bytes, counts, first, (int)key_runs, stream));
+  hipLaunchKernelGGL(f32_subkeys_kernel, grid, block, 0, stream, keys_out, first, key_runs, slots, (int)emax, keys_in,
+                     flags);
+  STIR_LAUNCH_CHECK();
+  bytes = rle_bytes;
+  STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(cub_tmp, bytes, keys_in, unique, counts, flags + 1, (int)slots,
+                                                 stream));
+  STIR_HIP(hipMemcpyAsync(host_flags, flags, sizeof(host_flags), hipMemcpyDeviceToHost, stream));
+  STIR_HIP(hipStreamSynchronize(stream));
+  STIR_REQUIRE(host_flags[0] == 0, "rgms_f32: a (relation, row) pair has too many edges for the tiled kernel");
   const int64_t pairs = host_flags[1];
   idx.pairs = pairs;
-  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, scan_bytes, counts, first, (int)pairs, stream));
-  STIR_HIP(hipMalloc(&idx.d_pairs, sizeof(PairF32) * (size_t)std::max<int64_t>(pairs, 1)));
-  hipLaunchKernelGGL(f32_pairs_kernel, dim3((unsigned)ceil_div(pairs, 256)), block, 0, stream, unique, counts, first,
-                     pairs, num_rels, static_cast<PairF32*>(idx.d_pairs));
-  STIR_LAUNCH_CHECK();
-  STIR_LAUNCH_CHECK();
-  // the (tile, relation) runs of pairs and their batches.  keys_in / vals_in / keys_out / vals_out are free again
-  uint64_t* run_of_pair = keys_in;   // pair key without the row
-  uint64_t* run_keys = keys_out;
+  bytes = scan_bytes;
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, bytes, counts, first, (int)pairs, stream));
+  // the (tile, relation) runs of pairs.  keys_out / vals_in / vals_out are free again; keys_in is
+  // once the run-length encoding above has read it (same stream)
+  uint64_t* run_of_pair = keys_out;
+  uint64_t* run_keys = keys_in;
   int32_t *run_pairs = vals_in, *run_first_pair = vals_out;
   int32_t *run_batches = nullptr, *run_first_batch = nullptr;
   if (tmp.get(&run_batches, pairs + 1) || tmp.get(&run_first_batch, pairs + 1)) return -1;
@@ -613,33 +673,74 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
   STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(nullptr, rle2, run_of_pair, run_keys, run_pairs, flags + 1, (int)pairs,
                                                  stream));
   STIR_HIP(hipcub::DeviceScan::ExclusiveSum(nullptr, scan2, run_pairs, run_first_pair, (int)pairs + 1, stream));
-  STIR_REQUIRE(std::max(rle2, scan2) <= std::max(sort_bytes, std::max(rle_bytes, scan_bytes)),
-               "rgms_f32: scratch of the index build is too small");
-  STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(cub_tmp, rle2, run_of_pair, run_keys, run_pairs, flags + 1, (int)pairs,
+  STIR_REQUIRE(std::max(rle2, scan2) <= cub_bytes, "rgms_f32: scratch of the index build is too small");
+  bytes = rle2;
+  STIR_HIP(hipcub::DeviceRunLengthEncode::Encode(cub_tmp, bytes, run_of_pair, run_keys, run_pairs, flags + 1, (int)pairs,
                                                  stream));
   STIR_HIP(hipMemcpyAsync(host_flags, flags, sizeof(host_flags), hipMemcpyDeviceToHost, stream));
   STIR_HIP(hipStreamSynchronize(stream));
   const int64_t runs = host_flags[1];
-  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, scan2, run_pairs, run_first_pair, (int)runs, stream));
-  hipLaunchKernelGGL(f32_batch_count_kernel, dim3((unsigned)ceil_div(runs, 256)), block, 0, stream, run_pairs, runs,
-                     run_batches);
+  bytes = scan2;
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, bytes, run_pairs, run_first_pair, (int)runs, stream));
+  const dim3 run_grid((unsigned)ceil_div(runs, 256));
+  hipLaunchKernelGGL(f32_batches_kernel<false>, run_grid, block, 0, stream, run_keys, run_pairs, run_first_pair,
+                     (const int32_t*)nullptr, runs, num_rels, (int)emax, unique, counts, first, run_batches,
+                     (BatchF32*)nullptr, (uint32_t*)nullptr);
   STIR_LAUNCH_CHECK();
   // one entry more than runs: the last one is the batch count (run_batches[runs] is not read as an addend)
   STIR_HIP(hipMemsetAsync(run_batches + runs, 0, sizeof(int32_t), stream));
-  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, scan2, run_batches, run_first_batch, (int)runs + 1, stream));
+  bytes = scan2;
+  STIR_HIP(hipcub::DeviceScan::ExclusiveSum(cub_tmp, bytes, run_batches, run_first_batch, (int)runs + 1, stream));
   int32_t total_batches = 0;
   STIR_HIP(hipMemcpyAsync(&total_batches, run_first_batch + runs, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
   STIR_HIP(hipStreamSynchronize(stream));
   idx.batches = total_batches;
   STIR_HIP(hipMalloc(&idx.d_batches, sizeof(BatchF32) * (size_t)std::max<int64_t>(total_batches, 1)));
-  hipLaunchKernelGGL(f32_batch_fill_kernel, dim3((unsigned)ceil_div(runs, 256)), block, 0, stream, run_keys, run_pairs,
-                     run_first_pair, run_first_batch, runs, num_rels, static_cast<BatchF32*>(idx.d_batches));
+  STIR_HIP(hipMalloc(&idx.d_pairs, sizeof(uint32_t) * (size_t)std::max<int64_t>(pairs, 1)));
+  hipLaunchKernelGGL(f32_batches_kernel<true>, run_grid, block, 0, stream, run_keys, run_pairs, run_first_pair,
+                     run_first_batch, runs, num_rels, (int)emax, unique, counts, first, (int32_t*)nullptr,
+                     static_cast<BatchF32*>(idx.d_batches), static_cast<uint32_t*>(idx.d_pairs));
   STIR_LAUNCH_CHECK();
   hipLaunchKernelGGL(f32_tile_batches_kernel, dim3((unsigned)ceil_div(tiles + 1, 256)), block, 0, stream, run_keys,
-                     run_first_batch, runs, (int64_t)total_batches, tiles, num_rels,
-                     static_cast<int64_t*>(idx.d_tile_pairs));
+                     run_first_batch, runs, (int64_t)total_batches, tiles, num_rels, tile_begin);
   STIR_LAUNCH_CHECK();
-  STIR_HIP(hipStreamSynchronize(stream));  // the scratch arrays go away
+  // units: a tile, or -- for a tile with more than 1.5 times `cap` batches -- pieces of at most
+  // `cap` batches, cap = twice the average of the tiles that have batches (at least 32)
+  std::vector<int64_t> tb((size_t)tiles + 1);
+  STIR_HIP(hipMemcpyAsync(tb.data(), tile_begin, sizeof(int64_t) * tb.size(), hipMemcpyDeviceToHost, stream));
+  STIR_HIP(hipStreamSynchronize(stream));  // also: the scratch arrays go away
+  int64_t busy = 0;
+  for (int64_t t = 0; t < tiles; ++t) busy += tb[(size_t)t + 1] > tb[(size_t)t];
+  const int64_t cap = std::max<int64_t>(32, busy ? 2 * ceil_div((int64_t)total_batches, busy) : 32);
+  std::vector<UnitF32> units;
+  std::vector<MultiF32> multi;
+  int64_t partial_tiles = 0;
+  for (int64_t t = 0; t < tiles; ++t) {
+    const int64_t lo = tb[(size_t)t], hi = tb[(size_t)t + 1];
+    if (hi <= lo) continue;
+    if (2 * (hi - lo) <= 3 * cap) {
+      units.push_back(UnitF32{(int32_t)t, (int32_t)lo, (int32_t)hi, -1});
+      continue;
+    }
+    const int64_t pieces = ceil_div(hi - lo, cap), len = ceil_div(hi - lo, pieces);
+    STIR_REQUIRE(partial_tiles + pieces < (int64_t(1) << 31), "rgms_f32: too many partial tiles");
+    multi.push_back(MultiF32{(int32_t)t, (int32_t)partial_tiles, (int32_t)pieces, 0});
+    for (int64_t p = 0; p < pieces; ++p)
+      units.push_back(UnitF32{(int32_t)t, (int32_t)(lo + p * len), (int32_t)std::min(hi, lo + (p + 1) * len),
+                              (int32_t)(partial_tiles + p)});
+    partial_tiles += pieces;
+  }
+  // the longest units first
+  std::stable_sort(units.begin(), units.end(), [](const UnitF32& a, const UnitF32& b) {
+    return a.batch_end - a.batch_begin > b.batch_end - b.batch_begin;
+  });
+  idx.units = (int64_t)units.size(), idx.multi = (int64_t)multi.size(), idx.partial_tiles = partial_tiles;
+  STIR_HIP(hipMalloc(&idx.d_units, sizeof(UnitF32) * std::max<size_t>(units.size(), 1)));
+  STIR_HIP(hipMemcpy(idx.d_units, units.data(), sizeof(UnitF32) * units.size(), hipMemcpyHostToDevice));
+  if (!multi.empty()) {
+    STIR_HIP(hipMalloc(&idx.d_multi, sizeof(MultiF32) * multi.size()));
+    STIR_HIP(hipMemcpy(idx.d_multi, multi.data(), sizeof(MultiF32) * multi.size(), hipMemcpyHostToDevice));
+  }
   return 0;
 }
 }  // namespace
@@ -648,10 +749,11 @@ int f32_tiles_launch(F32TileIndex& idx, int32_t feat_in, int32_t feat_out, const
                      float* d_Y, hipStream_t stream) {
   STIR_REQUIRE(f32_tiles_serves(feat_in, feat_out), "rgms_f32: feature sizes %d -> %d are not served by the tiled kernel",
                feat_in, feat_out);
-  if (idx.pairs == 0) return 0;
-  STIR_REQUIRE(idx.tiles < (int64_t(1) << 31), "rgms_f32: too many tiles for one launch");
+  STIR_REQUIRE(idx.emax == (feat_in <= 32 ? 32 : 16), "rgms_f32: the edge index was built for another feat_in");
+  if (idx.units == 0) return 0;
+  STIR_REQUIRE(idx.units < (int64_t(1) << 31), "rgms_f32: too many units for one launch");
   // the kernel's 32-bit byte offsets
-  STIR_REQUIRE((int64_t)idx.n * feat_in * 4 < (int64_t(1) << 32) && idx.edges * 16 < (int64_t(1) << 32),
+  STIR_REQUIRE(f32_tiles_fits(idx.n, feat_in, idx.edges),
                "rgms_f32: the tiled kernel addresses X and its index with 32-bit offsets");
   const int ks = feat_in <= 32 ? 1 : 2, nt = feat_out <= 32 ? 2 : 4;
   // W in operand order, rewritten by every launch (W may change between launches)
@@ -663,18 +765,26 @@ int f32_tiles_launch(F32TileIndex& idx, int32_t feat_in, int32_t feat_out, const
     STIR_HIP(hipMalloc(&idx.d_wpack, need));
     idx.wpack_bytes = need;
   }
+  const size_t partial_need = sizeof(float) * (size_t)idx.partial_tiles * kTileRows * (size_t)feat_out;
+  if (partial_need > idx.partial_bytes) {
+    if (idx.d_partials) STIR_HIP(hipFree(idx.d_partials));
+    idx.d_partials = nullptr, idx.partial_bytes = 0;
+    STIR_HIP(hipMalloc(&idx.d_partials, partial_need));
+    idx.partial_bytes = partial_need;
+  }
   float4* wp = static_cast<float4*>(idx.d_wpack);
   hipLaunchKernelGGL(f32_pack_w_kernel, dim3((unsigned)ceil_div(words, 256)), dim3(256), 0, stream, d_W, wp, words, nt, ks,
                      feat_in, feat_out);
   STIR_LAUNCH_CHECK();
-  const dim3 grid((unsigned)idx.tiles), block(256);
-  const int64_t* tp = static_cast<const int64_t*>(idx.d_tile_pairs);
+  const dim3 grid((unsigned)idx.units), block(256);  // longest units first: they go to whichever slot is free
+  const UnitF32* units = static_cast<const UnitF32*>(idx.d_units);
   const BatchF32* bts = static_cast<const BatchF32*>(idx.d_batches);
-  const PairF32* pairs = static_cast<const PairF32*>(idx.d_pairs);
+  const uint32_t* pinfo = static_cast<const uint32_t*>(idx.d_pairs);
   const EdgeF32* edges = static_cast<const EdgeF32*>(idx.d_edges);
-#define STIR_F32_TILE(KS, NT)                                                                                       \
-  hipLaunchKernelGGL((rgms_f32_tile_kernel<KS, NT>), grid, block, 0, stream, idx.m, feat_in, feat_out, idx.batches, tp, \
-                     bts, pairs, edges, wp, d_X, d_Y)
+  float* partials = static_cast<float*>(idx.d_partials);
+#define STIR_F32_TILE(KS, NT)                                                                                   \
+  hipLaunchKernelGGL((rgms_f32_tile_kernel<KS, NT>), grid, block, 0, stream, idx.m, feat_in, feat_out,          \
+                     (int)idx.batches, units, bts, pinfo, edges, wp, d_X, d_Y, partials)
   if (ks == 1) {
     if (nt == 2) STIR_F32_TILE(1, 2); else STIR_F32_TILE(1, 4);
   } else {
@@ -682,6 +792,11 @@ int f32_tiles_launch(F32TileIndex& idx, int32_t feat_in, int32_t feat_out, const
   }
 #undef STIR_F32_TILE
   STIR_LAUNCH_CHECK();
+  if (idx.multi > 0) {
+    hipLaunchKernelGGL(f32_sum_partials_kernel, dim3((unsigned)idx.multi), block, 0, stream,
+                       static_cast<const MultiF32*>(idx.d_multi), idx.m, feat_out, partials, d_Y);
+    STIR_LAUNCH_CHECK();
+  }
   return 0;
 }
 

@@ -46,9 +46,11 @@ def test_rgms_csf_f32(dev, fin, fout):
     _check(y.cpu().numpy().reshape(n, fout), want, scale, oracle.rgms_csf_f32(a, w, x, *csf, n), f"csf {fin}x{fout}")
 
 
-def test_rgms_csf_f32_long_row_and_empty_relations(dev):
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_rgms_csf_f32_long_row_and_empty_relations(dev, deterministic):
     """One stored row with thousands of edges (several 64-edge passes of one tile), relations
-    without rows, a single stored row in the last relation."""
+    without rows, a single stored row in the last relation.  (3005 edges: both settings run the
+    atomic kernel; the deterministic one through a plan.)"""
     n, fin, fout, R = 5000, 32, 32, 5
     rng = np.random.default_rng(3)
     long_cols = np.sort(rng.choice(n, 3000, replace=False)).astype(np.int32)
@@ -60,7 +62,7 @@ def test_rgms_csf_f32_long_row_and_empty_relations(dev):
     x = rng.standard_normal((n, fin), dtype=np.float32)
     w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
     a = rng.standard_normal(len(i1)).astype(np.float32)
-    f = ops.build_rgms_csf(n, n, R, fin, fout, len(i0), len(i1))
+    f = ops.build_rgms_csf(n, n, R, fin, fout, len(i0), len(i1), deterministic=deterministic)
     y = torch.zeros(n * fout, dtype=torch.float32, device=dev)
     f(_t(dev, a), _t(dev, w.ravel()), _t(dev, x.ravel()), y, *[_t(dev, c) for c in csf])
     torch.cuda.synchronize()
@@ -78,7 +80,7 @@ def test_rgms_csf_f32_empty(dev):
     assert torch.all(y == 3.0)
 
 
-def _run_ell3d(dev, csf, n, x, w, group, buckets, weighted, seed=0, deterministic=False):
+def _run_ell3d(dev, csf, n, x, w, group, buckets, weighted, seed=0, deterministic=True):
     R, fout, fin = w.shape
     rows_bkt = [max(1, group // b) for b in buckets]
     ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rows_bkt, buckets)
@@ -125,16 +127,17 @@ def test_rgms_ell3d_f32(dev, group, buckets, fin, fout, weighted):
         assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(ref) + 2e-5 * scale + 1e-30)
 
 
-def test_rgms_f32_config5_reduced_both_forms_agree(dev):
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_rgms_f32_config5_reduced_both_forms_agree(dev, deterministic):
     cfg = datasets.config5(n=4000, num_rels=65, num_edges=40000)
     csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
     n = cfg["n"]
     w = np.ascontiguousarray(cfg["w"].transpose(0, 2, 1))
-    got, bk = _run_ell3d(dev, csf, n, cfg["x"], w, 32, cfg["buckets"], False)
+    got, bk = _run_ell3d(dev, csf, n, cfg["x"], w, 32, cfg["buckets"], False, deterministic=deterministic)
     ones = np.ones(len(csf[3]), np.float32)
     want, scale = _closed_forms(csf, ones, cfg["x"], w, n)
     _check(got, want, scale, oracle.rgms_ell3d_f32(w, cfg["x"], bk, n), "config5 ell3d")
-    f = ops.build_rgms_csf(n, n, 65, 32, 32, len(csf[1]), len(csf[3]))
+    f = ops.build_rgms_csf(n, n, 65, 32, 32, len(csf[1]), len(csf[3]), deterministic=deterministic)
     y = torch.zeros(n * 32, dtype=torch.float32, device=dev)
     f(_t(dev, ones), _t(dev, w.ravel()), _t(dev, cfg["x"].ravel()), y, *[_t(dev, c) for c in csf])
     torch.cuda.synchronize()
