@@ -26,9 +26,9 @@
 //      this partial tile (LDS float atomics run at a third of a lane per clock and compute unit
 //      on this chip, slower than atomics in memory).
 // A batch is a chain of dependent loads (batch record -> edge records -> rows of X and weights),
-// so the records run ahead of the arithmetic: batch records four batches ahead, edge records and
-// pair words three, rows of X and weights one; the loop body has no branch around a load, so the
-// compiler's wait counts leave the younger loads in flight.
+// so everything is requested two of the wavefront's batches before the step of the chain that
+// needs it, into registers that are never copied while a load is in flight (two sets, a loop
+// unrolled by two); the loop body has no branch around a load.
 // At the end the four partial tiles are added up: into the tile's rows of Y, each element once,
 // or -- for a unit that is a piece of a tile -- into the plan's memory for partial tiles.
 #include "rgms_f32_tiles.h"
@@ -295,7 +295,8 @@ __global__ __launch_bounds__(256) void f32_pack_w_kernel(const float* __restrict
 // block.  Offsets into X and the edge records are 32-bit byte offsets from scalar bases (the
 // launch checks that they fit).
 template <int KS, int NT>
-__global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(KS == 1 && NT == 2 ? 3 : 1, 3)))
+void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
                                                             const UnitF32* __restrict__ units,
                                                             const BatchF32* __restrict__ batches,
                                                             const uint32_t* __restrict__ pinfo,
@@ -376,55 +377,74 @@ __global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int 
   };
   auto load_pair = [&](const Batch& bt) { return pinfo[bt.pair_begin + (i < bt.npairs ? (uint32_t)i : 0u)]; };
 
-  // the pipeline: batch records four ahead, edge records and pair words three, rows of X one
-  Batch bt0 = scalars(raw_batch(b), b), bt1 = scalars(raw_batch(b + 4), b + 4), bt2 = scalars(raw_batch(b + 8), b + 8);
-  BatchF32 raw3 = raw_batch(b + 12);
-  EdgesG eg1 = load_edges(bt1), eg2 = load_edges(bt2);
-  uint32_t pw0 = load_pair(bt0), pw1 = load_pair(bt1), pw2 = load_pair(bt2);
-  RowsG rw0;
-  {
-    const EdgesG eg0 = load_edges(bt0);
-    rw0 = load_rows(eg0);
-  }
-
-  while (bt0.npairs > 0) {  // the same for every lane
-    // requests: the next batch's rows, this batch's W, the records further ahead
-    const RowsG rw1 = load_rows(eg1);
-    float4 wq[NT][KS][2];
-    const float4* wrel = Wp + (int64_t)bt0.rel * (NT * KS * 2 * 64) + lane;
+  auto load_w = [&](float4 (&wq)[NT][KS][2], int rel) {  // B operands of `rel`, in lane order
+    const float4* wrel = Wp + (int64_t)rel * (NT * KS * 2 * 64) + lane;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int s = 0; s < KS; ++s)
 #pragma unroll
         for (int c = 0; c < 2; ++c) wq[nt][s][c] = wrel[((nt * KS + s) * 2 + c) * 64];
-    const Batch bt3 = scalars(raw3, b + 12);
-    const BatchF32 raw4 = raw_batch(b + 16);
-    const EdgesG eg3 = load_edges(bt3);
-    const uint32_t pw3 = load_pair(bt3);
+  };
 
+  // The pipeline.  Everything a batch needs is requested two of the wavefront's batches ahead of
+  // its use -- the record of batch j + 6 (so that its scalars exist at j + 4), the edge records of
+  // j + 4 (so that the rows of X of j + 2 can be requested at j), the rows, pair words and W
+  // operands of j + 2 -- into two sets of registers, one for the even and one for the odd batches:
+  // a set's registers are reloaded right after their last use, nothing in flight is ever copied,
+  // and the loop is unrolled by two.
+  struct Stage {
+    RowsG rw;              // rows of X and weights of batch j
+    EdgesG eg;             // edge records of batch j + 2
+    BatchF32 raw;          // record of batch j + 4
+    uint32_t pw;           // pair word of batch j
+    float4 wq[NT][KS][2];  // W operands of batch j
+  };
+  Batch bt0 = scalars(raw_batch(b), b), bt1 = scalars(raw_batch(b + 4), b + 4);
+  Batch bt2 = scalars(raw_batch(b + 8), b + 8), bt3 = scalars(raw_batch(b + 12), b + 12);
+  Stage even, odd;
+  even.raw = raw_batch(b + 16), odd.raw = raw_batch(b + 20);
+  even.eg = load_edges(bt2), odd.eg = load_edges(bt3);
+  even.pw = load_pair(bt0), odd.pw = load_pair(bt1);
+  load_w(even.wq, bt0.rel);
+  load_w(odd.wq, bt1.rel);
+  {
+    const EdgesG eg0 = load_edges(bt0), eg1 = load_edges(bt1);
+    even.rw = load_rows(eg0), odd.rw = load_rows(eg1);
+  }
+
+  auto batch = [&](Stage& st) {
     // 1. the weighted rows of this batch, into the edge tile.  Places behind the batch's last edge
     // get whatever was read: no pair reads them.  Chunks beyond feat_in are never written and stay
     // zero.
     if (chunk_live) {
 #pragma unroll
       for (int k = 0; k < NLOAD; ++k) {
-        const float w = rw0.w[k];
-        float4 v = rw0.x[k];
+        const float w = st.rw.w[k];
+        float4 v = st.rw.x[k];
         v.x *= w, v.y *= w, v.z *= w, v.w *= w;
         *reinterpret_cast<float4*>(et + (k * RPI + gr) * SS + 4 * gc) = v;
       }
     }
+    // requests for the batches to come
+    st.rw = load_rows(st.eg);
+    const Batch bt4 = scalars(st.raw, b + 16);
+    st.eg = load_edges(bt4);
+    st.raw = raw_batch(b + 24);
     // 2. the sums of the pairs, multiplying layout: lane (i, q) walks the edges of pair i; a lane
     // whose pair has fewer edges than the batch's longest reads the tile's row of zeros meanwhile
-    const int my_first = (int)((pw0 >> 16) & 255u), my_count = i < bt0.npairs ? (int)((pw0 >> 8) & 255u) : 0;
-    const int my_dl = (int)(pw0 & (kTileRows - 1));
+    const uint32_t pw = st.pw;
+    const int my_first = (int)((pw >> 16) & 255u), my_count = i < bt0.npairs ? (int)((pw >> 8) & 255u) : 0;
+    const int my_dl = (int)(pw & (kTileRows - 1));
     float4 sq[KS][2];
+    {  // every pair has a first edge; a lane without a pair takes the row of zeros
+      const float* row = et + (my_count > 0 ? my_first : EMAX) * SS + 8 * q;
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
+      for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int c = 0; c < 2; ++c) sq[s][c] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int t = 0; t < bt0.most; ++t) {  // the same for every lane
+        for (int c = 0; c < 2; ++c) sq[s][c] = *reinterpret_cast<const float4*>(row + 32 * s + 4 * c);
+    }
+    for (int t = 1; t < bt0.most; ++t) {  // the same for every lane
       const float* row = et + (t < my_count ? my_first + t : EMAX) * SS + 8 * q;
 #pragma unroll
       for (int s = 0; s < KS; ++s)
@@ -444,12 +464,13 @@ __global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int 
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-          const float4 wk = wq[nt][s][c], sk = sq[s][c];
+          const float4 wk = st.wq[nt][s][c], sk = sq[s][c];
           acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sk.x, wk.x, acc[nt], 0, 0, 0);
           acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sk.y, wk.y, acc[nt], 0, 0, 0);
           acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sk.z, wk.z, acc[nt], 0, 0, 0);
           acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sk.w, wk.w, acc[nt], 0, 0, 0);
         }
+    load_w(st.wq, bt2.rel);
     // 4. acc[nt][v]: pair 4 q + v of the batch, output 16 nt + i, which lives at float NT i + nt of
     // its row of the partial tile: a lane's NT outputs are neighbours, one read and one write.
     // The pairs of a batch end in different rows (a row cut into pieces has at most its last,
@@ -471,11 +492,20 @@ __global__ __launch_bounds__(256) void rgms_f32_tile_kernel(int m, int fin, int 
         }
       }
     }
+    st.pw = load_pair(bt2);  // last: the old word's row number was in use until here
     b += 4;
-    bt0 = bt1, bt1 = bt2, bt2 = bt3, raw3 = raw4;
-    eg1 = eg2, eg2 = eg3;
-    pw0 = pw1, pw1 = pw2, pw2 = pw3;
-    rw0 = rw1;
+    bt0 = bt1, bt1 = bt2, bt2 = bt3, bt3 = bt4;  // scalars: copies wait for nothing
+  };
+  // (With the way out between the two halves, the compiler's wait counts at the top of a round are
+  // "everything requested in the round before has arrived".  Without it -- both batches run
+  // whether the second exists or not, and the requests of the prologue waited for once before the
+  // loop -- the counts leave two batches' worth of loads in flight, and the launch is slower: 139
+  // against 130 us on 100k nodes / 65 relations / 2M edges.  The loop is bound by instruction
+  // issue, not by the latency of its loads.)
+  while (bt0.npairs > 0) {  // the same for every lane
+    batch(even);
+    if (bt0.npairs == 0) break;
+    batch(odd);
   }
 
   __syncthreads();
