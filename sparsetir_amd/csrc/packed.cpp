@@ -220,11 +220,13 @@ struct PlanCache {
 PlanCache<stir_hyb_plan> g_hyb_plans(stir_hyb_plan_destroy);
 PlanCache<stir_rgms_plan> g_rgms_plans(stir_rgms_plan_destroy);
 PlanCache<stir_rgms_f32_plan> g_rgms_f32_plans(stir_rgms_f32_plan_destroy);
+PlanCache<stir_rgms_csf_f32_plan> g_rgms_csf_plans(stir_rgms_csf_f32_plan_destroy);  // only under the promise below
 
 // Promises of the caller for the plans made from now on.  Without the first, a cached plan holds
 // addresses and sizes only and every call reads the index arrays afresh, as the reference's built
 // operators do; with it, plans may keep what they derive from the contents of the index arrays
-// (the verdict that drops atomics and the slot lists of hyb, the edge index of RGMS).
+// (the verdict that drops atomics and the slot lists of hyb, the edge index of RGMS; the fp32 RGMS
+// then sums every tile of Y on chip in a fixed order instead of adding with atomics).
 bool g_static_structure = false;
 bool g_rgms_static_weights = false;
 
@@ -517,6 +519,10 @@ static int packed_rgms_any(const char* name, bool f32, TVMValue* v, int* tc, int
       if (stir_rgms_f32_plan_create(&plan, nb, rb.data(), cb.data(), groups.data(), Af.data(), Rk.data(), Ck.data(),
                                     Mk.data()))
         return forward(-1);
+      if (g_static_structure && stir_rgms_f32_plan_set_deterministic(plan, 1)) {
+        stir_rgms_f32_plan_destroy(plan);
+        return forward(-1);
+      }
       g_rgms_f32_plans.insert(key, plan);
     }
     return forward(stir_rgms_f32(plan, mm, nn, rr, (int32_t)fin, (int32_t)fout, (const float*)W.data,
@@ -556,6 +562,7 @@ int stir_packed_invalidate_plans(TVMValue*, int*, int n, TVMRetValueHandle, void
   g_hyb_plans.clear();
   g_rgms_plans.clear();
   g_rgms_f32_plans.clear();
+  g_rgms_csf_plans.clear();
   return 0;
 }
 
@@ -571,6 +578,8 @@ int stir_packed_static_structure(TVMValue* v, int* tc, int n, TVMRetValueHandle,
     // the cached plans were made under the other setting
     g_hyb_plans.clear();
     g_rgms_plans.clear();
+    g_rgms_f32_plans.clear();
+    g_rgms_csf_plans.clear();
   }
   g_static_structure = on != 0;
   return 0;
@@ -611,6 +620,24 @@ int stir_packed_rgms_csf(TVMValue* v, int* tc, int n, TVMRetValueHandle, void*) 
   if (!fits_i32(Y.len / fout) || !fits_i32(X.len / fin) || !fits_i32(R)) return packed_fail("%s: sizes exceed int32", a.fn);
   DeviceGuard g;
   if (g.enter(a.dev_id)) return forward(-1);
+  {
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    if (g_static_structure) {  // the plan keeps an edge index made from the four index arrays
+      HybKey key;
+      for (const Arr* x : {&A, &Pi, &Ii, &Pj, &Ij}) key.ptrs.push_back((uintptr_t)x->data);
+      for (int64_t x : {Ii.len, A.len, Y.len / fout, X.len / fin, R, (int64_t)a.dev_id}) key.nums.push_back(x);
+      stir_rgms_csf_f32_plan* plan = g_rgms_csf_plans.find(key);
+      if (!plan) {
+        if (stir_rgms_csf_f32_plan_create(&plan, Ii.len, A.len, (const float*)A.data, (const int32_t*)Pi.data,
+                                          (const int32_t*)Ii.data, (const int32_t*)Pj.data, (const int32_t*)Ij.data))
+          return forward(-1);
+        g_rgms_csf_plans.insert(key, plan);
+      }
+      return forward(stir_rgms_csf_f32_planned(plan, (int32_t)(Y.len / fout), (int32_t)(X.len / fin), (int32_t)R,
+                                               (int32_t)fin, (int32_t)fout, (const float*)W.data,
+                                               (const float*)X.data, (float*)Y.data, g_stream));
+    }
+  }
   return forward(stir_rgms_csf_f32((int32_t)(Y.len / fout), (int32_t)(X.len / fin), (int32_t)R, (int32_t)fin,
                                    (int32_t)fout, Ii.len, A.len, (const float*)A.data, (const float*)W.data,
                                    (const float*)X.data, (float*)Y.data, (const int32_t*)Pi.data,

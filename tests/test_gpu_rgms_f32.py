@@ -248,3 +248,68 @@ def test_rgms_f32_tiled_rejects_bad_ids(dev):
     bad_rows[7] = n + 5
     with pytest.raises(SparseTIRError, match="row id"):
         f(a, w, x, torch.zeros(n * fout, device=dev), _t(dev, csf[0]), _t(dev, bad_rows), _t(dev, csf[2]), _t(dev, csf[3]))
+
+
+def test_packed_rgms_f32_static_structure_sums_in_tiles(dev):
+    """Under "sparsetir.static_structure"(1) the PackedFuncs sparsetir.rgms_f32 and
+    sparsetir.rgms_csf keep an edge index per set of arrays and sum every tile of Y on chip: the
+    closed form within tolerance, the same bits on every call, one plan per function for any
+    number of calls; edge values rewritten in place are read by the next call; without the promise
+    the same calls build no index."""
+    from sparsetir_amd import packed
+    promise = packed.get_global_func("sparsetir.static_structure")
+    inval = packed.get_global_func("sparsetir.invalidate_plans")
+    R, n, fin, fout, group, buckets = 7, 3000, 32, 32, 32, [1, 2, 4, 8, 16]
+    csf = random_csf(R, n, 40000, seed=77)
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((n, fin), dtype=np.float32)
+    w = rng.standard_normal((R, fout, fin), dtype=np.float32) * 0.1
+    a = 0.5 + rng.random(len(csf[3]), dtype=np.float32)
+    want, scale = _closed_forms(csf, a, x, w, n)
+    ones = np.ones(len(csf[3]), np.float32)
+    want1, scale1 = _closed_forms(csf, ones, x, w, n)
+    rb = [group // b for b in buckets]
+    iptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [_t(dev, mask[k].astype(np.float32).ravel()), _t(dev, rows[k].ravel()), _t(dev, cols[k].ravel())]
+        mids.append(_t(dev, np.repeat(np.arange(R, dtype=np.int32), np.diff(iptr[k]))))
+    assert sum(c.size for c in cols) >= 8192
+    dw, dx, da = _t(dev, w.ravel()), _t(dev, x.ravel()), _t(dev, a)
+    d_csf = [_t(dev, c) for c in csf]
+    f_ell, f_csf = packed.get_global_func("sparsetir.rgms_f32"), packed.get_global_func("sparsetir.rgms_csf")
+
+    def run_ell():
+        y = torch.zeros(n * fout, device=dev)
+        f_ell(dw, dx, y, *triples, *mids, fin, fout)
+        torch.cuda.synchronize()
+        return y
+
+    def run_csf():
+        y = torch.zeros(n * fout, device=dev)
+        f_csf(da, dw, dx, y, *d_csf, fin, fout)
+        torch.cuda.synchronize()
+        return y
+
+    inval()
+    promise(1)
+    try:
+        before = packed.plan_builds()
+        e0, e1, c0, c1 = run_ell(), run_ell(), run_csf(), run_csf()
+        assert packed.plan_builds() == before + 2
+        assert torch.equal(e0, e1) and torch.equal(c0, c1)
+        _check(e0.cpu().numpy().reshape(n, fout), want1, scale1, oracle.rgms_csf_f32(ones, w, x, *csf, n), "packed ell3d")
+        _check(c0.cpu().numpy().reshape(n, fout), want, scale, oracle.rgms_csf_f32(a, w, x, *csf, n), "packed csf")
+        da.mul_(2.0)
+        c2 = run_csf()
+        assert np.all(np.abs(c2.cpu().numpy().reshape(n, fout) - 2 * want) <= 2e-5 * np.abs(want) + 2e-5 * scale + 1e-30)
+        assert packed.plan_builds() == before + 2
+        da.mul_(0.5)
+        promise(0)  # the plans made under the promise go away
+        before = packed.plan_builds()
+        c3 = run_csf()
+        assert packed.plan_builds() == before  # stateless again
+        _check(c3.cpu().numpy().reshape(n, fout), want, scale, oracle.rgms_csf_f32(a, w, x, *csf, n), "packed csf, atomics")
+    finally:
+        promise(0)
+        inval()
