@@ -1,5 +1,6 @@
 """The entry point that allocates nothing (stir_hyb_spmm_f32_noalloc) against the plan-based pair
-it is a variant of (stir_hyb_plan_create + stir_hyb_spmm_f32), both called through the C ABI.
+it is a variant of (stir_hyb_plan_create + stir_hyb_spmm_f32), both called through the C ABI, and
+against the oracle's CSR product of the matrix the format was made from.
 
 Two calls in a row on one GPU, the second with a smaller input, so that descriptors left in the
 library's fixed device array by the first call would show.  Buckets that store (one partition,
@@ -12,6 +13,7 @@ import numpy as np
 import pytest
 import torch
 
+import oracle
 import sparsetir_amd as st
 from sparsetir_amd import _lib
 from helpers import random_csr
@@ -86,6 +88,9 @@ def test_noalloc_matches_plan_based_entry_point_twice(dev, parts, buckets, feat)
         x = torch.randn(n * feat, device=dev, generator=torch.Generator(device=dev).manual_seed(call))
         got, want = _both_ways(dev, m, n, feat, parts, buckets, A, R, C, nrows, x)
         _compare(dev, got, want, m, feat, indptr, vals, x, R, nrows, parts, len(buckets), f"call {call}")
+        # and the oracle: C = A @ X from the CSR arrays the decomposition was made from
+        ref = torch.from_numpy(oracle.csrmm(vals.cpu().numpy(), x.cpu().numpy(), indptr, indices, feat)).to(dev)
+        _compare(dev, got, ref.reshape(-1), m, feat, indptr, vals, x, R, nrows, 0, len(buckets), f"call {call} vs oracle")
 
 
 def test_noalloc_rejects_more_buckets_than_the_fixed_array_holds(dev):
