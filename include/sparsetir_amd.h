@@ -327,11 +327,13 @@ int stir_tc_spmm_f16(int32_t out_dtype, int32_t mb, int32_t tile_size, int32_t g
  * first, cut into pieces of at most 128 steps.  stir_tc_spmm_f16_planned then takes the arguments
  * of stir_tc_spmm_f16: the short tiles as there, then one workgroup per
  * piece -- none is started only to find its tile short, and the hub tiles of a power-law graph
- * are spread over many compute units from the start of the launch -- and, for the tiles of several
- * pieces, a launch that adds their fp32 partial tiles and rounds once (the sums are those of
- * stir_tc_spmm_f16 up to the order of the fp32 additions).  The partial tiles live in memory the
- * plan owns, sized by the first launch with a given feat (that launch allocates): launches with
- * one plan must not overlap on the GPU.  The plan describes the contents of d_indptr at its
+ * are spread over many compute units from the start of the launch.  The pieces of a tile leave
+ * fp32 partial tiles, and the workgroup that finishes last among them (a counter per tile and
+ * feature tile, which it sets back to zero) adds them in piece order and rounds once: no atomics
+ * on C, the same bits on every run (the sums are those of stir_tc_spmm_f16 up to the order of
+ * the fp32 additions).  The partial tiles and counters live in memory the plan owns, sized by the
+ * first launch with a given feat (that launch allocates): launches with one plan must not overlap
+ * on the GPU.  The plan describes the contents of d_indptr at its
  * creation; make a new one when they change.  It belongs to the device that was current at
  * its creation, and a launch with another device current is refused.
  */

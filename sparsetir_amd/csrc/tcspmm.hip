@@ -421,16 +421,29 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_long_kernel(int feat, 
 // hub tiles of a power-law graph are spread over many compute units from the start of the launch
 // and no workgroup is started only to find its tile short.  A tile that is one piece is written
 // as fp16 by its workgroup; the pieces of a longer tile leave fp32 partial tiles in the plan's
-// scratch memory, which tcspmm_pieces_sum_kernel adds up and rounds once.
+// scratch memory, and the workgroup that finishes last among the pieces of a tile (per feature
+// tile: a counter in device memory, which that workgroup sets back to zero) adds them up in piece
+// order and rounds once -- no launch of its own for the sums, and the same bits whichever
+// workgroup comes last.  The partial tiles are written and read with device-coherent accesses
+// (they pass the XCD's L2), so that no workgroup has to write back or invalidate a whole L2 --
+// which a release or acquire at device scope does, and which costs more than the extra launch.
 constexpr int kPieceSteps = 128;
 
 struct TcPiece {
   int32_t tile, step_begin, step_end;
-  int32_t slot;  // partial tile in the scratch memory, or -1: the piece is the whole tile
+  int32_t slot;        // partial tile in the scratch memory, or -1: the piece is the whole tile
+  int32_t first_slot;  // of the tile's pieces
+  int32_t pieces;      // of the tile
+  int32_t multi;       // number of the tile among the tiles of several pieces
+  int32_t pad;
 };
-struct TcMulti {
-  int32_t tile, first_slot, pieces, pad;
-};
+
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 template <int T, int NTL, int OUT>
 __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat, int f_tiles,
@@ -438,12 +451,15 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat
                                                                         const uint16_t* __restrict__ A,
                                                                         const uint16_t* __restrict__ B,
                                                                         void* __restrict__ C,
-                                                                        float* __restrict__ scratch,
+                                                                        float* scratch, uint32_t* arrived,
                                                                         const int32_t* __restrict__ indptr,
                                                                         const int32_t* __restrict__ indices) {
   extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+  __shared__ int last_of_tile;
+  constexpr int TF = 32 * NTL;
   const TcPiece pc = pieces[blockIdx.x / f_tiles];
-  const int f0 = (int)(blockIdx.x % f_tiles) * (32 * NTL);
+  const int f_tile = (int)(blockIdx.x % f_tiles);
+  const int f0 = f_tile * TF;
   const int64_t io = pc.tile;
   // a plan made from other contents of indptr: stay inside the tile as it is now
   const int s_end = min(pc.step_end, tile_steps(indptr, io));
@@ -458,43 +474,55 @@ __global__ __launch_bounds__(64 * (32 / NTL)) void tcspmm_pieces_kernel(int feat
                                   static_cast<uint16_t*>(C)[off] = __builtin_bit_cast(uint16_t, hv);
                                 }
                               });
-  } else {
-    float* part = scratch + (int64_t)pc.slot * T * feat;
-    tcspmm_long_steps<T, NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
-                              [&](int row, int fcol, float sum) { part[(int64_t)row * feat + fcol] = sum; });
+    return;
   }
-}
-
-// C[tile] = fp16(sum of the tile's partial tiles); grid (tiles cut into several pieces) x
-// (tile * feat / 1024): a thread owns four consecutive elements (feat is a multiple of 32)
-template <int OUT>
-__global__ __launch_bounds__(256) void tcspmm_pieces_sum_kernel(int tile, int feat, int chunks,
-                                                                const TcMulti* __restrict__ multi,
-                                                                const float* __restrict__ scratch,
-                                                                void* __restrict__ C) {
-  const TcMulti mt = multi[blockIdx.x / chunks];
-  const int64_t elems = (int64_t)tile * feat;
-  const int64_t e = ((int64_t)(blockIdx.x % chunks) * 256 + threadIdx.x) * 4;
-  if (e >= elems) return;
-  const float* part = scratch + (int64_t)mt.first_slot * elems + e;
-  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int p0 = 0; p0 < mt.pieces; p0 += 4) {
-    float4 x[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-      x[u] = p0 + u < mt.pieces ? *reinterpret_cast<const float4*>(part + (p0 + u) * elems)
-                                : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) sum.x += x[u].x, sum.y += x[u].y, sum.z += x[u].z, sum.w += x[u].w;
+  const int64_t elems = (int64_t)T * feat;
+  float* part = scratch + (int64_t)pc.slot * elems;
+  tcspmm_long_steps<T, NTL>(lds, feat, io, f0, pc.step_begin, s_end, A, B, indptr, indices,
+                            [&](int row, int fcol, float sum) { coherent_store(part + (int64_t)row * feat + fcol, sum); });
+  // Every wavefront waits until its stores have arrived, then one thread counts the workgroup
+  // in: whoever counts last finds the partial tiles of all the others in memory.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t* counter = arrived + (int64_t)pc.multi * f_tiles + f_tile;
+    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = before + 1 == (uint32_t)pc.pieces;
+    if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    last_of_tile = last;
   }
-  if constexpr (OUT == 1) {
-    *reinterpret_cast<float4*>(static_cast<float*>(C) + (int64_t)mt.tile * elems + e) = sum;
-  } else {
-    const _Float16 h0 = (_Float16)sum.x, h1 = (_Float16)sum.y, h2 = (_Float16)sum.z, h3 = (_Float16)sum.w;
-    uint2 out;
-    out.x = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
-    out.y = (uint32_t)__builtin_bit_cast(uint16_t, h2) | ((uint32_t)__builtin_bit_cast(uint16_t, h3) << 16);
-    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(C) + (int64_t)mt.tile * elems + e) = out;
+  __syncthreads();
+  if (!last_of_tile) return;
+  // C[tile, f0 .. f0 + TF) = the partial tiles added in piece order, rounded once; four
+  // consecutive features per thread (feat is a multiple of 32)
+  const float* first = scratch + (int64_t)pc.first_slot * elems;
+  for (int w = threadIdx.x; w < T * (TF / 4); w += 64 * (32 / NTL)) {
+    const int row = w / (TF / 4), fcol = f0 + (w % (TF / 4)) * 4;
+    if (fcol >= feat) continue;
+    const int64_t e = (int64_t)row * feat + fcol;
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int p0 = 0; p0 < pc.pieces; p0 += 4) {
+      float4 x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        x[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (p0 + u < pc.pieces) {
+          const float* at = first + (p0 + u) * elems + e;
+          x[u] = make_float4(coherent_load(at), coherent_load(at + 1), coherent_load(at + 2), coherent_load(at + 3));
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) sum.x += x[u].x, sum.y += x[u].y, sum.z += x[u].z, sum.w += x[u].w;
+    }
+    if constexpr (OUT == 1) {
+      *reinterpret_cast<float4*>(static_cast<float*>(C) + io * elems + e) = sum;
+    } else {
+      const _Float16 h0 = (_Float16)sum.x, h1 = (_Float16)sum.y, h2 = (_Float16)sum.z, h3 = (_Float16)sum.w;
+      uint2 out;
+      out.x = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+      out.y = (uint32_t)__builtin_bit_cast(uint16_t, h2) | ((uint32_t)__builtin_bit_cast(uint16_t, h3) << 16);
+      *reinterpret_cast<uint2*>(static_cast<uint16_t*>(C) + io * elems + e) = out;
+    }
   }
 }
 
@@ -542,9 +570,9 @@ int launch_unplanned(bool out32, int32_t mb, int32_t feat, const uint16_t* A, co
 }
 
 template <int T>
-int launch_planned(bool out32, int32_t mb, int32_t feat, int64_t n_pieces, int64_t n_multi, const TcPiece* d_pieces,
-                   const TcMulti* d_multi, float* d_scratch, const uint16_t* A, const uint16_t* B, void* d_C,
-                   const int32_t* d_indptr, const int32_t* d_indices, hipStream_t st) {
+int launch_planned(bool out32, int32_t mb, int32_t feat, int64_t n_pieces, const TcPiece* d_pieces, float* d_scratch,
+                   uint32_t* d_arrived, const uint16_t* A, const uint16_t* B, void* d_C, const int32_t* d_indptr,
+                   const int32_t* d_indices, hipStream_t st) {
   const int f_tiles = (int)stir::ceil_div(feat, kTileF);
   const int64_t blocks = (int64_t)mb * f_tiles;
   STIR_REQUIRE(blocks < (int64_t(1) << 31), "tc_spmm: too many tiles for one launch");
@@ -562,20 +590,12 @@ int launch_planned(bool out32, int32_t mb, int32_t feat, int64_t n_pieces, int64
   STIR_REQUIRE(long_blocks < (int64_t(1) << 31), "tc_spmm: too many pieces for one launch");
   if (out32)
     hipLaunchKernelGGL((tcspmm_pieces_kernel<T, kLongNT, 1>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
-                       kLongLds, st, feat, long_f_tiles, d_pieces, A, B, d_C, d_scratch, d_indptr, d_indices);
+                       kLongLds, st, feat, long_f_tiles, d_pieces, A, B, d_C, d_scratch, d_arrived, d_indptr,
+                       d_indices);
   else
     hipLaunchKernelGGL((tcspmm_pieces_kernel<T, kLongNT, 0>), dim3((unsigned)long_blocks), dim3(64 * kLongWaves),
-                       kLongLds, st, feat, long_f_tiles, d_pieces, A, B, d_C, d_scratch, d_indptr, d_indices);
-  STIR_LAUNCH_CHECK();
-  if (n_multi == 0) return 0;
-  const int chunks = (int)stir::ceil_div((int64_t)T * feat, 1024);
-  STIR_REQUIRE(n_multi * chunks < (int64_t(1) << 31), "tc_spmm: too many partial tiles for one launch");
-  if (out32)
-    hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<1>, dim3((unsigned)(n_multi * chunks)), dim3(256), 0, st, T, feat,
-                       chunks, d_multi, d_scratch, d_C);
-  else
-    hipLaunchKernelGGL(tcspmm_pieces_sum_kernel<0>, dim3((unsigned)(n_multi * chunks)), dim3(256), 0, st, T, feat,
-                       chunks, d_multi, d_scratch, d_C);
+                       kLongLds, st, feat, long_f_tiles, d_pieces, A, B, d_C, d_scratch, d_arrived, d_indptr,
+                       d_indices);
   STIR_LAUNCH_CHECK();
   return 0;
 }
@@ -603,15 +623,18 @@ struct stir_tc_plan {
   int device = 0;
   int64_t n_pieces = 0, n_multi = 0, slots = 0;
   TcPiece* d_pieces = nullptr;
-  TcMulti* d_multi = nullptr;
   float* d_scratch = nullptr;  // slots x 32 x feat floats, grown by the launch that needs more
   size_t scratch_bytes = 0;
+  // per tile of several pieces and feature tile: the pieces that have finished in the running
+  // launch; zero between launches (the workgroup that counts last clears its counter)
+  uint32_t* d_arrived = nullptr;
+  size_t arrived_count = 0;
 };
 
 extern "C" int stir_tc_plan_destroy(stir_tc_plan* plan) {
   if (!plan) return 0;
   if (plan->d_pieces) (void)hipFree(plan->d_pieces);
-  if (plan->d_multi) (void)hipFree(plan->d_multi);
+  if (plan->d_arrived) (void)hipFree(plan->d_arrived);
   if (plan->d_scratch) (void)hipFree(plan->d_scratch);
   delete plan;
   return 0;
@@ -636,33 +659,27 @@ extern "C" int stir_tc_plan_create(stir_tc_plan** plan, int32_t mb, const int32_
   std::stable_sort(longs.begin(), longs.end(),
                    [](const std::pair<int32_t, int32_t>& a, const std::pair<int32_t, int32_t>& b) { return a.first > b.first; });
   std::vector<TcPiece> pieces;
-  std::vector<TcMulti> multi;
-  int64_t slots = 0;
+  int64_t slots = 0, n_multi = 0;
   for (const auto& lt : longs) {
     const int32_t steps = lt.first, io = lt.second;
     const int32_t n = (steps + kPieceSteps - 1) / kPieceSteps;  // pieces of equal length
     const int32_t len = (steps + n - 1) / n;
     STIR_REQUIRE(slots + n < (int64_t(1) << 31), "tc_plan_create: too many pieces");
-    if (n > 1) multi.push_back(TcMulti{io, (int32_t)slots, n, 0});
     for (int32_t p = 0; p < n; ++p)
-      pieces.push_back(TcPiece{io, p * len, std::min(steps, (p + 1) * len), n > 1 ? (int32_t)(slots + p) : -1});
-    if (n > 1) slots += n;
+      pieces.push_back(TcPiece{io, p * len, std::min(steps, (p + 1) * len), n > 1 ? (int32_t)(slots + p) : -1,
+                               (int32_t)slots, n, (int32_t)n_multi, 0});
+    if (n > 1) slots += n, ++n_multi;
   }
   stir_tc_plan* p = new stir_tc_plan();
   p->mb = mb;
   p->n_pieces = (int64_t)pieces.size();
-  p->n_multi = (int64_t)multi.size();
+  p->n_multi = n_multi;
   p->slots = slots;
   hipError_t e = hipGetDevice(&p->device);
   if (e == hipSuccess && !pieces.empty()) {
     e = hipMalloc(reinterpret_cast<void**>(&p->d_pieces), sizeof(TcPiece) * pieces.size());
     if (e == hipSuccess)
       e = hipMemcpyAsync(p->d_pieces, pieces.data(), sizeof(TcPiece) * pieces.size(), hipMemcpyHostToDevice, st);
-  }
-  if (e == hipSuccess && !multi.empty()) {
-    e = hipMalloc(reinterpret_cast<void**>(&p->d_multi), sizeof(TcMulti) * multi.size());
-    if (e == hipSuccess)
-      e = hipMemcpyAsync(p->d_multi, multi.data(), sizeof(TcMulti) * multi.size(), hipMemcpyHostToDevice, st);
   }
   if (e == hipSuccess) e = hipStreamSynchronize(st);  // the host vectors go away
   if (e != hipSuccess) {
@@ -701,15 +718,24 @@ extern "C" int stir_tc_spmm_f16_planned(stir_tc_plan* plan, int32_t out_dtype, i
     STIR_HIP(hipMalloc(reinterpret_cast<void**>(&plan->d_scratch), need));
     plan->scratch_bytes = need;
   }
+  const size_t counters = size_t(plan->n_multi) * size_t(stir::ceil_div(feat, kLongTF));
+  if (counters > plan->arrived_count) {
+    if (plan->d_arrived) STIR_HIP(hipFree(plan->d_arrived));
+    plan->d_arrived = nullptr;
+    plan->arrived_count = 0;
+    STIR_HIP(hipMalloc(reinterpret_cast<void**>(&plan->d_arrived), counters * sizeof(uint32_t)));
+    STIR_HIP(hipMemsetAsync(plan->d_arrived, 0, counters * sizeof(uint32_t), st));
+    plan->arrived_count = counters;
+  }
   switch (tile_size) {
     case 8:
-      return launch_planned<8>(out32, mb, feat, plan->n_pieces, plan->n_multi, plan->d_pieces, plan->d_multi,
-                               plan->d_scratch, A, B, d_C, d_indptr, d_indices, st);
+      return launch_planned<8>(out32, mb, feat, plan->n_pieces, plan->d_pieces, plan->d_scratch, plan->d_arrived, A, B,
+                               d_C, d_indptr, d_indices, st);
     case 16:
-      return launch_planned<16>(out32, mb, feat, plan->n_pieces, plan->n_multi, plan->d_pieces, plan->d_multi,
-                                plan->d_scratch, A, B, d_C, d_indptr, d_indices, st);
+      return launch_planned<16>(out32, mb, feat, plan->n_pieces, plan->d_pieces, plan->d_scratch, plan->d_arrived, A,
+                                B, d_C, d_indptr, d_indices, st);
     default:
-      return launch_planned<32>(out32, mb, feat, plan->n_pieces, plan->n_multi, plan->d_pieces, plan->d_multi,
-                                plan->d_scratch, A, B, d_C, d_indptr, d_indices, st);
+      return launch_planned<32>(out32, mb, feat, plan->n_pieces, plan->d_pieces, plan->d_scratch, plan->d_arrived, A,
+                                B, d_C, d_indptr, d_indices, st);
   }
 }
