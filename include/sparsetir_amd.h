@@ -431,7 +431,7 @@ int stir_rgms_f32(const stir_rgms_f32_plan* plan, int32_t m, int32_t n, int32_t 
  * 64-row tile of Y, relation, row; it allocates and synchronises the stream, later launches only
  * rewrite a packed copy of W held by the plan; the index arrays must not change afterwards, the
  * weights may) and every tile of Y is summed on chip in a fixed order and written once, without
- * atomics: 140 us against 159 us on 100k nodes, 65 relations, 2M edges.  Inputs outside these
+ * atomics: 134 us against 159 us on 100k nodes, 65 relations, 2M edges.  Inputs outside these
  * limits, or whose index would not fit its 64-bit sort keys, run the atomic kernels.
  * A plan in this mode serves one call at a time.
  */
@@ -454,7 +454,7 @@ int stir_rgms_csf_f32(int32_t m, int32_t n, int32_t num_rels, int32_t feat_in, i
 
 /*
  * The same operator without atomics (no counterpart in the reference): sums that come out the
- * same, bit for bit, on every run, and faster than stir_rgms_csf_f32 (131 against 159 us on 100k
+ * same, bit for bit, on every run, and faster than stir_rgms_csf_f32 (122 against 159 us on 100k
  * nodes, 65 relations, 2M edges).  The plan keeps the pointers of the five arrays; from 8192 edges
  * on, with feat_in and feat_out of at most 64, its first launch builds the edge index described
  * at stir_rgms_f32_plan_set_deterministic from the four index arrays (they must not change

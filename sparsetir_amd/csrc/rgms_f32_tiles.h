@@ -5,8 +5,9 @@
 // 64 rows, relation, destination row); runs of equal key are the (relation, row) pairs, whose
 // weighted sums of X rows meet the relation's W on the matrix cores 16 pairs at a time
 // (v_mfma_f32_16x16x4_f32), and the products are added into a partial tile in LDS.  Tiles with
-// many more edges than the average are cut into pieces whose partial tiles a second launch adds
-// in a fixed order: the result does not depend on the order in which wavefronts run.
+// many more edges than the average are cut into pieces, and so are the few tiles beyond whole
+// rounds of resident workgroups; the piece of a tile that finishes last adds the pieces' partial
+// tiles in a fixed order: the result does not depend on the order in which wavefronts run.
 #pragma once
 #include <cstdint>
 #include <vector>
@@ -43,8 +44,8 @@ struct F32TileIndex {
   void* d_edges = nullptr;     // edges x 16 bytes, sorted
   void* d_pairs = nullptr;     // pairs x 4 bytes, sorted: row in tile | edges << 8 | first edge in its batch << 16
   void* d_batches = nullptr;   // batches x 16 bytes: up to 16 pairs and emax edges of one (tile, relation) each
-  void* d_units = nullptr;     // units x 16 bytes: a tile or a piece of one, as a range of batches; longest first
-  void* d_multi = nullptr;     // the tiles cut into several units
+  void* d_units = nullptr;     // units x 32 bytes: a tile or a piece of one, as a range of batches; longest first
+  void* d_arrived = nullptr;   // a counter per tile cut into several units (`multi` of them), zero between launches
   void* d_partials = nullptr;  // their partial tiles, rewritten by every launch
   size_t partial_bytes = 0;
   void* d_wpack = nullptr;     // W in the multiply's operand order, rewritten by every launch

@@ -6,8 +6,8 @@
 // into pieces of at most EMAX = 32 / KS edges (a second key: key << 20 | position in the run /
 // EMAX, run-length encoded).  The pairs of one (tile, relation) run are cut into batches of at
 // most 16 pairs and at most EMAX edges, listed per tile; a tile with many more batches than the
-// average is cut into several units, whose partial tiles go to memory of the plan and are added
-// up, in order, by a second small launch.
+// average is cut into several units, whose partial tiles go to memory of the plan; the unit of a
+// tile that finishes last adds them up, in the order of the units.
 // An edge record holds the source row and the address of the edge's weight (weights are read at
 // every launch); a pair is one word: row inside the tile, edges, first edge inside its batch.
 //
@@ -30,7 +30,11 @@
 // needs it, into registers that are never copied while a load is in flight (two sets, a loop
 // unrolled by two); the loop body has no branch around a load.
 // At the end the four partial tiles are added up: into the tile's rows of Y, each element once,
-// or -- for a unit that is a piece of a tile -- into the plan's memory for partial tiles.
+// or -- for a unit that is a piece of a tile -- into the plan's memory for partial tiles, with
+// device-coherent stores.  Such a unit then counts itself in (a counter per cut tile); the one
+// that counts last reads the partial tiles of all, coherently, adds them in unit order into Y and
+// sets the counter back to zero: no second launch, no fence that writes back or invalidates a
+// whole L2, and the same bits whichever unit comes last.
 #include "rgms_f32_tiles.h"
 
 #include <algorithm>
@@ -58,10 +62,9 @@ struct alignas(16) UnitF32 {
   int32_t tile;
   int32_t batch_begin, batch_end;
   int32_t partial;  // -1: the unit is a whole tile and adds to Y; else its place among the partial tiles
-};
-
-struct alignas(16) MultiF32 {  // a tile cut into several units
-  int32_t tile, first_partial, pieces, pad;
+  // of a unit that is a piece of a tile: the first partial tile of the tile, its pieces, and its
+  // number among the cut tiles (its counter)
+  int32_t first_partial, pieces, cut_tile, pad;
 };
 
 struct alignas(16) DevBucketF32 {
@@ -303,7 +306,7 @@ void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
                                                             const EdgeF32* __restrict__ edges,
                                                             const float4* __restrict__ Wp,
                                                             const float* __restrict__ X, float* __restrict__ Y,
-                                                            float* __restrict__ partials) {
+                                                            float* partials, uint32_t* arrived) {
   constexpr int FO = 16 * NT;      // floats per row of a partial tile
   constexpr int CPR = 8 * KS;      // lanes (16-byte chunks) per gathered row
   constexpr int RPI = 64 / CPR;    // rows per load instruction
@@ -314,6 +317,7 @@ void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
   static_assert(NT == 2 || NT == 4, "a lane's outputs are one 8- or 16-byte word of the partial tile");
   __shared__ __attribute__((aligned(16))) float ytile[4][kTileRows * FO];
   __shared__ __attribute__((aligned(16))) float etile[4][(EMAX + 1) * SS];  // the last row stays zero
+  __shared__ int last_of_tile;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i = lane & 15, q = lane >> 4;      // multiplying
@@ -510,6 +514,7 @@ void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
 
   __syncthreads();
   const int64_t row0 = (int64_t)u.tile * kTileRows;
+  const int64_t stride = (int64_t)kTileRows * fout;
   for (int e = tid; e < kTileRows * fout; e += 256) {
     const int r = e / fout, c = e - r * fout;
     if (row0 + r >= m) break;
@@ -518,22 +523,28 @@ void rgms_f32_tile_kernel(int m, int fin, int fout, int total_batches,
     if (u.partial < 0)
       Y[(row0 + r) * fout + c] += sum;
     else
-      partials[(int64_t)u.partial * (kTileRows * fout) + e] = sum;
+      __hip_atomic_store(partials + u.partial * stride + e, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-}
-
-// The tiles that were cut into several units: their partial tiles, in the order of the units, are
-// added to Y.  One workgroup per such tile.
-__global__ __launch_bounds__(256) void f32_sum_partials_kernel(const MultiF32* __restrict__ multi, int m, int fout,
-                                                               const float* __restrict__ partials,
-                                                               float* __restrict__ Y) {
-  const MultiF32 t = multi[blockIdx.x];
-  const int64_t row0 = (int64_t)t.tile * kTileRows;
-  const int64_t stride = (int64_t)kTileRows * fout;
-  for (int e = threadIdx.x; e < kTileRows * fout; e += 256) {
+  if (u.partial < 0) return;
+  // A piece of a tile.  Every wavefront waits until its stores have arrived, then one thread
+  // counts the unit in; the unit that counts last finds the partial tiles of all the others in
+  // memory (stores and loads of partial tiles pass the L2 of their XCD).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t* counter = arrived + u.cut_tile;
+    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = before + 1 == (uint32_t)u.pieces;
+    if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    last_of_tile = last;
+  }
+  __syncthreads();
+  if (!last_of_tile) return;
+  for (int e = tid; e < kTileRows * fout; e += 256) {
     if (row0 + e / fout >= m) break;
     float sum = 0.f;
-    for (int p = 0; p < t.pieces; ++p) sum += partials[(t.first_partial + p) * stride + e];
+    for (int p = 0; p < u.pieces; ++p)
+      sum += __hip_atomic_load(partials + (u.first_partial + p) * stride + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     Y[row0 * fout + e] += sum;
   }
 }
@@ -573,7 +584,7 @@ void f32_tiles_free(F32TileIndex& idx) {
   if (idx.d_pairs) (void)hipFree(idx.d_pairs);
   if (idx.d_batches) (void)hipFree(idx.d_batches);
   if (idx.d_units) (void)hipFree(idx.d_units);
-  if (idx.d_multi) (void)hipFree(idx.d_multi);
+  if (idx.d_arrived) (void)hipFree(idx.d_arrived);
   if (idx.d_partials) (void)hipFree(idx.d_partials);
   if (idx.d_wpack) (void)hipFree(idx.d_wpack);
   idx = F32TileIndex();
@@ -743,33 +754,66 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
   for (int64_t t = 0; t < tiles; ++t) busy += tb[(size_t)t + 1] > tb[(size_t)t];
   const int64_t cap = std::max<int64_t>(32, busy ? 2 * ceil_div((int64_t)total_batches, busy) : 32);
   std::vector<UnitF32> units;
-  std::vector<MultiF32> multi;
-  int64_t partial_tiles = 0;
+  int64_t partial_tiles = 0, cut_tiles = 0;
   for (int64_t t = 0; t < tiles; ++t) {
     const int64_t lo = tb[(size_t)t], hi = tb[(size_t)t + 1];
     if (hi <= lo) continue;
     if (2 * (hi - lo) <= 3 * cap) {
-      units.push_back(UnitF32{(int32_t)t, (int32_t)lo, (int32_t)hi, -1});
+      units.push_back(UnitF32{(int32_t)t, (int32_t)lo, (int32_t)hi, -1, 0, 0, 0, 0});
       continue;
     }
     const int64_t pieces = ceil_div(hi - lo, cap), len = ceil_div(hi - lo, pieces);
     STIR_REQUIRE(partial_tiles + pieces < (int64_t(1) << 31), "rgms_f32: too many partial tiles");
-    multi.push_back(MultiF32{(int32_t)t, (int32_t)partial_tiles, (int32_t)pieces, 0});
     for (int64_t p = 0; p < pieces; ++p)
       units.push_back(UnitF32{(int32_t)t, (int32_t)(lo + p * len), (int32_t)std::min(hi, lo + (p + 1) * len),
-                              (int32_t)(partial_tiles + p)});
-    partial_tiles += pieces;
+                              (int32_t)(partial_tiles + p), (int32_t)partial_tiles, (int32_t)pieces,
+                              (int32_t)cut_tiles, 0});
+    partial_tiles += pieces, ++cut_tiles;
   }
   // the longest units first
   std::stable_sort(units.begin(), units.end(), [](const UnitF32& a, const UnitF32& b) {
     return a.batch_end - a.batch_begin > b.batch_end - b.batch_begin;
   });
-  idx.units = (int64_t)units.size(), idx.multi = (int64_t)multi.size(), idx.partial_tiles = partial_tiles;
+  // A few units beyond whole rounds of resident workgroups (three per CU) would run when the
+  // others are done, each as slowly as a unit alone: those are cut into four pieces that run side
+  // by side (100k nodes, 65 relations, 2M edges: 1563 units on 768 resident workgroups, 27 beyond
+  // two rounds; 133 -> 127 us).  Only when they are few and of ordinary length.
+  {
+    int dev = 0, cus = 0;
+    STIR_HIP(hipGetDevice(&dev));
+    STIR_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int64_t resident = 3 * (int64_t)cus, count = (int64_t)units.size();
+    const int64_t beyond = resident > 0 ? count % resident : 0;
+    constexpr int64_t kPieces = 4;  // 3 to 4 measured best; 6 and 8 give the gain back
+    if (count > resident && beyond > 0 && 8 * beyond <= resident) {
+      const int64_t ordinary = total_batches / (2 * count);  // half the average length
+      std::vector<UnitF32> cut;
+      int64_t kept = 0;
+      for (int64_t k = count - beyond; k < count; ++k) {
+        const UnitF32 whole = units[(size_t)k];
+        const int64_t lo = whole.batch_begin, hi = whole.batch_end;
+        if (whole.partial >= 0 || hi - lo < std::max<int64_t>(ordinary, 2 * kPieces) ||
+            partial_tiles + kPieces >= (int64_t(1) << 31)) {
+          units[(size_t)(count - beyond + kept++)] = whole;
+          continue;
+        }
+        const int64_t len = ceil_div(hi - lo, kPieces);
+        for (int64_t p = 0; p < kPieces; ++p)
+          cut.push_back(UnitF32{whole.tile, (int32_t)(lo + p * len), (int32_t)std::min(hi, lo + (p + 1) * len),
+                                (int32_t)(partial_tiles + p), (int32_t)partial_tiles, (int32_t)kPieces,
+                                (int32_t)cut_tiles, 0});
+        partial_tiles += kPieces, ++cut_tiles;
+      }
+      units.resize((size_t)(count - beyond + kept));
+      units.insert(units.end(), cut.begin(), cut.end());
+    }
+  }
+  idx.units = (int64_t)units.size(), idx.multi = cut_tiles, idx.partial_tiles = partial_tiles;
   STIR_HIP(hipMalloc(&idx.d_units, sizeof(UnitF32) * std::max<size_t>(units.size(), 1)));
   STIR_HIP(hipMemcpy(idx.d_units, units.data(), sizeof(UnitF32) * units.size(), hipMemcpyHostToDevice));
-  if (!multi.empty()) {
-    STIR_HIP(hipMalloc(&idx.d_multi, sizeof(MultiF32) * multi.size()));
-    STIR_HIP(hipMemcpy(idx.d_multi, multi.data(), sizeof(MultiF32) * multi.size(), hipMemcpyHostToDevice));
+  if (cut_tiles > 0) {  // the counters of the cut tiles: zero between launches
+    STIR_HIP(hipMalloc(&idx.d_arrived, sizeof(uint32_t) * (size_t)cut_tiles));
+    STIR_HIP(hipMemset(idx.d_arrived, 0, sizeof(uint32_t) * (size_t)cut_tiles));
   }
   return 0;
 }
@@ -814,7 +858,8 @@ int f32_tiles_launch(F32TileIndex& idx, int32_t feat_in, int32_t feat_out, const
   float* partials = static_cast<float*>(idx.d_partials);
 #define STIR_F32_TILE(KS, NT)                                                                                   \
   hipLaunchKernelGGL((rgms_f32_tile_kernel<KS, NT>), grid, block, 0, stream, idx.m, feat_in, feat_out,          \
-                     (int)idx.batches, units, bts, pinfo, edges, wp, d_X, d_Y, partials)
+                     (int)idx.batches, units, bts, pinfo, edges, wp, d_X, d_Y, partials,                        \
+                     static_cast<uint32_t*>(idx.d_arrived))
   if (ks == 1) {
     if (nt == 2) STIR_F32_TILE(1, 2); else STIR_F32_TILE(1, 4);
   } else {
@@ -822,11 +867,6 @@ int f32_tiles_launch(F32TileIndex& idx, int32_t feat_in, int32_t feat_out, const
   }
 #undef STIR_F32_TILE
   STIR_LAUNCH_CHECK();
-  if (idx.multi > 0) {
-    hipLaunchKernelGGL(f32_sum_partials_kernel, dim3((unsigned)idx.multi), block, 0, stream,
-                       static_cast<const MultiF32*>(idx.d_multi), idx.m, feat_out, partials, d_Y);
-    STIR_LAUNCH_CHECK();
-  }
   return 0;
 }
 

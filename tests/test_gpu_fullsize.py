@@ -118,6 +118,53 @@ def test_config3_sddmm_edge_sample(dev, cfg3):
     assert bool(((out2 - ev * out).abs() <= 1e-6 * (ev * out).abs() + 1e-30).all())
 
 
+@pytest.mark.parametrize("deterministic", [True, False])
+def test_config5_rgms_f32_full(dev, deterministic):
+    """Config 5 in fp32, both front ends, against the float64 closed form (|err| <= 1e-5 of the
+    summed magnitudes).  The tile form at this size runs 1563 units, of which the few beyond whole
+    rounds of resident workgroups are cut into pieces whose partial tiles the last piece adds up:
+    two calls give the same bits."""
+    cfg = datasets.config5()
+    R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
+    csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(11)
+    a = (0.5 + rng.random(len(csf[3]))).astype(np.float32)
+    w = np.ascontiguousarray(cfg["w"].transpose(0, 2, 1))  # [R, fout, fin]
+    want = rgms_f64(*csf, a, cfg["x"], cfg["w"], n)
+    scale = rgms_f64(*csf, np.abs(a), np.abs(cfg["x"]), np.abs(cfg["w"]), n)
+    f = ops.build_rgms_csf(n, n, R, fin, fout, len(csf[1]), len(csf[3]), deterministic=deterministic)
+    d = [t(a), t(w.ravel()), t(cfg["x"].ravel())] + [t(c) for c in csf]
+    ys = [torch.zeros(n * fout, device=dev) for _ in range(2)]
+    for y in ys:
+        f(d[0], d[1], d[2], y, *d[3:])
+    torch.cuda.synchronize()
+    got = ys[0].cpu().numpy().reshape(n, fout)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-5 * scale + 1e-30)
+    if deterministic:
+        assert torch.equal(ys[0], ys[1])
+    # ELL3D buckets of the same graph (weights 1)
+    buckets, group = cfg["buckets"], 32
+    rb = [max(1, group // b) for b in buckets]
+    ptr, rows, cols, mask = st.csf_to_ell3d(*csf, rb, buckets)
+    triples, mids = [], []
+    for k in range(len(buckets)):
+        triples += [t(mask[k].astype(np.float32).ravel()), t(rows[k].ravel()), t(cols[k].ravel())]
+        mids.append(t(np.repeat(np.arange(R, dtype=np.int32), np.diff(ptr[k]))))
+    ones = np.ones(len(csf[3]), np.float32)
+    want1 = rgms_f64(*csf, ones, cfg["x"], cfg["w"], n)
+    scale1 = rgms_f64(*csf, ones, np.abs(cfg["x"]), np.abs(cfg["w"]), n)
+    g = ops.build_rgms_f32(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols], deterministic=deterministic)
+    ys = [torch.zeros(n * fout, device=dev) for _ in range(2)]
+    for y in ys:
+        g(d[1], d[2], y, *triples, *mids)
+    torch.cuda.synchronize()
+    got = ys[0].cpu().numpy().reshape(n, fout)
+    assert np.all(np.abs(got - want1) <= 1e-5 * np.abs(want1) + 1e-5 * scale1 + 1e-30)
+    if deterministic:
+        assert torch.equal(ys[0], ys[1])
+
+
 def test_config5_rgms_full(dev):
     cfg = datasets.config5()
     R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
