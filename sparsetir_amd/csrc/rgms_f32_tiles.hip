@@ -813,7 +813,8 @@ int build_index(F32TileIndex& idx, const F32Source& src, int32_t m, int32_t n, i
   STIR_HIP(hipMemcpy(idx.d_units, units.data(), sizeof(UnitF32) * units.size(), hipMemcpyHostToDevice));
   if (cut_tiles > 0) {  // the counters of the cut tiles: zero between launches
     STIR_HIP(hipMalloc(&idx.d_arrived, sizeof(uint32_t) * (size_t)cut_tiles));
-    STIR_HIP(hipMemset(idx.d_arrived, 0, sizeof(uint32_t) * (size_t)cut_tiles));
+    STIR_HIP(hipMemsetAsync(idx.d_arrived, 0, sizeof(uint32_t) * (size_t)cut_tiles, stream));
+    STIR_HIP(hipStreamSynchronize(stream));  // done before a launch on any stream
   }
   return 0;
 }
