@@ -225,8 +225,9 @@ PlanCache<stir_rgms_csf_f32_plan> g_rgms_csf_plans(stir_rgms_csf_f32_plan_destro
 // Promises of the caller for the plans made from now on.  Without the first, a cached plan holds
 // addresses and sizes only and every call reads the index arrays afresh, as the reference's built
 // operators do; with it, plans may keep what they derive from the contents of the index arrays
-// (the single-writer finding that drops atomics and the slot lists of hyb, the edge index of RGMS; the fp32 RGMS
-// then sums every tile of Y on chip in a fixed order instead of adding with atomics).
+// (the single-writer finding that drops atomics and the slot lists of hyb, the edge index of
+// RGMS; the fp32 RGMS then sums every tile of Y on chip in a fixed order instead of adding with
+// atomics).
 bool g_static_structure = false;
 bool g_rgms_static_weights = false;
 
