@@ -304,6 +304,27 @@ def test_hyb_spmm_caller_built_arrays_sharing_output_rows(dev, where):
     assert np.all(np.abs(got - want) <= 2 * RTOL * scale + 1e-30)
 
 
+def test_fused_launch_of_two_row_sums(dev):
+    """The reference's one numeric unit test (tests/python/sparsetir/test_horizontal_fuse.py:177-215):
+    two row-sum kernels, over a 128 x 128 and a 64 x 128 matrix, fused into one launch and compared
+    with numpy at rtol = atol = 1e-5.  Here the two "kernels" are two ELL buckets of one fused hyb
+    launch: the matrices' entries are the slot weights, every slot gathers a row of ones, and the
+    buckets write disjoint output rows (the second one, as the last bucket, by adding)."""
+    rng = np.random.default_rng(0)
+    x_np = rng.random((128, 128), dtype=np.float32)
+    y_np = rng.random((64, 128), dtype=np.float32)
+    feat, n = 4, 256
+    cols0 = np.tile(np.arange(128, dtype=np.int32), (128, 1))
+    y_pad = np.concatenate([y_np, np.zeros((64, 128), np.float32)], axis=1)  # width 256, half of it padding
+    cols1 = np.concatenate([np.tile(np.arange(128, 256, dtype=np.int32), (64, 1)), np.zeros((64, 128), np.int32)], axis=1)
+    triples = [(x_np, np.arange(128, dtype=np.int32), cols0), (y_pad, np.arange(128, 192, dtype=np.int32), cols1)]
+    ones = np.ones((n, feat), np.float32)
+    got, _ = _run_hyb(dev, 192, n, feat, 1, [128, 256], triples, ones)
+    for k in range(feat):
+        np.testing.assert_allclose(got[:128, k], x_np.sum(axis=-1), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(got[128:, k], y_np.sum(axis=-1), rtol=1e-5, atol=1e-5)
+
+
 def test_hyb_plan_rejects_row_ids_out_of_range(dev):
     m, n, feat, parts, buckets = 16, 32, 32, 2, [1, 2]
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
