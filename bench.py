@@ -251,6 +251,27 @@ def config2_sweep(torch, dev, ops, st, datasets, time_steps):
                               "hyb_alg_GBps": byts / dh / 1e9, "hyb_suggested_us": ds * 1e6,
                               "hyb_suggested_alg_GBps": byts / ds / 1e9,
                               "roofline": side_roofline("hbm", byts / dh / 1e9, f"config2/p{parts}/f{feat}")}
+    if not PROFILE_RUN:
+        # the same graph cut into 1 ... 16 column partitions (widths 1..512), as the plan runs them
+        # (phases up to 4 partitions, rows merged across partitions above), at 128 and 256 features
+        sweep = {}
+        for sp in (1, 2, 4, 8, 16):
+            prow, pcol, pmask = st.column_part_hyb(m, n, d_ptr, d_idx, sp, buckets)
+            ptriples, pnrows, slots = [], [], 0
+            for p in range(sp):
+                for b in range(len(buckets)):
+                    ptriples += [pmask[p][b].reshape(-1).float(), prow[p][b], pcol[p][b].reshape(-1)]
+                    pnrows.append(int(prow[p][b].shape[0]))
+                    slots += int(pcol[p][b].numel())
+            entry = {"slots_per_edge": slots / nnz, "ell_rows_per_row": sum(pnrows) / m}
+            for feat in (128, 256):
+                x = torch.randn(n * feat, device=dev)
+                c = torch.zeros(m * feat, device=dev)
+                f = ops.build_hyb_csrmm(m, n, feat, sp, buckets, pnrows)
+                _, dp, _ = time_steps(lambda: f(x, c, *ptriples), 50, 2, torch)
+                entry[f"feat{feat}_us"] = dp * 1e6
+            sweep[f"parts{sp}"] = entry
+        out["partition_sweep"] = sweep
     return out
 
 
