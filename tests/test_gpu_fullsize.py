@@ -123,7 +123,7 @@ def test_config5_rgms_f32_full(dev, deterministic):
     """Config 5 in fp32, both front ends, against the float64 closed form (|err| <= 1e-5 of the
     summed magnitudes).  The tile form at this size runs 1563 units, of which the few beyond whole
     rounds of resident workgroups are cut into pieces whose partial tiles the last piece adds up:
-    two calls give the same bits."""
+    eight calls back to back give the same bits."""
     cfg = datasets.config5()
     R, n, fin, fout = cfg["num_rels"], cfg["n"], cfg["feat_in"], cfg["feat_out"]
     csf = (cfg["indptr0"], cfg["indices0"], cfg["indptr1"], cfg["indices1"])
@@ -135,14 +135,14 @@ def test_config5_rgms_f32_full(dev, deterministic):
     scale = rgms_f64(*csf, np.abs(a), np.abs(cfg["x"]), np.abs(cfg["w"]), n)
     f = ops.build_rgms_csf(n, n, R, fin, fout, len(csf[1]), len(csf[3]), deterministic=deterministic)
     d = [t(a), t(w.ravel()), t(cfg["x"].ravel())] + [t(c) for c in csf]
-    ys = [torch.zeros(n * fout, device=dev) for _ in range(2)]
+    ys = [torch.zeros(n * fout, device=dev) for _ in range(8)]
     for y in ys:
         f(d[0], d[1], d[2], y, *d[3:])
     torch.cuda.synchronize()
     got = ys[0].cpu().numpy().reshape(n, fout)
     assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-5 * scale + 1e-30)
     if deterministic:
-        assert torch.equal(ys[0], ys[1])
+        assert all(torch.equal(ys[0], y) for y in ys[1:])
     # ELL3D buckets of the same graph (weights 1)
     buckets, group = cfg["buckets"], 32
     rb = [max(1, group // b) for b in buckets]
@@ -155,14 +155,14 @@ def test_config5_rgms_f32_full(dev, deterministic):
     want1 = rgms_f64(*csf, ones, cfg["x"], cfg["w"], n)
     scale1 = rgms_f64(*csf, ones, np.abs(cfg["x"]), np.abs(cfg["w"]), n)
     g = ops.build_rgms_f32(n, n, R, fin, fout, rb, buckets, [c.shape[0] for c in cols], deterministic=deterministic)
-    ys = [torch.zeros(n * fout, device=dev) for _ in range(2)]
+    ys = [torch.zeros(n * fout, device=dev) for _ in range(8)]
     for y in ys:
         g(d[1], d[2], y, *triples, *mids)
     torch.cuda.synchronize()
     got = ys[0].cpu().numpy().reshape(n, fout)
     assert np.all(np.abs(got - want1) <= 1e-5 * np.abs(want1) + 1e-5 * scale1 + 1e-30)
     if deterministic:
-        assert torch.equal(ys[0], ys[1])
+        assert all(torch.equal(ys[0], y) for y in ys[1:])
 
 
 def test_config5_rgms_full(dev):
