@@ -57,7 +57,8 @@ def build_probes():
     return PROBES_LIB
 
 
-PROBE_SYMBOLS = ("bench_probe_copy", "bench_probe_gather", "bench_probe_atomic_rows", "bench_probe_mfma_f16")
+PROBE_SYMBOLS = ("bench_probe_copy", "bench_probe_gather", "bench_probe_atomic_rows", "bench_probe_mfma_f16",
+                 "bench_probe_bsr_lds")
 
 
 def load_probes():
@@ -78,6 +79,7 @@ def load_probes():
     L.bench_probe_atomic_rows.restype, L.bench_probe_atomic_rows.argtypes = I32, [VP, I64, I64, VP]
     L.bench_probe_mfma_f16.restype = I32
     L.bench_probe_mfma_f16.argtypes = [I32, I32, I32, VP, ctypes.POINTER(ctypes.c_double), VP]
+    L.bench_probe_bsr_lds.restype, L.bench_probe_bsr_lds.argtypes = I32, [I32, VP, VP]
     return L
 
 
@@ -129,6 +131,9 @@ def parse():
     ap.add_argument("--profile", action="store_true",
                     help="few launches per kernel and no graph replays: for runs under rocprofv3 --pmc, "
                          "which serialises and slows every launch")
+    ap.add_argument("--lds-probes", action="store_true",
+                    help="only launch the LDS access-class kernels of the BSR tile body (bench_probes.hip), for a "
+                         "run under rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_ACTIVE_INST_LDS SQ_INSTS_LDS")
     ap.add_argument("--cpu-rows", type=int, default=10**9,
                     help="rows in the cpu_baseline sample (default: every row, about 6 s on one core)")
     return ap.parse_args()
@@ -655,6 +660,13 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     feat = args.feat
+    if args.lds_probes:
+        out = torch.zeros(512, dtype=torch.int32, device=dev)
+        rc = load_probes().bench_probe_bsr_lds(2000, ctypes.c_void_p(out.data_ptr()),
+                                               ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        print(json.dumps({"lds_probes": "launched" if rc == 0 else "failed"}))
+        sys.exit(0 if rc == 0 else 1)
 
     wl = hyb_workload(args, args.columns, torch, dev, st, datasets, ops)
     m, n, nnz = wl["m"], wl["n"], wl["nnz"]

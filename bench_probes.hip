@@ -99,9 +99,91 @@ __global__ __launch_bounds__(256) void probe_mfma_f16_kernel(int iters, float* _
   if (sum == 1.2345e38f) sink[0] = sum;
 }
 
+// ---- LDS access classes of the BSR tile body (sparsetir_amd/csrc/bsr.hip, bsr_tile), each in a
+// kernel of its own with the tile body's addresses, for SQ_LDS_BANK_CONFLICT / SQ_ACTIVE_INST_LDS /
+// SQ_INSTS_LDS: CLS 0 the 16-byte stores of the X tile, 1 the 8-byte stores of the A block, 2 the
+// 16-byte reads of the A fragment, 3 the transposing reads of X (ds_read_b64_tr_b16), 4 the 16-byte
+// stores of the A block of two 32-row slices.  VAR: the column swizzle of the X tile, 0 = column ^
+// 2 (k & 3), 1 = none, 2 = column ^ 4 (k & 3) (what the kernels use).  NT: 128 NT features per tile.
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t probe_u32x2 __attribute__((ext_vector_type(2)));
+typedef __fp16 probe_tr16x4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+
+template <int NT, int CLS, int VAR>
+__global__ __launch_bounds__(256) void probe_bsr_lds_kernel(int iters, uint32_t* out) {
+  constexpr int TF = 128 * NT, FCN = TF / 8, XB = 32 * TF * 2;
+  __shared__ __attribute__((aligned(16))) char lds[XB + 4096];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  for (int i = tid; i < (XB + 4096) / 4; i += 256) reinterpret_cast<uint32_t*>(lds)[i] = i;
+  __syncthreads();
+  auto swizzle = [](int c, int k) { return VAR == 0 ? c ^ (2 * k) : VAR == 1 ? c : c ^ (4 * k); };
+  uint32_t xdst[2 * NT];
+  for (int q = 0; q < 2 * NT; ++q) {
+    const int idx = 64 * (wave * 2 * NT + q) + lane, c = idx % FCN, kk = idx / FCN;
+    xdst[q] = (uint32_t)(((kk >> 2) * 4 * FCN + (kk & 3) * FCN + swizzle(c, kk & 3)) * 16);
+  }
+  const int sl = lane & 15, half16 = (lane >> 4) & 1;
+  uint32_t bread[NT];
+  for (int t = 0; t < NT; ++t) {
+    const int kr = sl >> 2, c = (wave * NT + t) * 4 + 2 * half16 + ((sl & 3) >> 1);
+    bread[t] = (uint32_t)(((2 * h) * 4 * FCN + kr * FCN + swizzle(c, kr)) * 16 + (sl & 1) * 8);
+  }
+  const uint32_t aread = XB + (h * 32 + n) * 16;
+  probe_u32x4 acc = {0, 0, 0, 0};
+  probe_u32x4 v = {(uint32_t)tid, 1, 2, 3};
+  for (int it = 0; it < iters; ++it) {
+    if (CLS == 0) {
+#pragma unroll
+      for (int q = 0; q < 2 * NT; ++q) *reinterpret_cast<probe_u32x4*>(lds + xdst[q]) = v;
+      v[0] += 1;
+    } else if (CLS == 1) {
+      *reinterpret_cast<probe_u32x2*>(lds + XB + tid * 8) = probe_u32x2{v[0], v[1]};
+      v[0] += 1;
+    } else if (CLS == 2) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m) acc += *reinterpret_cast<const probe_u32x4*>(lds + aread + m * 1024);
+    } else if (CLS == 3) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          typedef __attribute__((address_space(3))) probe_tr16x4 LdsTr;
+          const char* bp = lds + bread[t] + (4 * m) * FCN * 64;
+          const probe_tr16x4 t0 = __builtin_amdgcn_ds_read_tr16_b64_v4f16((LdsTr*)(bp));
+          const probe_tr16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4f16((LdsTr*)(bp + FCN * 64));
+          const probe_u32x2 lo = __builtin_bit_cast(probe_u32x2, t0), hi = __builtin_bit_cast(probe_u32x2, t1);
+          acc += probe_u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    } else {
+      *reinterpret_cast<probe_u32x4*>(lds + XB + tid * 16) = v;
+      v[0] += 1;
+    }
+    asm volatile("" ::: "memory");
+  }
+  __syncthreads();
+  if (acc[0] + acc[1] + acc[2] + acc[3] == 0x12345678u) out[tid] = acc[0] + lds[tid];
+  if (CLS < 2 || CLS == 4) out[256 + tid] = reinterpret_cast<uint32_t*>(lds)[tid * 3];
+}
+
 }  // namespace
 
 extern "C" {
+
+// Launches the LDS access-class kernels of the BSR tile body one after the other (256 workgroups
+// of 256 threads, `iters` rounds each; d_out: 512 words): for a counter run, see
+// probe_bsr_lds_kernel.  The order of the launches is the order of the template arguments below.
+int bench_probe_bsr_lds(int32_t iters, uint32_t* d_out, void* stream) {
+  if (!(iters > 0 && d_out)) return -1;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define BENCH_LDS(NT, CLS, VAR) \
+  hipLaunchKernelGGL((probe_bsr_lds_kernel<NT, CLS, VAR>), dim3(256), dim3(256), 0, st, iters, d_out)
+  BENCH_LDS(2, 0, 2); BENCH_LDS(2, 1, 2); BENCH_LDS(2, 2, 2); BENCH_LDS(2, 3, 2); BENCH_LDS(2, 4, 2);
+  BENCH_LDS(1, 0, 2); BENCH_LDS(1, 3, 2);
+  BENCH_LDS(2, 3, 0); BENCH_LDS(2, 3, 1);
+#undef BENCH_LDS
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
 
 // waves_per_simd (1..8) wavefronts on every SIMD of `cus` compute units, each issuing iters x 4
 // MFMAs of 32x32x16 (2*32*32*16 flop each); *flop receives the flop of the whole launch.
